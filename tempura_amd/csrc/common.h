@@ -1,0 +1,106 @@
+// Shared helpers of the gfx950 kernels: element types, reductions, error reporting.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#define TP_WAVE 64
+
+// Element type codes of the C interface.
+enum TpDtype { TP_F32 = 0, TP_BF16 = 1 };
+
+// bfloat16 as its 16 bits; conversions are explicit so rounding is in one place.
+struct bf16_t {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float bf16_to_float(bf16_t v) {
+  union {
+    uint32_t u;
+    float f;
+  } c;
+  c.u = ((uint32_t)v.bits) << 16;
+  return c.f;
+}
+
+// Round to nearest, ties to even; NaN stays NaN.
+__host__ __device__ inline bf16_t float_to_bf16(float f) {
+  union {
+    uint32_t u;
+    float f;
+  } c;
+  c.f = f;
+  bf16_t r;
+  if ((c.u & 0x7fffffffu) > 0x7f800000u) {
+    r.bits = (uint16_t)((c.u >> 16) | 0x0040u);
+    return r;
+  }
+  c.u += 0x7fffu + ((c.u >> 16) & 1u);
+  r.bits = (uint16_t)(c.u >> 16);
+  return r;
+}
+
+__device__ inline float to_float(float v) { return v; }
+__device__ inline float to_float(bf16_t v) { return bf16_to_float(v); }
+__device__ inline void from_float(float* p, float v) { *p = v; }
+__device__ inline void from_float(bf16_t* p, float v) { *p = float_to_bf16(v); }
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int o = TP_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TP_WAVE);
+  return v;
+}
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int o = TP_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, TP_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `scratch` is shared memory of at least 32 floats; safe to call repeatedly.
+__device__ inline float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  const int nwaves = (blockDim.x + TP_WAVE - 1) / TP_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nwaves; ++i) t += scratch[i];
+  return t;
+}
+
+__device__ inline float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  const int nwaves = (blockDim.x + TP_WAVE - 1) / TP_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = scratch[0];
+  for (int i = 1; i < nwaves; ++i) t = fmaxf(t, scratch[i]);
+  return t;
+}
+
+// ---- host-side error reporting ------------------------------------------------
+// Every entry point returns 0 on success; otherwise tp_last_error() says why.
+void tp_set_error(const char* fmt, ...);
+
+#define TP_REQUIRE(cond, ...)    \
+  do {                           \
+    if (!(cond)) {               \
+      tp_set_error(__VA_ARGS__); \
+      return 1;                  \
+    }                            \
+  } while (0)
+
+#define TP_CHECK_LAUNCH(name)                                          \
+  do {                                                                 \
+    hipError_t e_ = hipGetLastError();                                 \
+    if (e_ != hipSuccess) {                                            \
+      tp_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+      return 2;                                                        \
+    }                                                                  \
+  } while (0)

@@ -1,0 +1,209 @@
+// Memory-bound kernels of the step: embedding gather, RMSNorm, rotary + cache
+// write, SwiGLU.  Every kernel takes any size (no power-of-two assumptions).
+#include <stdarg.h>
+
+#include "common.h"
+
+static thread_local char g_error[512] = "";
+
+void tp_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* tp_last_error() { return g_error; }
+
+// ---- embedding ------------------------------------------------------------------
+// out[t, :] = table[token[t], :] widened to float32 (the residual stream).
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
+                             float* __restrict__ out, int hidden) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)tokens[t] * hidden;
+  float* o = out + (size_t)t * hidden;
+  for (int j = threadIdx.x; j < hidden; j += blockDim.x) o[j] = to_float(row[j]);
+}
+
+extern "C" int tp_embed(const int* tokens, const void* table, int table_dt, float* out, int n,
+                        int hidden, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && hidden > 0, "embed: bad sizes n=%d hidden=%d", n, hidden);
+  if (n == 0) return 0;
+  if (table_dt == TP_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(256), 0, s, tokens, (const float*)table, out, hidden);
+  else if (table_dt == TP_BF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(256), 0, s, tokens, (const bf16_t*)table, out, hidden);
+  else
+    TP_REQUIRE(false, "embed: unknown dtype %d", table_dt);
+  TP_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ---- RMSNorm ---------------------------------------------------------------------
+// y = x * (1 / sqrt(mean(x^2) + eps)) * w, all in float32; one block per output row.
+// `rows` (optional) picks the input row of each output row.
+template <typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               const int* __restrict__ rows, TO* __restrict__ out, int hidden, float eps) {
+  __shared__ float scratch[32];
+  const int r = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * hidden;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+    const float v = xr[j];
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+  TO* o = out + (size_t)r * hidden;
+  for (int j = threadIdx.x; j < hidden; j += blockDim.x) from_float(o + j, xr[j] * scale * w[j]);
+}
+
+extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void* out, int out_dt,
+                          int n_out, int hidden, float eps, hipStream_t s) {
+  TP_REQUIRE(n_out >= 0 && hidden > 0, "rmsnorm: bad sizes");
+  if (n_out == 0) return 0;
+  const int threads = hidden >= 2048 ? 1024 : (hidden >= 512 ? 256 : 64);
+  if (out_dt == TP_F32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n_out), dim3(threads), 0, s, x, w, rows, (float*)out, hidden, eps);
+  else if (out_dt == TP_BF16)
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(n_out), dim3(threads), 0, s, x, w, rows, (bf16_t*)out, hidden, eps);
+  else
+    TP_REQUIRE(false, "rmsnorm: unknown dtype %d", out_dt);
+  TP_CHECK_LAUNCH("rmsnorm");
+  return 0;
+}
+
+// ---- rotary position encoding + cache write -----------------------------------------
+// One block per token.  qkv row: [q heads | k heads | v heads] x head_dim, float32.
+// Pair (d, d + rotary_dim/2) of each q and k head turns by angle pos * inv_freq[d]; the
+// angle is formed in float64 from the integer position.  q goes to q_out, rotated k and raw
+// v go to the cache row `slots[t]` (page * page_size + offset) of the paged pools
+// [page, kv_head, page_size, head_dim].  With slots == nullptr only q is produced
+// (the row then holds q heads only).
+template <typename TQ, typename TC>
+__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stride,
+                                     const int* __restrict__ positions, const int* __restrict__ slots,
+                                     const double* __restrict__ inv_freq, int rotary_dim, float factor,
+                                     int n_heads, int n_kv, int head_dim, TQ* __restrict__ q_out,
+                                     TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size) {
+  extern __shared__ float cs[];  // cos[half], sin[half]
+  const int t = blockIdx.x;
+  const int half = rotary_dim / 2;
+  const double pos = (double)positions[t];
+  for (int d = threadIdx.x; d < half; d += blockDim.x) {
+    const double ang = pos * inv_freq[d];
+    cs[d] = (float)cos(ang) * factor;
+    cs[half + d] = (float)sin(ang) * factor;
+  }
+  __syncthreads();
+  const float* row = qkv + (size_t)t * row_stride;
+  const int rot_heads = n_heads + (slots ? n_kv : 0);
+  long slot = 0;
+  size_t page = 0, off = 0;
+  if (slots) {
+    slot = slots[t];
+    page = (size_t)(slot / page_size);
+    off = (size_t)(slot % page_size);
+  }
+  // rotated part of q and k heads
+  for (int i = threadIdx.x; i < rot_heads * half; i += blockDim.x) {
+    const int h = i / half, d = i % half;
+    const float x0 = row[h * head_dim + d], x1 = row[h * head_dim + d + half];
+    const float c = cs[d], sn = cs[half + d];
+    const float y0 = x0 * c - x1 * sn, y1 = x0 * sn + x1 * c;
+    if (h < n_heads) {
+      TQ* o = q_out + ((size_t)t * n_heads + h) * head_dim;
+      from_float(o + d, y0);
+      from_float(o + d + half, y1);
+    } else {
+      TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+      from_float(o + d, y0);
+      from_float(o + d + half, y1);
+    }
+  }
+  // elements past the rotary part pass through
+  const int tail = head_dim - rotary_dim;
+  if (tail > 0) {
+    for (int i = threadIdx.x; i < rot_heads * tail; i += blockDim.x) {
+      const int h = i / tail, d = rotary_dim + i % tail;
+      const float x = row[h * head_dim + d];
+      if (h < n_heads)
+        from_float(q_out + ((size_t)t * n_heads + h) * head_dim + d, x);
+      else
+        from_float(k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim + d, x);
+    }
+  }
+  if (slots) {
+    const float* vrow = row + (size_t)(n_heads + n_kv) * head_dim;
+    for (int i = threadIdx.x; i < n_kv * head_dim; i += blockDim.x) {
+      const int h = i / head_dim, d = i % head_dim;
+      from_float(v_cache + ((page * n_kv + h) * page_size + off) * head_dim + d, vrow[i]);
+    }
+  }
+}
+
+extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* positions, const int* slots,
+                                const double* inv_freq, int rotary_dim, float factor, int n, int n_heads,
+                                int n_kv, int head_dim, void* q_out, int q_dt, void* k_cache, void* v_cache,
+                                int cache_dt, int page_size, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && n_heads > 0 && n_kv >= 0 && head_dim > 0, "rope_kv_write: bad sizes");
+  TP_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim,
+             "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, head_dim);
+  TP_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope_kv_write: no frequency table");
+  TP_REQUIRE(slots == nullptr || (k_cache && v_cache && page_size > 0), "rope_kv_write: cache missing");
+  TP_REQUIRE(row_stride >= (n_heads + (slots ? 2 * n_kv : 0)) * head_dim, "rope_kv_write: row too short");
+  if (n == 0) return 0;
+  const size_t shmem = (size_t)(rotary_dim > 0 ? rotary_dim : 1) * sizeof(float);
+#define LAUNCH(TQ, TC)                                                                                   \
+  hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), dim3(n), dim3(256), shmem, s, qkv, row_stride,       \
+                     positions, slots, inv_freq, rotary_dim, factor, n_heads, n_kv, head_dim, (TQ*)q_out, \
+                     (TC*)k_cache, (TC*)v_cache, page_size)
+  if (q_dt == TP_F32 && cache_dt == TP_F32)
+    LAUNCH(float, float);
+  else if (q_dt == TP_BF16 && cache_dt == TP_BF16)
+    LAUNCH(bf16_t, bf16_t);
+  else if (q_dt == TP_F32 && cache_dt == TP_BF16)
+    LAUNCH(float, bf16_t);
+  else if (q_dt == TP_BF16 && cache_dt == TP_F32)
+    LAUNCH(bf16_t, float);
+  else
+    TP_REQUIRE(false, "rope_kv_write: unknown dtypes %d %d", q_dt, cache_dt);
+#undef LAUNCH
+  TP_CHECK_LAUNCH("rope_kv_write");
+  return 0;
+}
+
+// ---- SwiGLU --------------------------------------------------------------------------
+// out[m, i] = silu(gu[m, i]) * gu[m, I + i], silu(x) = x / (1 + exp(-x)).
+template <typename TI, typename TO>
+__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t m = idx / inter;
+  const int i = (int)(idx % inter);
+  const float g = to_float(gu[m * 2 * inter + i]);
+  const float u = to_float(gu[m * 2 * inter + inter + i]);
+  from_float(out + idx, g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int tp_swiglu(const void* gu, int in_dt, void* out, int out_dt, int m, int inter, hipStream_t s) {
+  TP_REQUIRE(m >= 0 && inter > 0, "swiglu: bad sizes");
+  if (m == 0) return 0;
+  const size_t total = (size_t)m * inter;
+  const dim3 grid((unsigned)((total + 255) / 256));
+#define LAUNCH(TI, TO) \
+  hipLaunchKernelGGL((swiglu_kernel<TI, TO>), grid, dim3(256), 0, s, (const TI*)gu, (TO*)out, inter, total)
+  if (in_dt == TP_F32 && out_dt == TP_F32)
+    LAUNCH(float, float);
+  else if (in_dt == TP_BF16 && out_dt == TP_BF16)
+    LAUNCH(bf16_t, bf16_t);
+  else if (in_dt == TP_F32 && out_dt == TP_BF16)
+    LAUNCH(float, bf16_t);
+  else
+    TP_REQUIRE(false, "swiglu: unsupported dtypes %d -> %d", in_dt, out_dt);
+#undef LAUNCH
+  TP_CHECK_LAUNCH("swiglu");
+  return 0;
+}

@@ -1,0 +1,174 @@
+// out[M, N] (+)= x[M, K] * w[N, K]^T with float32 accumulation.
+//
+// gemm_tiled_kernel is the general kernel: any M, N, K, float32 or bfloat16 operands,
+// plain FMA in float32 (no reduced-precision matrix mode), LDS-tiled 64x64x16 with a
+// 4x4 register block per thread.  The k loop runs in ascending order for every output
+// element, so a row's result does not depend on how many rows are in the batch.
+// bfloat16 products at model sizes go to the MFMA kernels in gemm_mfma.hip.
+#include "common.h"
+
+#define BM 64
+#define BN 64
+#define BK 16
+
+template <typename TI, typename TO, bool ACC>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const TI* __restrict__ x, const TI* __restrict__ w,
+                                                         TO* __restrict__ out, int M, int N, int K) {
+  __shared__ float xs[BK][BM + 4];
+  __shared__ float ws[BK][BN + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  // loader mapping: 64 rows x 16 k, four consecutive k per thread
+  const int lrow = tid / 4, lk = (tid % 4) * 4;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    {
+      const int gm = m0 + lrow;
+      const TI* p = x + (size_t)gm * K + k0 + lk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xs[lk + j][lrow] = (gm < M && k0 + lk + j < K) ? to_float(p[j]) : 0.f;
+      const int gn = n0 + lrow;
+      const TI* q = w + (size_t)gn * K + k0 + lk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ws[lk + j][lrow] = (gn < N && k0 + lk + j < K) ? to_float(q[j]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = xs[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ws[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gm = m0 + ty * 4 + i;
+    if (gm >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gn = n0 + tx * 4 + j;
+      if (gn >= N) continue;
+      TO* o = out + (size_t)gm * N + gn;
+      if (ACC)
+        from_float(o, to_float(*o) + acc[i][j]);
+      else
+        from_float(o, acc[i][j]);
+    }
+  }
+}
+
+// Skinny kernel for a handful of rows (decode): one wave per output column, lanes
+// stride over K, float32 FMA, wave reduction.  The x rows are staged in LDS in chunks.
+// Result per (row, column) is independent of the other rows in the batch.
+#define SK_COLS 16   // output columns per block (4 waves x 4 columns)
+#define SK_KC 512    // K chunk staged in LDS
+#define SK_MAXM 8
+
+template <typename TI, typename TO, bool ACC>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const TI* __restrict__ x, const TI* __restrict__ w,
+                                                          TO* __restrict__ out, int M, int N, int K) {
+  __shared__ float xs[SK_MAXM][SK_KC];
+  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  const int n_base = blockIdx.x * SK_COLS + wave * 4;
+  float acc[4][SK_MAXM];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int m = 0; m < SK_MAXM; ++m) acc[c][m] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += SK_KC) {
+    const int kc = min(SK_KC, K - k0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < M * SK_KC; i += blockDim.x) {
+      const int m = i / SK_KC, k = i % SK_KC;
+      xs[m][k] = (k < kc) ? to_float(x[(size_t)m * K + k0 + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int n = n_base + c;
+      if (n >= N) continue;
+      const TI* wr = w + (size_t)n * K + k0;
+      for (int k = lane; k < kc; k += TP_WAVE) {
+        const float wv = to_float(wr[k]);
+#pragma unroll
+        for (int m = 0; m < SK_MAXM; ++m)
+          if (m < M) acc[c][m] = fmaf(wv, xs[m][k], acc[c][m]);
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int n = n_base + c;
+#pragma unroll
+    for (int m = 0; m < SK_MAXM; ++m) {
+      const float v = wave_sum(acc[c][m]);
+      if (lane == 0 && n < N && m < M) {
+        TO* o = out + (size_t)m * N + n;
+        if (ACC)
+          from_float(o, to_float(*o) + v);
+        else
+          from_float(o, v);
+      }
+    }
+  }
+}
+
+template <typename TI, typename TO, bool ACC>
+static void launch_generic(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t s) {
+  if (M <= SK_MAXM) {
+    dim3 grid((N + SK_COLS - 1) / SK_COLS);
+    hipLaunchKernelGGL((gemm_skinny_kernel<TI, TO, ACC>), grid, dim3(256), 0, s, (const TI*)x, (const TI*)w,
+                       (TO*)out, M, N, K);
+  } else {
+    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+    hipLaunchKernelGGL((gemm_tiled_kernel<TI, TO, ACC>), grid, dim3(256), 0, s, (const TI*)x, (const TI*)w,
+                       (TO*)out, M, N, K);
+  }
+}
+
+// Defined in gemm_mfma.hip; returns 0 when it took the product, -1 when the sizes are
+// not its own (the general kernel then runs), >0 on error.
+int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
+                   hipStream_t s);
+
+extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
+                         int N, int K, int allow_mfma, hipStream_t s) {
+  TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
+  TP_REQUIRE(!accumulate || out_dt == TP_F32, "linear: accumulating output must be float32");
+  TP_REQUIRE((size_t)M * N < ((size_t)1 << 40), "linear: output too large");
+  if (M == 0) return 0;
+  if (in_dt == TP_BF16 && allow_mfma) {
+    const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, s);
+    if (r >= 0) return r;
+  }
+  if (in_dt == TP_F32 && out_dt == TP_F32) {
+    if (accumulate)
+      launch_generic<float, float, true>(x, w, out, M, N, K, s);
+    else
+      launch_generic<float, float, false>(x, w, out, M, N, K, s);
+  } else if (in_dt == TP_BF16 && out_dt == TP_F32) {
+    if (accumulate)
+      launch_generic<bf16_t, float, true>(x, w, out, M, N, K, s);
+    else
+      launch_generic<bf16_t, float, false>(x, w, out, M, N, K, s);
+  } else if (in_dt == TP_BF16 && out_dt == TP_BF16) {
+    launch_generic<bf16_t, bf16_t, false>(x, w, out, M, N, K, s);
+  } else {
+    TP_REQUIRE(false, "linear: unsupported dtypes in=%d out=%d", in_dt, out_dt);
+  }
+  TP_CHECK_LAUNCH("linear");
+  return 0;
+}

@@ -1,0 +1,50 @@
+"""From a model folder to a model on the device."""
+from __future__ import annotations
+
+import torch
+
+from ..config import load_config
+from ..weights.loader import load_into
+from ..weights.random_init import random_tensor
+from .model import CausalLM
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype must be bfloat16 or float32, got {dtype}")
+        return dtype
+    try:
+        return _DTYPES[str(dtype)]
+    except KeyError:
+        raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}") from None
+
+
+def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> CausalLM:
+    """Read ``config.json``, pick the architecture from the registry, build it, load its weights."""
+    config = load_config(model_dir)
+    model = CausalLM(config.build_spec(), parse_dtype(dtype), torch.device(device))
+    model.config = config
+    load_into(model, model_dir)
+    return model
+
+
+def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: float = 0.02,
+                 norm_jitter: float = 0.0) -> CausalLM:
+    """A model with seeded random weights made tensor by tensor, never written to disk
+    (for sizes whose folder would be tens of gigabytes)."""
+    td = parse_dtype(dtype)
+    model = CausalLM(config.build_spec(), td, torch.device(device))
+    model.config = config
+    expected = model.expected_weights()
+
+    def get(name, optional=False):
+        info = expected[name]
+        if info.init == "skip":
+            return None
+        return random_tensor(name, info, seed, std, norm_jitter, torch.bfloat16 if td == torch.bfloat16 else torch.float32)
+
+    model.load_weights(get)
+    return model

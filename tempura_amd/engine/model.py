@@ -1,0 +1,124 @@
+"""The decoder built from a ``ModelSpec``: embedding, blocks in their run order,
+final norm and output head.
+
+The forward pass follows the reference's order
+(/root/reference/engine/src/model.rs:643-1399): gather embeddings, run each
+layer on the float32 residual stream, normalise and project.  Unlike the
+reference, which projects the last row only (model.rs:1389-1396), logits are
+produced at every requested row of the batch.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, List, Optional, Tuple
+
+import torch
+
+from ..config.spec import ModelSpec
+from ..parts.base import CacheSpec, StateSpec, WeightInfo, build_part, part_class
+
+
+def expected_weights(spec: ModelSpec) -> Dict[str, WeightInfo]:
+    """Every checkpoint tensor the model reads, by name (no device needed)."""
+    out: Dict[str, WeightInfo] = {}
+    out.update(part_class("embedding", spec.embedding.kind).expected_weights(
+        spec.embedding, spec.hidden_size, spec.vocab_size))
+    for ls in spec.layers:
+        out.update(part_class("block", ls.block).expected_weights(ls, spec.hidden_size))
+    out.update(part_class("norm", spec.final_norm.kind).expected_weights(spec.final_norm, spec.hidden_size))
+    out.update(part_class("lm_head", spec.lm_head.kind).expected_weights(
+        spec.lm_head, spec.hidden_size, spec.vocab_size))
+    return out
+
+
+class CausalLM:
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"compute dtype must be bfloat16 or float32, got {dtype}")
+        self.spec = spec
+        self.dtype = dtype
+        self.device = device
+        h = spec.hidden_size
+        self.embedding = part_class("embedding", spec.embedding.kind)(spec.embedding, h, dtype, device, spec.vocab_size)
+        self.layers = [part_class("block", ls.block)(ls, h, dtype, device) for ls in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm, h, dtype, device)
+        self.lm_head = part_class("lm_head", spec.lm_head.kind)(spec.lm_head, h, dtype, device, spec.vocab_size)
+        self.order = spec.resolved_order()
+        self._plan_caches()
+
+    # ---- caches --------------------------------------------------------
+    def _plan_caches(self) -> None:
+        """Group cache slots by what their mixers need."""
+        n_slots = 1 + max((c.cache for c in self.order), default=-1)
+        owner: List[Optional[int]] = [None] * n_slots     # order index of the call that writes the slot
+        self.call_writes: List[bool] = []
+        for i, call in enumerate(self.order):
+            if owner[call.cache] is None:
+                owner[call.cache] = i
+                self.call_writes.append(True)
+            else:
+                self.call_writes.append(False)
+        self.cache_groups: List[CacheSpec] = []
+        self.slot_group: List[Tuple[int, int]] = []        # slot -> (group, index within group)
+        self.state_specs: Dict[int, StateSpec] = {}
+        counts: List[int] = []
+        for slot in range(n_slots):
+            mixer = self.layers[self.order[owner[slot]].layer].mixer
+            cs = mixer.cache_spec()
+            if cs is None:
+                self.slot_group.append((-1, 0))
+            else:
+                if cs not in self.cache_groups:
+                    self.cache_groups.append(cs)
+                    counts.append(0)
+                g = self.cache_groups.index(cs)
+                self.slot_group.append((g, counts[g]))
+                counts[g] += 1
+            ss = mixer.state_spec()
+            if ss is not None:
+                self.state_specs[slot] = ss
+        self.slots_per_group = counts
+        for i, call in enumerate(self.order):
+            if not self.call_writes[i]:
+                mine = self.layers[call.layer].mixer.cache_spec()
+                theirs = self.layers[self.order[owner[call.cache]].layer].mixer.cache_spec()
+                if mine != theirs:
+                    raise ValueError(f"run order entry {i} reads cache slot {call.cache} whose layout differs from its own")
+
+    # ---- weights -------------------------------------------------------
+    def expected_weights(self) -> Dict[str, WeightInfo]:
+        return expected_weights(self.spec)
+
+    def load_weights(self, get: Callable) -> None:
+        self.embedding.load_weights(get)
+        for layer in self.layers:
+            layer.load_weights(get)
+        self.final_norm.load_weights(get)
+        self.lm_head.load_weights(get, self.embedding)
+
+    def weight_bytes(self, include_embedding: bool = True) -> int:
+        seen, total = set(), 0
+
+        def add(t):
+            nonlocal total
+            if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+        objs = [self.final_norm, self.lm_head]
+        if include_embedding:
+            objs.append(self.embedding)
+        for layer in self.layers:
+            objs.extend(layer.parts())
+        for o in objs:
+            for v in vars(o).values():
+                add(v)
+        return total
+
+    # ---- forward -------------------------------------------------------
+    def forward(self, tokens: torch.Tensor, ctx, caches) -> torch.Tensor:
+        """``tokens`` int32 [n]; ``caches[i]`` is the ``LayerCache`` of run-order entry i.
+        Returns float32 logits [len(ctx.logit_rows), vocab]."""
+        h = self.embedding.forward(tokens)
+        for i, call in enumerate(self.order):
+            self.layers[call.layer].forward(h, ctx, caches[i])
+        x = self.final_norm.forward(h, ctx.logit_rows)
+        return self.lm_head.forward(x)

@@ -1,0 +1,212 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A batch may hold portions of prompts beside single decoded tokens, cut anywhere.
+Only the tokens given are run; everything earlier comes from the cache pages that
+earlier steps wrote.  The reference has three disjoint calls instead (one
+sequence of n tokens, or m sequences of exactly one token,
+/root/reference/engine/src/model.rs:305-448) and never mixes them in a forward
+(/root/reference/server/src/engine_task.rs:748-778).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, CachePools, LayerCache, PagesExhausted
+from .model import CausalLM
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens and the places (indices into
+    ``tokens``) whose logits are wanted."""
+
+    rid: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class StepContext:
+    """Everything a part may read about the batch.  Device tensors are int32.
+
+    positions[n]      absolute position of each token in its request
+    token_req[n]      index (row of this batch) of the request each token belongs to
+    cu_seqlens[r+1]   where each request's tokens start in the flattened batch
+    context_lens[r]   tokens of the request in the cache once this step is written
+    block_tables[g]   [r, width] logical page -> physical page, per cache group
+    slot_mapping[g]   [n] physical cache row (page * page_size + offset) of each new token
+    state_slots[r]    row of the per-request state tensors
+    logit_rows[m]     flattened token indices whose logits are returned
+    Host copies (``q_starts``, ``q_lens``, ``ctx_lens``, ``state_slot_list``) serve parts
+    that loop over requests on the host.
+    """
+
+    def __init__(self):
+        self.num_tokens = 0
+        self.num_requests = 0
+        self.positions = None
+        self.token_req = None
+        self.cu_seqlens = None
+        self.context_lens = None
+        self.block_tables: List[torch.Tensor] = []
+        self.slot_mapping: List[torch.Tensor] = []
+        self.state_slots = None
+        self.logit_rows = None
+        self.max_q_len = 0
+        self.max_context_len = 0
+        self.page_size = 0
+        self.q_starts: List[int] = []
+        self.q_lens: List[int] = []
+        self.ctx_lens: List[int] = []
+        self.state_slot_list: List[int] = []
+
+
+class ModelRunner:
+    def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
+                 cache_dtype: Optional[torch.dtype] = None):
+        self.model = model
+        self.device = model.device
+        self.page_size = int(page_size)
+        n_groups = len(model.cache_groups)
+        if isinstance(num_pages, int):
+            num_pages = [num_pages] * n_groups
+        self.cache = CacheManager(model.cache_groups, self.page_size, list(num_pages), max_requests)
+        self.pools = CachePools(model.cache_groups, model.slots_per_group, self.page_size, list(num_pages),
+                                cache_dtype or model.dtype, self.device, model.state_specs, max_requests)
+        self.layer_caches: List[LayerCache] = []
+        for i, call in enumerate(model.order):
+            g, idx = model.slot_group[call.cache]
+            k = v = None
+            if g >= 0:
+                k = self.pools.kv[g][idx, 0]
+                v = self.pools.kv[g][idx, 1]
+            self.layer_caches.append(LayerCache(g, k, v, model.call_writes[i], self.page_size,
+                                                self.pools.state.get(call.cache)))
+        self.steps_run = 0
+        self.tokens_run = 0
+
+    # ---- request lifetime ---------------------------------------------
+    def has_request(self, rid) -> bool:
+        return self.cache.has(rid)
+
+    def add_request(self, rid) -> None:
+        self.cache.add(rid)
+
+    def end_request(self, rid) -> None:
+        self.cache.release(rid)
+
+    def num_cached(self, rid) -> int:
+        return self.cache.num_tokens(rid)
+
+    # ---- the step ------------------------------------------------------
+    def _check_entries(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        seen = set()
+        vocab = self.model.spec.vocab_size
+        for e in entries:
+            if e.rid in seen:
+                raise ValueError(f"request {e.rid!r} appears twice in one step")
+            seen.add(e.rid)
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.rid!r}: a step entry needs at least one token")
+            for t in e.tokens:
+                if t < 0 or t >= vocab:
+                    raise ValueError(f"request {e.rid!r}: token id {t} outside the vocabulary of {vocab}")
+            for w in e.want:
+                if w < 0 or w >= len(e.tokens):
+                    raise ValueError(f"request {e.rid!r}: wanted place {w} outside its {len(e.tokens)} tokens")
+            if not self.cache.has(e.rid):
+                raise ValueError(f"request {e.rid!r} is not live; add_request first")
+            end = self.cache.num_tokens(e.rid) + len(e.tokens)
+            if end > self.model.spec.max_positions:
+                raise ValueError(f"request {e.rid!r}: {end} tokens exceed max positions {self.model.spec.max_positions}")
+
+    def reserve(self, entries: Sequence[StepEntry]) -> None:
+        """Pages for every entry, or ``PagesExhausted`` with nothing changed."""
+        n_groups = len(self.cache.groups)
+        total = [0] * n_groups
+        for e in entries:
+            for g, n in enumerate(self.cache.pages_needed(e.rid, len(e.tokens))):
+                total[g] += n
+        free = self.cache.free_pages()
+        for g in range(n_groups):
+            if total[g] > free[g]:
+                raise PagesExhausted(total[g], free[g], g)
+        for e in entries:
+            self.cache.reserve(e.rid, len(e.tokens))
+
+    def build_context(self, entries: Sequence[StepEntry]):
+        """Host side of a step: flatten the batch and describe it (pages must be reserved)."""
+        n_groups = len(self.cache.groups)
+        R = len(entries)
+        q_lens = [len(e.tokens) for e in entries]
+        starts = [self.cache.num_tokens(e.rid) for e in entries]
+        N = sum(q_lens)
+        cu = np.zeros(R + 1, dtype=np.int32)
+        cu[1:] = np.cumsum(q_lens)
+        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+        positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, q_lens)])
+        token_req = np.repeat(np.arange(R, dtype=np.int32), q_lens)
+        ctx_lens = np.asarray([s + n for s, n in zip(starts, q_lens)], dtype=np.int32)
+        state_slots = np.asarray([self.cache.state_slot(e.rid) for e in entries], dtype=np.int32)
+        rows: List[int] = []
+        for r, e in enumerate(entries):
+            rows.extend(int(cu[r]) + int(w) for w in e.want)
+        logit_rows = np.asarray(rows, dtype=np.int32)
+        tables, slots = [], []
+        for g in range(n_groups):
+            width = max(1, max(len(self.cache.table(e.rid, g)) for e in entries))
+            bt = np.full((R, width), self.pools.scratch_page(g), dtype=np.int32)
+            for r, e in enumerate(entries):
+                t = np.asarray(self.cache.table(e.rid, g), dtype=np.int32)
+                # Pages a window has given back stay pointed at the scratch page; no query reads them.
+                bt[r, : len(t)] = np.where(t >= 0, t, self.pools.scratch_page(g))
+            tables.append(bt)
+            slots.append(np.concatenate([self.cache.slots(e.rid, g, s, n)
+                                         for e, s, n in zip(entries, starts, q_lens)]).astype(np.int32))
+
+        # One packed host buffer, one copy to the device, then views.
+        pieces = [tokens, positions, token_req, cu, ctx_lens, state_slots, logit_rows] + \
+                 [t.reshape(-1) for t in tables] + slots
+        offs = np.cumsum([0] + [p.size for p in pieces])
+        packed = torch.from_numpy(np.concatenate(pieces)).to(self.device)
+        view = [packed[offs[i]: offs[i + 1]] for i in range(len(pieces))]
+
+        ctx = StepContext()
+        ctx.num_tokens, ctx.num_requests = N, R
+        tok_dev, ctx.positions, ctx.token_req, ctx.cu_seqlens, ctx.context_lens, ctx.state_slots, ctx.logit_rows = view[:7]
+        ctx.block_tables = [view[7 + g].view(R, tables[g].shape[1]) for g in range(n_groups)]
+        ctx.slot_mapping = view[7 + n_groups: 7 + 2 * n_groups]
+        ctx.max_q_len = max(q_lens)
+        ctx.max_context_len = int(ctx_lens.max())
+        ctx.page_size = self.page_size
+        ctx.q_starts = [int(c) for c in cu[:-1]]
+        ctx.q_lens = q_lens
+        ctx.ctx_lens = [int(c) for c in ctx_lens]
+        ctx.state_slot_list = [int(s) for s in state_slots]
+        return tok_dev, ctx, starts
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the batch; returns float32 logits [sum of wanted places, vocab] on the device,
+        ordered by entry and then by ``want``."""
+        entries = list(entries)
+        self._check_entries(entries)
+        self.reserve(entries)
+        tok_dev, ctx, starts = self.build_context(entries)
+        # A request that starts at position 0 gets a cleared state (also after a recompute).
+        if self.pools.state:
+            fresh = [ctx.state_slot_list[r] for r, s in enumerate(starts) if s == 0]
+            if fresh:
+                idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
+                for t in self.pools.state.values():
+                    t.index_fill_(0, idx, 0)
+        logits = self.model.forward(tok_dev, ctx, self.layer_caches)
+        for e in entries:
+            self.cache.commit(e.rid, len(e.tokens))
+        self.steps_run += 1
+        self.tokens_run += ctx.num_tokens
+        return logits

@@ -1,0 +1,248 @@
+"""The operations the parts are written against, bound to the gfx950 kernel library.
+
+Every function checks shapes, dtypes, contiguity and device on the host before a
+kernel is launched (a kernel never sees an operand it was not written for), then
+calls the library's C entry point on the current stream.  There is no CPU path:
+without the compiled library or without a GPU the first call raises.
+
+Tests may install another backend with ``set_backend`` (an object with the same
+functions) to exercise the engine's bookkeeping on the host; nothing in the
+product does.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+_F32, _BF16 = 0, 1
+_backend = None
+
+
+def set_backend(backend) -> None:
+    """Install an object providing this module's functions (tests only); None restores the library."""
+    global _backend
+    _backend = backend
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+class _Library:
+    """The compiled kernel library, loaded on first use."""
+
+    _lib = None
+
+    @classmethod
+    def get(cls):
+        if cls._lib is None:
+            if not torch.cuda.is_available():
+                raise KernelError("tempura_amd needs a GPU: torch.cuda.is_available() is False and there is no CPU path")
+            from ..csrc.build import ensure_built
+            path = ensure_built()
+            try:
+                lib = ctypes.CDLL(path)
+            except OSError as e:
+                raise KernelError(f"cannot load the kernel library {path}: {e}") from e
+            lib.tp_last_error.restype = ctypes.c_char_p
+            cls._lib = lib
+            cls.path = path
+        return cls._lib
+
+
+def library():
+    return _Library.get()
+
+
+def _call(name: str, *args) -> None:
+    lib = _Library.get()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise KernelError(f"{name}: {lib.tp_last_error().decode()}")
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return _F32
+    if t.dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError(f"unsupported dtype {t.dtype}")
+
+
+def _dtcode(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _F32
+    if dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError(f"unsupported dtype {dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev_ok(*ts) -> None:
+    for t in ts:
+        if t is not None:
+            _need(t.is_cuda, "operand is not on the GPU")
+            _need(t.is_contiguous(), "operand is not contiguous")
+
+
+def _i32(t: torch.Tensor, n: int, what: str) -> None:
+    _need(t.dtype == torch.int32 and t.numel() >= n and t.dim() >= 1, f"{what}: need int32 with {n} elements")
+
+
+# ---------------------------------------------------------------------------------
+def embed(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """int32 [n] , [vocab, hidden] -> float32 [n, hidden]."""
+    if _backend is not None:
+        return _backend.embed(tokens, table)
+    _dev_ok(tokens, table)
+    n = tokens.numel()
+    _i32(tokens, n, "embed tokens")
+    _need(table.dim() == 2, "embed: table must be [vocab, hidden]")
+    out = torch.empty((n, table.shape[1]), dtype=torch.float32, device=table.device)
+    _call("tp_embed", _ptr(tokens), _ptr(table), _dt(table), _ptr(out), n, table.shape[1], _stream())
+    return out
+
+
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [n, hidden] -> out_dtype [n or len(rows), hidden]."""
+    if _backend is not None:
+        return _backend.rmsnorm(h, weight, eps, out_dtype, rows)
+    _dev_ok(h, weight, rows)
+    _need(h.dtype == torch.float32 and h.dim() == 2, "rmsnorm: input must be float32 [n, hidden]")
+    _need(weight.dtype == torch.float32 and weight.numel() == h.shape[1], "rmsnorm: weight must be float32 [hidden]")
+    n_out = h.shape[0]
+    if rows is not None:
+        n_out = rows.numel()
+        _i32(rows, n_out, "rmsnorm rows") if n_out else None
+    out = torch.empty((n_out, h.shape[1]), dtype=out_dtype, device=h.device)
+    _call("tp_rmsnorm", _ptr(h), _ptr(weight), _ptr(rows), _ptr(out), _dtcode(out_dtype), n_out, h.shape[1],
+          ctypes.c_float(eps), _stream())
+    return out
+
+
+#: bfloat16 products may use the matrix-core kernels (tests switch this off to grade the general kernel)
+allow_mfma = True
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
+           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [m, k] @ w[n, k]^T -> out_dtype [m, n]; with ``residual`` (float32 [m, n]) the product is
+    added into it in place and it is returned."""
+    if _backend is not None:
+        return _backend.linear(x, w, out_dtype, residual)
+    _dev_ok(x, w, residual)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
+    _need(x.dtype == w.dtype, f"linear: operand dtypes differ ({x.dtype}, {w.dtype})")
+    m, k = x.shape
+    n = w.shape[0]
+    if residual is not None:
+        _need(residual.dtype == torch.float32 and tuple(residual.shape) == (m, n), "linear: residual must be float32 [m, n]")
+        out, acc = residual, 1
+    else:
+        out, acc = torch.empty((m, n), dtype=out_dtype, device=x.device), 0
+    _call("tp_linear", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _stream())
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                  inv_freq: Optional[torch.Tensor], rotary_dim: int, factor: float, num_heads: int,
+                  num_kv_heads: int, head_dim: int, k_cache: Optional[torch.Tensor],
+                  v_cache: Optional[torch.Tensor], q_dtype: torch.dtype) -> torch.Tensor:
+    """Rotate q and k of float32 rows [n, (heads + 2 kv_heads) * head_dim], store k and v into the
+    cache rows ``slots`` and return q as q_dtype [n, heads, head_dim].  With ``slots`` None the rows
+    hold q only and nothing is stored."""
+    if _backend is not None:
+        return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,
+                                      num_kv_heads, head_dim, k_cache, v_cache, q_dtype)
+    _dev_ok(qkv, positions, slots, inv_freq, k_cache, v_cache)
+    _need(qkv.dtype == torch.float32 and qkv.dim() == 2, "rope_kv_write: rows must be float32 [n, width]")
+    n = qkv.shape[0]
+    width = (num_heads + (2 * num_kv_heads if slots is not None else 0)) * head_dim
+    _need(qkv.shape[1] == width, f"rope_kv_write: row width {qkv.shape[1]} != {width}")
+    _i32(positions, n, "positions") if n else None
+    page_size, cache_dt = 1, _F32
+    if slots is not None:
+        _i32(slots, n, "slots") if n else None
+        _need(k_cache is not None and v_cache is not None and k_cache.shape == v_cache.shape and k_cache.dim() == 4,
+              "rope_kv_write: caches must be [pages, kv_heads, page_size, head_dim]")
+        _need(k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim, "rope_kv_write: cache layout mismatch")
+        _need(k_cache.dtype == v_cache.dtype, "rope_kv_write: cache dtypes differ")
+        page_size, cache_dt = k_cache.shape[2], _dt(k_cache)
+    if rotary_dim:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float64 and inv_freq.numel() == rotary_dim // 2,
+              "rope_kv_write: inv_freq must be float64 [rotary_dim / 2]")
+    q = torch.empty((n, num_heads, head_dim), dtype=q_dtype, device=qkv.device)
+    _call("tp_rope_kv_write", _ptr(qkv), qkv.shape[1], _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
+          ctypes.c_float(factor), n, num_heads, num_kv_heads, head_dim, _ptr(q), _dtcode(q_dtype),
+          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, _stream())
+    return q
+
+
+#: bfloat16 attention may use the matrix-core kernels
+allow_fast_attention = True
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                    cu_seqlens: torch.Tensor, context_lens: torch.Tensor, token_req: torch.Tensor,
+                    scale: float, window: int, max_q_len: int, max_context_len: int) -> torch.Tensor:
+    """q [n, heads, head_dim] over caches [pages, kv_heads, page_size, head_dim] -> [n, heads * head_dim]."""
+    if _backend is not None:
+        return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
+                                        token_req, scale, window, max_q_len, max_context_len)
+    _dev_ok(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens, token_req)
+    _need(q.dim() == 3 and k_cache.dim() == 4 and k_cache.shape == v_cache.shape, "paged_attention: bad operand ranks")
+    n, heads, d = q.shape
+    pages, kvh, page_size, d2 = k_cache.shape
+    _need(d == d2, "paged_attention: head_dim of q and cache differ")
+    _need(q.dtype == k_cache.dtype == v_cache.dtype, "paged_attention: q and cache dtypes differ")
+    _need(block_tables.dim() == 2 and block_tables.dtype == torch.int32, "paged_attention: block_tables must be int32 [r, width]")
+    r, width = block_tables.shape
+    _i32(cu_seqlens, r + 1, "cu_seqlens")
+    _i32(context_lens, r, "context_lens")
+    _i32(token_req, n, "token_req") if n else None
+    _need(pages * kvh * page_size < 2 ** 31, "paged_attention: cache pool too large for 32-bit row indices")
+    _need(max_context_len <= width * page_size, "paged_attention: block table narrower than the longest context")
+    out = torch.empty((n, heads * d), dtype=q.dtype, device=q.device)
+    _call("tp_paged_attention", _ptr(q), _dt(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), width,
+          _ptr(cu_seqlens), _ptr(context_lens), _ptr(token_req), _ptr(out), n, r, heads, kvh, d, page_size,
+          ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(allow_fast_attention),
+          _stream())
+    return out
+
+
+def swiglu(gu: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """[m, 2i] (gate columns then up columns) -> out_dtype [m, i]."""
+    if _backend is not None:
+        return _backend.swiglu(gu, out_dtype)
+    _dev_ok(gu)
+    _need(gu.dim() == 2 and gu.shape[1] % 2 == 0, "swiglu: input must be [m, 2i]")
+    m, i2 = gu.shape
+    out = torch.empty((m, i2 // 2), dtype=out_dtype, device=gu.device)
+    _call("tp_swiglu", _ptr(gu), _dt(gu), _ptr(out), _dtcode(out_dtype), m, i2 // 2, _stream())
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """float32 [m, vocab] -> int32 [m]; the last maximum wins on exact ties."""
+    if _backend is not None:
+        return _backend.argmax(logits)
+    _dev_ok(logits)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "argmax: logits must be float32 [m, vocab]")
+    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    _call("tp_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
+    return out

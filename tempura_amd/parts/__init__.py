@@ -1,0 +1,6 @@
+from .base import (Part, Mixer, FeedForward, Norm, PositionEncoding, Block, CacheSpec, StateSpec,
+                   WeightInfo, register_part, part_class, build_part)
+from . import norm, rope, attention, ffn, block, embedding  # noqa: F401  (register the built-in parts)
+
+__all__ = ["Part", "Mixer", "FeedForward", "Norm", "PositionEncoding", "Block", "CacheSpec",
+           "StateSpec", "WeightInfo", "register_part", "part_class", "build_part"]

@@ -1,0 +1,88 @@
+"""Grouped-query attention over the paged cache.
+
+Per token: q, k, v projections (no bias), position encoding on q and k, k and v
+stored into the cache pages, causal (optionally windowed) softmax attention
+over the request's cached keys with ``kv_head = head // (heads / kv_heads)``,
+output projection added into the residual stream
+(/root/reference/engine/src/model.rs:1007-1152,
+/root/reference/kernels/src/attention.rs:28-87).
+A window of ``w`` lets query position p see keys p-w+1 .. p
+(/root/reference/kernels/src/attention.rs:55-59).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import CacheSpec, Mixer, WeightInfo, build_part, register_part
+
+
+class PagedAttention(Mixer):
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        p = spec.params
+        self.num_heads = int(p["num_heads"])
+        self.num_kv_heads = int(p["num_kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        if self.num_heads % self.num_kv_heads != 0:
+            raise ValueError("attention: heads must be a multiple of kv heads")
+        self.scale = float(p["scale"])
+        self.window = p.get("window")
+        self.q_dim = self.num_heads * self.head_dim
+        self.kv_dim = self.num_kv_heads * self.head_dim
+        self.position = build_part("position", p["position"], hidden_size, dtype, device)
+        self.wqkv = None
+        self.wo = None
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        p, w = spec.params, spec.weights
+        q_dim = p["num_heads"] * p["head_dim"]
+        kv_dim = p["num_kv_heads"] * p["head_dim"]
+        return {
+            w["q"]: WeightInfo((q_dim, hidden_size)),
+            w["k"]: WeightInfo((kv_dim, hidden_size)),
+            w["v"]: WeightInfo((kv_dim, hidden_size)),
+            w["o"]: WeightInfo((hidden_size, q_dim)),
+        }
+
+    def load_weights(self, get):
+        w = self.spec.weights
+        # One [q_dim + 2 kv_dim, hidden] matrix: one product instead of three.
+        parts = [get(w["q"]), get(w["k"]), get(w["v"])]
+        self.wqkv = torch.cat([self._to_device(t) for t in parts], dim=0).contiguous()
+        self.wo = self._to_device(get(w["o"]))
+
+    def cache_spec(self):
+        kind = "window" if self.window is not None else "full"
+        return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, ctx, cache, residual):
+        rot = self.position.rotary()
+        if cache.writes:
+            qkv = ops.linear(x, self.wqkv, torch.float32)
+        else:
+            # A call that reads another call's cache needs queries only.
+            qkv = ops.linear(x, self.wqkv[: self.q_dim], torch.float32)
+        if rot is None:
+            q = qkv[:, : self.q_dim]
+            k = qkv[:, self.q_dim: self.q_dim + self.kv_dim] if cache.writes else None
+            q2, k2 = self.position.apply(q, k, ctx.positions)
+            if cache.writes:
+                qkv = torch.cat([q2, k2, qkv[:, self.q_dim + self.kv_dim:]], dim=1).contiguous()
+            else:
+                qkv = q2.contiguous()
+            inv_freq, rotary_dim, factor = None, 0, 1.0
+        else:
+            inv_freq, rotary_dim, factor = rot
+        q = ops.rope_kv_write(
+            qkv, ctx.positions, ctx.slot_mapping[cache.group] if cache.writes else None,
+            inv_freq, rotary_dim, factor, self.num_heads, self.num_kv_heads, self.head_dim,
+            cache.k if cache.writes else None, cache.v if cache.writes else None, self.dtype)
+        a = ops.paged_attention(
+            q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
+            ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len)
+        ops.linear(a, self.wo, torch.float32, residual=residual)
+
+
+register_part("mixer", "attention", PagedAttention)
