@@ -1,0 +1,140 @@
+"""Shared pieces of the tests: tiny configurations, model folders, step schedules."""
+from __future__ import annotations
+
+import os
+import random
+from typing import Dict, List, Sequence, Tuple
+
+import torch
+
+import plain
+from tempura_amd.config import LlamaConfig, RopeScaling
+from tempura_amd.weights import write_random_model
+
+# Two tiny configurations that differ in every size and option, plus a windowed one.
+# A: groups of 2, head size 16, untied, plain rope.
+# B: one kv head (MQA), head size 12 (no power of two, no multiple of 8), hidden 96, vocabulary
+#    384, tied, llama3 scaling whose original length (64) is passed so all three branches are hit.
+# C: head size 48, 6 heads in 3 groups, hidden 80 (!= heads * head size), a window of 24 on
+#    alternating layers, vocabulary 300.
+CONFIGS: Dict[str, LlamaConfig] = {
+    "A": LlamaConfig(hidden_size=64, intermediate_size=192, num_hidden_layers=2, num_attention_heads=4,
+                     num_key_value_heads=2, head_dim=16, vocab_size=256, max_position_embeddings=2048,
+                     rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=False),
+    "B": LlamaConfig(hidden_size=96, intermediate_size=320, num_hidden_layers=3, num_attention_heads=8,
+                     num_key_value_heads=1, head_dim=12, vocab_size=384, max_position_embeddings=1024,
+                     rms_norm_eps=1e-6, rope_theta=500000.0,
+                     rope_scaling=RopeScaling("llama3", 8.0, 1.0, 4.0, 64), tie_word_embeddings=True),
+    "C": LlamaConfig(hidden_size=80, intermediate_size=136, num_hidden_layers=4, num_attention_heads=6,
+                     num_key_value_heads=3, head_dim=48, vocab_size=300, max_position_embeddings=512,
+                     rms_norm_eps=3e-6, rope_theta=25000.0,
+                     rope_scaling=RopeScaling("llama3", 4.0, 1.0, 2.0, 32), tie_word_embeddings=False,
+                     sliding_window=24,
+                     layer_types=["sliding_attention", "full_attention", "sliding_attention", "full_attention"]),
+}
+#: weights are N(0, STD): large enough that attention is peaked and faults show
+STD = 0.15
+
+
+class TinyModels:
+    def __init__(self, root):
+        self.root = str(root)
+        self._made = {}
+
+    def path(self, name: str, dtype: str = "float32") -> str:
+        key = (name, dtype)
+        if key not in self._made:
+            d = os.path.join(self.root, f"{name}_{dtype}")
+            cfg = LlamaConfig.from_dict(CONFIGS[name].to_dict())
+            write_random_model(cfg, d, seed={"A": 11, "B": 23, "C": 37}[name], std=STD, norm_jitter=0.2, dtype=dtype)
+            self._made[key] = d
+        return self._made[key]
+
+    def plain_model(self, name: str, dtype: str = "float32"):
+        return plain.read_model_dir(self.path(name, dtype))
+
+
+def random_tokens(vocab: int, n: int, seed: int) -> List[int]:
+    g = random.Random(seed)
+    return [g.randrange(vocab) for _ in range(n)]
+
+
+def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """Largest difference relative to the largest reference logit."""
+    return float((got.double() - ref.double()).abs().max() / ref.double().abs().max().clamp_min(1e-30))
+
+
+#: bounds on rel_err against the plain float64 implementation
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+# ---- step schedules ---------------------------------------------------------------------------
+# A schedule is a list of steps; a step is (entries, end) with entries = [(rid, start, count)].
+def roundup(n: int, m: int) -> int:
+    return (n + m - 1) // m * m
+
+
+def schedule_whole(lengths: Dict[str, int]):
+    return [([(rid, 0, n)], [rid]) for rid, n in lengths.items()]
+
+
+def schedule_bulk_tail(lengths: Dict[str, int], tail: int = 32):
+    steps = []
+    for rid, n in lengths.items():
+        t = min(tail, n - 1) if n > 1 else 0
+        if n - t > 0:
+            steps.append(([(rid, 0, n - t)], []))
+        for i in range(n - t, n):
+            steps.append(([(rid, i, 1)], []))
+        steps[-1] = (steps[-1][0], [rid])
+    return steps
+
+
+def schedule_portions(lengths: Dict[str, int], sizes=(7, 2, 16, 3, 2, 31, 5, 2, 64, 9, 2, 17)):
+    steps = []
+    k = 0
+    for rid, n in lengths.items():
+        i = 0
+        while i < n:
+            c = min(sizes[k % len(sizes)], n - i)
+            k += 1
+            steps.append(([(rid, i, c)], []))
+            i += c
+        steps[-1] = (steps[-1][0], [rid])
+    return steps
+
+
+def schedule_mixed(lengths: Dict[str, int], max_tokens: int, seed: int, max_live: int = 4):
+    """Up to ``max_live`` requests at a time, portions of some beside single tokens of others;
+    a request is admitted only while the live ones (each rounded up to 64) fit ``max_tokens``."""
+    g = random.Random(seed)
+    waiting = list(lengths.items())
+    live: Dict[str, int] = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, n = waiting[0]
+            held = sum(roundup(lengths[r], 64) for r in live)
+            if held + roundup(n, 64) > max_tokens:
+                break
+            live[rid] = 0
+            waiting.pop(0)
+        assert live, "max_tokens too small for the next request"
+        entries, end = [], []
+        for rid in list(live):
+            done, n = live[rid], lengths[rid]
+            if len(live) > 1 and g.random() < 0.2:
+                continue                      # left out of this step, goes on later
+            rest = n - done
+            if rest > 32:
+                c = min(g.choice([2, 3, 5, 8, 13, 16, 17, 31, 40]), rest - 32)
+            else:
+                c = 1                         # the tail is decoded token by token
+            entries.append((rid, done, c))
+            live[rid] = done + c
+            if live[rid] == n:
+                end.append(rid)
+                del live[rid]
+        if entries:
+            steps.append((entries, end))
+    return steps

@@ -1,0 +1,186 @@
+"""Each HIP kernel alone against its plain PyTorch reference (tests/emu_ops.py), at sizes other
+than the engine's: widths and vocabularies that are no power of two, odd head counts and groups,
+head sizes in steps of 16 and below, ragged batches, shuffled pages."""
+import math
+
+import pytest
+import torch
+
+from emu_ops import EmuOps
+
+pytestmark = pytest.mark.gpu
+emu = EmuOps()
+DEV = "cuda:0"
+
+
+def _ops():
+    from tempura_amd.kernels import ops
+    ops.set_backend(None)
+    return ops
+
+
+def _close(got, ref, tol, what=""):
+    err = float((got.double().cpu() - ref.double()).abs().max())
+    scale = float(ref.double().abs().max()) or 1.0
+    assert err <= tol * scale, f"{what}: max error {err:.3e} against scale {scale:.3e} (tol {tol})"
+
+
+def _tol(dtype):
+    return 1e-5 if dtype == torch.float32 else 1.2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,hidden,vocab", [(1, 64, 256), (7, 100, 301), (33, 4096, 1000)])
+def test_embed(dtype, n, hidden, vocab):
+    ops = _ops()
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(vocab, hidden, generator=g).to(dtype)
+    tok = torch.randint(0, vocab, (n,), generator=g, dtype=torch.int32)
+    got = ops.embed(tok.to(DEV), table.to(DEV))
+    assert torch.equal(got.cpu(), emu.embed(tok, table))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,hidden,eps", [(1, 16, 1e-5), (4, 64, 1e-6), (8, 256, 1e-5), (3, 100, 1e-2), (5, 4096, 1e-5), (2, 5000, 1e-6)])
+def test_rmsnorm(out_dtype, n, hidden, eps):
+    ops = _ops()
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(n, hidden, generator=g) * 3
+    x[0] *= 1e-3                                  # a near-zero row: eps placement matters
+    w = 1 + 0.3 * torch.randn(hidden, generator=g)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, out_dtype)
+    _close(got, emu.rmsnorm(x, w, eps, torch.float64), _tol(out_dtype), "rmsnorm")
+    rows = torch.tensor([n - 1, 0], dtype=torch.int32)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, out_dtype, rows.to(DEV))
+    _close(got, emu.rmsnorm(x, w, eps, torch.float64, rows), _tol(out_dtype), "rmsnorm rows")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(1, 16, 8), (4, 32, 16), (8, 64, 64), (1, 1024, 512), (3, 96, 320), (9, 12, 96),
+                                   (17, 100, 36), (64, 384, 96), (65, 130, 70), (130, 257, 129), (2, 301, 1000)])
+def test_linear(dtype, m, n, k):
+    ops = _ops()
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    w = torch.randn(n, k, generator=g).to(dtype)
+    ref = x.double() @ w.double().T
+    for out_dtype in ([torch.float32] if dtype == torch.float32 else [torch.float32, torch.bfloat16]):
+        got = ops.linear(x.to(DEV), w.to(DEV), out_dtype)
+        _close(got, ref, 1e-5 if out_dtype == torch.float32 else 1e-2, f"linear {out_dtype}")
+    res = torch.randn(m, n, generator=g)
+    got = ops.linear(x.to(DEV), w.to(DEV), torch.float32, residual=res.clone().to(DEV))
+    _close(got, ref + res.double(), 1e-5, "linear residual")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv,d,rot,page", [(4, 2, 16, 16, 16), (8, 1, 12, 12, 8), (6, 3, 48, 48, 32), (3, 3, 80, 32, 4), (32, 8, 128, 128, 16)])
+def test_rope_kv_write(dtype, heads, kv, d, rot, page):
+    ops = _ops()
+    from tempura_amd.parts.rope import rotary_inv_freq
+    g = torch.Generator().manual_seed(4)
+    n, pages = 19, 7
+    qkv = torch.randn(n, (heads + 2 * kv) * d, generator=g)
+    pos = torch.randint(0, 100000, (n,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(pages * page, generator=g)[:n].to(torch.int32)
+    inv = rotary_inv_freq(d, 500000.0, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                        "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}, rot)
+    kc = torch.zeros(pages, kv, page, d, dtype=dtype)
+    vc = torch.zeros_like(kc)
+    kr, vr = kc.clone(), vc.clone()
+    qr = emu.rope_kv_write(qkv, pos, slots, inv, rot, 1.0, heads, kv, d, kr, vr, torch.float64)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    q = ops.rope_kv_write(qkv.to(DEV), pos.to(DEV), slots.to(DEV), inv.to(DEV), rot, 1.0, heads, kv, d, kd, vd, dtype)
+    tol = 2e-6 if dtype == torch.float32 else 8e-3
+    _close(q, qr, tol, "q")
+    _close(kd, kr, tol, "k cache")
+    _close(vd, vr, tol, "v cache")
+    # queries only (a call that reads another call's cache)
+    q2 = ops.rope_kv_write(qkv[:, : heads * d].contiguous().to(DEV), pos.to(DEV), None, inv.to(DEV), rot, 1.0,
+                           heads, kv, d, None, None, dtype)
+    assert torch.equal(q2, q)
+
+
+def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, allow_fast=True):
+    ops = _ops()
+    g = torch.Generator().manual_seed(seed)
+    R = len(q_lens)
+    n = sum(q_lens)
+    pages_needed = sum((c + page - 1) // page for c in ctx_lens)
+    pages = pages_needed + 3
+    perm = torch.randperm(pages, generator=g).tolist()            # shuffled, non-monotonic tables
+    width = max((c + page - 1) // page for c in ctx_lens) + 1
+    bt = torch.full((R, width), perm[-1], dtype=torch.int32)
+    it = iter(perm)
+    for r, c in enumerate(ctx_lens):
+        for i in range((c + page - 1) // page):
+            bt[r, i] = next(it)
+    kc = (torch.randn(pages, kv, page, d, generator=g) * 1.5).to(dtype)
+    vc = torch.randn(pages, kv, page, d, generator=g).to(dtype)
+    q = (torch.randn(n, heads, d, generator=g) * 1.5).to(dtype)
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    cl = torch.tensor(ctx_lens, dtype=torch.int32)
+    tr = torch.repeat_interleave(torch.arange(R, dtype=torch.int32), torch.tensor(q_lens))
+    scale = 1.0 / math.sqrt(d)
+    ref = emu.paged_attention(q, kc, vc, bt, cu, cl, tr, scale, window, max(q_lens), max(ctx_lens)).double()
+    ops.allow_fast_attention = allow_fast
+    try:
+        got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), cu.to(DEV), cl.to(DEV), tr.to(DEV),
+                                  scale, window, max(q_lens), max(ctx_lens))
+    finally:
+        ops.allow_fast_attention = True
+    _close(got, ref, 2e-5 if dtype == torch.float32 else 1.2e-2, f"attention h{heads} kv{kv} d{d} page{page}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv,d,page", [(4, 4, 8, 4), (8, 2, 16, 16), (4, 4, 32, 8), (8, 1, 12, 8), (6, 3, 48, 32), (5, 5, 80, 16), (32, 8, 128, 16), (3, 1, 256, 64)])
+def test_attention_general(dtype, heads, kv, d, page):
+    # ragged: a whole prompt, a portion after a cached prefix, single decoded tokens, a one-token request
+    _attention_case(dtype, heads, kv, d, page, [37, 9, 1, 1, 1], [37, 64, 33, 130, 1], 0, seed=5, allow_fast=False)
+    _attention_case(dtype, heads, kv, d, page, [20, 1, 6], [50, 77, 6], 13, seed=6, allow_fast=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_far_key_stands_out(dtype):
+    """One far key among hundreds carries the whole answer: scale one query/key pair so its score dominates."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(7)
+    heads, kv, d, page, ctx = 4, 2, 64, 16, 700
+    pages = (ctx + page - 1) // page
+    kc = torch.randn(pages, kv, page, d, generator=g) * 0.1
+    vc = torch.randn(pages, kv, page, d, generator=g)
+    q = torch.randn(1, heads, d, generator=g) * 0.1
+    far = 3                                                 # a key in the first page
+    kc[far // page, :, far % page] = q[0, ::2] * 400.0      # aligned with the query of each group's first head
+    bt = torch.arange(pages, dtype=torch.int32)[None]
+    cu = torch.tensor([0, 1], dtype=torch.int32)
+    cl = torch.tensor([ctx], dtype=torch.int32)
+    tr = torch.zeros(1, dtype=torch.int32)
+    kc, vc, q = kc.to(dtype), vc.to(dtype), q.to(dtype)
+    ref = emu.paged_attention(q, kc, vc, bt, cu, cl, tr, 1.0, 0, 1, ctx).double()
+    got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), cu.to(DEV), cl.to(DEV), tr.to(DEV), 1.0, 0, 1, ctx)
+    _close(got, ref, 2e-5 if dtype == torch.float32 else 1.2e-2, "far key")
+    # the answer of heads 0 and 2 is (almost) the far key's value row
+    assert float((ref.reshape(heads, d)[0] - vc[far // page, 0, far % page].double()).abs().max()) < 0.05
+
+
+@pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("m,inter", [(1, 192), (7, 320), (3, 137), (64, 14336)])
+def test_swiglu(in_dtype, out_dtype, m, inter):
+    ops = _ops()
+    g = torch.Generator().manual_seed(8)
+    gu = (torch.randn(m, 2 * inter, generator=g) * 4).to(in_dtype)
+    gu[0, :4] = torch.tensor([0.0, 80.0, -80.0, 1e4]).to(in_dtype)
+    got = ops.swiglu(gu.to(DEV), out_dtype)
+    assert torch.isfinite(got.float()).all()
+    _close(got, emu.swiglu(gu, torch.float64), _tol(out_dtype), "swiglu")
+
+
+@pytest.mark.parametrize("m,vocab", [(1, 256), (5, 301), (3, 128256)])
+def test_argmax_last_max_wins(m, vocab):
+    ops = _ops()
+    g = torch.Generator().manual_seed(9)
+    lg = torch.randn(m, vocab, generator=g)
+    lg[0, 7] = lg[0, vocab - 3] = 50.0                      # an exact tie: the later index wins
+    got = ops.argmax(lg.to(DEV)).cpu()
+    assert torch.equal(got, emu.argmax(lg))
+    assert int(got[0]) == vocab - 3
