@@ -45,3 +45,303 @@ extern "C" int tp_argmax(const float* logits, int* out, int rows, int vocab, hip
   TP_CHECK_LAUNCH("argmax");
   return 0;
 }
+
+// ---- penalties ----------------------------------------------------------------------
+// entries: (row, token, count, in_window).  Presence/frequency penalties subtract
+// frequency * count + presence (/root/reference/kernel-api/src/lib.rs:292-308); the
+// repetition penalty multiplies non-positive logits and divides positive ones
+// (/root/reference/kernels/src/sampler_chain.rs:222-246).  The reference applies
+// presence/frequency to the raw logits and the repetition penalty after the temperature;
+// dividing by a positive temperature keeps signs, so applying it to the raw logits and
+// scaling afterwards gives the same values.
+__global__ void penalties_kernel(float* __restrict__ logits, int vocab, const int* __restrict__ rows,
+                                 const int* __restrict__ tokens, const int* __restrict__ counts,
+                                 const int* __restrict__ in_window, const float* __restrict__ presence,
+                                 const float* __restrict__ frequency, const float* __restrict__ repeat, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int r = rows[i], tok = tokens[i];
+  if (tok < 0 || tok >= vocab) return;
+  float* p = logits + (size_t)r * vocab + tok;
+  float v = *p;
+  if (counts[i] > 0) v -= frequency[r] * (float)counts[i] + presence[r];
+  if (in_window[i] && repeat[r] != 1.0f) v = (v <= 0.f) ? v * repeat[r] : v / repeat[r];
+  *p = v;
+}
+
+extern "C" int tp_apply_penalties(float* logits, int vocab, const int* rows, const int* tokens, const int* counts,
+                                  const int* in_window, const float* presence, const float* frequency,
+                                  const float* repeat, int n, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && vocab > 0, "apply_penalties: bad sizes");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(penalties_kernel, dim3((n + 255) / 256), dim3(256), 0, s, logits, vocab, rows, tokens, counts,
+                     in_window, presence, frequency, repeat, n);
+  TP_CHECK_LAUNCH("apply_penalties");
+  return 0;
+}
+
+// ---- filtered sampling ----------------------------------------------------------------
+// One block of 1024 threads per row:
+//   x = logit / temperature; drop x < max + ln(min_p); keep the top_k largest; softmax;
+//   keep the shortest prefix (by descending probability) whose mass reaches top_p;
+//   renormalise; walk the survivors in INDEX order and return the first index whose
+//   cumulative mass exceeds r (/root/reference/kernels/src/sampling.rs:229-333).
+// There is no sort: the k-th largest value and the top-p cut are found by radix selection
+// over the order-preserving integer image of the floats (4 passes of 8 bits), counting
+// elements for top-k and probability mass for top-p.  Mass is summed as 40-bit fixed point
+// integers, so every sum is exact and independent of the order of additions: the same row,
+// parameters and r always give the same token.  Ties at a cut are admitted in index order.
+// temperature == 0 returns the argmax (last maximum wins).
+#define SMP_THREADS 1024
+#define SMP_WAVES (SMP_THREADS / TP_WAVE)
+#define SMP_FIX 1099511627776.0f  // 2^40
+
+__device__ inline unsigned int float_key(float f) {
+  const unsigned int u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ inline unsigned long long fix_mass(float x, float maxv) {
+  return (unsigned long long)(expf(x - maxv) * SMP_FIX);
+}
+
+// Exclusive prefix sum over the block in thread order; *total gets the block's sum.
+__device__ inline unsigned long long block_excl_scan(unsigned long long v, unsigned long long* lds,
+                                                     unsigned long long* total) {
+  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  unsigned long long inc = v;
+#pragma unroll
+  for (int o = 1; o < TP_WAVE; o <<= 1) {
+    const unsigned long long t = __shfl_up(inc, o, TP_WAVE);
+    if (lane >= o) inc += t;
+  }
+  __syncthreads();
+  if (lane == TP_WAVE - 1) lds[wave] = inc;
+  __syncthreads();
+  unsigned long long base = 0, tot = 0;
+  for (int i = 0; i < SMP_WAVES; ++i) {
+    const unsigned long long w = lds[i];
+    if (i < wave) base += w;
+    tot += w;
+  }
+  *total = tot;
+  return base + inc - v;
+}
+
+// Radix selection from the top: finds the key K such that weight(key > K) < target <=
+// weight(key >= K), where an element's weight is 1 (MASS = false) or its fixed-point mass.
+// Only elements with key >= floor_key take part.  Returns K; *gt = weight(key > K),
+// *eq_count = number of elements with key == K.
+template <bool MASS>
+__device__ unsigned int radix_select(const float* __restrict__ x, int n, float maxv, unsigned int floor_key,
+                                     unsigned long long target, unsigned long long* hist /*256*/,
+                                     unsigned int* cnt /*256*/, unsigned long long* sh /*4*/,
+                                     unsigned long long* gt_out, unsigned int* eq_count) {
+  unsigned int prefix = 0;
+  unsigned long long gt = 0;
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    __syncthreads();
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) {
+      hist[i] = 0;
+      cnt[i] = 0;
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < n; j += blockDim.x) {
+      const float v = x[j];
+      const unsigned int key = float_key(v);
+      if (key < floor_key) continue;
+      if (pass > 0 && (key >> (shift + 8)) != prefix) continue;
+      const unsigned int bin = (key >> shift) & 255u;
+      atomicAdd(&cnt[bin], 1u);
+      if (MASS)
+        atomicAdd(&hist[bin], fix_mass(v, maxv));
+      else
+        atomicAdd(&hist[bin], 1ull);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long run = gt;
+      int b = 255;
+      for (; b > 0; --b) {
+        if (run + hist[b] >= target) break;
+        run += hist[b];
+      }
+      sh[0] = run;
+      sh[1] = (unsigned long long)b;
+      sh[2] = (unsigned long long)cnt[b];
+    }
+    __syncthreads();
+    gt = sh[0];
+    prefix = (prefix << 8) | (unsigned int)sh[1];
+  }
+  *gt_out = gt;
+  *eq_count = (unsigned int)sh[2];
+  return prefix;
+}
+
+// Keep only the first `quota` elements (index order) among those with key == K: the others
+// become -inf.  Threads own contiguous index ranges so that ranks follow the index.
+__device__ void drop_surplus_ties(float* __restrict__ x, int n, unsigned int K, unsigned long long quota,
+                                  unsigned long long* lds) {
+  const int per = (n + SMP_THREADS - 1) / SMP_THREADS;
+  const int lo = min(n, (int)threadIdx.x * per), hi = min(n, lo + per);
+  unsigned long long mine = 0;
+  for (int j = lo; j < hi; ++j) mine += (float_key(x[j]) == K) ? 1ull : 0ull;
+  unsigned long long total;
+  unsigned long long rank = block_excl_scan(mine, lds, &total);
+  for (int j = lo; j < hi; ++j) {
+    if (float_key(x[j]) == K) {
+      if (rank >= quota) x[j] = -INFINITY;
+      ++rank;
+    }
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
+    const float* __restrict__ logits, float* __restrict__ work, int vocab, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
+    const float* __restrict__ rnd, int* __restrict__ out) {
+  __shared__ unsigned long long hist[256];
+  __shared__ unsigned int cnt[256];
+  __shared__ unsigned long long sh[4];
+  __shared__ unsigned long long scan[SMP_WAVES];
+  __shared__ float fscratch[32];
+  __shared__ int ibest[SMP_WAVES];
+  __shared__ float vbest[SMP_WAVES];
+  const int row = blockIdx.x;
+  const float* lg = logits + (size_t)row * vocab;
+  float* x = work + (size_t)row * vocab;
+  const float T = temperature[row];
+
+  if (!(T > 0.f)) {  // greedy: argmax, last maximum wins
+    float bv = -INFINITY;
+    int bi = -1;
+    for (int j = threadIdx.x; j < vocab; j += blockDim.x) argmax_merge(bv, bi, lg[j], j);
+    for (int o = TP_WAVE / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, TP_WAVE);
+      const int oi = __shfl_xor(bi, o, TP_WAVE);
+      argmax_merge(bv, bi, ov, oi);
+    }
+    if (threadIdx.x % TP_WAVE == 0) {
+      vbest[threadIdx.x / TP_WAVE] = bv;
+      ibest[threadIdx.x / TP_WAVE] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int i = 1; i < SMP_WAVES; ++i) argmax_merge(bv, bi, vbest[i], ibest[i]);
+      out[row] = bi < 0 ? vocab - 1 : bi;
+    }
+    return;
+  }
+
+  // 1. scale by the temperature, find the maximum
+  float mx = -INFINITY;
+  for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
+    float v = lg[j];
+    if (T != 1.0f) v = v / T;
+    if (!(v == v)) v = -INFINITY;  // NaN never survives
+    x[j] = v;
+    mx = fmaxf(mx, v);
+  }
+  const float maxv = block_max(mx, fscratch);
+  __syncthreads();
+  if (maxv == -INFINITY) {  // nothing to choose from: the reference falls through to the last index
+    if (threadIdx.x == 0) out[row] = vocab - 1;
+    return;
+  }
+
+  // 2. min_p: drop x < max + ln(min_p)
+  unsigned int floor_key = float_key(-INFINITY) + 1u;  // everything finite
+  const float mp = min_p[row];
+  if (mp > 0.f) {
+    const float thr = maxv + logf(mp);
+    const unsigned int k2 = float_key(thr);
+    if (k2 > floor_key) floor_key = k2;
+  }
+
+  // 3. top_k: the k-th largest value among the survivors
+  const int k = top_k[row];
+  if (k > 0 && k < vocab) {
+    unsigned long long gt;
+    unsigned int eq;
+    const unsigned int K = radix_select<false>(x, vocab, maxv, floor_key, (unsigned long long)k, hist, cnt, sh, &gt, &eq);
+    // fewer than k survivors: K lands on the smallest surviving bin and nothing is cut
+    if (gt + eq > (unsigned long long)k) drop_surplus_ties(x, vocab, K, (unsigned long long)k - gt, scan);
+    if (K > floor_key) floor_key = K;
+  }
+
+  // 4. total mass of the survivors
+  unsigned long long part = 0;
+  for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
+    const float v = x[j];
+    if (float_key(v) >= floor_key) part += fix_mass(v, maxv);
+  }
+  unsigned long long Z;
+  block_excl_scan(part, scan, &Z);
+
+  // 5. top_p: the shortest prefix by descending probability whose mass reaches top_p
+  const float tp = top_p[row];
+  if (tp < 1.0f && tp > 0.f) {
+    unsigned long long target = (unsigned long long)((double)tp * (double)Z);
+    if (target < 1) target = 1;
+    unsigned long long gt;
+    unsigned int eq;
+    const unsigned int K = radix_select<true>(x, vocab, maxv, floor_key, target, hist, cnt, sh, &gt, &eq);
+    // each tie at K has the same mass q; take as many as the target still needs
+    float kv;
+    {
+      const unsigned int u = (K & 0x80000000u) ? (K & 0x7fffffffu) : ~K;
+      kv = __uint_as_float(u);
+    }
+    const unsigned long long q = fix_mass(kv, maxv);
+    unsigned long long need = 1;
+    if (q > 0 && target > gt) need = (target - gt + q - 1) / q;
+    if (need < 1) need = 1;
+    if ((unsigned long long)eq > need) drop_surplus_ties(x, vocab, K, need, scan);
+    if (K > floor_key) floor_key = K;
+    Z = gt + (need < (unsigned long long)eq ? need : (unsigned long long)eq) * q;
+  }
+
+  // 6. draw: first index (index order) whose cumulative mass exceeds r * Z
+  const float r = rnd[row];
+  unsigned long long t = (unsigned long long)((double)r * (double)Z);
+  if (t >= Z) t = Z - 1;
+  const int per = (vocab + SMP_THREADS - 1) / SMP_THREADS;
+  const int lo = min(vocab, (int)threadIdx.x * per), hi = min(vocab, lo + per);
+  unsigned long long mine = 0;
+  for (int j = lo; j < hi; ++j) {
+    const float v = x[j];
+    if (float_key(v) >= floor_key) mine += fix_mass(v, maxv);
+  }
+  unsigned long long total;
+  unsigned long long base = block_excl_scan(mine, scan, &total);
+  if (threadIdx.x == 0 && total == 0) out[row] = vocab - 1;
+  if (mine > 0 && base <= t && t < base + mine) {
+    unsigned long long c = base;
+    int pick = hi - 1;
+    for (int j = lo; j < hi; ++j) {
+      const float v = x[j];
+      if (float_key(v) >= floor_key) {
+        c += fix_mass(v, maxv);
+        if (c > t) {
+          pick = j;
+          break;
+        }
+      }
+    }
+    out[row] = pick;
+  }
+}
+
+extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
+                         const int* top_k, const float* top_p, const float* min_p, const float* rnd, int* out,
+                         hipStream_t s) {
+  TP_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, work, vocab, temperature, top_k,
+                     top_p, min_p, rnd, out);
+  TP_CHECK_LAUNCH("sample");
+  return 0;
+}

@@ -1,0 +1,161 @@
+"""The Python entry point: a model folder (or a configuration with random weights) to tokens.
+
+Shaped after the reference's ``InferenceModel`` (``forward``, ``generate``,
+/root/reference/engine/src/model.rs:305-448) and its serving loop
+(/root/reference/server/src/engine_task.rs:581-875), with option names taken from the
+reference's ``ServeArgs`` where it has them (``max_batch_size``, ``max_seq_len``,
+/root/reference/server/src/lib.rs:45-110).
+"""
+from __future__ import annotations
+
+import itertools
+import time
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple, Union
+
+import torch
+
+from ..config import load_config
+from ..sampling import Sampler, SamplingParams
+from .loading import load_model, parse_dtype, random_model
+from .model import CausalLM
+from .runner import ModelRunner, StepEntry
+from .scheduler import Request, RequestState, Scheduler, SchedulerConfig
+
+
+class Engine:
+    def __init__(self, model: Union[str, object], dtype: str = "bfloat16", random_weights: bool = False,
+                 seed: int = 0, page_size: int = 16, kv_pages: Optional[int] = None,
+                 gpu_memory_utilization: float = 0.9, max_batch_size: int = 64,
+                 max_seq_len: Optional[int] = None, max_num_batched_tokens: int = 2048,
+                 prefill_chunk_size: int = 512, device: str = "cuda:0", use_graph: bool = True):
+        """``model``: a folder with config.json and safetensors, or (with ``random_weights``) a typed
+        configuration such as ``LlamaConfig``/``PRESETS[name]``.
+        ``kv_pages``: cache pages per group; by default as many as ``gpu_memory_utilization`` of the
+        free memory holds, but no more than ``max_batch_size`` requests of ``max_seq_len`` need."""
+        self.device = torch.device(device)
+        if isinstance(model, str):
+            if random_weights:
+                self.model = random_model(load_config(model), seed, dtype, device)
+            else:
+                self.model = load_model(model, dtype, device)
+        elif isinstance(model, CausalLM):
+            self.model = model
+        else:
+            if not random_weights:
+                raise ValueError("a configuration without a folder needs random_weights=True")
+            self.model = random_model(model, seed, dtype, device)
+        spec = self.model.spec
+        self.max_seq_len = min(int(max_seq_len or spec.max_positions), spec.max_positions)
+        self.page_size = int(page_size)
+        if kv_pages is None:
+            kv_pages = self._pages_from_memory(gpu_memory_utilization, max_batch_size)
+        self.runner = ModelRunner(self.model, self.page_size, int(kv_pages), max_requests=max_batch_size,
+                                  use_graph=use_graph)
+        self.scheduler = Scheduler(
+            SchedulerConfig(max_num_seqs=max_batch_size, max_num_batched_tokens=max_num_batched_tokens,
+                            prefill_chunk_size=prefill_chunk_size, max_model_len=self.max_seq_len),
+            self.runner.cache)
+        self.sampler = Sampler(spec.vocab_size, self.device, default_seed=seed)
+        self._ids = itertools.count()
+        self._requests: Dict[Hashable, Request] = {}
+        self.counters = {"steps": 0, "prompt_tokens": 0, "generated_tokens": 0, "batched_tokens": 0}
+
+    def _pages_from_memory(self, utilization: float, max_batch_size: int) -> int:
+        m = self.model
+        elem = 2 if m.dtype == torch.bfloat16 else 4
+        per_page = sum(n * 2 * g.num_kv_heads * self.page_size * g.head_dim * elem
+                       for g, n in zip(m.cache_groups, m.slots_per_group)) or 1
+        pages_cap = max_batch_size * ((self.max_seq_len + self.page_size - 1) // self.page_size)
+        if self.device.type != "cuda":
+            return pages_cap
+        free, _total = torch.cuda.mem_get_info(self.device)
+        workspace = 2 << 30            # activations of the largest step, logits, sampler scratch
+        budget = int(free * utilization) - workspace
+        return max(1, min(pages_cap, budget // per_page))
+
+    # ---- requests ------------------------------------------------------------
+    def add_request(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
+                    rid: Optional[Hashable] = None) -> Hashable:
+        params = params or SamplingParams()
+        if rid is None:
+            rid = next(self._ids)
+        if rid in self._requests and self._requests[rid].state != RequestState.FINISHED:
+            raise ValueError(f"request id {rid!r} is in use")
+        vocab = self.model.spec.vocab_size
+        for t in prompt_ids:
+            if t < 0 or t >= vocab:
+                raise ValueError(f"token id {t} outside the vocabulary of {vocab}")
+        eos = params.eos_token_id if params.eos_token_id is not None else self.model.spec.eos_token_ids
+        req = Request(rid, [int(t) for t in prompt_ids], params, tuple(int(e) for e in eos))
+        self.scheduler.add_request(req)
+        self._requests[rid] = req
+        self.counters["prompt_tokens"] += len(req.prompt)
+        return rid
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    def step(self) -> List[Tuple[Hashable, int, bool]]:
+        """One scheduler decision, one model step, one sampling pass.
+        Returns (request id, new token, finished) for every request that got a token."""
+        items = self.scheduler.schedule()
+        if not items:
+            return []
+        entries = []
+        for it in items:
+            toks = it.request.tokens[it.start: it.start + it.count]
+            entries.append(StepEntry(it.request.rid, toks, [it.count - 1] if it.samples else []))
+        logits = self.runner.step(entries)
+        self.counters["steps"] += 1
+        self.counters["batched_tokens"] += sum(it.count for it in items)
+        for it in items:
+            self.scheduler.advance(it)
+        sampling = [it.request for it in items if it.samples]
+        out: List[Tuple[Hashable, int, bool]] = []
+        if sampling:
+            tokens = self.sampler.sample(
+                logits, [r.params for r in sampling], [len(r.output) for r in sampling],
+                [r.prompt for r in sampling], [r.output for r in sampling])
+            for req, tok in zip(sampling, tokens):
+                done = self.scheduler.append_token(req, tok)
+                self.counters["generated_tokens"] += 1
+                if done:
+                    self.scheduler.finish(req)
+                out.append((req.rid, int(tok), done))
+        return out
+
+    def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None
+                 ) -> List[List[int]]:
+        """Generate for every prompt (token ids in, token ids out); continuous batching inside."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt")
+        rids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        while self.has_unfinished():
+            self.step()
+        return [list(self._requests[r].output) for r in rids]
+
+    def forward(self, token_ids: Sequence[int]) -> torch.Tensor:
+        """Logits [vocab] (float32, host) after a whole prompt of a fresh request
+        (the reference's ``forward``, /root/reference/engine/src/model.rs:308)."""
+        rid = ("forward", next(self._ids))
+        self.runner.add_request(rid)
+        try:
+            logits = self.runner.step([StepEntry(rid, list(token_ids), [len(token_ids) - 1])])
+        finally:
+            self.runner.end_request(rid)
+        return logits[0].cpu()
+
+    def request(self, rid) -> Request:
+        return self._requests[rid]
+
+    def stats(self) -> Dict[str, object]:
+        s = dict(self.counters)
+        s["preemptions"] = self.scheduler.num_preemptions
+        s["pages_high_water"] = list(self.scheduler.pages_high_water)
+        s["pages_total"] = [p.num_pages for p in self.runner.cache.pools]
+        s["cache_bytes"] = self.runner.pools.bytes()
+        s["weight_bytes"] = self.model.weight_bytes()
+        s["graph_steps"] = self.runner.graph_steps
+        return s

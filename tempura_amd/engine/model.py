@@ -15,19 +15,7 @@ import torch
 
 from ..config.spec import ModelSpec
 from ..parts.base import CacheSpec, StateSpec, WeightInfo, build_part, part_class
-
-
-def expected_weights(spec: ModelSpec) -> Dict[str, WeightInfo]:
-    """Every checkpoint tensor the model reads, by name (no device needed)."""
-    out: Dict[str, WeightInfo] = {}
-    out.update(part_class("embedding", spec.embedding.kind).expected_weights(
-        spec.embedding, spec.hidden_size, spec.vocab_size))
-    for ls in spec.layers:
-        out.update(part_class("block", ls.block).expected_weights(ls, spec.hidden_size))
-    out.update(part_class("norm", spec.final_norm.kind).expected_weights(spec.final_norm, spec.hidden_size))
-    out.update(part_class("lm_head", spec.lm_head.kind).expected_weights(
-        spec.lm_head, spec.hidden_size, spec.vocab_size))
-    return out
+from ..parts.inventory import expected_weights
 
 
 class CausalLM:

@@ -66,7 +66,7 @@ class StepContext:
 
 class ModelRunner:
     def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
-                 cache_dtype: Optional[torch.dtype] = None):
+                 cache_dtype: Optional[torch.dtype] = None, use_graph: bool = False):
         self.model = model
         self.device = model.device
         self.page_size = int(page_size)
@@ -87,6 +87,8 @@ class ModelRunner:
                                                 self.pools.state.get(call.cache)))
         self.steps_run = 0
         self.tokens_run = 0
+        self.use_graph = use_graph
+        self.graph_steps = 0
 
     # ---- request lifetime ---------------------------------------------
     def has_request(self, rid) -> bool:

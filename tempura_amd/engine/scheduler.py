@@ -1,0 +1,218 @@
+"""Continuous batching above the step function: admit, cut prompts into portions under
+a token budget, decode, finish and free.
+
+Every step is ONE mixed batch: first one token for every decoding request, then prompt
+portions in admission order while the token budget lasts.  The reference instead runs one
+512-token chunk per prefilling session per tick, each its own forward, and then one batched
+decode (/root/reference/server/src/engine_task.rs:748-778; chunk size engine_task.rs:11,
+queues and states /root/reference/server/src/batch.rs:13-56).
+
+When pages run out the most recently admitted running request is preempted: its pages are
+given back and it returns to the FRONT of the waiting queue with prompt + output so far as its
+new prompt (recompute; the reference requeues preempted work first, batch.rs:137-142,214-229,
+and otherwise swaps a victim out to host memory, engine_task.rs:261-289 — there is no host
+tier here).  Its sampler draws are indexed by output length, so its continuation is unchanged.
+A request that could never fit the pool alone is refused when it is added.
+
+This module is host logic only; it needs a cache manager's bookkeeping, no GPU.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from enum import Enum
+from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
+
+from ..cache import CacheManager
+from ..sampling.params import SamplingParams
+
+
+class RequestState(Enum):
+    WAITING = "waiting"
+    RUNNING = "running"
+    FINISHED = "finished"
+
+
+@dataclass
+class Request:
+    rid: Hashable
+    prompt: List[int]
+    params: SamplingParams
+    eos_token_ids: Tuple[int, ...] = ()
+    output: List[int] = field(default_factory=list)
+    state: RequestState = RequestState.WAITING
+    num_computed: int = 0            # tokens of prompt + output whose keys/values are cached
+    preemptions: int = 0
+    finish_reason: Optional[str] = None
+    arrival: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def num_tokens(self) -> int:
+        return len(self.prompt) + len(self.output)
+
+    @property
+    def is_decoding(self) -> bool:
+        """Only the newest token is not yet cached."""
+        return self.num_tokens - self.num_computed == 1 and len(self.output) > 0
+
+
+@dataclass
+class SchedulerConfig:
+    max_num_seqs: int = 64                  # the reference's --max-batch-size (server/src/lib.rs:45-110)
+    max_num_batched_tokens: int = 2048      # token budget of one step
+    prefill_chunk_size: int = 512           # largest prompt portion (engine_task.rs:11)
+    max_model_len: int = 4096               # the reference's --max-seq-len
+
+
+@dataclass
+class ScheduledItem:
+    request: Request
+    start: int          # first position run in this step
+    count: int          # tokens run in this step
+    samples: bool       # the step reaches the request's newest token: a token is sampled
+
+
+class Scheduler:
+    def __init__(self, config: SchedulerConfig, cache: CacheManager):
+        if config.max_num_batched_tokens < 1 or config.prefill_chunk_size < 1 or config.max_num_seqs < 1:
+            raise ValueError("scheduler limits must be positive")
+        self.config = config
+        self.cache = cache
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []      # in admission order
+        self.finished: List[Request] = []
+        self._arrivals = 0
+        self.num_preemptions = 0
+        self.pages_high_water = [0] * len(cache.pools)
+
+    # ---- intake --------------------------------------------------------
+    def add_request(self, req: Request) -> None:
+        if not req.prompt:
+            raise ValueError(f"request {req.rid!r}: empty prompt")
+        total = len(req.prompt) + req.params.max_new_tokens
+        limit = self.config.max_model_len
+        if len(req.prompt) >= limit and req.params.max_new_tokens > 0:
+            raise ValueError(f"request {req.rid!r}: prompt of {len(req.prompt)} tokens leaves no room under max length {limit}")
+        # It must fit the pool when it is the only request, or it could never finish.
+        need_tokens = min(total, limit)
+        ps = self.cache.page_size
+        for g, pool in enumerate(self.cache.pools):
+            spec = self.cache.groups[g]
+            tokens_held = need_tokens
+            if spec.kind == "window" and spec.window is not None:
+                tokens_held = min(need_tokens, spec.window + min(self.config.prefill_chunk_size,
+                                                                 self.config.max_num_batched_tokens) + ps)
+            if (tokens_held + ps - 1) // ps > pool.num_pages:
+                raise ValueError(
+                    f"request {req.rid!r}: needs {(tokens_held + ps - 1) // ps} pages of cache group {g}, the pool has {pool.num_pages}")
+        req.arrival = self._arrivals
+        self._arrivals += 1
+        req.state = RequestState.WAITING
+        self.waiting.append(req)
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # ---- one step's plan -------------------------------------------------
+    def _portion(self, req: Request, budget: int) -> int:
+        rest = req.num_tokens - req.num_computed
+        return min(rest, self.config.prefill_chunk_size, budget)
+
+    def _fits(self, req: Request, count: int, planned: List[int]) -> bool:
+        need = self.cache.pages_needed(req.rid, count)
+        free = self.cache.free_pages()
+        return all(n + p <= f for n, p, f in zip(need, planned, free))
+
+    def _preempt(self, victim: Request) -> None:
+        self.cache.release(victim.rid)
+        victim.num_computed = 0
+        victim.state = RequestState.WAITING
+        victim.preemptions += 1
+        self.num_preemptions += 1
+        self.running.remove(victim)
+        self.waiting.appendleft(victim)
+
+    def schedule(self) -> List[ScheduledItem]:
+        """Decide the next step.  Pages are only counted here; the step function reserves them."""
+        budget = self.config.max_num_batched_tokens
+        planned = [0] * len(self.cache.pools)          # pages promised to items already in the plan
+        items: List[ScheduledItem] = []
+
+        def take(req: Request, count: int) -> None:
+            nonlocal budget
+            need = self.cache.pages_needed(req.rid, count)
+            for g, n in enumerate(need):
+                planned[g] += n
+            items.append(ScheduledItem(req, req.num_computed, count, req.num_computed + count == req.num_tokens))
+            budget -= count
+
+        # 1. running requests, decoding ones first, then prompt portions, each in admission order
+        order = [r for r in self.running if r.is_decoding] + [r for r in self.running if not r.is_decoding]
+        for req in order:
+            if req not in self.running:          # preempted while serving an earlier one
+                continue
+            if budget <= 0:
+                break
+            count = 1 if req.is_decoding else self._portion(req, budget)
+            while not self._fits(req, count, planned):
+                # give back the pages of the most recently admitted request that is not in the plan yet
+                victims = [r for r in reversed(self.running) if r is not req and all(it.request is not r for it in items)]
+                if not victims:
+                    break
+                self._preempt(victims[0])
+            else:
+                take(req, count)
+                continue
+            # nothing left to preempt: skip this request in this step unless it is the only work
+            if not items and len(self.running) == 1:
+                raise RuntimeError(f"request {req.rid!r} cannot get pages although it runs alone")
+
+        # 2. admit waiting requests (preempted ones are at the front)
+        while self.waiting and budget > 0 and len(self.running) < self.config.max_num_seqs:
+            req = self.waiting[0]
+            if not self.cache.has(req.rid):
+                if len(self.cache.live_requests()) >= self.cache.max_requests:
+                    break
+                self.cache.add(req.rid)
+            count = self._portion(req, budget)
+            if not self._fits(req, count, planned):
+                self.cache.release(req.rid)
+                break
+            self.waiting.popleft()
+            req.state = RequestState.RUNNING
+            self.running.append(req)
+            take(req, count)
+
+        for g, pool in enumerate(self.cache.pools):
+            self.pages_high_water[g] = max(self.pages_high_water[g], pool.num_held + planned[g])
+        return items
+
+    # ---- after the step ---------------------------------------------------
+    def advance(self, item: ScheduledItem) -> None:
+        """The step wrote ``item.count`` tokens of the request."""
+        item.request.num_computed += item.count
+
+    def append_token(self, req: Request, token: int) -> bool:
+        """Record a sampled token; returns True when the request is finished
+        (/root/reference/server/src/engine_task.rs:64-66: token budget or EOS; the EOS token is kept)."""
+        req.output.append(int(token))
+        if not req.params.ignore_eos and int(token) in req.eos_token_ids:
+            req.finish_reason = "eos"
+        elif len(req.output) >= req.params.max_new_tokens:
+            req.finish_reason = "length"
+        elif req.num_tokens >= self.config.max_model_len:
+            req.finish_reason = "max_model_len"
+        return req.finish_reason is not None
+
+    def finish(self, req: Request) -> None:
+        """Give back the request's pages and state slot at once."""
+        if req in self.running:
+            self.running.remove(req)
+        if self.cache.has(req.rid):
+            self.cache.release(req.rid)
+        req.state = RequestState.FINISHED
+        self.finished.append(req)

@@ -246,3 +246,49 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
     _call("tp_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
     return out
+
+
+def _dev_array(values, dtype, device) -> torch.Tensor:
+    import numpy as np
+    return torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=dtype))).to(device)
+
+
+def apply_penalties(logits: torch.Tensor, rows, tokens, counts, in_window, presence, frequency, repeat) -> None:
+    """In place on float32 [m, vocab]: for entry i, logits[rows[i], tokens[i]] gets the presence/frequency
+    penalty when counts[i] > 0 and the repetition penalty when in_window[i]; penalties are per row."""
+    if _backend is not None:
+        return _backend.apply_penalties(logits, rows, tokens, counts, in_window, presence, frequency, repeat)
+    import numpy as np
+    _dev_ok(logits)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "apply_penalties: logits must be float32 [m, vocab]")
+    m, vocab = logits.shape
+    n = len(rows)
+    _need(len(tokens) == n and len(counts) == n and len(in_window) == n, "apply_penalties: entry lists differ in length")
+    _need(len(presence) == m and len(frequency) == m and len(repeat) == m, "apply_penalties: one penalty per row")
+    _need(all(0 <= r < m for r in rows), "apply_penalties: row out of range")
+    dev = logits.device
+    ints = _dev_array([rows, tokens, counts, in_window], np.int32, dev)
+    fl = _dev_array([presence, frequency, repeat], np.float32, dev)
+    _call("tp_apply_penalties", _ptr(logits), vocab, _ptr(ints[0]), _ptr(ints[1]), _ptr(ints[2]), _ptr(ints[3]),
+          _ptr(fl[0]), _ptr(fl[1]), _ptr(fl[2]), n, _stream())
+
+
+def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, min_p, rnd) -> torch.Tensor:
+    """float32 [m, vocab] and per-row options (host arrays) -> int32 [m] chosen tokens.
+    ``work`` is float32 scratch of at least [m, vocab].  temperature 0 rows return the argmax."""
+    if _backend is not None:
+        return _backend.sample(logits, work, temperature, top_k, top_p, min_p, rnd)
+    import numpy as np
+    _dev_ok(logits, work)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits must be float32 [m, vocab]")
+    m, vocab = logits.shape
+    _need(work.dtype == torch.float32 and work.numel() >= m * vocab, "sample: work buffer too small")
+    for a in (temperature, top_k, top_p, min_p, rnd):
+        _need(len(a) == m, "sample: one option per row")
+    dev = logits.device
+    fl = _dev_array([temperature, top_p, min_p, rnd], np.float32, dev)
+    tk = _dev_array(top_k, np.int32, dev)
+    out = torch.empty((m,), dtype=torch.int32, device=dev)
+    _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
+          _ptr(fl[3]), _ptr(out), _stream())
+    return out

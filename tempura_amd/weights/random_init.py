@@ -15,7 +15,7 @@ from typing import Callable, Dict, Optional
 
 import torch
 
-from ..engine.model import expected_weights
+from ..parts.inventory import expected_weights
 from ..parts.base import WeightInfo
 from .safetensors_io import write_safetensors
 
