@@ -1,9 +1,12 @@
 """Device memory behind the cache manager: page pools and state slots.
 
-One allocation per group, ``[slots, 2 (k, v), pages + 1, kv_heads, page_size,
+One allocation per group, ``[slots, 2 (k, v), pages + 1, kv_heads, page_size *
 head_dim]``: a physical page id addresses the same page for every cache slot of
 the group, and within a page each kv head's rows lie together so that a head's
-keys of one page are one contiguous run.  The extra last page is never handed
+keys of one page are one contiguous run.  Keys are ``[page_size, head_dim]`` per
+head and page; values are kept transposed, ``[head_dim, page_size]``, so that
+the attention kernels fetch eight consecutive keys of one value element with one
+16-byte load.  The extra last page is never handed
 out; padded rows of a fixed-size decode batch write there.  State tensors are
 ``[max_requests + 1, *shape]`` per stateful cache slot, the extra row likewise.
 """
@@ -23,7 +26,7 @@ class LayerCache:
 
     group: int                       # index of the cache group (-1: the mixer has no paged cache)
     k: Optional[torch.Tensor]        # [pages + 1, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor]
+    v: Optional[torch.Tensor]        # [pages + 1, kv_heads, head_dim, page_size]
     writes: bool                     # False: this call only reads a slot another call writes
     page_size: int
     state: Optional[torch.Tensor]    # [max_requests + 1, *shape] or None

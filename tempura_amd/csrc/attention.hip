@@ -43,11 +43,13 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
   for (int j0 = lo; j0 <= pos; j0 += TP_WAVE) {
     const int j = j0 + lane;
     const bool valid = j <= pos;
-    int row = 0;  // cache row of this lane's key: (page * n_kv + kvh) * page_size + offset
+    int row = 0;   // cache row of this lane's key: (page * n_kv + kvh) * page_size + offset
+    int vbase = 0; // its value column: values are stored [page, kv_head, head_dim, page_size]
     float s = -INFINITY;
     if (valid) {
       const int page = table[j / page_size];
       row = (page * n_kv + kvh) * page_size + j % page_size;
+      vbase = (page * n_kv + kvh);
       const T* kr = k_cache + (size_t)row * head_dim;
       float dot = 0.f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
@@ -63,12 +65,12 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
     const int n_valid = min(TP_WAVE, pos - j0 + 1);
     for (int jj = 0; jj < n_valid; ++jj) {
       const float pj = __shfl(p, jj, TP_WAVE);
-      const int vrow = __shfl(row, jj, TP_WAVE);
-      const T* vr = v_cache + (size_t)vrow * head_dim;
+      const int vb = __shfl(vbase, jj, TP_WAVE);
+      const T* vr = v_cache + (size_t)vb * head_dim * page_size + (j0 + jj) % page_size;
 #pragma unroll
       for (int i = 0; i < ATT_MAX_ACC; ++i) {
         const int d = lane + i * TP_WAVE;
-        if (d < head_dim) acc[i] = fmaf(pj, to_float(vr[d]), acc[i]);
+        if (d < head_dim) acc[i] = fmaf(pj, to_float(vr[(size_t)d * page_size]), acc[i]);
       }
     }
   }
@@ -83,16 +85,18 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
 
 // Defined in attention_mfma.hip: takes bfloat16 shapes it is built for, returns -1 otherwise.
 int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
-                            int table_width, const int* cu_seqlens, const int* context_lens,
-                            const int* token_req, void* out, int n_tokens, int n_req, int n_heads, int n_kv,
-                            int head_dim, int page_size, float scale, int window, int max_q_len, int max_ctx,
-                            hipStream_t s);
+                            int table_width, const int* cu_seqlens, const int* context_lens, void* out, int n_tokens,
+                            int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
+                            int max_q_len, int num_single, int num_splits, float* scratch, hipStream_t s);
 
 extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, const void* v_cache,
                                   const int* block_tables, int table_width, const int* cu_seqlens,
                                   const int* context_lens, const int* token_req, void* out, int n_tokens,
                                   int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale,
-                                  int window, int max_q_len, int max_ctx, int allow_fast, hipStream_t s) {
+                                  int window, int max_q_len, int max_ctx, int allow_fast, int num_single,
+                                  int num_splits, float* scratch, hipStream_t s) {
+  // num_single: how many requests bring exactly one token (they go to the split decode kernel,
+  // which needs `scratch` of n_req * n_heads * num_splits * (head_dim + 2) floats).
   TP_REQUIRE(n_tokens >= 0 && n_req >= 0 && n_heads > 0 && n_kv > 0 && head_dim > 0 && page_size > 0,
              "paged_attention: bad sizes");
   TP_REQUIRE(n_heads % n_kv == 0, "paged_attention: %d heads is not a multiple of %d kv heads", n_heads, n_kv);
@@ -103,8 +107,8 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   if (n_tokens == 0) return 0;
   if (dt == TP_BF16 && allow_fast) {
     const int rc = tp_paged_attention_fast(q, k_cache, v_cache, block_tables, table_width, cu_seqlens,
-                                           context_lens, token_req, out, n_tokens, n_req, n_heads, n_kv,
-                                           head_dim, page_size, scale, window, max_q_len, max_ctx, s);
+                                           context_lens, out, n_tokens, n_req, n_heads, n_kv, head_dim,
+                                           page_size, scale, window, max_q_len, num_single, num_splits, scratch, s);
     if (rc >= 0) return rc;
   }
   const dim3 grid(n_tokens, n_heads);

@@ -79,9 +79,11 @@ extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void*
 // One block per token.  qkv row: [q heads | k heads | v heads] x head_dim, float32.
 // Pair (d, d + rotary_dim/2) of each q and k head turns by angle pos * inv_freq[d]; the
 // angle is formed in float64 from the integer position.  q goes to q_out, rotated k and raw
-// v go to the cache row `slots[t]` (page * page_size + offset) of the paged pools
-// [page, kv_head, page_size, head_dim].  With slots == nullptr only q is produced
-// (the row then holds q heads only).
+// v go to the cache place `slots[t]` (page * page_size + offset) of the paged pools: keys
+// as [page, kv_head, page_size, head_dim], values TRANSPOSED as [page, kv_head, head_dim,
+// page_size] so that the attention kernels read eight consecutive keys of one value
+// element with one 16-byte load.  With slots == nullptr only q is produced (the row then
+// holds q heads only).
 template <typename TQ, typename TC>
 __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stride,
                                      const int* __restrict__ positions, const int* __restrict__ slots,
@@ -139,7 +141,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
     const float* vrow = row + (size_t)(n_heads + n_kv) * head_dim;
     for (int i = threadIdx.x; i < n_kv * head_dim; i += blockDim.x) {
       const int h = i / head_dim, d = i % head_dim;
-      from_float(v_cache + ((page * n_kv + h) * page_size + off) * head_dim + d, vrow[i]);
+      from_float(v_cache + ((page * n_kv + h) * head_dim + d) * page_size + off, vrow[i]);
     }
   }
 }
@@ -205,5 +207,42 @@ extern "C" int tp_swiglu(const void* gu, int in_dt, void* out, int out_dt, int m
     TP_REQUIRE(false, "swiglu: unsupported dtypes %d -> %d", in_dt, out_dt);
 #undef LAUNCH
   TP_CHECK_LAUNCH("swiglu");
+  return 0;
+}
+
+// ---- seeded normal fill ------------------------------------------------------------------
+// out[i] = mean + std * N(0, 1) where the normal deviate of element i depends only on
+// (seed, i): a SplitMix64 hash gives two uniforms, Box-Muller turns them into a deviate.
+// Used to make random weights of large models directly in device memory.
+__device__ inline unsigned long long splitmix64(unsigned long long z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+template <typename T>
+__global__ void fill_normal_kernel(T* __restrict__ out, size_t n, unsigned long long seed, float mean, float std) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const unsigned long long h = splitmix64(seed ^ splitmix64((unsigned long long)i));
+  const float u1 = ((float)(unsigned int)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
+  const float u2 = (float)(unsigned int)((h >> 8) & 0xffffffu) * (1.0f / 16777216.0f);
+  const float z = sqrtf(-2.0f * logf(u1)) * cosf(6.283185307179586f * u2);
+  from_float(out + i, mean + std * z);
+}
+
+extern "C" int tp_fill_normal(void* out, int dt, size_t n, unsigned long long seed, float mean, float std,
+                              hipStream_t s) {
+  if (n == 0) return 0;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  TP_REQUIRE((n + 255) / 256 < ((size_t)1 << 31), "fill_normal: tensor too large");
+  if (dt == TP_F32)
+    hipLaunchKernelGGL(fill_normal_kernel<float>, grid, dim3(256), 0, s, (float*)out, n, seed, mean, std);
+  else if (dt == TP_BF16)
+    hipLaunchKernelGGL(fill_normal_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)out, n, seed, mean, std);
+  else
+    TP_REQUIRE(false, "fill_normal: unknown dtype %d", dt);
+  TP_CHECK_LAUNCH("fill_normal");
   return 0;
 }

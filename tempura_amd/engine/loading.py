@@ -32,19 +32,35 @@ def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> CausalLM:
 
 
 def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: float = 0.02,
-                 norm_jitter: float = 0.0) -> CausalLM:
+                 norm_jitter: float = 0.0, on_device: bool = None) -> CausalLM:
     """A model with seeded random weights made tensor by tensor, never written to disk
-    (for sizes whose folder would be tens of gigabytes)."""
+    (for sizes whose folder would be tens of gigabytes).  With ``on_device`` (the default on a
+    GPU) each tensor is filled by a kernel in device memory; its values then differ from the
+    host generator's that ``write_random_model`` uses."""
+    from ..kernels import ops
+    from ..weights.random_init import _tensor_seed
     td = parse_dtype(dtype)
-    model = CausalLM(config.build_spec(), td, torch.device(device))
+    dev = torch.device(device)
+    if on_device is None:
+        on_device = dev.type == "cuda"
+    model = CausalLM(config.build_spec(), td, dev)
     model.config = config
     expected = model.expected_weights()
+    store = torch.bfloat16 if td == torch.bfloat16 else torch.float32
 
     def get(name, optional=False):
         info = expected[name]
         if info.init == "skip":
             return None
-        return random_tensor(name, info, seed, std, norm_jitter, torch.bfloat16 if td == torch.bfloat16 else torch.float32)
+        if not on_device:
+            return random_tensor(name, info, seed, std, norm_jitter, store)
+        if info.init == "ones":
+            t = torch.ones(info.shape, dtype=torch.float32, device=dev)
+            if norm_jitter:
+                ops.fill_normal(t, _tensor_seed(seed, name), 1.0, norm_jitter)
+            return t
+        t = torch.empty(info.shape, dtype=store, device=dev)
+        return ops.fill_normal(t, _tensor_seed(seed, name), 0.0, std)
 
     model.load_weights(get)
     return model

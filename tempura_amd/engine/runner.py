@@ -57,6 +57,7 @@ class StepContext:
         self.logit_rows = None
         self.max_q_len = 0
         self.max_context_len = 0
+        self.num_single = 0          # requests that bring exactly one token
         self.page_size = 0
         self.q_starts: List[int] = []
         self.q_lens: List[int] = []
@@ -81,8 +82,9 @@ class ModelRunner:
             g, idx = model.slot_group[call.cache]
             k = v = None
             if g >= 0:
+                spec = model.cache_groups[g]
                 k = self.pools.kv[g][idx, 0]
-                v = self.pools.kv[g][idx, 1]
+                v = self.pools.kv[g][idx, 1].view(-1, spec.num_kv_heads, spec.head_dim, self.page_size)
             self.layer_caches.append(LayerCache(g, k, v, model.call_writes[i], self.page_size,
                                                 self.pools.state.get(call.cache)))
         self.steps_run = 0
@@ -184,6 +186,7 @@ class ModelRunner:
         ctx.block_tables = [view[7 + g].view(R, tables[g].shape[1]) for g in range(n_groups)]
         ctx.slot_mapping = view[7 + n_groups: 7 + 2 * n_groups]
         ctx.max_q_len = max(q_lens)
+        ctx.num_single = sum(1 for n in q_lens if n == 1)
         ctx.max_context_len = int(ctx_lens.max())
         ctx.page_size = self.page_size
         ctx.q_starts = [int(c) for c in cu[:-1]]

@@ -178,8 +178,9 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[to
     page_size, cache_dt = 1, _F32
     if slots is not None:
         _i32(slots, n, "slots") if n else None
-        _need(k_cache is not None and v_cache is not None and k_cache.shape == v_cache.shape and k_cache.dim() == 4,
-              "rope_kv_write: caches must be [pages, kv_heads, page_size, head_dim]")
+        _need(k_cache is not None and v_cache is not None and k_cache.dim() == 4 and v_cache.dim() == 4
+              and tuple(v_cache.shape) == (k_cache.shape[0], k_cache.shape[1], k_cache.shape[3], k_cache.shape[2]),
+              "rope_kv_write: caches must be k [pages, kv_heads, page_size, head_dim], v [pages, kv_heads, head_dim, page_size]")
         _need(k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim, "rope_kv_write: cache layout mismatch")
         _need(k_cache.dtype == v_cache.dtype, "rope_kv_write: cache dtypes differ")
         page_size, cache_dt = k_cache.shape[2], _dt(k_cache)
@@ -199,15 +200,20 @@ allow_fast_attention = True
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     cu_seqlens: torch.Tensor, context_lens: torch.Tensor, token_req: torch.Tensor,
-                    scale: float, window: int, max_q_len: int, max_context_len: int) -> torch.Tensor:
-    """q [n, heads, head_dim] over caches [pages, kv_heads, page_size, head_dim] -> [n, heads * head_dim]."""
+                    scale: float, window: int, max_q_len: int, max_context_len: int,
+                    num_single: Optional[int] = None) -> torch.Tensor:
+    """q [n, heads, head_dim] over k [pages, kv_heads, page_size, head_dim] and transposed
+    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim]."""
     if _backend is not None:
         return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
                                         token_req, scale, window, max_q_len, max_context_len)
+    # num_single: requests that bring exactly one token (None: all of them iff max_q_len == 1, else unknown
+    # and every request is treated as a portion).
     _dev_ok(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens, token_req)
-    _need(q.dim() == 3 and k_cache.dim() == 4 and k_cache.shape == v_cache.shape, "paged_attention: bad operand ranks")
+    _need(q.dim() == 3 and k_cache.dim() == 4 and v_cache.dim() == 4, "paged_attention: bad operand ranks")
     n, heads, d = q.shape
     pages, kvh, page_size, d2 = k_cache.shape
+    _need(tuple(v_cache.shape) == (pages, kvh, d2, page_size), "paged_attention: v cache must be [pages, kv_heads, head_dim, page_size]")
     _need(d == d2, "paged_attention: head_dim of q and cache differ")
     _need(q.dtype == k_cache.dtype == v_cache.dtype, "paged_attention: q and cache dtypes differ")
     _need(block_tables.dim() == 2 and block_tables.dtype == torch.int32, "paged_attention: block_tables must be int32 [r, width]")
@@ -218,10 +224,20 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _need(pages * kvh * page_size < 2 ** 31, "paged_attention: cache pool too large for 32-bit row indices")
     _need(max_context_len <= width * page_size, "paged_attention: block table narrower than the longest context")
     out = torch.empty((n, heads * d), dtype=q.dtype, device=q.device)
+    if num_single is None:
+        num_single = r if max_q_len == 1 else 0
+    _need(0 <= num_single <= r, "paged_attention: num_single out of range")
+    fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0
+    splits, scratch = 1, None
+    if fast and num_single > 0:
+        # enough blocks to fill 256 CUs, but at least 128 keys per block
+        blocks_per_split = num_single * kvh * ((heads // kvh + 15) // 16)
+        splits = max(1, min(64, -(-1024 // blocks_per_split), max(1, max_context_len // 128)))
+        scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
     _call("tp_paged_attention", _ptr(q), _dt(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), width,
           _ptr(cu_seqlens), _ptr(context_lens), _ptr(token_req), _ptr(out), n, r, heads, kvh, d, page_size,
-          ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(allow_fast_attention),
-          _stream())
+          ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(fast),
+          int(num_single), int(splits), _ptr(scratch), _stream())
     return out
 
 
@@ -291,4 +307,14 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
     out = torch.empty((m,), dtype=torch.int32, device=dev)
     _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
           _ptr(fl[3]), _ptr(out), _stream())
+    return out
+
+
+def fill_normal(out: torch.Tensor, seed: int, mean: float, std: float) -> torch.Tensor:
+    """Fill a device tensor with mean + std * N(0, 1); element i depends only on (seed, i)."""
+    if _backend is not None:
+        return _backend.fill_normal(out, seed, mean, std)
+    _dev_ok(out)
+    _call("tp_fill_normal", _ptr(out), _dt(out), ctypes.c_size_t(out.numel()), ctypes.c_ulonglong(seed & (2 ** 64 - 1)),
+          ctypes.c_float(mean), ctypes.c_float(std), _stream())
     return out

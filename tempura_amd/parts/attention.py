@@ -81,7 +81,8 @@ class PagedAttention(Mixer):
             cache.k if cache.writes else None, cache.v if cache.writes else None, self.dtype)
         a = ops.paged_attention(
             q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
-            ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len)
+            ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
+            ctx.num_single)
         ops.linear(a, self.wo, torch.float32, residual=residual)
 
 

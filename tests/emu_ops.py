@@ -48,11 +48,11 @@ class EmuOps:
             ps = k_cache.shape[2]
             page, off = slots.long() // ps, slots.long() % ps
             k_cache[page, :, off] = k.to(k_cache.dtype)
-            v_cache[page, :, off] = v.to(v_cache.dtype)
+            v_cache[page, :, :, off] = v.to(v_cache.dtype)          # values are kept transposed
         return q
 
     def paged_attention(self, q, k_cache, v_cache, block_tables, cu_seqlens, context_lens, token_req, scale,
-                        window, max_q_len, max_context_len):
+                        window, max_q_len, max_context_len, num_single=None):
         n, heads, d = q.shape
         kvh, ps = k_cache.shape[1], k_cache.shape[2]
         group = heads // kvh
@@ -65,7 +65,7 @@ class EmuOps:
             j = torch.arange(ctx)
             rows_page, rows_off = pages[j // ps], j % ps
             K = k_cache[rows_page, :, rows_off].double()      # [ctx, kvh, d]
-            V = v_cache[rows_page, :, rows_off].double()
+            V = v_cache[rows_page, :, :, rows_off].double()      # [ctx, kvh, d]
             for t in range(qs, qe):
                 pos = ctx - (qe - qs) + (t - qs)
                 lo = max(0, pos - window + 1) if window > 0 else 0

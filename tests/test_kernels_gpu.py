@@ -85,7 +85,7 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
     inv = rotary_inv_freq(d, 500000.0, {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                                         "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}, rot)
     kc = torch.zeros(pages, kv, page, d, dtype=dtype)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(pages, kv, d, page, dtype=dtype)
     kr, vr = kc.clone(), vc.clone()
     qr = emu.rope_kv_write(qkv, pos, slots, inv, rot, 1.0, heads, kv, d, kr, vr, torch.float64)
     kd, vd = kc.to(DEV), vc.to(DEV)
@@ -115,7 +115,7 @@ def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, a
         for i in range((c + page - 1) // page):
             bt[r, i] = next(it)
     kc = (torch.randn(pages, kv, page, d, generator=g) * 1.5).to(dtype)
-    vc = torch.randn(pages, kv, page, d, generator=g).to(dtype)
+    vc = torch.randn(pages, kv, d, page, generator=g).to(dtype)
     q = (torch.randn(n, heads, d, generator=g) * 1.5).to(dtype)
     cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
     cl = torch.tensor(ctx_lens, dtype=torch.int32)
@@ -147,7 +147,7 @@ def test_attention_far_key_stands_out(dtype):
     heads, kv, d, page, ctx = 4, 2, 64, 16, 700
     pages = (ctx + page - 1) // page
     kc = torch.randn(pages, kv, page, d, generator=g) * 0.1
-    vc = torch.randn(pages, kv, page, d, generator=g)
+    vc = torch.randn(pages, kv, d, page, generator=g)
     q = torch.randn(1, heads, d, generator=g) * 0.1
     far = 3                                                 # a key in the first page
     kc[far // page, :, far % page] = q[0, ::2] * 400.0      # aligned with the query of each group's first head
@@ -160,7 +160,7 @@ def test_attention_far_key_stands_out(dtype):
     got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), cu.to(DEV), cl.to(DEV), tr.to(DEV), 1.0, 0, 1, ctx)
     _close(got, ref, 2e-5 if dtype == torch.float32 else 1.2e-2, "far key")
     # the answer of heads 0 and 2 is (almost) the far key's value row
-    assert float((ref.reshape(heads, d)[0] - vc[far // page, 0, far % page].double()).abs().max()) < 0.05
+    assert float((ref.reshape(heads, d)[0] - vc[far // page, 0, :, far % page].double()).abs().max()) < 0.05
 
 
 @pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16)])
@@ -184,3 +184,47 @@ def test_argmax_last_max_wins(m, vocab):
     got = ops.argmax(lg.to(DEV)).cpu()
     assert torch.equal(got, emu.argmax(lg))
     assert int(got[0]) == vocab - 3
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 16, 32), (1, 4096, 4096), (8, 200, 96), (16, 6144, 4096), (17, 48, 64),
+                                   (33, 1000, 320), (48, 130, 2048), (64, 4096, 1024), (65, 128, 64),
+                                   (200, 300, 96), (257, 384, 160), (512, 1024, 4096)])
+def test_linear_mfma(m, n, k):
+    """The matrix-core kernels (decode and prefill shapes) against float64, and against the general kernel."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    ref = x.double() @ w.double().T
+    xd, wd = x.to(DEV), w.to(DEV)
+    got = ops.linear(xd, wd, torch.float32)
+    _close(got, ref, 2e-5, "mfma f32 out")
+    _close(ops.linear(xd, wd, torch.bfloat16), ref, 1e-2, "mfma bf16 out")
+    res = torch.randn(m, n, generator=g)
+    _close(ops.linear(xd, wd, torch.float32, residual=res.clone().to(DEV)), ref + res.double(), 2e-5, "mfma residual")
+    ops.allow_mfma = False
+    try:
+        general = ops.linear(xd, wd, torch.float32)
+    finally:
+        ops.allow_mfma = True
+    _close(got, general.double().cpu(), 2e-5, "mfma vs general kernel")
+    # a row's result does not depend on the other rows of the batch (same kernel family)
+    if m > 1 and m <= 16:
+        one = ops.linear(xd[:1].contiguous(), wd, torch.float32)
+        assert torch.equal(one[0], got[0])
+
+
+@pytest.mark.parametrize("heads,kv,d,page", [(4, 2, 32, 8), (8, 2, 64, 16), (6, 3, 96, 32), (32, 8, 128, 16), (8, 8, 128, 64),
+                                             (20, 1, 64, 16), (5, 1, 128, 8)])
+def test_attention_mfma(heads, kv, d, page):
+    """The matrix-core kernels: portions (with and without a cached prefix) beside single decoded tokens."""
+    bf = torch.bfloat16
+    _attention_case(bf, heads, kv, d, page, [37, 9, 1, 1, 1], [37, 64, 33, 130, 1], 0, seed=11)      # mixed
+    _attention_case(bf, heads, kv, d, page, [1, 1, 1], [700, 31, 257], 0, seed=12)                     # decode only, split context
+    _attention_case(bf, heads, kv, d, page, [70, 33], [70, 97], 0, seed=13)                            # portions only
+    _attention_case(bf, heads, kv, d, page, [20, 1, 6, 1], [50, 77, 6, 300], 13, seed=14)              # window
+    _attention_case(bf, heads, kv, d, page, [40, 1], [200, 200], 64, seed=15)                          # window longer than a step
+
+
+def test_attention_mfma_long_decode():
+    _attention_case(torch.bfloat16, 8, 2, 128, 16, [1, 1], [3000, 2049], 0, seed=16)
