@@ -65,6 +65,54 @@ class StepContext:
         self.state_slot_list: List[int] = []
 
 
+class _DecodeGraph:
+    """A captured decode step for a fixed number of rows and a bound on the context length.
+
+    Every per-step value lives in ``packed`` (one int32 device buffer refreshed by one copy
+    from pinned host memory); the kernels read lengths, tables and slots from there, so a
+    replay runs the new step without any host-side launch work.  The reference's batch
+    graphs are keyed by batch size with all per-step values device-read in the same way
+    (/root/reference/engine/src/cutile_gpu_forward.rs:939-953)."""
+
+    def __init__(self, runner: "ModelRunner", rows: int, ctx_bound: int):
+        self.rows = rows
+        self.ctx_bound = ctx_bound
+        self.width = (ctx_bound + runner.page_size - 1) // runner.page_size
+        n_groups = len(runner.cache.groups)
+        # layout: tokens, positions, context_lens, state_slots | per group: table, slots
+        self.sizes = [rows, rows, rows, rows] + [rows * self.width] * n_groups + [rows] * n_groups
+        self.offs = np.cumsum([0] + self.sizes)
+        total = int(self.offs[-1])
+        self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.packed = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        self.fixed = torch.arange(rows + 1, dtype=torch.int32, device=runner.device)
+        self.copied = torch.cuda.Event()
+        self.graph = None
+        self.logits = None
+
+    def view(self, i: int) -> torch.Tensor:
+        return self.packed[int(self.offs[i]): int(self.offs[i + 1])]
+
+    def context(self, runner: "ModelRunner") -> "StepContext":
+        n_groups = len(runner.cache.groups)
+        ctx = StepContext()
+        ctx.num_tokens = ctx.num_requests = self.rows
+        ctx.positions = self.view(1)
+        ctx.context_lens = self.view(2)
+        ctx.state_slots = self.view(3)
+        ctx.token_req = self.fixed[: self.rows]
+        ctx.cu_seqlens = self.fixed
+        ctx.logit_rows = None                     # every row
+        ctx.block_tables = [self.view(4 + g).view(self.rows, self.width) for g in range(n_groups)]
+        ctx.slot_mapping = [self.view(4 + n_groups + g) for g in range(n_groups)]
+        ctx.max_q_len = 1
+        ctx.num_single = self.rows
+        ctx.max_context_len = self.width * runner.page_size
+        ctx.page_size = runner.page_size
+        return ctx
+
+
 class ModelRunner:
     def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
                  cache_dtype: Optional[torch.dtype] = None, use_graph: bool = False):
@@ -89,8 +137,12 @@ class ModelRunner:
                                                 self.pools.state.get(call.cache)))
         self.steps_run = 0
         self.tokens_run = 0
-        self.use_graph = use_graph
+        # Decode-only steps replay a captured graph when every part of the model allows it.
+        self.use_graph = bool(use_graph) and self.device.type == "cuda" and not model.state_specs and \
+            all(getattr(p, "graph_safe", False) for layer in model.layers for p in layer.parts())
         self.graph_steps = 0
+        self._graphs: Dict[tuple, _DecodeGraph] = {}
+        self._graph_pool = None
 
     # ---- request lifetime ---------------------------------------------
     def has_request(self, rid) -> bool:
@@ -195,12 +247,88 @@ class ModelRunner:
         ctx.state_slot_list = [int(s) for s in state_slots]
         return tok_dev, ctx, starts
 
+    # ---- decode steps as a graph -----------------------------------------
+    def _graph_for(self, rows: int, ctx_len: int) -> Optional[_DecodeGraph]:
+        bucket = 1
+        while bucket < rows:
+            bucket *= 2
+        bound = 256
+        while bound < ctx_len:
+            bound *= 2
+        bound = min(bound, (self.model.spec.max_positions + self.page_size - 1) // self.page_size * self.page_size)
+        key = (bucket, bound)
+        g = self._graphs.get(key)
+        if g is None:
+            g = _DecodeGraph(self, bucket, bound)
+            self._graphs[key] = g
+        return g
+
+    def _fill_graph_inputs(self, g: _DecodeGraph, entries: Sequence[StepEntry]) -> None:
+        n_groups = len(self.cache.groups)
+        g.copied.synchronize()                     # the last copy out of the pinned buffer has finished
+        h, offs = g.host_np, g.offs
+        n = len(entries)
+        starts = [self.cache.num_tokens(e.rid) for e in entries]
+        tok, pos, ctxl, slot = (h[offs[i]: offs[i + 1]] for i in range(4))
+        tok[:] = 0
+        pos[:] = 0
+        ctxl[:] = 1                                 # padded rows: one key, in the scratch page
+        slot[:] = self.cache.max_requests
+        tok[:n] = [e.tokens[0] for e in entries]
+        pos[:n] = starts
+        ctxl[:n] = [s + 1 for s in starts]
+        slot[:n] = [self.cache.state_slot(e.rid) for e in entries]
+        for gi in range(n_groups):
+            scratch = self.pools.scratch_page(gi)
+            bt = h[offs[4 + gi]: offs[5 + gi]].reshape(g.rows, g.width)
+            bt[:] = scratch
+            for r, e in enumerate(entries):
+                t = np.asarray(self.cache.table(e.rid, gi), dtype=np.int32)
+                bt[r, : len(t)] = np.where(t >= 0, t, scratch)
+            sl = h[offs[4 + n_groups + gi]: offs[5 + n_groups + gi]]
+            sl[:] = scratch * self.page_size
+            for r, (e, s0) in enumerate(zip(entries, starts)):
+                sl[r] = self.cache.slots(e.rid, gi, s0, 1)[0]
+        g.packed.copy_(g.host, non_blocking=True)
+        g.copied.record()
+
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        ctx_len = max(self.cache.num_tokens(e.rid) for e in entries) + 1
+        g = self._graph_for(len(entries), ctx_len)
+        self._fill_graph_inputs(g, entries)
+        if g.graph is None:
+            ctx = g.context(self)
+            tok = g.view(0)
+            # one eager run first: lazy initialisation must not happen under capture
+            self.model.forward(tok, ctx, self.layer_caches)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                g.logits = self.model.forward(tok, ctx, self.layer_caches)
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
+            g.graph = graph
+        g.graph.replay()
+        self.graph_steps += 1
+        rows = [r for r, e in enumerate(entries) if len(e.want) > 0]
+        if len(rows) == len(entries):
+            return g.logits[: len(entries)]
+        return g.logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows else g.logits[:0]
+
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the batch; returns float32 logits [sum of wanted places, vocab] on the device,
-        ordered by entry and then by ``want``."""
+        ordered by entry and then by ``want``.  After a decode-only step the result is a view of
+        the graph's output buffer: use it before the next step."""
         entries = list(entries)
         self._check_entries(entries)
         self.reserve(entries)
+        if self.use_graph and all(len(e.tokens) == 1 for e in entries):
+            logits = self._graph_step(entries)
+            for e in entries:
+                self.cache.commit(e.rid, 1)
+            self.steps_run += 1
+            self.tokens_run += len(entries)
+            return logits
         tok_dev, ctx, starts = self.build_context(entries)
         # A request that starts at position 0 gets a cleared state (also after a recompute).
         if self.pools.state:

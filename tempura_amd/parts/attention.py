@@ -18,6 +18,8 @@ from .base import CacheSpec, Mixer, WeightInfo, build_part, register_part
 
 
 class PagedAttention(Mixer):
+    graph_safe = True      # only kernels on device-resident step data: may be captured in a graph
+
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
         p = spec.params

@@ -52,6 +52,9 @@ class Part:
     """Base of every part.  ``spec`` carries sizes, constants and tensor names."""
 
     category = ""
+    #: True when ``forward`` only launches kernels that read the step's data from device memory
+    #: (no host-side values of the batch, no host loops): decode steps may then replay a captured graph.
+    graph_safe = False
 
     def __init__(self, spec: PartSpec, hidden_size: int, dtype: torch.dtype, device):
         self.spec = spec

@@ -11,6 +11,8 @@ from .base import FeedForward, WeightInfo, register_part
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True      # only kernels on device-resident step data: may be captured in a graph
+
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
         self.intermediate_size = int(spec.params["intermediate_size"])

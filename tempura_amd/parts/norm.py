@@ -13,6 +13,8 @@ from .base import Norm, WeightInfo, register_part
 
 
 class RMSNorm(Norm):
+    graph_safe = True      # only kernels on device-resident step data: may be captured in a graph
+
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
         self.eps = float(spec.params["eps"])
