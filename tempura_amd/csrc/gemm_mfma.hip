@@ -35,65 +35,178 @@ __device__ inline void store_out(void* out, int mode, size_t idx, float v) {
 }
 
 // ---- skinny ---------------------------------------------------------------------------
-template <int MT, int WAVES>
+// MT: 16-row tiles of activations; NT: 16-row tiles of weights per block; WAVES: waves that
+// split K.  A wave takes K in runs of four consecutive 32-wide steps (256 contiguous bytes of
+// each weight row), run r going to wave r % WAVES.
+template <int MT, int NT, int WAVES, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16_t* __restrict__ x,
                                                                       const bf16_t* __restrict__ w,
                                                                       void* __restrict__ out, int mode, int M,
                                                                       int N, int K) {
-  __shared__ float red[WAVES][MT][256];
+  __shared__ float red[WAVES][NT * MT][256];
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-  const int n0 = blockIdx.x * 16;
-  const int wrow = min(n0 + (lane & 15), N - 1);
+  const int n0 = blockIdx.x * 16 * NT;
   const int kofs = (lane >> 4) * 8;
-  const u32x4_t* wp = (const u32x4_t*)(w + (size_t)wrow * K + kofs);
+  const u32x4_t* wp[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int wrow = min(n0 + j * 16 + (lane & 15), N - 1);
+    wp[j] = (const u32x4_t*)(w + (size_t)wrow * K + kofs);
+  }
   const u32x4_t* xp[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int xrow = min(t * 16 + (lane & 15), M - 1);
     xp[t] = (const u32x4_t*)(x + (size_t)xrow * K + kofs);
   }
-  f32x4_t acc[MT];
+  f32x4_t acc[NT][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[j][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  const int steps = K / 32;  // a step is 32 k = 4 u32x4_t per row
-  int s = wave;
-  // four steps in flight per wave
-  for (; s + 3 * WAVES < steps; s += 4 * WAVES) {
-    u32x4_t a[4];
+  const int steps = K / 32;  // a step is 32 k = 4 u32x4 per row
+  // DEPTH runs of four steps are fetched before any of them is multiplied: 4 * DEPTH * NT loads
+  // of 16 bytes per lane are in flight, which is what keeps the memory system busy.
+  for (int s0 = wave * 4; s0 < steps; s0 += WAVES * 4 * DEPTH) {
+    u32x4_t a[DEPTH][NT][4];
+    u32x4_t b[DEPTH][MT][4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) a[u] = __builtin_nontemporal_load(wp + (size_t)(s + u * WAVES) * 4);
+    for (int d = 0; d < DEPTH; ++d)
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < 4; ++u) {
+        // steps past the end repeat the last one; their products are dropped below
+        const int sidx = min(s0 + d * WAVES * 4 + u, steps - 1);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const u32x4_t b = xp[t][(size_t)(s + u * WAVES) * 4];
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(a[u]), as_frag(b), acc[t], 0, 0, 0);
+        for (int j = 0; j < NT; ++j) a[d][j][u] = wp[j][(size_t)sidx * 4];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) b[d][t][u] = xp[t][(size_t)sidx * 4];
       }
-    }
-  }
-  for (; s < steps; s += WAVES) {
-    const u32x4_t a = __builtin_nontemporal_load(wp + (size_t)s * 4);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const u32x4_t b = xp[t][(size_t)s * 4];
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(a), as_frag(b), acc[t], 0, 0, 0);
-    }
+    for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (s0 + d * WAVES * 4 + u < steps) {
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+              acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(a[d][j][u]), as_frag(b[d][t][u]), acc[j][t], 0, 0, 0);
+        }
+      }
   }
   // sum the waves' partial tiles in wave order
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+  for (int j = 0; j < NT; ++j)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][t][lane * 4 + r] = acc[t][r];
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][j * MT + t][lane * 4 + r] = acc[j][t][r];
   __syncthreads();
-  for (int e = threadIdx.x; e < MT * 256; e += WAVES * 64) {
-    const int t = e / 256, q = e % 256;
+  for (int e = threadIdx.x; e < NT * MT * 256; e += WAVES * 64) {
+    const int jt = e / 256, q = e % 256;
+    const int j = jt / MT, t = jt % MT;
     float v = 0.f;
 #pragma unroll
-    for (int i = 0; i < WAVES; ++i) v += red[i][t][q];
+    for (int i = 0; i < WAVES; ++i) v += red[i][jt][q];
     const int l = q / 4, r = q % 4;
-    const int n = n0 + (l >> 4) * 4 + r;   // weight row = output column
+    const int n = n0 + j * 16 + (l >> 4) * 4 + r;   // weight row = output column
     const int m = t * 16 + (l & 15);
+    if (n < N && m < M) store_out(out, mode, (size_t)m * N + n, v);
+  }
+}
+
+// ---- skinny, activations through LDS (M <= 16) ------------------------------------------
+// With more than one activation row the second operand is a gather of short pieces of several
+// rows, and the address path, not HBM, limits the kernel.  Here the block copies the
+// activations of one K chunk (1,024 wide) into LDS with wide coalesced loads and every wave
+// reads its operand fragments from there; the weight stream is as above, one run of four steps
+// per wave and chunk, the next chunk's weights and activations already in flight while this
+// chunk is multiplied.  Two LDS buffers, one barrier per chunk.
+#define LKC 1024            // K elements per chunk
+#define LLD (LKC + 8)       // padded LDS row (bf16 elements): 16-byte reads of 16 rows hit 64 banks
+
+template <int NT>
+__global__ __launch_bounds__(512) void gemm_skinny_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                              void* __restrict__ out, int mode, int M, int N, int K) {
+  constexpr int WAVES = 8;
+  __shared__ __attribute__((aligned(16))) uint16_t xs[2][16 * LLD];
+  __shared__ float red[WAVES][NT][256];
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int n0 = blockIdx.x * 16 * NT;
+  const int kofs = (lane >> 4) * 8;
+  const u32x4_t* wp[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int wrow = min(n0 + j * 16 + (lane & 15), N - 1);
+    wp[j] = (const u32x4_t*)(w + (size_t)wrow * K + kofs);
+  }
+  // copy mapping: 32 threads per activation row, 16 bytes each, four passes of 256 elements
+  const int xrow = tid / 32, xcol = (tid % 32) * 8;
+  const bool xload = xrow < M;
+  const bf16_t* xsrc = x + (size_t)min(xrow, M - 1) * K + xcol;
+
+  f32x4_t acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const int steps = K / 32;
+  const int chunks = (K + LKC - 1) / LKC;
+
+  u32x4_t a[NT][4], xr[4];
+  auto load_chunk = [&](int ch) {
+    const int s0 = ch * (LKC / 32) + wave * 4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int sidx = min(s0 + u, steps - 1);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) a[j][u] = wp[j][(size_t)sidx * 4];
+    }
+    if (xload) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int k = ch * LKC + p * 256 + xcol;
+        xr[p] = (k < K) ? *(const u32x4_t*)(xsrc + (size_t)ch * LKC + p * 256) : (u32x4_t){0u, 0u, 0u, 0u};
+      }
+    }
+  };
+  load_chunk(0);
+  for (int ch = 0; ch < chunks; ++ch) {
+    const int buf = ch & 1;
+    if (xload) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) *(u32x4_t*)(&xs[buf][xrow * LLD + p * 256 + xcol]) = xr[p];
+    }
+    u32x4_t cur[NT][4];
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) cur[j][u] = a[j][u];
+    __syncthreads();
+    if (ch + 1 < chunks) load_chunk(ch + 1);
+    const int s0 = ch * (LKC / 32) + wave * 4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (s0 + u < steps) {
+        const u32x4_t b = *(const u32x4_t*)(&xs[buf][(lane & 15) * LLD + (wave * 4 + u) * 32 + kofs]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(cur[j][u]), as_frag(b), acc[j], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][j][lane * 4 + r] = acc[j][r];
+  __syncthreads();
+  for (int e = tid; e < NT * 256; e += 512) {
+    const int j = e / 256, q = e % 256;
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < WAVES; ++i) v += red[i][j][q];
+    const int l = q / 4, r = q % 4;
+    const int n = n0 + j * 16 + (l >> 4) * 4 + r;
+    const int m = l & 15;
     if (n < N && m < M) store_out(out, mode, (size_t)m * N + n, v);
   }
 }
@@ -184,16 +297,76 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __re
 // In the skinny kernel x is the second operand, so the result lane holds weight rows
 // (l / 16) * 4 + r and activation row l % 16; see the index arithmetic there.
 
+// Tuning knobs of the skinny kernel (0 = choose by shape); set through tp_linear_tune.
+static int g_tune_waves = 0, g_tune_nt = 0, g_tune_depth = 0;   // depth 9 selects the LDS kernel
+
+extern "C" void tp_linear_tune(int waves, int nt, int depth) {
+  g_tune_waves = waves;
+  g_tune_nt = nt;
+  g_tune_depth = depth;
+}
+
+template <int MT, int NT, int WAVES, int DEPTH>
+static void launch_skinny4(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s) {
+  const int blocks = (N + 16 * NT - 1) / (16 * NT);
+  hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, NT, WAVES, DEPTH>), dim3(blocks), dim3(WAVES * 64), 0, s, x, w, out,
+                     mode, M, N, K);
+}
+
 template <int MT>
 static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s) {
-  const int blocks = (N + 15) / 16;
-  // enough waves to keep loads in flight, but every wave should get at least a few steps
-  if (K / 32 >= 64 && MT <= 2)
-    hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, 16>), dim3(blocks), dim3(16 * 64), 0, s, x, w, out, mode, M, N, K);
-  else if (K / 32 >= 16)
-    hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, 8>), dim3(blocks), dim3(8 * 64), 0, s, x, w, out, mode, M, N, K);
-  else
-    hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, 2>), dim3(blocks), dim3(2 * 64), 0, s, x, w, out, mode, M, N, K);
+  // every wave should get at least one run of four steps; small N wants many waves per block
+  // (one block per 16 columns is all the parallelism there is), large N fewer and two row tiles
+  // Measured on MI355X at Llama-8B shapes: eight waves with two runs in flight each stream
+  // fastest (5.7-6.3 TB/s with one activation row); wider blocks or two row tiles never won.
+  const int runs = K / 128;
+  int waves = runs >= 8 ? 8 : (runs >= 4 ? 4 : 2);
+  int nt = 1;
+  int depth = (runs >= 2 * waves && MT <= 2) ? 2 : 1;
+  if (g_tune_waves) waves = g_tune_waves;
+  if (g_tune_nt) nt = g_tune_nt;
+  if (g_tune_depth) depth = g_tune_depth;
+  if constexpr (MT == 1) {
+    // several activation rows: feed them through LDS, unless K is so long that the barrier per
+    // chunk costs more than the gather (measured: K = 14336 is faster without)
+    bool lds = M > 1 && K >= 2 * LKC && K <= 8 * LKC;
+    if (g_tune_depth) lds = g_tune_depth == 9;
+    if (lds) {
+      if (nt > 2) nt = 2;
+      const int blocks = (N + 16 * nt - 1) / (16 * nt);
+      if (nt == 2)
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K);
+      else
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K);
+      return;
+    }
+  }
+  if (MT > 2 && waves > 8) waves = 8;       // LDS for the partial tiles
+  if (MT > 1) nt = 1;
+  if (MT > 2 || nt > 2) depth = 1;           // registers
+#define CASE(NT_, W_, D_) \
+  if (nt == NT_ && waves == W_ && depth == D_) return launch_skinny4<MT, NT_, W_, D_>(x, w, out, mode, M, N, K, s)
+  CASE(1, 16, 1);
+  CASE(1, 8, 1);
+  CASE(1, 4, 1);
+  CASE(1, 2, 1);
+  if constexpr (MT <= 2) {
+    CASE(1, 16, 2);
+    CASE(1, 8, 2);
+    CASE(1, 4, 2);
+  }
+  if constexpr (MT == 1) {
+    CASE(2, 16, 1);
+    CASE(2, 8, 1);
+    CASE(2, 4, 1);
+    CASE(2, 16, 2);
+    CASE(2, 8, 2);
+    CASE(2, 4, 2);
+    CASE(4, 8, 1);
+    CASE(4, 4, 1);
+  }
+#undef CASE
+  launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, s);
 }
 
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
