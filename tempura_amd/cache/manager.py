@@ -166,6 +166,8 @@ class CacheManager:
         """Physical cache rows (page * page_size + offset) of positions start..start+n-1."""
         table = self._requests[rid].tables[g]
         pos = np.arange(start, start + n, dtype=np.int64)
+        if start < 0 or (start + n - 1) // self.page_size >= len(table):
+            raise RuntimeError(f"request {rid!r}: positions {start}..{start + n - 1} have no page reserved")
         pages = np.asarray(table, dtype=np.int64)[pos // self.page_size]
         if (pages < 0).any():
             raise RuntimeError(f"request {rid!r}: positions {start}..{start + n - 1} have no page reserved")

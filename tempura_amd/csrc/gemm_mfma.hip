@@ -21,7 +21,11 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
-enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_ACC_F32 = 2 };
+// OUT_SWIGLU: the weight rows alternate eight gate rows and eight up rows; output column
+// 8*b + i is silu(row 16*b + i) * (row 16*b + 8 + i), stored as bfloat16 [M, N / 2].
+enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_ACC_F32 = 2, OUT_SWIGLU = 3 };
+
+__device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
 __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 
@@ -112,7 +116,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
     const int l = q / 4, r = q % 4;
     const int n = n0 + j * 16 + (l >> 4) * 4 + r;   // weight row = output column
     const int m = t * 16 + (l & 15);
-    if (n < N && m < M) store_out(out, mode, (size_t)m * N + n, v);
+    if (mode == OUT_SWIGLU) {
+      if ((l >> 4) < 2 && n + 8 < N && m < M) {       // a gate row: its up row is eight further on
+        float u = 0.f;
+#pragma unroll
+        for (int i = 0; i < WAVES; ++i) u += red[i][jt][q + 128];
+        ((bf16_t*)out)[(size_t)m * (N / 2) + (n0 + j * 16) / 2 + (l >> 4) * 4 + r] = float_to_bf16(silu_mul(v, u));
+      }
+    } else if (n < N && m < M) {
+      store_out(out, mode, (size_t)m * N + n, v);
+    }
   }
 }
 
@@ -207,7 +220,16 @@ __global__ __launch_bounds__(512) void gemm_skinny_lds_kernel(const bf16_t* __re
     const int l = q / 4, r = q % 4;
     const int n = n0 + j * 16 + (l >> 4) * 4 + r;
     const int m = l & 15;
-    if (n < N && m < M) store_out(out, mode, (size_t)m * N + n, v);
+    if (mode == OUT_SWIGLU) {
+      if ((l >> 4) < 2 && n + 8 < N && m < M) {
+        float u = 0.f;
+#pragma unroll
+        for (int i = 0; i < WAVES; ++i) u += red[i][j][q + 128];
+        ((bf16_t*)out)[(size_t)m * (N / 2) + (n0 + j * 16) / 2 + (l >> 4) * 4 + r] = float_to_bf16(silu_mul(v, u));
+      }
+    } else if (n < N && m < M) {
+      store_out(out, mode, (size_t)m * N + n, v);
+    }
   }
 }
 
@@ -288,7 +310,13 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __re
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int n = n0 + wn * 64 + j * 16 + (lane & 15);
-        if (n < N) store_out(out, mode, (size_t)m * N + n, acc[i][j][r]);
+        if (mode == OUT_SWIGLU) {
+          const float u = __shfl_xor(acc[i][j][r], 8, 64);   // the up row sits eight columns to the right
+          if ((lane & 8) == 0 && n + 8 < N)
+            ((bf16_t*)out)[(size_t)m * (N / 2) + (n0 + wn * 64 + j * 16) / 2 + (lane & 7)] = float_to_bf16(silu_mul(acc[i][j][r], u));
+        } else if (n < N) {
+          store_out(out, mode, (size_t)m * N + n, acc[i][j][r]);
+        }
       }
     }
   }
@@ -369,11 +397,13 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
   launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, s);
 }
 
+// accumulate: 0 store, 1 add into the float32 output, 2 gated-SiLU epilogue (see OUT_SWIGLU)
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
                    hipStream_t s) {
   if (K % 32 != 0) return -1;
   if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return -1;
-  const int mode = accumulate ? OUT_ACC_F32 : (out_dt == TP_F32 ? OUT_F32 : OUT_BF16);
+  if (accumulate == 2 && (N % 16 != 0 || out_dt != TP_BF16)) return -1;
+  const int mode = accumulate == 2 ? OUT_SWIGLU : (accumulate ? OUT_ACC_F32 : (out_dt == TP_F32 ? OUT_F32 : OUT_BF16));
   const bf16_t* xb = (const bf16_t*)x;
   const bf16_t* wb = (const bf16_t*)w;
   if (M <= 64) {

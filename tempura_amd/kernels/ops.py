@@ -139,6 +139,34 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
 allow_mfma = True
 
 
+def gated_layout_ok(n_rows: int, k: int) -> bool:
+    """Whether ``linear_swiglu`` takes a weight of 2 * n_rows rows and k columns."""
+    return n_rows % 8 == 0 and k % 32 == 0
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """[i, k], [i, k] -> [2i, k] with eight gate rows and eight up rows in turn, the layout
+    ``linear_swiglu`` reads."""
+    i, k = gate.shape
+    return torch.stack([gate.reshape(i // 8, 8, k), up.reshape(i // 8, 8, k)], dim=1).reshape(2 * i, k).contiguous()
+
+
+def linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """bfloat16 x [m, k], interleaved gate/up weight [2i, k] -> bfloat16 [m, i] = silu(x g^T) * (x u^T),
+    the gate applied to the float32 accumulators (no rounding in between)."""
+    if _backend is not None:
+        return _backend.linear_swiglu(x, w)
+    _dev_ok(x, w)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_swiglu: shapes {tuple(x.shape)} x {tuple(w.shape)}")
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "linear_swiglu: operands must be bfloat16")
+    m, k = x.shape
+    n = w.shape[0]
+    _need(n % 16 == 0 and k % 32 == 0, "linear_swiglu: needs 2i % 16 == 0 and k % 32 == 0")
+    out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    _call("tp_linear", _ptr(x), _ptr(w), _BF16, _ptr(out), _BF16, 2, m, n, k, 1, _stream())
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
            residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x [m, k] @ w[n, k]^T -> out_dtype [m, n]; with ``residual`` (float32 [m, n]) the product is

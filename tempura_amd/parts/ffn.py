@@ -30,13 +30,22 @@ class SwiGLU(FeedForward):
 
     def load_weights(self, get):
         w = self.spec.weights
-        # gate rows then up rows in one matrix: one product instead of two.
-        self.w13 = torch.cat([self._to_device(get(w["gate"])), self._to_device(get(w["up"]))], dim=0).contiguous()
+        gate, up = self._to_device(get(w["gate"])), self._to_device(get(w["up"]))
+        # One matrix, one product instead of two.  In bfloat16 the rows alternate eight of gate and
+        # eight of up, so that the product's epilogue applies silu(g) * u to its float32 sums.
+        self.fused = self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
+        if self.fused:
+            self.w13 = ops.interleave_gate_up(gate, up)
+        else:
+            self.w13 = torch.cat([gate, up], dim=0).contiguous()
         self.w2 = self._to_device(get(w["down"]))
 
     def forward(self, x, ctx, residual):
-        gu = ops.linear(x, self.w13, torch.float32 if self.dtype == torch.float32 else self.dtype)
-        a = ops.swiglu(gu, self.dtype)
+        if self.fused:
+            a = ops.linear_swiglu(x, self.w13)
+        else:
+            gu = ops.linear(x, self.w13, torch.float32)
+            a = ops.swiglu(gu, self.dtype)
         ops.linear(a, self.w2, torch.float32, residual=residual)
 
 

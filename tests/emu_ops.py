@@ -28,6 +28,11 @@ class EmuOps:
             return residual
         return y.to(out_dtype)
 
+    def linear_swiglu(self, x, w):
+        y = (x.double() @ w.double().T).reshape(x.shape[0], -1, 2, 8)      # eight gate rows, eight up rows in turn
+        g, u = y[:, :, 0].reshape(x.shape[0], -1), y[:, :, 1].reshape(x.shape[0], -1)
+        return (g / (1.0 + torch.exp(-g)) * u).to(torch.bfloat16)
+
     def rope_kv_write(self, qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads, num_kv_heads,
                       head_dim, k_cache, v_cache, q_dtype):
         n = qkv.shape[0]

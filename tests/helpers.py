@@ -138,3 +138,58 @@ def schedule_mixed(lengths: Dict[str, int], max_tokens: int, seed: int, max_live
         if entries:
             steps.append((entries, end))
     return steps
+
+
+# ---- replaying a schedule through a runner -----------------------------------------------------
+LENGTHS = {"A": {"a0": 5, "a1": 17, "a2": 33, "a3": 150, "a4": 97, "a5": 64},
+           "B": {"b0": 1, "b1": 9, "b2": 40, "b3": 63, "b4": 120, "b5": 201},
+           "C": {"c0": 3, "c1": 49, "c2": 130, "c3": 75, "c4": 25, "c5": 88}}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 32}
+
+
+def requests_for(name: str) -> Dict[str, List[int]]:
+    vocab = CONFIGS[name].vocab_size
+    return {rid: random_tokens(vocab, n, seed=1000 + i) for i, (rid, n) in enumerate(LENGTHS[name].items())}
+
+
+def schedule_for(name: str, mode: str):
+    """(steps, max_tokens) of a replay mode for a configuration's requests."""
+    lengths = LENGTHS[name]
+    if mode == "mixed":
+        # room for about three of the requests: pages of finished ones must be used again
+        max_tokens = sum(sorted(roundup(n, 64) for n in lengths.values())[-2:]) + 64
+        return schedule_mixed(lengths, max_tokens, seed=5), max_tokens
+    max_tokens = max(roundup(n, 64) for n in lengths.values())
+    fn = {"whole": schedule_whole, "bulk_tail": schedule_bulk_tail, "portions": schedule_portions}[mode]
+    return fn(lengths), max_tokens
+
+
+def run_schedule(runner, requests, steps):
+    """Run a schedule asking for logits everywhere; returns {rid: [len, vocab] float32 on the host}."""
+    from tempura_amd.engine.runner import StepEntry
+    got = {rid: [None] * len(t) for rid, t in requests.items()}
+    for entries, end in steps:
+        batch = []
+        for rid, start, count in entries:
+            if not runner.has_request(rid):
+                runner.add_request(rid)
+            assert runner.num_cached(rid) == start
+            batch.append(StepEntry(rid, requests[rid][start:start + count], list(range(count))))
+        logits = runner.step(batch).cpu()
+        row = 0
+        for rid, start, count in entries:
+            for i in range(count):
+                got[rid][start + i] = logits[row].clone()
+                row += 1
+        for rid in end:
+            runner.end_request(rid)
+        runner.cache.check()
+    return {rid: torch.stack(rows) for rid, rows in got.items()}
+
+
+def first_difference(got: torch.Tensor, ref: torch.Tensor, tol: float):
+    """Index of the first position whose logits differ by more than tol (relative to the largest logit), or None."""
+    scale = float(ref.double().abs().max())
+    err = (got.double() - ref.double()).abs().amax(dim=-1) / scale
+    bad = torch.nonzero(err > tol)
+    return None if bad.numel() == 0 else int(bad[0])

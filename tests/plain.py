@@ -142,8 +142,11 @@ def layer_window(cfg: dict, layer: int) -> Optional[int]:
     return None
 
 
-def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=torch.float64) -> torch.Tensor:
+def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=torch.float64,
+            position_offset: int = 0) -> torch.Tensor:
     """Logits [T, vocab] at every position of one whole sequence, no cache.
+    ``position_offset`` shifts every position (positions are session.position + t,
+    /root/reference/engine/src/model.rs:686-688); only distances count, so logits must not change.
     Order inside a layer: norm, q/k/v, rope on q and k, attention, o, add, norm, feed-forward, add
     (/root/reference/engine/src/model.rs:952-1314); then final norm and output projection
     (model.rs:1355-1398), the output matrix being the embedding when the file has none
@@ -160,7 +163,7 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
         rs = None
     inv_freq = rope_inv_freq(D, theta, rs)
     T = len(tokens)
-    pos = torch.arange(T)
+    pos = torch.arange(T) + position_offset
     h = W["model.embed_tokens.weight"][torch.tensor(tokens)]           # model.rs:672-684, no scaling
     scale = 1.0 / math.sqrt(D)                                          # model.rs:1078
     for l in range(cfg["num_hidden_layers"]):

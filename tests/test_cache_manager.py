@@ -1,0 +1,152 @@
+"""The cache manager's bookkeeping (CPU): no page lost, held twice or freed twice, under random
+orders of requests; windows give pages back; reservations fail without side effects."""
+import random
+
+import pytest
+
+from tempura_amd.cache import CacheManager, PagePool, PagesExhausted
+from tempura_amd.parts import CacheSpec
+
+FULL = CacheSpec("full", 2, 16)
+WIN = CacheSpec("window", 2, 16, window=24)
+
+
+def test_page_pool_conservation_and_double_free():
+    # invariant available + in_use == total (/root/reference/kernel-api/src/lib.rs:604-618)
+    p = PagePool(4)
+    a, b = p.alloc(), p.alloc()
+    assert p.num_free == 2 and p.num_held == 2 and a != b
+    p.free(a)
+    with pytest.raises(ValueError, match="freed twice"):
+        p.free(a)
+    with pytest.raises(ValueError, match="out of range"):
+        p.free(9)
+    assert p.alloc() == a                       # most recently freed page is used again first
+    p.alloc(), p.alloc()
+    with pytest.raises(PagesExhausted):
+        p.alloc()
+    p.check()
+
+
+def test_reserve_commit_release():
+    m = CacheManager([FULL], page_size=8, num_pages=6, max_requests=2)
+    m.add("a")
+    assert m.pages_needed("a", 17) == [3]
+    m.reserve("a", 17)
+    m.commit("a", 17)
+    assert m.num_tokens("a") == 17 and len(m.table("a", 0)) == 3 and m.free_pages() == [3]
+    assert m.pages_needed("a", 7) == [0] and m.pages_needed("a", 8) == [1]
+    slots = m.slots("a", 0, 15, 2)             # positions 15, 16: last row of page 1, first of page 2
+    t = m.table("a", 0)
+    assert list(slots) == [t[1] * 8 + 7, t[2] * 8 + 0]
+    m.add("b")
+    with pytest.raises(PagesExhausted) as ei:
+        m.reserve("b", 8 * 4)
+    assert ei.value.need == 4 and ei.value.free == 3
+    assert m.table("b", 0) == [] and m.free_pages() == [3]        # nothing changed
+    m.check()
+    m.release("a")
+    assert m.free_pages() == [6]
+    with pytest.raises(ValueError, match="not live"):
+        m.release("a")
+    with pytest.raises(RuntimeError, match="no page reserved"):
+        m.slots("b", 0, 0, 1)
+    m.check()
+
+
+def test_state_slots():
+    m = CacheManager([FULL], 8, 4, max_requests=2)
+    s0, s1 = m.add("a"), m.add("b")
+    assert {s0, s1} == {0, 1}
+    with pytest.raises(RuntimeError, match="no free state slot"):
+        m.add("c")
+    with pytest.raises(ValueError, match="already live"):
+        m.add("a")
+    m.release("a")
+    assert m.add("c") == s0
+    m.check()
+
+
+def test_window_group_gives_pages_back():
+    m = CacheManager([FULL, WIN], page_size=8, num_pages=[32, 12], max_requests=1)
+    m.add("a")
+    n = 0
+    for chunk in [5, 20, 3, 1, 1, 40, 1, 1, 1, 17, 1]:
+        m.reserve("a", chunk)
+        m.commit("a", chunk)
+        n += chunk
+        t_full, t_win = m.table("a", 0), m.table("a", 1)
+        assert all(p >= 0 for p in t_full) and len(t_full) == (n + 7) // 8
+        first_visible = max(0, n - 24 + 1)       # the next query (position n) sees keys from here
+        for lp, p in enumerate(t_win):
+            if (lp + 1) * 8 <= first_visible:
+                assert p == -1, f"page {lp} should be free after {n} tokens"
+            else:
+                assert p >= 0
+        m.check()
+    # between steps the window group holds the window and a page of slack, whatever the length
+    assert m.pools[1].num_held <= 24 // 8 + 2
+    m.release("a")
+    assert m.free_pages() == [32, 12]
+
+
+def test_window_pool_smaller_than_sequence():
+    """A long request runs in a window pool far smaller than its length, because pages come back."""
+    m = CacheManager([WIN], page_size=8, num_pages=6, max_requests=1)
+    m.add("a")
+    for _ in range(300):
+        m.reserve("a", 1)
+        m.commit("a", 1)
+    assert m.num_tokens("a") == 300 and m.pools[0].num_held <= 4
+    m.check()
+
+
+def test_truncate():
+    m = CacheManager([FULL], 8, 8, 1)
+    m.add("a")
+    m.reserve("a", 30)
+    m.commit("a", 30)
+    m.truncate("a", 9)
+    assert m.num_tokens("a") == 9 and len(m.table("a", 0)) == 2 and m.free_pages() == [6]
+    m.check()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_of_requests(seed):
+    """Requests arrive, grow by random portions, end in random order; the invariants hold throughout and
+    every page comes back."""
+    g = random.Random(seed)
+    groups = [FULL, WIN] if seed % 2 else [FULL]
+    m = CacheManager(groups, page_size=g.choice([4, 8, 16]), num_pages=40, max_requests=5)
+    live = {}
+    next_id = 0
+    for _ in range(400):
+        op = g.random()
+        if op < 0.15 and len(live) < 5:
+            m.add(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif op < 0.85 and live:
+            rid = g.choice(list(live))
+            n = g.choice([1, 1, 1, 2, 3, 7, 16, 33])
+            before = (m.free_pages(), [list(t) for t in m._requests[rid].tables])
+            try:
+                m.reserve(rid, n)
+            except PagesExhausted:
+                assert (m.free_pages(), [list(t) for t in m._requests[rid].tables]) == before
+                victim = g.choice(list(live))
+                m.release(victim)
+                del live[victim]
+            else:
+                m.commit(rid, n)
+                live[rid] += n
+                assert m.num_tokens(rid) == live[rid]
+        elif live:
+            rid = g.choice(list(live))
+            m.release(rid)
+            del live[rid]
+        m.check()
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert m.free_pages() == [40] * len(groups)

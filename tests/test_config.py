@@ -1,0 +1,117 @@
+"""Configuration and registry (CPU)."""
+import json
+
+import pytest
+
+from tempura_amd.config import (ConfigError, LlamaConfig, PRESETS, architecture_names, load_config,
+                                register_architecture)
+
+BASE = {"architectures": ["LlamaForCausalLM"], "hidden_size": 64, "num_attention_heads": 4, "num_hidden_layers": 2,
+        "intermediate_size": 192, "vocab_size": 256}
+
+
+def test_llama_json_and_defaults():
+    # defaults as in /root/reference/engine/src/config.rs:400-432
+    c = LlamaConfig.from_json(json.dumps(BASE))
+    assert (c.hidden_size, c.num_attention_heads, c.num_hidden_layers, c.intermediate_size, c.vocab_size) == (64, 4, 2, 192, 256)
+    assert c.num_key_value_heads == 4 and c.head_dim == 16 and c.max_position_embeddings == 4096
+    assert c.rope_theta == 10000.0 and c.rms_norm_eps == 1e-5 and c.rope_scaling is None
+    assert not c.tie_word_embeddings and c.sliding_window is None
+
+
+def test_every_key_is_read():
+    d = dict(BASE, num_key_value_heads=2, head_dim=24, max_position_embeddings=777, rope_theta=5e5, rms_norm_eps=3e-6,
+             tie_word_embeddings=True, eos_token_id=[7, 9], bos_token_id=1, sliding_window=32,
+             rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                           "original_max_position_embeddings": 64})
+    c = LlamaConfig.from_dict(d)
+    assert (c.num_key_value_heads, c.head_dim, c.max_position_embeddings) == (2, 24, 777)
+    assert c.rope_theta == 5e5 and c.rms_norm_eps == 3e-6 and c.tie_word_embeddings
+    assert c.eos_token_id == [7, 9] and c.bos_token_id == 1 and c.sliding_window == 32
+    assert c.rope_scaling.factor == 8.0 and c.rope_scaling.original_max_position_embeddings == 64
+    # and survives a round trip through its own config.json
+    c2 = LlamaConfig.from_json(c.to_json())
+    assert c2 == c
+
+
+def test_rope_scaling_type_and_rope_type_keys():
+    # the reference reads "type" only (config.rs:466); released files say "rope_type"
+    for key in ("type", "rope_type"):
+        c = LlamaConfig.from_dict(dict(BASE, rope_scaling={key: "llama3", "factor": 2.0}))
+        assert c.rope_scaling.rope_type == "llama3" and c.rope_scaling.factor == 2.0
+        assert c.rope_scaling.low_freq_factor == 1.0 and c.rope_scaling.high_freq_factor == 4.0
+        assert c.rope_scaling.original_max_position_embeddings == 4096      # defaults to max positions
+    with pytest.raises(ConfigError, match="yarn"):
+        LlamaConfig.from_dict(dict(BASE, rope_scaling={"type": "yarn", "factor": 2.0}))
+
+
+def test_layer_norm_eps_fallback_key():
+    assert LlamaConfig.from_dict(dict(BASE, layer_norm_eps=1e-3)).rms_norm_eps == 1e-3
+
+
+@pytest.mark.parametrize("key", ["hidden_size", "num_attention_heads", "num_hidden_layers", "intermediate_size", "vocab_size"])
+def test_missing_field(key):
+    d = dict(BASE)
+    del d[key]
+    with pytest.raises(ConfigError, match=key):
+        LlamaConfig.from_dict(d)
+
+
+def test_malformed_and_invalid():
+    with pytest.raises(ConfigError, match="malformed"):
+        LlamaConfig.from_json("{not json")
+    with pytest.raises(ConfigError, match="multiple"):
+        LlamaConfig.from_dict(dict(BASE, num_key_value_heads=3))
+    with pytest.raises(ConfigError, match="even"):
+        LlamaConfig.from_dict(dict(BASE, head_dim=15))
+    with pytest.raises(ConfigError, match="hidden_act"):
+        LlamaConfig.from_dict(dict(BASE, hidden_act="gelu"))
+    with pytest.raises(ConfigError, match="attention_bias"):
+        LlamaConfig.from_dict(dict(BASE, attention_bias=True))
+    with pytest.raises(ConfigError, match="integer"):
+        LlamaConfig.from_dict(dict(BASE, hidden_size="64"))
+    with pytest.raises(ConfigError, match="layer_types"):
+        LlamaConfig.from_dict(dict(BASE, sliding_window=8, layer_types=["full_attention"]))
+
+
+def test_registry(tmp_path):
+    assert "LlamaForCausalLM" in architecture_names() and "llama" in architecture_names()
+    (tmp_path / "config.json").write_text(json.dumps(BASE))
+    assert isinstance(load_config(str(tmp_path)), LlamaConfig)
+    (tmp_path / "config.json").write_text(json.dumps(dict(BASE, architectures=["MysteryForCausalLM"])))
+    with pytest.raises(ConfigError, match="unknown architecture"):      # no silent default to Llama
+        load_config(str(tmp_path))
+    d = dict(BASE)
+    del d["architectures"]
+    (tmp_path / "config.json").write_text(json.dumps(dict(d, model_type="llama")))
+    assert isinstance(load_config(str(tmp_path)), LlamaConfig)
+    with pytest.raises(ConfigError, match="cannot read"):
+        load_config(str(tmp_path / "nowhere"))
+
+    class Other(LlamaConfig):
+        pass
+    register_architecture("OtherForCausalLM", Other)
+    (tmp_path / "config.json").write_text(json.dumps(dict(BASE, architectures=["OtherForCausalLM"])))
+    assert type(load_config(str(tmp_path))) is Other
+
+
+def test_spec_names_and_windows():
+    c = LlamaConfig.from_dict(dict(BASE, num_hidden_layers=3, sliding_window=16,
+                                   layer_types=["sliding_attention", "full_attention", "sliding_attention"]))
+    spec = c.build_spec()
+    assert len(spec.layers) == 3 and [call.layer for call in spec.order] == [0, 1, 2]
+    assert [l.mixer.params["window"] for l in spec.layers] == [16, None, 16]
+    assert spec.layers[1].mixer.weights["q"] == "model.layers.1.self_attn.q_proj.weight"
+    assert spec.layers[2].ffn.weights["down"] == "model.layers.2.mlp.down_proj.weight"
+    assert spec.final_norm.weights["weight"] == "model.norm.weight"
+    from tempura_amd.parts import expected_weights
+    names = expected_weights(spec)
+    assert len([n for n, i in names.items() if not i.optional]) == 2 + 9 * 3     # 3 + 9 L with lm_head (weights.rs:205-228)
+    assert names["lm_head.weight"].optional
+
+
+def test_presets_match_published_sizes():
+    c = PRESETS["llama-3.1-8b"]
+    assert abs(c.num_parameters() - 8.03e9) < 0.01e9
+    assert c.kv_bytes_per_token(2) == 128 * 1024           # 128 KiB per token (/root/reference/AGENTS.md:396-397)
+    assert abs(PRESETS["llama-3.1-70b"].num_parameters() - 70.55e9) < 0.05e9

@@ -1,0 +1,171 @@
+"""The engine's bookkeeping on the host (CPU): with the kernel operations replaced by their plain PyTorch
+stand-ins (tests/emu_ops.py), every way of cutting and batching must reproduce the plain implementation.
+A difference here is a fault of the cache or the batch, not of a kernel."""
+import pytest
+import torch
+
+import helpers
+import plain
+from emu_ops import EmuOps
+
+
+@pytest.fixture(autouse=True)
+def host_ops():
+    from tempura_amd.kernels import ops
+    ops.set_backend(EmuOps())
+    yield
+    ops.set_backend(None)
+
+
+def _runner(tiny_dirs, name, max_tokens):
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    ps = helpers.PAGE_SIZE[name]
+    model = load_model(tiny_dirs.path(name, "float32"), "float32", "cpu")
+    return ModelRunner(model, ps, (max_tokens + ps - 1) // ps, max_requests=4)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
+def test_every_cutting_matches_plain(tiny_dirs, name, mode):
+    cfg, W = tiny_dirs.plain_model(name)
+    requests = helpers.requests_for(name)
+    steps, max_tokens = helpers.schedule_for(name, mode)
+    runner = _runner(tiny_dirs, name, max_tokens)
+    got = helpers.run_schedule(runner, requests, steps)
+    for rid, toks in requests.items():
+        ref = plain.forward(cfg, W, toks)
+        bad = helpers.first_difference(got[rid], ref, 1e-6)
+        assert bad is None, f"{name}/{mode}: request {rid} first differs at position {bad}"
+    assert not runner.cache.live_requests()
+    assert runner.cache.free_pages() == [p.num_pages for p in runner.cache.pools]
+
+
+def test_mixed_schedule_really_reuses_pages(tiny_dirs):
+    steps, max_tokens = helpers.schedule_for("A", "mixed")
+    runner = _runner(tiny_dirs, "A", max_tokens)
+    seen, reused = {}, 0
+    requests = helpers.requests_for("A")
+    from tempura_amd.engine.runner import StepEntry
+    for entries, end in steps:
+        batch = []
+        for rid, s, c in entries:
+            if not runner.has_request(rid):
+                runner.add_request(rid)
+            batch.append(StepEntry(rid, requests[rid][s:s + c], []))
+        runner.step(batch)
+        for rid, _, _ in entries:
+            for p in runner.cache.table(rid, 0):
+                if p in seen and seen[p] != rid:
+                    reused += 1
+                seen[p] = rid
+        assert max(len(e) for e, _ in steps) >= 3
+        for rid in end:
+            runner.end_request(rid)
+    assert reused > 0, "the pool is so small that pages pass from finished requests to later ones"
+    assert max(len(entries) for entries, _ in steps) == 4
+
+
+def test_layer_order_is_data(tiny_dirs):
+    """A run order that names a layer twice (its second call has a cache slot of its own) and lets a call read
+    the cache another call wrote, against the same thing written out with the plain parts."""
+    import math
+    from tempura_amd.config import LayerCall, LlamaConfig
+    from tempura_amd.engine.model import CausalLM
+    from tempura_amd.engine.runner import ModelRunner, StepEntry
+    from tempura_amd.weights import random_weights
+    cfg = LlamaConfig.from_dict(helpers.CONFIGS["A"].to_dict())
+    spec = cfg.build_spec()
+    spec.order = [LayerCall(0, cache=0), LayerCall(1, cache=1), LayerCall(0, cache=2), LayerCall(1, cache=1)]
+    model = CausalLM(spec, torch.float32, torch.device("cpu"))
+    assert model.call_writes == [True, True, True, False] and model.slots_per_group == [3]
+    W = {k: v.double() for k, v in random_weights(cfg, seed=5, std=helpers.STD, norm_jitter=0.2, dtype="float32").items()}
+    model.load_weights(lambda n, optional=False: W[n].float())
+    runner = ModelRunner(model, 16, 8, 2)
+    toks = helpers.random_tokens(cfg.vocab_size, 37, seed=9)
+    runner.add_request("x")
+    got = torch.cat([runner.step([StepEntry("x", toks[:20], list(range(20)))]),
+                     runner.step([StepEntry("x", toks[20:], list(range(17)))])])
+
+    T, D, nH, nKV = 37, 16, 4, 2
+    inv = plain.rope_inv_freq(D, 10000.0, None)
+    pos = torch.arange(T)
+    h = W["model.embed_tokens.weight"][torch.tensor(toks)]
+    kv_of_slot = {}
+    for layer, slot, writes in [(0, 0, True), (1, 1, True), (0, 2, True), (1, 1, False)]:
+        p = f"model.layers.{layer}."
+        x = plain.rmsnorm(h, W[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        q = plain.rope((x @ W[p + "self_attn.q_proj.weight"].T).reshape(T, nH, D), pos, inv)
+        if writes:
+            k = plain.rope((x @ W[p + "self_attn.k_proj.weight"].T).reshape(T, nKV, D), pos, inv)
+            v = (x @ W[p + "self_attn.v_proj.weight"].T).reshape(T, nKV, D)
+            kv_of_slot[slot] = (k, v)
+        k, v = kv_of_slot[slot]
+        h = h + plain.attention(q, k, v, 1 / math.sqrt(D)) @ W[p + "self_attn.o_proj.weight"].T
+        x = plain.rmsnorm(h, W[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
+        h = h + plain.swiglu_ffn(x, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+    ref = plain.rmsnorm(h, W["model.norm.weight"], cfg.rms_norm_eps) @ W["lm_head.weight"].T
+    assert helpers.rel_err(got, ref) < 1e-6
+
+
+def test_step_rejects_bad_batches(tiny_dirs):
+    from tempura_amd.cache import PagesExhausted
+    from tempura_amd.engine.runner import StepEntry
+    runner = _runner(tiny_dirs, "A", 64)
+    runner.add_request("a")
+    with pytest.raises(ValueError, match="not live"):
+        runner.step([StepEntry("nobody", [1], [0])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.step([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(ValueError, match="vocabulary"):
+        runner.step([StepEntry("a", [256], [])])
+    with pytest.raises(ValueError, match="wanted place"):
+        runner.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(ValueError, match="at least one token"):
+        runner.step([StepEntry("a", [], [])])
+    with pytest.raises(PagesExhausted):
+        runner.step([StepEntry("a", [1] * 65, [])])
+    assert runner.num_cached("a") == 0 and runner.cache.free_pages() == [4]      # nothing happened
+    runner.cache.check()
+
+
+def test_generate_and_preemption_on_host(tiny_dirs):
+    from tempura_amd.engine import Engine
+    from tempura_amd.sampling import SamplingParams
+    cfg, W = tiny_dirs.plain_model("A")
+    prompts = [helpers.random_tokens(256, n, seed=700 + n) for n in (5, 17, 33, 26)]
+    params = SamplingParams(temperature=0.0, max_new_tokens=12)
+    kw = dict(dtype="float32", device="cpu", page_size=16, max_batch_size=4, max_num_batched_tokens=24, prefill_chunk_size=16)
+    want = [plain.greedy_generate(cfg, W, p, 12) for p in prompts]
+    roomy = Engine(tiny_dirs.path("A"), kv_pages=32, **kw)
+    assert roomy.generate(prompts, params) == want
+    tight = Engine(tiny_dirs.path("A"), kv_pages=6, **kw)
+    assert tight.generate(prompts, params) == want
+    assert tight.stats()["preemptions"] > 0 and tight.runner.cache.free_pages() == [6]
+
+
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    """A mixer defined in the tests, with per-request state and no paged cache, in an architecture of its own."""
+    import toy_parts
+    from tempura_amd.config import load_config
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner, StepEntry
+    from tempura_amd.weights import write_random_model
+    cfg = toy_parts.ToyConfig()
+    d = write_random_model(cfg, str(tmp_path / "toy"), seed=4, std=0.2, norm_jitter=0.1, dtype="float32")
+    assert type(load_config(d)) is toy_parts.ToyConfig
+    model = load_model(d, "float32", "cpu")
+    assert sorted(model.state_specs) == [0, 2] and model.slots_per_group == [1]     # two state layers, one attention layer
+    _, W = plain.read_model_dir(d)
+    runner = ModelRunner(model, 8, 12, max_requests=3)
+    reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30}.items())}
+    ref = {r: toy_parts.plain_toy_forward(cfg, W, t) for r, t in reqs.items()}
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
+             ([("p", 10, 11), ("r", 17, 13)], ["p", "r"])]
+    got = helpers.run_schedule(runner, reqs, steps)
+    for r in reqs:
+        assert helpers.first_difference(got[r], ref[r], 1e-6) is None, r
+    # a state slot used again starts from zero
+    runner.add_request("again")
+    lg = runner.step([StepEntry("again", reqs["q"], list(range(9)))])
+    assert helpers.rel_err(lg, ref["q"]) < 1e-6

@@ -1,0 +1,113 @@
+"""Generation through the entry point on the GPU: greedy tokens against the plain implementation,
+temperature sampling, preemption under a tiny pool, the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import helpers
+import plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _engine(tiny_dirs, name, dtype="float32", **kw):
+    from tempura_amd.engine import Engine
+    from tempura_amd.kernels import ops
+    ops.set_backend(None)
+    args = dict(page_size=helpers.PAGE_SIZE[name], kv_pages=64, max_batch_size=4, max_num_batched_tokens=48,
+                prefill_chunk_size=16)
+    args.update(kw)
+    return Engine(tiny_dirs.path(name, dtype), dtype=dtype, **args)
+
+
+@pytest.mark.parametrize("name,prompt_lens,n_new", [("A", [5, 17, 33], 16), ("B", [1, 9, 40, 63, 120], 24)])
+def test_greedy_generation_matches_plain(tiny_dirs, name, prompt_lens, n_new):
+    from tempura_amd.sampling import SamplingParams
+    cfg, W = tiny_dirs.plain_model(name)
+    prompts = [helpers.random_tokens(cfg["vocab_size"], n, seed=200 + i) for i, n in enumerate(prompt_lens)]
+    eng = _engine(tiny_dirs, name)
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=n_new))
+    for p, o in zip(prompts, outs):
+        assert o == plain.greedy_generate(cfg, W, p, n_new)
+    st = eng.stats()
+    assert st["generated_tokens"] == n_new * len(prompts) and st["graph_steps"] > 0
+    assert eng.runner.cache.free_pages() == [64] * len(eng.runner.cache.pools)
+    # forward(): the last position's logits of a fresh request
+    lg = eng.forward(prompts[1])
+    assert helpers.rel_err(lg, plain.forward(cfg, W, prompts[1])[-1]) <= helpers.TOL["float32"]
+
+
+def test_bfloat16_greedy_generation_runs_and_is_repeatable(tiny_dirs):
+    from tempura_amd.sampling import SamplingParams
+    prompts = [helpers.random_tokens(300, n, seed=300 + n) for n in (3, 50, 21)]
+    a = _engine(tiny_dirs, "C", "bfloat16").generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=20))
+    b = _engine(tiny_dirs, "C", "bfloat16", use_graph=False).generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=20))
+    assert a == b and all(len(o) == 20 for o in a)
+
+
+def test_preemption_by_recompute_keeps_tokens(tiny_dirs):
+    """So few pages that running requests are preempted: every request still gets exactly the tokens it gets
+    with plenty of pages, in greedy and in seeded temperature sampling."""
+    from tempura_amd.sampling import SamplingParams
+    prompts = [helpers.random_tokens(256, n, seed=400 + n) for n in (30, 45, 38, 20)]
+    for params in (SamplingParams(temperature=0.0, max_new_tokens=40),
+                   SamplingParams(temperature=0.8, top_k=0, seed=2, max_new_tokens=40)):
+        roomy = _engine(tiny_dirs, "A", kv_pages=64)
+        want = roomy.generate(prompts, params)
+        assert roomy.stats()["preemptions"] == 0
+        tight = _engine(tiny_dirs, "A", kv_pages=11)        # 176 tokens of cache for 333 tokens of work
+        got = tight.generate(prompts, params)
+        assert tight.stats()["preemptions"] > 0
+        assert got == want
+        assert tight.runner.cache.free_pages() == [11]
+
+
+def test_temperature_sampling_seeded(tiny_dirs):
+    from tempura_amd.sampling import SamplingParams
+    prompts = [helpers.random_tokens(384, n, seed=500 + n) for n in (1, 9, 40)]
+    eng = _engine(tiny_dirs, "B")
+    p = SamplingParams(temperature=0.8, top_k=0, seed=2, max_new_tokens=24)
+    a = eng.generate(prompts, p)
+    b = _engine(tiny_dirs, "B").generate(prompts, p)
+    c = _engine(tiny_dirs, "B").generate(prompts, SamplingParams(temperature=0.8, top_k=0, seed=3, max_new_tokens=24))
+    assert a == b, "same seed, same tokens"
+    assert a != c, "another seed, other tokens"
+    # alone or in a batch: the same tokens (draws depend on the seed and the draw's number only)
+    alone = _engine(tiny_dirs, "B").generate([prompts[2]], p)
+    assert alone[0] == a[2]
+
+
+def test_eos_and_length_limits(tiny_dirs):
+    from tempura_amd.sampling import SamplingParams
+    cfg, W = tiny_dirs.plain_model("A")
+    prompt = helpers.random_tokens(256, 12, seed=600)
+    ref = plain.greedy_generate(cfg, W, prompt, 10)
+    eng = _engine(tiny_dirs, "A")
+    out = eng.generate([prompt], SamplingParams(temperature=0.0, max_new_tokens=10, eos_token_id=[ref[3]]))[0]
+    stop = ref.index(ref[3])
+    assert out == ref[:stop + 1], "generation stops after the first EOS token, which is kept"
+    out = eng.generate([prompt], SamplingParams(temperature=0.0, max_new_tokens=10, eos_token_id=[ref[3]], ignore_eos=True))[0]
+    assert out == ref
+
+
+def test_command_line(tiny_dirs, tmp_path):
+    cfg, W = tiny_dirs.plain_model("A")
+    model = tiny_dirs.path("A", "float32")
+    tempura = os.path.join(ROOT, "bin", "tempura")
+    p = subprocess.run([sys.executable, tempura, "inspect", model, "--json"], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr
+    info = json.loads(p.stdout)
+    assert info["hidden_size"] == 64 and info["kv_heads"] == 2 and info["architecture"] == "LlamaForCausalLM"
+    prompt = helpers.random_tokens(256, 7, seed=601)
+    p = subprocess.run([sys.executable, tempura, "run", "--model", model, "--dtype", "float32", "--prompt-ids",
+                        ",".join(map(str, prompt)), "--max-new-tokens", "6", "--temperature", "0", "--kv-blocks", "16",
+                        "--max-batch-size", "2", "--stats"], capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    rec = json.loads(p.stdout.strip().splitlines()[-1])
+    assert rec["output_ids"] == plain.greedy_generate(cfg, W, prompt, 6) and rec["finish_reason"] == "length"
+    assert '"stats"' in p.stderr

@@ -231,3 +231,51 @@ def test_attention_mfma(heads, kv, d, page):
 
 def test_attention_mfma_long_decode():
     _attention_case(torch.bfloat16, 8, 2, 128, 16, [1, 1], [3000, 2049], 0, seed=16)
+
+
+@pytest.mark.parametrize("dtype,fast", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+def test_attention_window_edge(dtype, fast):
+    """Two keys carry huge scores: the one exactly at the window's edge (position p - w + 1) must be seen,
+    the one just outside (p - w) must not.  A window off by one in either direction changes the answer."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(17)
+    heads, kv, d, page, ctx, w = 2, 1, 64, 16, 200, 37
+    pages = (ctx + page - 1) // page
+    q = torch.randn(1, heads, d, generator=g) * 0.1
+    kc = torch.randn(pages, kv, page, d, generator=g) * 0.1
+    vc = torch.randn(pages, kv, d, page, generator=g)
+    pos = ctx - 1
+    edge, outside = pos - w + 1, pos - w
+    for j, gain in ((edge, 300.0), (outside, 600.0)):
+        kc[j // page, 0, j % page] = q[0, 0] * gain
+    bt = torch.arange(pages, dtype=torch.int32)[None]
+    cu = torch.tensor([0, 1], dtype=torch.int32)
+    cl = torch.tensor([ctx], dtype=torch.int32)
+    tr = torch.zeros(1, dtype=torch.int32)
+    q, kc, vc = q.to(dtype), kc.to(dtype), vc.to(dtype)
+    ref = emu.paged_attention(q, kc, vc, bt, cu, cl, tr, 1.0, w, 1, ctx).double()
+    assert float((ref.reshape(heads, d)[0] - vc[edge // page, 0, :, edge % page].double()).abs().max()) < 0.05
+    ops.allow_fast_attention = fast
+    try:
+        got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), cu.to(DEV), cl.to(DEV), tr.to(DEV), 1.0, w, 1, ctx)
+    finally:
+        ops.allow_fast_attention = True
+    _close(got, ref, 2e-5 if dtype == torch.float32 else 1.2e-2, "window edge")
+
+
+@pytest.mark.parametrize("m,inter,k", [(1, 192, 64), (8, 14336, 4096), (16, 320, 96), (40, 136, 160), (64, 1024, 2048), (300, 200, 128), (2048, 512, 256)])
+def test_linear_swiglu(m, inter, k):
+    """The gated epilogue of the matrix-core products, on the interleaved gate/up layout."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(20)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    wg = (torch.randn(inter, k, generator=g) * 0.3).to(torch.bfloat16)
+    wu = (torch.randn(inter, k, generator=g) * 0.3).to(torch.bfloat16)
+    w = ops.interleave_gate_up(wg, wu)
+    assert torch.equal(w[:8], wg[:8]) and torch.equal(w[8:16], wu[:8]) and torch.equal(w[16:24], wg[8:16])
+    gd, ud = x.double() @ wg.double().T, x.double() @ wu.double().T
+    ref = gd / (1 + torch.exp(-gd)) * ud
+    got = ops.linear_swiglu(x.to(DEV), w.to(DEV))
+    assert got.shape == (m, inter)
+    _close(got, ref, 6e-3, "linear_swiglu")
+    assert torch.equal(emu.linear_swiglu(x, w), ref.to(torch.bfloat16))

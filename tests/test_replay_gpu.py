@@ -15,45 +15,15 @@ import plain
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": {"a0": 5, "a1": 17, "a2": 33, "a3": 150, "a4": 97, "a5": 64},
-           "B": {"b0": 1, "b1": 9, "b2": 40, "b3": 63, "b4": 120, "b5": 201},
-           "C": {"c0": 3, "c1": 49, "c2": 130, "c3": 75, "c4": 25, "c5": 88}}
 
 
-def _requests(name):
-    vocab = helpers.CONFIGS[name].vocab_size
-    return {rid: helpers.random_tokens(vocab, n, seed=1000 + i)
-            for i, (rid, n) in enumerate(LENGTHS[name].items())}
-
-
-def _runner(tiny_dirs, name, dtype, max_tokens, page_size=16):
+def _runner(tiny_dirs, name, dtype, max_tokens, page_size=16, use_graph=False):
     from tempura_amd.engine.loading import load_model
     from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.kernels import ops
+    ops.set_backend(None)
     model = load_model(tiny_dirs.path(name, dtype), dtype, "cuda:0")
-    return ModelRunner(model, page_size, (max_tokens + page_size - 1) // page_size, max_requests=4)
-
-
-def _run(runner, requests, steps):
-    """Run a schedule asking for logits everywhere; returns {rid: [len, vocab] float32}."""
-    from tempura_amd.engine.runner import StepEntry
-    got = {rid: [None] * len(t) for rid, t in requests.items()}
-    for entries, end in steps:
-        batch = []
-        for rid, start, count in entries:
-            if not runner.has_request(rid):
-                runner.add_request(rid)
-            assert runner.num_cached(rid) == start
-            batch.append(StepEntry(rid, requests[rid][start:start + count], list(range(count))))
-        logits = runner.step(batch).cpu()
-        row = 0
-        for rid, start, count in entries:
-            for i in range(count):
-                got[rid][start + i] = logits[row]
-                row += 1
-        for rid in end:
-            runner.end_request(rid)
-        runner.cache.check()
-    return {rid: torch.stack(rows) for rid, rows in got.items()}
+    return ModelRunner(model, page_size, (max_tokens + page_size - 1) // page_size, max_requests=4, use_graph=use_graph)
 
 
 _REF = {}
@@ -63,35 +33,123 @@ def _reference(tiny_dirs, name, dtype):
     key = (name, dtype)
     if key not in _REF:
         cfg, W = tiny_dirs.plain_model(name, dtype)
-        _REF[key] = {rid: plain.forward(cfg, W, toks) for rid, toks in _requests(name).items()}
+        _REF[key] = {rid: plain.forward(cfg, W, toks) for rid, toks in helpers.requests_for(name).items()}
     return _REF[key]
 
 
 def _compare(got, ref, dtype, what):
     for rid in ref:
         err = helpers.rel_err(got[rid], ref[rid])
-        assert err <= helpers.TOL[dtype], f"{what}: request {rid} differs from the plain implementation by {err:.3e}"
-        # the first wrong token, if any, for the report
-    return True
+        bad = helpers.first_difference(got[rid], ref[rid], helpers.TOL[dtype])
+        assert err <= helpers.TOL[dtype], \
+            f"{what}: request {rid} differs from the plain implementation by {err:.3e}, first at position {bad}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_replay_modes(tiny_dirs, name, dtype, mode):
-    requests = _requests(name)
-    lengths = LENGTHS[name]
-    if mode == "mixed":
-        # room for about three of the requests: pages of finished ones must be used again
-        max_tokens = sum(sorted(helpers.roundup(n, 64) for n in lengths.values())[-2:]) + 64
-        steps = helpers.schedule_mixed(lengths, max_tokens, seed=5)
-    else:
-        max_tokens = max(helpers.roundup(n, 64) for n in lengths.values())
-        steps = {"whole": helpers.schedule_whole, "bulk_tail": helpers.schedule_bulk_tail,
-                 "portions": helpers.schedule_portions}[mode](lengths)
-    page_size = {"A": 16, "B": 8, "C": 32}[name]
-    runner = _runner(tiny_dirs, name, dtype, max_tokens, page_size)
-    got = _run(runner, requests, steps)
+    requests = helpers.requests_for(name)
+    steps, max_tokens = helpers.schedule_for(name, mode)
+    runner = _runner(tiny_dirs, name, dtype, max_tokens, helpers.PAGE_SIZE[name])
+    got = helpers.run_schedule(runner, requests, steps)
     assert not runner.cache.live_requests()
     assert runner.cache.free_pages() == [p.num_pages for p in runner.cache.pools]
     _compare(got, _reference(tiny_dirs, name, dtype), dtype, f"{name}/{dtype}/{mode}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_graph_replays_match_eager(tiny_dirs, name, dtype):
+    """Decode steps replayed as a captured graph give the eager steps' logits, replay after replay, with
+    eager steps (prompt portions of other requests) and synchronisations between the replays."""
+    requests = helpers.requests_for(name)
+    steps, max_tokens = helpers.schedule_for(name, "mixed")
+    eager = helpers.run_schedule(_runner(tiny_dirs, name, dtype, max_tokens, helpers.PAGE_SIZE[name]), requests, steps)
+    runner = _runner(tiny_dirs, name, dtype, max_tokens, helpers.PAGE_SIZE[name], use_graph=True)
+    assert runner.use_graph
+    graphed = helpers.run_schedule(runner, requests, steps)
+    assert runner.graph_steps >= 32, "decode-only steps went through the graph"
+    for rid in eager:
+        assert torch.equal(graphed[rid], eager[rid]), f"request {rid}: graph replay differs from the eager step"
+    _compare(graphed, _reference(tiny_dirs, name, dtype), dtype, f"{name}/{dtype}/graph")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(tiny_dirs, dtype):
+    """700 tokens decoded one by one after a short prompt (config A, 44 pages of 16)."""
+    cfg, W = tiny_dirs.plain_model("A", dtype)
+    toks = helpers.random_tokens(cfg["vocab_size"], 700, seed=77)
+    ref = plain.forward(cfg, W, toks)
+    runner = _runner(tiny_dirs, "A", dtype, 704, 16, use_graph=True)
+    steps = [([("x", 0, 9)], [])] + [([("x", i, 1)], []) for i in range(9, 700)]
+    got = helpers.run_schedule(runner, {"x": toks}, steps)
+    _compare(got, {"x": ref}, dtype, f"long decode {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens(tiny_dirs, name, dtype):
+    """The first tokens of a sequence, one by one from position 0 (one key, then two, ...)."""
+    cfg, W = tiny_dirs.plain_model(name, dtype)
+    toks = helpers.random_tokens(cfg["vocab_size"], 6, seed=78)
+    ref = plain.forward(cfg, W, toks)
+    runner = _runner(tiny_dirs, name, dtype, 64, helpers.PAGE_SIZE[name])
+    got = helpers.run_schedule(runner, {"x": toks}, [([("x", i, 1)], []) for i in range(6)])
+    _compare(got, {"x": ref}, dtype, f"first tokens {name} {dtype}")
+
+
+def test_window_layers_give_pages_back(tiny_dirs):
+    """Config C has a window of 24 on two of its four layers: portions and single tokens cross the window's
+    edge at every offset, logits match the plain implementation, and the windowed group holds one page where
+    the full group holds three."""
+    cfg, W = tiny_dirs.plain_model("C", "float32")
+    toks = helpers.random_tokens(cfg["vocab_size"], 90, seed=79)
+    ref = plain.forward(cfg, W, toks)
+    runner = _runner(tiny_dirs, "C", "float32", 128, 32)
+    steps = [([("x", 0, 38)], []), ([("x", 38, 5)], [])] + [([("x", i, 1)], []) for i in range(43, 90)]
+    got = helpers.run_schedule(runner, {"x": toks}, steps)
+    _compare(got, {"x": ref}, "float32", "window edge")
+    kinds = [g.kind for g in runner.cache.groups]
+    held = {k: p.num_held for k, p in zip(kinds, runner.cache.pools)}
+    assert held == {"window": 1, "full": 3}
+    runner.end_request("x")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tiny_dirs, tmp_path, dtype):
+    """bin/trace_run as a user runs it: JSON steps on standard input, logits files out."""
+    name = "B"
+    requests = helpers.requests_for(name)
+    steps, max_tokens = helpers.schedule_for(name, "mixed")
+    out_dir = tmp_path / "out"
+    lines = []
+    for i, (entries, end) in enumerate(steps):
+        want_all = i % 3 != 1
+        lines.append(json.dumps({"step": i, "end": end, "entries": [
+            {"id": rid, "tokens": requests[rid][s:s + c], "want": list(range(c)) if want_all else []}
+            for rid, s, c in entries]}))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", tiny_dirs.path(name, dtype),
+                        "--dtype", dtype, "--out", str(out_dir), "--max-tokens", str(max_tokens)],
+                       input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(steps))]
+    ref = _reference(tiny_dirs, name, dtype)
+    vocab = helpers.CONFIGS[name].vocab_size
+    checked = 0
+    for i, (entries, end) in enumerate(steps):
+        path = out_dir / f"{i}.f32"
+        if i % 3 == 1:
+            assert not path.exists(), "a step in which nothing is wanted writes no file"
+            continue
+        arr = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(-1, vocab))
+        row = 0
+        for rid, s, c in entries:
+            # the same measure as everywhere: the difference relative to the request's largest logit
+            err = float((arr[row:row + c].double() - ref[rid][s:s + c]).abs().max() / ref[rid].abs().max())
+            assert err <= helpers.TOL[dtype], f"step {i} request {rid}: {err:.3e}"
+            row += c
+            checked += c
+        assert row == arr.shape[0]
+    assert checked > 200

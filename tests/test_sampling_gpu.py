@@ -1,0 +1,133 @@
+"""The sampling kernels against the reference's rules written out plainly in Python."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def plain_sample(logits, temperature, top_k, top_p, min_p, r):
+    """temperature scale, min-p, top-k, softmax over the kept, top-p prefix, renormalise, walk the
+    probabilities in INDEX order and return the first index whose cumulative sum exceeds r
+    (/root/reference/kernels/src/sampling.rs:229-333, min-p /root/reference/kernels/src/sampler_chain.rs:54-80)."""
+    x = logits.double().clone()
+    if temperature == 0:
+        mx = x.max()
+        return int(torch.nonzero(x == mx).max())
+    if temperature != 1.0:
+        x = x / temperature
+    if min_p > 0:
+        x[x < x.max() + math.log(min_p)] = -math.inf
+    V = x.numel()
+    order = torch.argsort(x, descending=True, stable=True)
+    k = V if top_k <= 0 else min(top_k, V)
+    keep = order[:k]
+    p = torch.zeros(V, dtype=torch.float64)
+    p[keep] = torch.exp(x[keep] - x.max())
+    p /= p.sum()
+    if top_p < 1.0:
+        o2 = torch.argsort(p, descending=True, stable=True)
+        cs = torch.cumsum(p[o2], 0)
+        cut = int(torch.nonzero(cs >= top_p)[0]) + 1
+        mask = torch.zeros(V, dtype=torch.bool)
+        mask[o2[:cut]] = True
+        p[~mask] = 0
+        p /= p.sum()
+    cs = torch.cumsum(p, 0)
+    hit = torch.nonzero(cs > r)
+    return int(hit[0]) if hit.numel() else V - 1
+
+
+def _sample(logits, temperature, top_k, top_p, min_p, r):
+    from tempura_amd.kernels import ops
+    ops.set_backend(None)
+    m, v = logits.shape
+    work = torch.empty(m, v, device=DEV)
+    full = lambda a: [a] * m if not isinstance(a, (list, tuple)) else list(a)
+    return ops.sample(logits.to(DEV), work, full(temperature), full(top_k), full(top_p), full(min_p), full(r)).tolist()
+
+
+@pytest.mark.parametrize("vocab", [16, 301, 4099])
+@pytest.mark.parametrize("temperature,top_k,top_p,min_p", [(1.0, 0, 1.0, 0.0), (0.8, 0, 1.0, 0.0), (1.0, 5, 1.0, 0.0), (0.7, 50, 0.9, 0.0),
+                                                            (1.3, 0, 0.5, 0.0), (1.0, 0, 1.0, 0.1), (0.9, 40, 0.95, 0.05), (0.0, 50, 0.9, 0.0)])
+def test_sample_matches_plain_rules(vocab, temperature, top_k, top_p, min_p):
+    g = torch.Generator().manual_seed(vocab + int(top_k))
+    logits = torch.randn(24, vocab, generator=g) * 2.5
+    rs = [(i + 0.37) / 24 for i in range(24)]
+    got = _sample(logits, temperature, top_k, top_p, min_p, rs)
+    want = [plain_sample(logits[i], temperature, top_k, top_p, min_p, rs[i]) for i in range(24)]
+    assert got == want
+
+
+def test_greedy_ties_and_fallthrough():
+    lg = torch.zeros(3, 100)
+    lg[0, 5] = lg[0, 70] = 3.0                       # tie: the later index wins (model.rs:459-473)
+    lg[1] = -math.inf                                 # nothing to choose from: the last index (sampling.rs:496-520)
+    lg[2, 9] = 1.0
+    assert _sample(lg, [0.0, 1.0, 0.0], 0, 1.0, 0.0, 0.5) == [70, 99, 9]
+
+
+def test_temperature_to_zero_converges_to_argmax():
+    g = torch.Generator().manual_seed(1)
+    lg = torch.randn(16, 500, generator=g)
+    got = _sample(lg, 1e-4, 0, 1.0, 0.0, [i / 16 + 0.01 for i in range(16)])
+    assert got == lg.argmax(dim=1).tolist()
+
+
+def test_top_k_keeps_at_most_k_even_with_ties():
+    lg = torch.zeros(1, 64)                           # all equal: ties at the cut are admitted in index order
+    seen = set()
+    for i in range(200):
+        seen.update(_sample(lg, 1.0, 5, 1.0, 0.0, (i + 0.5) / 200))
+    assert seen == {0, 1, 2, 3, 4}
+    lg[0, 40:] = 1.0
+    seen = set()
+    for i in range(200):
+        seen.update(_sample(lg, 1.0, 30, 1.0, 0.0, (i + 0.5) / 200))
+    assert seen == set(range(40, 64)) | set(range(6))
+
+
+def test_frequencies_follow_softmax():
+    """Chi-square of 20,000 draws against softmax(logits / T) on a vocabulary of 16."""
+    from tempura_amd.sampling import uniform_draw
+    g = torch.Generator().manual_seed(2)
+    lg = torch.randn(1, 16, generator=g) * 1.5
+    p = torch.softmax(lg[0].double() / 0.8, 0)
+    n = 20000
+    rows = lg.expand(2000, 16).contiguous()
+    counts = torch.zeros(16)
+    for b in range(n // 2000):
+        rs = [uniform_draw(123, b * 2000 + i) for i in range(2000)]
+        counts += torch.bincount(torch.tensor(_sample(rows, 0.8, 0, 1.0, 0.0, rs)), minlength=16)
+    chi2 = float(((counts - n * p) ** 2 / (n * p)).sum())
+    assert chi2 < 45.0, f"chi-square {chi2:.1f} with 15 degrees of freedom"        # p ~ 1e-4
+
+
+def test_penalties():
+    from tempura_amd.kernels import ops
+    ops.set_backend(None)
+    lg = torch.tensor([[1.0, -2.0, 3.0, 0.5, -1.0], [1.0, -2.0, 3.0, 0.5, -1.0]])
+    d = lg.clone().to(DEV)
+    # row 0: token 2 generated twice, token 1 once; tokens 0 and 1 in the repetition window
+    ops.apply_penalties(d, [0, 0, 0], [2, 1, 0], [2, 1, 0], [0, 1, 1], [0.5, 0.0], [0.25, 0.0], [2.0, 1.0])
+    want = lg.clone()
+    want[0, 2] -= 0.25 * 2 + 0.5           # frequency * count + presence (kernel-api/src/lib.rs:292-308)
+    want[0, 1] = (want[0, 1] - (0.25 + 0.5)) * 2.0      # non-positive logits are multiplied (sampler_chain.rs:239-243)
+    want[0, 0] = want[0, 0] / 2.0                        # positive ones divided
+    assert torch.allclose(d.cpu(), want)
+
+
+def test_sampler_class_rows_with_different_options():
+    from tempura_amd.sampling import Sampler, SamplingParams
+    g = torch.Generator().manual_seed(3)
+    lg = torch.randn(3, 300, generator=g).to(DEV)
+    s = Sampler(300, torch.device(DEV), default_seed=9)
+    ps = [SamplingParams(temperature=0.0), SamplingParams(temperature=0.9, top_k=10, seed=4),
+          SamplingParams(temperature=1.0, top_k=0, presence_penalty=100.0)]
+    out = s.sample(lg, ps, [0, 3, 1], [[], [], []], [[], [], [int(lg[2].argmax())]])
+    assert out[0] == int(lg[0].argmax())
+    assert out[1] in lg[1].topk(10).indices.tolist()
+    assert out[2] != int(lg[2].argmax()), "a huge presence penalty bans the generated token"
+    assert s.sample(lg, ps, [0, 3, 1], [[], [], []], [[], [], [int(lg[2].argmax())]]) == out

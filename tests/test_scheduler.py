@@ -1,0 +1,156 @@
+"""The scheduler's decisions (CPU): admission, portions under a token budget, decoding first,
+finishing and freeing, and what happens when pages run out."""
+import random
+
+import pytest
+
+from tempura_amd.cache import CacheManager
+from tempura_amd.engine.scheduler import Request, RequestState, Scheduler, SchedulerConfig
+from tempura_amd.parts import CacheSpec
+from tempura_amd.sampling import SamplingParams
+
+FULL = CacheSpec("full", 2, 16)
+
+
+def make(num_pages=64, page_size=8, **cfg):
+    cache = CacheManager([FULL], page_size, num_pages, max_requests=cfg.get("max_num_seqs", 8))
+    return Scheduler(SchedulerConfig(**{"max_num_seqs": 8, "max_num_batched_tokens": 32, "prefill_chunk_size": 16,
+                                        "max_model_len": 512, **cfg}), cache), cache
+
+
+def req(rid, n_prompt, max_new=4, **kw):
+    return Request(rid, list(range(1, n_prompt + 1)), SamplingParams(temperature=0, max_new_tokens=max_new, **kw))
+
+
+def run(sched, cache, token_of=lambda r: 7, max_steps=10000, on_step=None):
+    """Drive the scheduler as the engine does, with a stand-in for the model (reserve/commit only)."""
+    steps = []
+    while sched.has_unfinished():
+        items = sched.schedule()
+        assert items, "the scheduler made no progress"
+        assert len({id(it.request) for it in items}) == len(items), "a request was scheduled twice in one step"
+        for it in items:
+            assert it.start == it.request.num_computed == cache.num_tokens(it.request.rid)
+            cache.reserve(it.request.rid, it.count)
+        for it in items:
+            cache.commit(it.request.rid, it.count)
+            sched.advance(it)
+        for it in items:
+            if it.samples:
+                if sched.append_token(it.request, token_of(it.request)):
+                    sched.finish(it.request)
+        cache.check()
+        steps.append([(it.request.rid, it.start, it.count, it.samples) for it in items])
+        if on_step:
+            on_step(items)
+        assert len(steps) < max_steps
+    return steps
+
+
+def test_portions_under_budget_then_decode():
+    sched, cache = make()
+    sched.add_request(req("a", 40, max_new=3))
+    steps = run(sched, cache)
+    # 40 prompt tokens in portions of at most 16, the last portion samples; then one token per step
+    assert steps[0] == [("a", 0, 16, False)] and steps[1] == [("a", 16, 16, False)] and steps[2] == [("a", 32, 8, True)]
+    assert steps[3] == [("a", 40, 1, True)] and steps[4] == [("a", 41, 1, True)] and len(steps) == 5
+    r = sched.finished[0]
+    assert r.output == [7, 7, 7] and r.finish_reason == "length" and r.state == RequestState.FINISHED
+    assert cache.free_pages() == [64] and not cache.live_requests()
+
+
+def test_mixed_steps_decoding_first_and_budget():
+    sched, cache = make(max_num_batched_tokens=20)
+    sched.add_request(req("a", 5, max_new=30))
+    sched.add_request(req("b", 50, max_new=2))
+    sched.add_request(req("c", 9, max_new=2))
+    seen_mixed = False
+
+    def check(items):
+        nonlocal seen_mixed
+        assert sum(it.count for it in items) <= 20
+        kinds = [it.request.is_decoding or it.count == 1 and it.samples for it in items]
+        dec = [i for i, it in enumerate(items) if it.count == 1 and it.start >= len(it.request.prompt)]
+        if dec and len(dec) < len(items):
+            seen_mixed = True
+            assert dec == list(range(len(dec))), "decoding requests come first in the batch"
+    steps = run(sched, cache, on_step=check)
+    assert seen_mixed, "prompt portions ran beside decoded tokens"
+    assert sorted(r.rid for r in sched.finished) == ["a", "b", "c"]
+    assert [len(r.output) for r in sorted(sched.finished, key=lambda r: r.rid)] == [30, 2, 2]
+    # first step: a's whole prompt (5) then 15 of b's tokens fill the budget of 20
+    assert steps[0] == [("a", 0, 5, True), ("b", 0, 15, False)]
+
+
+def test_eos_stops_and_is_kept():
+    sched, cache = make()
+    r = req("a", 3, max_new=10)
+    r.eos_token_ids = (99,)
+    sched.add_request(r)
+    toks = iter([5, 99, 6])
+    run(sched, cache, token_of=lambda _r: next(toks))
+    assert r.output == [5, 99] and r.finish_reason == "eos"      # the EOS token is kept (model.rs:9765)
+    r2 = req("b", 3, max_new=3, ignore_eos=True)
+    r2.eos_token_ids = (99,)
+    sched.add_request(r2)
+    run(sched, cache, token_of=lambda _r: 99)
+    assert r2.output == [99, 99, 99] and r2.finish_reason == "length"
+
+
+def test_max_num_seqs_and_fifo():
+    sched, cache = make(max_num_seqs=2)
+    for i in range(5):
+        sched.add_request(req(i, 4, max_new=2))
+    order = []
+    run(sched, cache, on_step=lambda items: order.extend(it.request.rid for it in items if it.start == 0))
+    assert order == [0, 1, 2, 3, 4]
+    assert len(sched.finished) == 5
+
+
+def test_request_that_can_never_fit_is_refused():
+    sched, cache = make(num_pages=4, page_size=8)
+    with pytest.raises(ValueError, match="pages"):
+        sched.add_request(req("big", 30, max_new=10))
+    with pytest.raises(ValueError, match="empty prompt"):
+        sched.add_request(Request("e", [], SamplingParams()))
+    with pytest.raises(ValueError, match="no room"):
+        sched.add_request(req("long", 512, max_new=1))
+
+
+def test_pages_run_out_preempt_newest_and_recompute():
+    """Two requests outgrow the pool: the one admitted last is preempted (pages back, front of the queue,
+    prompt + output recomputed) and both finish with every token they were promised."""
+    sched, cache = make(num_pages=8, page_size=8, max_num_batched_tokens=64, prefill_chunk_size=64)
+    a, b = req("a", 20, max_new=30), req("b", 20, max_new=30)     # each needs 50 tokens = 7 pages; the pool has 8
+    sched.add_request(a)
+    sched.add_request(b)
+    counter = {"n": 0}
+
+    def tok(r):
+        counter["n"] += 1
+        return len(r.output) + 100 * (1 if r.rid == "a" else 2)
+    run(sched, cache, token_of=tok)
+    assert sched.num_preemptions >= 1
+    assert b.preemptions >= 1 and a.preemptions == 0, "the most recently admitted request is the victim"
+    assert a.output == [100 + i for i in range(30)] and b.output == [200 + i for i in range(30)]
+    assert cache.free_pages() == [8] and not cache.live_requests()
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_no_request_lost_under_a_tiny_pool(seed):
+    # the reference's test_no_silent_drops (/root/reference/server/src/batch.rs:641-654)
+    g = random.Random(seed)
+    sched, cache = make(num_pages=12, page_size=4, max_num_seqs=4, max_num_batched_tokens=24, prefill_chunk_size=8,
+                        max_model_len=64)
+    want = {}
+    for i in range(12):
+        n, k = g.randint(1, 20), g.randint(1, 15)
+        if n + k > 40:
+            continue
+        sched.add_request(req(i, n, max_new=k))
+        want[i] = k
+    run(sched, cache)
+    got = {r.rid: len(r.output) for r in sched.finished}
+    assert got == want
+    assert cache.free_pages() == [12]
+    assert sched.pages_high_water[0] <= 12

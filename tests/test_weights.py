@@ -1,0 +1,127 @@
+"""Weights: by-name loading, kept dtypes, one error for every fault, random-weights mode (CPU)."""
+import json
+import os
+
+import pytest
+import torch
+
+import helpers
+from tempura_amd.config import LlamaConfig
+from tempura_amd.engine.model import CausalLM
+from tempura_amd.weights import (Checkpoint, SafetensorsError, SafetensorsFile, WeightsError, check_checkpoint,
+                                 load_into, random_weights, write_random_model, write_safetensors)
+
+
+def _model(name="A", dtype=torch.float32):
+    cfg = LlamaConfig.from_dict(helpers.CONFIGS[name].to_dict())
+    return cfg, CausalLM(cfg.build_spec(), dtype, torch.device("cpu"))
+
+
+def test_random_model_folder_loads(tmp_path):
+    cfg, model = _model("A")
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=3, dtype="bfloat16")
+    assert sorted(os.listdir(d)) == ["config.json", "model.safetensors"]
+    load_into(model, d)
+    assert model.layers[0].mixer.wqkv.shape == ((4 + 2 * 2) * 16, 64)
+    assert model.lm_head.weight.data_ptr() != model.embedding.weight.data_ptr()
+    # same seed, same values; another seed, other values; norm weights are 1.0
+    w1, w2, w3 = random_weights(cfg, 3), random_weights(cfg, 3), random_weights(cfg, 4)
+    assert all(torch.equal(w1[k], w2[k]) for k in w1)
+    assert not torch.equal(w1["model.embed_tokens.weight"], w3["model.embed_tokens.weight"])
+    assert torch.all(w1["model.norm.weight"] == 1.0)
+    assert abs(float(w1["model.embed_tokens.weight"].float().std()) - 0.02) < 2e-3
+
+
+def test_tied_model_has_no_output_matrix(tmp_path):
+    cfg, model = _model("B")
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=1, dtype="float32")
+    names = SafetensorsFile(os.path.join(d, "model.safetensors")).names()
+    assert "lm_head.weight" not in names
+    load_into(model, d)
+    assert model.lm_head.weight.data_ptr() == model.embedding.weight.data_ptr()      # same buffer, no copy
+
+
+def test_untied_config_without_output_matrix_falls_back_to_embedding(tmp_path):
+    # the reference decides tying by the tensor's absence (/root/reference/engine/src/weights.rs:156-166)
+    cfg, model = _model("A")
+    w = random_weights(cfg, 0, dtype="float32")
+    del w["lm_head.weight"]
+    os.makedirs(tmp_path / "m")
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), w.items())
+    load_into(model, str(tmp_path / "m"))
+    assert model.lm_head.weight.data_ptr() == model.embedding.weight.data_ptr()
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    cfg, model = _model("A")
+    w = random_weights(cfg, 0, dtype="float32")
+    del w["model.layers.1.mlp.up_proj.weight"]
+    del w["model.norm.weight"]
+    w["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    w["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(64, 64)        # should be [32, 64]
+    w["model.embed_tokens.weight"] = torch.zeros(64, 256)                     # right count, wrong shape
+    os.makedirs(tmp_path / "m")
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), w.items())
+    with pytest.raises(WeightsError) as ei:
+        load_into(model, str(tmp_path / "m"))
+    e = ei.value
+    assert e.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
+    assert e.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert set(e.wrong_shape) == {"model.layers.0.self_attn.k_proj.weight", "model.embed_tokens.weight"}
+    assert e.wrong_shape["model.embed_tokens.weight"] == ((256, 64), (64, 256))
+    for needle in ("model.norm.weight", "rotary_emb.inv_freq", "k_proj.weight expected [32, 64] found [64, 64]"):
+        assert needle in str(e)
+
+
+def test_no_files_and_bad_files(tmp_path):
+    with pytest.raises(WeightsError, match="no .safetensors"):
+        Checkpoint(str(tmp_path))
+    (tmp_path / "x.safetensors").write_bytes(b"\x05")
+    with pytest.raises(SafetensorsError, match="too short"):
+        SafetensorsFile(str(tmp_path / "x.safetensors"))
+    (tmp_path / "x.safetensors").write_bytes((10 ** 6).to_bytes(8, "little") + b"{}")
+    with pytest.raises(SafetensorsError, match="header length"):
+        SafetensorsFile(str(tmp_path / "x.safetensors"))
+    hdr = json.dumps({"t": {"dtype": "F8_E4M3", "shape": [1], "data_offsets": [0, 1]}}).encode()
+    (tmp_path / "x.safetensors").write_bytes(len(hdr).to_bytes(8, "little") + hdr + b"\0")
+    with pytest.raises(SafetensorsError, match="unsupported dtype"):
+        SafetensorsFile(str(tmp_path / "x.safetensors"))
+
+
+def test_kept_dtypes_and_exact_widening(tmp_path):
+    g = torch.Generator().manual_seed(0)
+    f32 = torch.randn(5, 7, generator=g)
+    tensors = {"bf": f32.to(torch.bfloat16), "f32": f32, "f16": f32.to(torch.float16),
+               "i64": torch.arange(6, dtype=torch.int64).reshape(2, 3), "i32": torch.arange(4, dtype=torch.int32)}
+    # subnormal and special float16 values widen exactly (/root/reference/engine/src/loader.rs:62-93)
+    tensors["f16s"] = torch.tensor([6e-8, -6e-8, 65504.0, float("inf"), 0.0], dtype=torch.float16)
+    write_safetensors(str(tmp_path / "a.safetensors"), tensors.items())
+    ck = Checkpoint(str(tmp_path))
+    assert ck.tensor("bf").dtype == torch.bfloat16 and torch.equal(ck.tensor("bf"), tensors["bf"])
+    assert ck.tensor("f32").dtype == torch.float32 and torch.equal(ck.tensor("f32"), f32)      # 32-bit stays 32-bit
+    assert ck.tensor("f16").dtype == torch.float32 and torch.equal(ck.tensor("f16"), tensors["f16"].float())
+    assert torch.equal(ck.tensor("f16s"), tensors["f16s"].float())
+    assert ck.tensor("i64").dtype == torch.int32 and ck.tensor("i64").tolist() == [[0, 1, 2], [3, 4, 5]]
+    assert ck.tensor("i32").dtype == torch.int32
+
+
+def test_shards_in_path_order_later_overwrites(tmp_path):
+    write_safetensors(str(tmp_path / "model-00001.safetensors"), [("a", torch.ones(2)), ("b", torch.ones(3))])
+    write_safetensors(str(tmp_path / "model-00002.safetensors"), [("b", torch.zeros(3)), ("c", torch.ones(1))])
+    ck = Checkpoint(str(tmp_path))
+    assert sorted(ck.names()) == ["a", "b", "c"]
+    assert torch.equal(ck.tensor("b"), torch.zeros(3))
+
+
+def test_compute_dtype_conversion(tmp_path):
+    """Stored bfloat16 runs in float32 exactly widened; stored float32 runs in bfloat16 rounded; norms stay float32."""
+    cfg, m32 = _model("A", torch.float32)
+    d = write_random_model(cfg, str(tmp_path / "bf"), seed=2, dtype="bfloat16")
+    load_into(m32, d)
+    stored = Checkpoint(d).tensor("model.layers.0.self_attn.o_proj.weight")
+    assert m32.layers[0].mixer.wo.dtype == torch.float32 and torch.equal(m32.layers[0].mixer.wo, stored.float())
+    _, mbf = _model("A", torch.bfloat16)
+    d2 = write_random_model(cfg, str(tmp_path / "f32"), seed=2, dtype="float32")
+    load_into(mbf, d2)
+    assert mbf.layers[0].mixer.wo.dtype == torch.bfloat16
+    assert mbf.final_norm.weight.dtype == torch.float32
