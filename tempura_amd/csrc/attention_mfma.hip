@@ -272,24 +272,27 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 }
 
 // out[token, head, :] = sum_s 2^(m_s - m) O_s / sum_s 2^(m_s - m) l_s, splits in ascending order.
-// grid: (requests, heads); block: D threads (rounded up to a wave).
-__global__ void attn_combine_kernel(const float* __restrict__ scratch, const int* __restrict__ cu_seqlens,
-                                    bf16_t* __restrict__ out, int n_heads, int D, int num_splits) {
-  const int r = blockIdx.x, h = blockIdx.y;
+// grid: (requests, heads); block: one wave.  Lane s holds split s's statistics (num_splits <= 64).
+__global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ scratch,
+                                                          const int* __restrict__ cu_seqlens,
+                                                          bf16_t* __restrict__ out, int n_heads, int D,
+                                                          int num_splits) {
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int q_start = cu_seqlens[r];
   if (cu_seqlens[r + 1] - q_start != 1) return;
   const float* base = scratch + ((size_t)r * n_heads + h) * num_splits * (D + 2);
-  float mg = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) mg = fmaxf(mg, base[(size_t)s * (D + 2) + D]);
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < num_splits) {
+    ms = base[(size_t)lane * (D + 2) + D];
+    ls = base[(size_t)lane * (D + 2) + D + 1];
+  }
+  const float mg = wave_max(ms);
   const float mu = (mg == -INFINITY) ? 0.f : mg;
-  float lsum = 0.f;
-  for (int s = 0; s < num_splits; ++s)
-    lsum += __builtin_amdgcn_exp2f(base[(size_t)s * (D + 2) + D] - mu) * base[(size_t)s * (D + 2) + D + 1];
-  const float inv = 1.0f / lsum;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+  const float ws = __builtin_amdgcn_exp2f(ms - mu);   // 0 for lanes without a split
+  const float inv = 1.0f / wave_sum(ws * ls);
+  for (int d = lane; d < D; d += 64) {
     float acc = 0.f;
-    for (int s = 0; s < num_splits; ++s)
-      acc += __builtin_amdgcn_exp2f(base[(size_t)s * (D + 2) + D] - mu) * base[(size_t)s * (D + 2) + d];
+    for (int s = 0; s < num_splits; ++s) acc = fmaf(__shfl(ws, s, 64), base[(size_t)s * (D + 2) + d], acc);
     out[((size_t)q_start * n_heads + h) * D + d] = float_to_bf16(acc * inv);
   }
 }
@@ -303,8 +306,8 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
     const dim3 grid(n_req, a.n_kv * ((group + 15) / 16), a.num_splits);
     hipLaunchKernelGGL(attn_decode_kernel<D>, grid, dim3(256), 0, s, a);
     const dim3 cgrid(n_req, a.n_heads);
-    hipLaunchKernelGGL(attn_combine_kernel, cgrid, dim3(D <= 64 ? 64 : 128), 0, s, a.scratch, a.cu_seqlens, a.out,
-                       a.n_heads, D, a.num_splits);
+    hipLaunchKernelGGL(attn_combine_kernel, cgrid, dim3(64), 0, s, a.scratch, a.cu_seqlens, a.out, a.n_heads, D,
+                       a.num_splits);
   }
   if (has_multi) {
     constexpr int NQ = (D <= 128) ? 2 : 1;
@@ -320,7 +323,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int max_q_len, int num_single, int num_splits, float* scratch, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
   if (n_req > 65535 || n_req <= 0) return -1;
-  if (num_single > 0 && (scratch == nullptr || num_splits < 1)) return -1;
+  if (num_single > 0 && (scratch == nullptr || num_splits < 1 || num_splits > 64)) return -1;
   AttnArgs a;
   a.q = (const bf16_t*)q;
   a.k_cache = (const bf16_t*)k_cache;

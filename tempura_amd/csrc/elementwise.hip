@@ -42,13 +42,43 @@ extern "C" int tp_embed(const int* tokens, const void* table, int table_dt, floa
 
 // ---- RMSNorm ---------------------------------------------------------------------
 // y = x * (1 / sqrt(mean(x^2) + eps)) * w, all in float32; one block per output row.
-// `rows` (optional) picks the input row of each output row.
+// `rows` (optional) picks the input row of each output row.  The row is kept in registers
+// between the two passes when it fits (hidden <= 4 * VEC_ITEMS * threads).
+#define RMS_ITEMS 4
 template <typename TO>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                const int* __restrict__ rows, TO* __restrict__ out, int hidden, float eps) {
   __shared__ float scratch[32];
   const int r = blockIdx.x;
   const float* xr = x + (size_t)(rows ? rows[r] : r) * hidden;
+  TO* o = out + (size_t)r * hidden;
+  const bool vec = (hidden % 4 == 0) && hidden <= 4 * RMS_ITEMS * (int)blockDim.x;
+  if (vec) {
+    float4 v[RMS_ITEMS];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < RMS_ITEMS; ++i) {
+      const int j = (threadIdx.x + i * blockDim.x) * 4;
+      if (j < hidden) {
+        v[i] = *(const float4*)(xr + j);
+        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+      }
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+#pragma unroll
+    for (int i = 0; i < RMS_ITEMS; ++i) {
+      const int j = (threadIdx.x + i * blockDim.x) * 4;
+      if (j < hidden) {
+        const float4 wv = *(const float4*)(w + j);
+        from_float(o + j, v[i].x * scale * wv.x);
+        from_float(o + j + 1, v[i].y * scale * wv.y);
+        from_float(o + j + 2, v[i].z * scale * wv.z);
+        from_float(o + j + 3, v[i].w * scale * wv.w);
+      }
+    }
+    return;
+  }
   float ss = 0.f;
   for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
     const float v = xr[j];
@@ -56,7 +86,6 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
   }
   ss = block_sum(ss, scratch);
   const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
-  TO* o = out + (size_t)r * hidden;
   for (int j = threadIdx.x; j < hidden; j += blockDim.x) from_float(o + j, xr[j] * scale * w[j]);
 }
 
@@ -64,7 +93,7 @@ extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void*
                           int n_out, int hidden, float eps, hipStream_t s) {
   TP_REQUIRE(n_out >= 0 && hidden > 0, "rmsnorm: bad sizes");
   if (n_out == 0) return 0;
-  const int threads = hidden >= 2048 ? 1024 : (hidden >= 512 ? 256 : 64);
+  const int threads = hidden >= 8192 ? 1024 : (hidden >= 1024 ? 256 : 64);
   if (out_dt == TP_F32)
     hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n_out), dim3(threads), 0, s, x, w, rows, (float*)out, hidden, eps);
   else if (out_dt == TP_BF16)
@@ -95,9 +124,13 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
   const int half = rotary_dim / 2;
   const double pos = (double)positions[t];
   for (int d = threadIdx.x; d < half; d += blockDim.x) {
-    const double ang = pos * inv_freq[d];
-    cs[d] = (float)cos(ang) * factor;
-    cs[half + d] = (float)sin(ang) * factor;
+    // the angle in float64, reduced to [0, 2 pi) there; sine and cosine of the small rest in float32
+    const double turns = pos * inv_freq[d] * 0.15915494309189535;
+    const float rest = (float)((turns - floor(turns)) * 6.283185307179586);
+    float sn, c;
+    sincosf(rest, &sn, &c);
+    cs[d] = c * factor;
+    cs[half + d] = sn * factor;
   }
   __syncthreads();
   const float* row = qkv + (size_t)t * row_stride;
@@ -109,9 +142,10 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
     page = (size_t)(slot / page_size);
     off = (size_t)(slot % page_size);
   }
-  // rotated part of q and k heads
-  for (int i = threadIdx.x; i < rot_heads * half; i += blockDim.x) {
-    const int h = i / half, d = i % half;
+  // rotated part of q and k heads: a thread keeps its pair index d and walks over heads
+  const int hstride = half > 0 ? max(1, (int)blockDim.x / half) : 1;
+  const int h_first = half > 0 ? threadIdx.x / half : rot_heads, d = half > 0 ? threadIdx.x % half : 0;
+  for (int h = h_first; h < rot_heads && h_first < hstride; h += hstride) {
     const float x0 = row[h * head_dim + d], x1 = row[h * head_dim + d + half];
     const float c = cs[d], sn = cs[half + d];
     const float y0 = x0 * c - x1 * sn, y1 = x0 * sn + x1 * c;
@@ -154,6 +188,7 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
   TP_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim,
              "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, head_dim);
   TP_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope_kv_write: no frequency table");
+  TP_REQUIRE(rotary_dim <= 512, "rope_kv_write: rotary_dim %d exceeds 512", rotary_dim);
   TP_REQUIRE(slots == nullptr || (k_cache && v_cache && page_size > 0), "rope_kv_write: cache missing");
   TP_REQUIRE(row_stride >= (n_heads + (slots ? 2 * n_kv : 0)) * head_dim, "rope_kv_write: row too short");
   if (n == 0) return 0;

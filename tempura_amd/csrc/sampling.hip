@@ -13,13 +13,19 @@ __device__ inline void argmax_merge(float& bv, int& bi, float v, int i) {
   }
 }
 
-__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+// Stage 1: grid (rows, chunks): each block scans its share of the row; stage 2 (chunks == 1 or the
+// second launch) merges.  `part` holds (value, index) per (row, chunk).
+__global__ void argmax_kernel(const float* __restrict__ logits, int vocab, int chunks, float* __restrict__ part_v,
+                              int* __restrict__ part_i, int* __restrict__ out) {
   __shared__ float sv[16];
   __shared__ int si[16];
-  const float* row = logits + (size_t)blockIdx.x * vocab;
+  const int rowi = blockIdx.x, chunk = blockIdx.y;
+  const float* row = logits + (size_t)rowi * vocab;
+  const int per = (vocab + chunks - 1) / chunks;
+  const int lo = chunk * per, hi = min(vocab, lo + per);
   float bv = -INFINITY;
   int bi = -1;
-  for (int j = threadIdx.x; j < vocab; j += blockDim.x) argmax_merge(bv, bi, row[j], j);
+  for (int j = lo + threadIdx.x; j < hi; j += blockDim.x) argmax_merge(bv, bi, row[j], j);
   for (int o = TP_WAVE / 2; o > 0; o >>= 1) {
     const float ov = __shfl_xor(bv, o, TP_WAVE);
     const int oi = __shfl_xor(bi, o, TP_WAVE);
@@ -34,14 +40,40 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict_
   if (threadIdx.x == 0) {
     const int nw = (blockDim.x + TP_WAVE - 1) / TP_WAVE;
     for (int i = 1; i < nw; ++i) argmax_merge(bv, bi, sv[i], si[i]);
-    out[blockIdx.x] = bi < 0 ? vocab - 1 : bi;  // all -inf / NaN: the last index
+    if (chunks == 1) {
+      out[rowi] = bi < 0 ? vocab - 1 : bi;  // all -inf / NaN: the last index
+    } else {
+      part_v[rowi * chunks + chunk] = bv;
+      part_i[rowi * chunks + chunk] = bi;
+    }
   }
 }
 
-extern "C" int tp_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t s) {
+__global__ void argmax_merge_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i, int chunks,
+                                    int vocab, int* __restrict__ out) {
+  const int rowi = blockIdx.x;
+  float bv = -INFINITY;
+  int bi = -1;
+  for (int c = threadIdx.x; c < chunks; c += TP_WAVE) argmax_merge(bv, bi, part_v[rowi * chunks + c], part_i[rowi * chunks + c]);
+  for (int o = TP_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, TP_WAVE);
+    const int oi = __shfl_xor(bi, o, TP_WAVE);
+    argmax_merge(bv, bi, ov, oi);
+  }
+  if (threadIdx.x == 0) out[rowi] = bi < 0 ? vocab - 1 : bi;
+}
+
+// `part` is scratch of rows * 64 floats followed by rows * 64 ints (may be null for small vocabularies).
+extern "C" int tp_argmax(const float* logits, int* out, int rows, int vocab, void* part, hipStream_t s) {
   TP_REQUIRE(rows >= 0 && vocab > 0, "argmax: bad sizes");
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, s, logits, out, vocab);
+  int chunks = 1;
+  if (part != nullptr && vocab >= 16384) chunks = min(64, max(1, 512 / rows));
+  float* pv = (float*)part;
+  int* pi = (int*)(pv + (size_t)rows * 64);
+  hipLaunchKernelGGL(argmax_kernel, dim3(rows, chunks), dim3(chunks == 1 ? 1024 : 256), 0, s, logits, vocab, chunks, pv,
+                     pi, out);
+  if (chunks > 1) hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(TP_WAVE), 0, s, pv, pi, chunks, vocab, out);
   TP_CHECK_LAUNCH("argmax");
   return 0;
 }

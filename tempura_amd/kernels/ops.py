@@ -288,7 +288,8 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     _dev_ok(logits)
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "argmax: logits must be float32 [m, vocab]")
     out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-    _call("tp_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
+    part = torch.empty((logits.shape[0] * 128,), dtype=torch.float32, device=logits.device)
+    _call("tp_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _ptr(part), _stream())
     return out
 
 
