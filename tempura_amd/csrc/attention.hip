@@ -96,7 +96,8 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
                                   int window, int max_q_len, int max_ctx, int allow_fast, int num_single,
                                   int num_splits, float* scratch, hipStream_t s) {
   // num_single: how many requests bring exactly one token (they go to the split decode kernel,
-  // which needs `scratch` of n_req * n_heads * num_splits * (head_dim + 2) floats).
+  // which, with more than one split, needs `scratch` of n_req * n_heads * num_splits * (head_dim + 2)
+  // floats).
   TP_REQUIRE(n_tokens >= 0 && n_req >= 0 && n_heads > 0 && n_kv > 0 && head_dim > 0 && page_size > 0,
              "paged_attention: bad sizes");
   TP_REQUIRE(n_heads % n_kv == 0, "paged_attention: %d heads is not a multiple of %d kv heads", n_heads, n_kv);

@@ -262,6 +262,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       acc += f * red_o[w][d][col];
       lsum += f * red_l[w][col];
     }
+    if (a.num_splits == 1) {  // nothing to combine: this is the answer
+      a.out[((size_t)q_start * a.n_heads + (kvh * group + h0 + col)) * D + d] = float_to_bf16(acc / lsum);
+      continue;
+    }
     float* part = a.scratch + (((size_t)r * a.n_heads + (kvh * group + h0 + col)) * a.num_splits + blockIdx.z) * (D + 2);
     part[d] = acc;
     if (d == 0) {
@@ -273,6 +277,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 
 // out[token, head, :] = sum_s 2^(m_s - m) O_s / sum_s 2^(m_s - m) l_s, splits in ascending order.
 // grid: (requests, heads); block: one wave.  Lane s holds split s's statistics (num_splits <= 64).
+// (Combining inside the decode kernel by whichever block finishes last was tried and is far
+// slower: the L2 caches of the eight XCDs are not coherent with each other, so partial results
+// would have to travel through memory with device-scope fences.)
 __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ scratch,
                                                           const int* __restrict__ cu_seqlens,
                                                           bf16_t* __restrict__ out, int n_heads, int D,
@@ -288,11 +295,19 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   }
   const float mg = wave_max(ms);
   const float mu = (mg == -INFINITY) ? 0.f : mg;
-  const float ws = __builtin_amdgcn_exp2f(ms - mu);   // 0 for lanes without a split
+  const float ws = __builtin_amdgcn_exp2f(ms - mu);  // 0 for lanes without a split
   const float inv = 1.0f / wave_sum(ws * ls);
   for (int d = lane; d < D; d += 64) {
     float acc = 0.f;
-    for (int s = 0; s < num_splits; ++s) acc = fmaf(__shfl(ws, s, 64), base[(size_t)s * (D + 2) + d], acc);
+    int s = 0;
+    for (; s + 8 <= num_splits; s += 8) {   // eight independent loads in flight
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = base[(size_t)(s + u) * (D + 2) + d];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc = fmaf(__shfl(ws, s + u, 64), v[u], acc);
+    }
+    for (; s < num_splits; ++s) acc = fmaf(__shfl(ws, s, 64), base[(size_t)s * (D + 2) + d], acc);
     out[((size_t)q_start * n_heads + h) * D + d] = float_to_bf16(acc * inv);
   }
 }
@@ -305,9 +320,11 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
   if (num_single > 0) {
     const dim3 grid(n_req, a.n_kv * ((group + 15) / 16), a.num_splits);
     hipLaunchKernelGGL(attn_decode_kernel<D>, grid, dim3(256), 0, s, a);
-    const dim3 cgrid(n_req, a.n_heads);
-    hipLaunchKernelGGL(attn_combine_kernel, cgrid, dim3(64), 0, s, a.scratch, a.cu_seqlens, a.out, a.n_heads, D,
-                       a.num_splits);
+    if (a.num_splits > 1) {
+      const dim3 cgrid(n_req, a.n_heads);
+      hipLaunchKernelGGL(attn_combine_kernel, cgrid, dim3(64), 0, s, a.scratch, a.cu_seqlens, a.out, a.n_heads, D,
+                         a.num_splits);
+    }
   }
   if (has_multi) {
     constexpr int NQ = (D <= 128) ? 2 : 1;
@@ -323,7 +340,8 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int max_q_len, int num_single, int num_splits, float* scratch, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
   if (n_req > 65535 || n_req <= 0) return -1;
-  if (num_single > 0 && (scratch == nullptr || num_splits < 1 || num_splits > 64)) return -1;
+  if (num_single > 0 && (num_splits < 1 || num_splits > 64)) return -1;
+  if (num_single > 0 && num_splits > 1 && scratch == nullptr) return -1;
   AttnArgs a;
   a.q = (const bf16_t*)q;
   a.k_cache = (const bf16_t*)k_cache;

@@ -17,23 +17,26 @@ extern "C" const char* tp_last_error() { return g_error; }
 
 // ---- embedding ------------------------------------------------------------------
 // out[t, :] = table[token[t], :] widened to float32 (the residual stream).
+// grid: (tokens, column blocks of 256); every thread moves one element, so all loads of a
+// row are in flight at once.
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
                              float* __restrict__ out, int hidden) {
   const int t = blockIdx.x;
-  const T* row = table + (size_t)tokens[t] * hidden;
-  float* o = out + (size_t)t * hidden;
-  for (int j = threadIdx.x; j < hidden; j += blockDim.x) o[j] = to_float(row[j]);
+  const int j = blockIdx.y * blockDim.x + threadIdx.x;
+  if (j < hidden) out[(size_t)t * hidden + j] = to_float(table[(size_t)tokens[t] * hidden + j]);
 }
 
 extern "C" int tp_embed(const int* tokens, const void* table, int table_dt, float* out, int n,
                         int hidden, hipStream_t s) {
   TP_REQUIRE(n >= 0 && hidden > 0, "embed: bad sizes n=%d hidden=%d", n, hidden);
   if (n == 0) return 0;
+  const dim3 grid(n, (hidden + 255) / 256);
+  TP_REQUIRE(grid.y <= 65535, "embed: hidden size too large");
   if (table_dt == TP_F32)
-    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(256), 0, s, tokens, (const float*)table, out, hidden);
+    hipLaunchKernelGGL(embed_kernel<float>, grid, dim3(256), 0, s, tokens, (const float*)table, out, hidden);
   else if (table_dt == TP_BF16)
-    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(256), 0, s, tokens, (const bf16_t*)table, out, hidden);
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, dim3(256), 0, s, tokens, (const bf16_t*)table, out, hidden);
   else
     TP_REQUIRE(false, "embed: unknown dtype %d", table_dt);
   TP_CHECK_LAUNCH("embed");
@@ -105,78 +108,69 @@ extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void*
 }
 
 // ---- rotary position encoding + cache write -----------------------------------------
-// One block per token.  qkv row: [q heads | k heads | v heads] x head_dim, float32.
-// Pair (d, d + rotary_dim/2) of each q and k head turns by angle pos * inv_freq[d]; the
-// angle is formed in float64 from the integer position.  q goes to q_out, rotated k and raw
-// v go to the cache place `slots[t]` (page * page_size + offset) of the paged pools: keys
-// as [page, kv_head, page_size, head_dim], values TRANSPOSED as [page, kv_head, head_dim,
-// page_size] so that the attention kernels read eight consecutive keys of one value
-// element with one 16-byte load.  With slots == nullptr only q is produced (the row then
-// holds q heads only).
+// qkv row: [q heads | k heads | v heads] x head_dim, float32.  Pair (d, d + rotary_dim/2) of
+// each q and k head turns by the angle pos * inv_freq[d]: the product is formed in float64 and
+// reduced to [0, 2 pi) there, sine and cosine of the small rest are float32.  q goes to
+// q_out, rotated k and raw v go to the cache place `slots[t]` (page * page_size + offset) of
+// the paged pools: keys as [page, kv_head, page_size, head_dim], values TRANSPOSED as
+// [page, kv_head, head_dim, page_size] so that the attention kernels read eight consecutive
+// keys of one value element with one 16-byte load.  With slots == nullptr only q is produced
+// (the row then holds q heads only).
+// grid: (tokens, head blocks); a thread owns one pair (or two plain elements) of one head, so
+// every load of the row is in flight at once.
 template <typename TQ, typename TC>
 __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stride,
                                      const int* __restrict__ positions, const int* __restrict__ slots,
                                      const double* __restrict__ inv_freq, int rotary_dim, float factor,
                                      int n_heads, int n_kv, int head_dim, TQ* __restrict__ q_out,
-                                     TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size) {
-  extern __shared__ float cs[];  // cos[half], sin[half]
+                                     TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size,
+                                     int pairs, int heads_per_block) {
   const int t = blockIdx.x;
+  const int hl = threadIdx.x / pairs, d = threadIdx.x % pairs;   // pairs = head_dim / 2
+  const int h = blockIdx.y * heads_per_block + hl;
+  const int total_heads = n_heads + (slots ? 2 * n_kv : 0);
+  if (hl >= heads_per_block || h >= total_heads) return;
   const int half = rotary_dim / 2;
-  const double pos = (double)positions[t];
-  for (int d = threadIdx.x; d < half; d += blockDim.x) {
-    // the angle in float64, reduced to [0, 2 pi) there; sine and cosine of the small rest in float32
-    const double turns = pos * inv_freq[d] * 0.15915494309189535;
-    const float rest = (float)((turns - floor(turns)) * 6.283185307179586);
-    float sn, c;
-    sincosf(rest, &sn, &c);
-    cs[d] = c * factor;
-    cs[half + d] = sn * factor;
+  const float* row = qkv + (size_t)t * row_stride + (size_t)h * head_dim;
+  // the two elements this thread moves: a rotary pair, or two pass-through elements
+  int i0, i1;
+  if (d < half) {
+    i0 = d;
+    i1 = d + half;
+  } else {
+    i0 = rotary_dim + 2 * (d - half);
+    i1 = i0 + 1;
   }
-  __syncthreads();
-  const float* row = qkv + (size_t)t * row_stride;
-  const int rot_heads = n_heads + (slots ? n_kv : 0);
-  long slot = 0;
+  float y0 = row[i0], y1 = row[i1];
   size_t page = 0, off = 0;
   if (slots) {
-    slot = slots[t];
+    const int slot = slots[t];
     page = (size_t)(slot / page_size);
     off = (size_t)(slot % page_size);
   }
-  // rotated part of q and k heads: a thread keeps its pair index d and walks over heads
-  const int hstride = half > 0 ? max(1, (int)blockDim.x / half) : 1;
-  const int h_first = half > 0 ? threadIdx.x / half : rot_heads, d = half > 0 ? threadIdx.x % half : 0;
-  for (int h = h_first; h < rot_heads && h_first < hstride; h += hstride) {
-    const float x0 = row[h * head_dim + d], x1 = row[h * head_dim + d + half];
-    const float c = cs[d], sn = cs[half + d];
-    const float y0 = x0 * c - x1 * sn, y1 = x0 * sn + x1 * c;
-    if (h < n_heads) {
-      TQ* o = q_out + ((size_t)t * n_heads + h) * head_dim;
-      from_float(o + d, y0);
-      from_float(o + d + half, y1);
-    } else {
-      TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
-      from_float(o + d, y0);
-      from_float(o + d + half, y1);
-    }
+  if (h < n_heads + n_kv && d < half) {  // q and k heads rotate
+    const double turns = (double)positions[t] * inv_freq[d] * 0.15915494309189535;
+    const float rest = (float)((turns - floor(turns)) * 6.283185307179586);
+    float sn, c;
+    sincosf(rest, &sn, &c);
+    c *= factor;
+    sn *= factor;
+    const float x0 = y0, x1 = y1;
+    y0 = x0 * c - x1 * sn;
+    y1 = x0 * sn + x1 * c;
   }
-  // elements past the rotary part pass through
-  const int tail = head_dim - rotary_dim;
-  if (tail > 0) {
-    for (int i = threadIdx.x; i < rot_heads * tail; i += blockDim.x) {
-      const int h = i / tail, d = rotary_dim + i % tail;
-      const float x = row[h * head_dim + d];
-      if (h < n_heads)
-        from_float(q_out + ((size_t)t * n_heads + h) * head_dim + d, x);
-      else
-        from_float(k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim + d, x);
-    }
-  }
-  if (slots) {
-    const float* vrow = row + (size_t)(n_heads + n_kv) * head_dim;
-    for (int i = threadIdx.x; i < n_kv * head_dim; i += blockDim.x) {
-      const int h = i / head_dim, d = i % head_dim;
-      from_float(v_cache + ((page * n_kv + h) * head_dim + d) * page_size + off, vrow[i]);
-    }
+  if (h < n_heads) {
+    TQ* o = q_out + ((size_t)t * n_heads + h) * head_dim;
+    from_float(o + i0, y0);
+    from_float(o + i1, y1);
+  } else if (h < n_heads + n_kv) {
+    TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+    from_float(o + i0, y0);
+    from_float(o + i1, y1);
+  } else {
+    TC* o = v_cache + ((page * n_kv + (h - n_heads - n_kv)) * head_dim) * page_size + off;
+    from_float(o + (size_t)i0 * page_size, y0);
+    from_float(o + (size_t)i1 * page_size, y1);
   }
 }
 
@@ -185,18 +179,23 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
                                 int n_kv, int head_dim, void* q_out, int q_dt, void* k_cache, void* v_cache,
                                 int cache_dt, int page_size, hipStream_t s) {
   TP_REQUIRE(n >= 0 && n_heads > 0 && n_kv >= 0 && head_dim > 0, "rope_kv_write: bad sizes");
+  TP_REQUIRE(head_dim % 2 == 0 && head_dim <= 1024, "rope_kv_write: head_dim %d must be even and <= 1024", head_dim);
   TP_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim,
              "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, head_dim);
   TP_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope_kv_write: no frequency table");
-  TP_REQUIRE(rotary_dim <= 512, "rope_kv_write: rotary_dim %d exceeds 512", rotary_dim);
   TP_REQUIRE(slots == nullptr || (k_cache && v_cache && page_size > 0), "rope_kv_write: cache missing");
   TP_REQUIRE(row_stride >= (n_heads + (slots ? 2 * n_kv : 0)) * head_dim, "rope_kv_write: row too short");
   if (n == 0) return 0;
-  const size_t shmem = (size_t)(rotary_dim > 0 ? rotary_dim : 1) * sizeof(float);
-#define LAUNCH(TQ, TC)                                                                                   \
-  hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), dim3(n), dim3(256), shmem, s, qkv, row_stride,       \
-                     positions, slots, inv_freq, rotary_dim, factor, n_heads, n_kv, head_dim, (TQ*)q_out, \
-                     (TC*)k_cache, (TC*)v_cache, page_size)
+  const int pairs = head_dim / 2;
+  const int threads = pairs <= 256 ? 256 : 512;
+  const int hpb = threads / pairs;
+  const int total_heads = n_heads + (slots ? 2 * n_kv : 0);
+  const dim3 grid(n, (total_heads + hpb - 1) / hpb);
+  TP_REQUIRE(grid.y <= 65535, "rope_kv_write: too many heads");
+#define LAUNCH(TQ, TC)                                                                                    \
+  hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), grid, dim3(threads), 0, s, qkv, row_stride, positions, \
+                     slots, inv_freq, rotary_dim, factor, n_heads, n_kv, head_dim, (TQ*)q_out, (TC*)k_cache, \
+                     (TC*)v_cache, page_size, pairs, hpb)
   if (q_dt == TP_F32 && cache_dt == TP_F32)
     LAUNCH(float, float);
   else if (q_dt == TP_BF16 && cache_dt == TP_BF16)

@@ -261,7 +261,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         # enough blocks to fill 256 CUs, but at least 128 keys per block
         blocks_per_split = num_single * kvh * ((heads // kvh + 15) // 16)
         splits = max(1, min(64, -(-1024 // blocks_per_split), max(1, max_context_len // 128)))
-        scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
+        if splits > 1:
+            scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
     _call("tp_paged_attention", _ptr(q), _dt(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), width,
           _ptr(cu_seqlens), _ptr(context_lens), _ptr(token_req), _ptr(out), n, r, heads, kvh, d, page_size,
           ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(fast),
