@@ -142,22 +142,23 @@ static void launch_generic(const void* x, const void* w, void* out, int M, int N
 // Defined in gemm_mfma.hip; returns 0 when it took the product, -1 when the sizes are
 // not its own (the general kernel then runs), >0 on error.
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
-                   hipStream_t s);
+                   float* scratch, size_t scratch_floats, hipStream_t s);
 
+// `scratch` (optional, `scratch_floats` float32): room for split-K partial sums of mid-sized products.
 extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
-                         int N, int K, int allow_mfma, hipStream_t s) {
+                         int N, int K, int allow_mfma, float* scratch, size_t scratch_floats, hipStream_t s) {
   TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(accumulate != 1 || out_dt == TP_F32, "linear: accumulating output must be float32");
   if (accumulate == 2) {  // gated-SiLU epilogue: only the matrix-core kernels have it
     TP_REQUIRE(in_dt == TP_BF16 && allow_mfma, "linear: the gated epilogue needs bfloat16 operands");
-    const int r = tp_linear_mfma(x, w, out, out_dt, 2, M, N, K, s);
+    const int r = tp_linear_mfma(x, w, out, out_dt, 2, M, N, K, scratch, scratch_floats, s);
     TP_REQUIRE(r >= 0, "linear: sizes M=%d N=%d K=%d do not fit the gated epilogue", M, N, K);
     return r;
   }
   TP_REQUIRE((size_t)M * N < ((size_t)1 << 40), "linear: output too large");
   if (M == 0) return 0;
   if (in_dt == TP_BF16 && allow_mfma) {
-    const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, s);
+    const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, scratch, scratch_floats, s);
     if (r >= 0) return r;
   }
   if (in_dt == TP_F32 && out_dt == TP_F32) {

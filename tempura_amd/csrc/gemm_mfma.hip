@@ -234,86 +234,105 @@ __global__ __launch_bounds__(512) void gemm_skinny_lds_kernel(const bf16_t* __re
 }
 
 // ---- tiled ----------------------------------------------------------------------------
-#define TBM 128
-#define TBN 128
-
-template <int BK>
+// Block of four waves (2 x 2); a wave owns WMT x WNT result tiles of 16 x 16, so the block
+// tile is (32 WMT) x (32 WNT).  blockIdx.z splits K: with more than one split every block
+// writes its float32 partial tile to `partial` [split, M, N] and a second kernel adds the
+// splits in ascending order and applies the epilogue (so the result does not depend on timing).
+// Measured on MI355X: two blocks per CU matter more than a larger tile (a 256 x 128 tile or
+// a second set of prefetch registers drops occupancy to one wave per SIMD and loses a third).
+template <int BK, int WMT, int WNT>
 __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __restrict__ x,
                                                               const bf16_t* __restrict__ w, void* __restrict__ out,
-                                                              int mode, int M, int N, int K) {
+                                                              float* __restrict__ partial, int mode, int M, int N,
+                                                              int K) {
+  constexpr int BM = 32 * WMT, BN = 32 * WNT;
   constexpr int LD = BK + 8;            // padded row, in bf16 elements (conflict-free 16-byte reads)
   constexpr int CPR = BK / 8;           // 16-byte chunks per tile row
-  constexpr int CPT = TBM * CPR / 256;  // chunks per thread per operand
-  __shared__ __attribute__((aligned(16))) uint16_t xs[TBM * LD];
-  __shared__ __attribute__((aligned(16))) uint16_t ws[TBN * LD];
+  constexpr int XCPT = BM * CPR / 256;  // chunks per thread, x tile
+  constexpr int WCPT = BN * CPR / 256;  // chunks per thread, w tile
+  __shared__ __attribute__((aligned(16))) uint16_t xs[BM * LD];
+  __shared__ __attribute__((aligned(16))) uint16_t ws[BN * LD];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * TBM, n0 = blockIdx.x * TBN;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  // this block's share of K, in tiles
+  const int KT_all = K / BK;
+  const int per = (KT_all + gridDim.z - 1) / gridDim.z;
+  const int kt_begin = blockIdx.z * per, kt_end = min(KT_all, kt_begin + per);
 
-  f32x4_t acc[4][4];
+  f32x4_t acc[WMT][WNT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < WMT; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < WNT; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  u32x4_t xr[CPT], wr[CPT];
+  u32x4_t xr[XCPT], wr[WCPT];
   auto load_global = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
+    for (int i = 0; i < XCPT; ++i) {
       const int c = tid + 256 * i;
-      const int row = c / CPR, kc = c % CPR;
-      const int gm = min(m0 + row, M - 1), gn = min(n0 + row, N - 1);
-      xr[i] = *(const u32x4_t*)(x + (size_t)gm * K + k0 + kc * 8);
-      wr[i] = *(const u32x4_t*)(w + (size_t)gn * K + k0 + kc * 8);
+      const int gm = min(m0 + c / CPR, M - 1);
+      xr[i] = *(const u32x4_t*)(x + (size_t)gm * K + k0 + (c % CPR) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < WCPT; ++i) {
+      const int c = tid + 256 * i;
+      const int gn = min(n0 + c / CPR, N - 1);
+      wr[i] = *(const u32x4_t*)(w + (size_t)gn * K + k0 + (c % CPR) * 8);
     }
   };
   auto store_lds = [&]() {
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
+    for (int i = 0; i < XCPT; ++i) {
       const int c = tid + 256 * i;
-      const int row = c / CPR, kc = c % CPR;
-      *(u32x4_t*)(&xs[row * LD + kc * 8]) = xr[i];
-      *(u32x4_t*)(&ws[row * LD + kc * 8]) = wr[i];
+      *(u32x4_t*)(&xs[(c / CPR) * LD + (c % CPR) * 8]) = xr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < WCPT; ++i) {
+      const int c = tid + 256 * i;
+      *(u32x4_t*)(&ws[(c / CPR) * LD + (c % CPR) * 8]) = wr[i];
     }
   };
 
   // The next tile travels from global memory into registers while this one is multiplied.
-  const int KT = K / BK;
-  load_global(0);
-  for (int kt = 0; kt < KT; ++kt) {
+  if (kt_begin < kt_end) load_global(kt_begin * BK);
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
     store_lds();
     __syncthreads();
-    if (kt + 1 < KT) load_global((kt + 1) * BK);
+    if (kt + 1 < kt_end) load_global((kt + 1) * BK);
 #pragma unroll
     for (int kk = 0; kk < BK / 32; ++kk) {
-      bf16x8_t a[4], b[4];
+      bf16x8_t b[WNT];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        a[i] = as_frag(*(const u32x4_t*)(&xs[(wm * 64 + i * 16 + (lane & 15)) * LD + kk * 32 + (lane >> 4) * 8]));
+      for (int j = 0; j < WNT; ++j)
+        b[j] = as_frag(*(const u32x4_t*)(&ws[(wn * 16 * WNT + j * 16 + (lane & 15)) * LD + kk * 32 + (lane >> 4) * 8]));
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        b[j] = as_frag(*(const u32x4_t*)(&ws[(wn * 64 + j * 16 + (lane & 15)) * LD + kk * 32 + (lane >> 4) * 8]));
+      for (int i = 0; i < WMT; ++i) {
+        const bf16x8_t a =
+            as_frag(*(const u32x4_t*)(&xs[(wm * 16 * WMT + i * 16 + (lane & 15)) * LD + kk * 32 + (lane >> 4) * 8]));
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WNT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j], acc[i][j], 0, 0, 0);
+      }
     }
     __syncthreads();
   }
   // result lane l: rows (l / 16) * 4 + r of the x tile (m), column l % 16 of the w tile (n)
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < WMT; ++i) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int m = m0 + wm * 64 + i * 16 + (lane >> 4) * 4 + r;
+      const int m = m0 + wm * 16 * WMT + i * 16 + (lane >> 4) * 4 + r;
       if (m >= M) continue;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int n = n0 + wn * 64 + j * 16 + (lane & 15);
-        if (mode == OUT_SWIGLU) {
+      for (int j = 0; j < WNT; ++j) {
+        const int nt = n0 + wn * 16 * WNT + j * 16;   // first column of this 16-wide tile
+        const int n = nt + (lane & 15);
+        if (gridDim.z > 1) {
+          if (n < N) partial[((size_t)blockIdx.z * M + m) * N + n] = acc[i][j][r];
+        } else if (mode == OUT_SWIGLU) {
           const float u = __shfl_xor(acc[i][j][r], 8, 64);   // the up row sits eight columns to the right
           if ((lane & 8) == 0 && n + 8 < N)
-            ((bf16_t*)out)[(size_t)m * (N / 2) + (n0 + wn * 64 + j * 16) / 2 + (lane & 7)] = float_to_bf16(silu_mul(acc[i][j][r], u));
+            ((bf16_t*)out)[(size_t)m * (N / 2) + nt / 2 + (lane & 7)] = float_to_bf16(silu_mul(acc[i][j][r], u));
         } else if (n < N) {
           store_out(out, mode, (size_t)m * N + n, acc[i][j][r]);
         }
@@ -322,11 +341,42 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __re
   }
 }
 
+// Adds the K splits of `partial` [splits, M, N] in ascending order and applies the epilogue.
+__global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out, int mode,
+                                          int splits, int M, int N) {
+  const size_t total = (size_t)M * N;
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (mode == OUT_SWIGLU) {
+    // one thread per output element: column 8 b + i pairs rows 16 b + i and 16 b + 8 + i
+    const int half = N / 2;
+    if (idx >= (size_t)M * half) return;
+    const int m = (int)(idx / half), c = (int)(idx % half);
+    const int ng = (c / 8) * 16 + (c % 8);
+    float g = 0.f, u = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      g += partial[(size_t)s * total + (size_t)m * N + ng];
+      u += partial[(size_t)s * total + (size_t)m * N + ng + 8];
+    }
+    ((bf16_t*)out)[idx] = float_to_bf16(silu_mul(g, u));
+    return;
+  }
+  if (idx >= total) return;
+  float v = 0.f;
+  for (int s = 0; s < splits; ++s) v += partial[(size_t)s * total + idx];
+  store_out(out, mode, idx, v);
+}
+
 // In the skinny kernel x is the second operand, so the result lane holds weight rows
 // (l / 16) * 4 + r and activation row l % 16; see the index arithmetic there.
 
 // Tuning knobs of the skinny kernel (0 = choose by shape); set through tp_linear_tune.
 static int g_tune_waves = 0, g_tune_nt = 0, g_tune_depth = 0;   // depth 9 selects the LDS kernel
+static int g_tune_splits = 0, g_tune_mid = 0;                    // mid = 1: 17..64 rows stay on the skinny kernel
+
+extern "C" void tp_linear_tune_mid(int mid, int splits) {
+  g_tune_mid = mid;
+  g_tune_splits = splits;
+}
 
 extern "C" void tp_linear_tune(int waves, int nt, int depth) {
   g_tune_waves = waves;
@@ -399,14 +449,15 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
 
 // accumulate: 0 store, 1 add into the float32 output, 2 gated-SiLU epilogue (see OUT_SWIGLU)
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
-                   hipStream_t s) {
+                   float* scratch, size_t scratch_floats, hipStream_t s) {
   if (K % 32 != 0) return -1;
   if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return -1;
   if (accumulate == 2 && (N % 16 != 0 || out_dt != TP_BF16)) return -1;
   const int mode = accumulate == 2 ? OUT_SWIGLU : (accumulate ? OUT_ACC_F32 : (out_dt == TP_F32 ? OUT_F32 : OUT_BF16));
   const bf16_t* xb = (const bf16_t*)x;
   const bf16_t* wb = (const bf16_t*)w;
-  if (M <= 64) {
+  const bool mid_ok = scratch != nullptr && g_tune_mid != 1;
+  if (M <= 16 || (M <= 64 && !mid_ok)) {
     if (M <= 16)
       launch_skinny<1>(xb, wb, out, mode, M, N, K, s);
     else if (M <= 32)
@@ -416,12 +467,32 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
     else
       launch_skinny<4>(xb, wb, out, mode, M, N, K, s);
   } else {
-    const dim3 grid((N + TBN - 1) / TBN, (M + TBM - 1) / TBM);
-    if (grid.y > 65535) return -1;
-    if (K % 64 == 0)
-      hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64>), grid, dim3(256), 0, s, xb, wb, out, mode, M, N, K);
-    else
-      hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32>), grid, dim3(256), 0, s, xb, wb, out, mode, M, N, K);
+    // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
+    // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.
+    if (M > 128 || scratch == nullptr) {
+      const dim3 grid((N + 127) / 128, (M + 127) / 128);
+      if (grid.y > 65535) return -1;
+      if (K % 64 == 0)
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K);
+      else
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K);
+    } else {
+      const int nb = (N + 127) / 128, mb = (M + 63) / 64;
+      int splits = g_tune_splits ? g_tune_splits : (512 + nb * mb - 1) / (nb * mb);
+      const int kt = K / (K % 64 == 0 ? 64 : 32);
+      splits = max(1, min(splits, min(16, kt / 4)));
+      while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
+      const dim3 grid(nb, mb, splits);
+      if (K % 64 == 0)
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K);
+      else
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K);
+      if (splits > 1) {
+        const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out,
+                           mode, splits, M, N);
+      }
+    }
   }
   TP_CHECK_LAUNCH("linear (mfma)");
   return 0;

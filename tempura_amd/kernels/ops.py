@@ -163,8 +163,18 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     n = w.shape[0]
     _need(n % 16 == 0 and k % 32 == 0, "linear_swiglu: needs 2i % 16 == 0 and k % 32 == 0")
     out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
-    _call("tp_linear", _ptr(x), _ptr(w), _BF16, _ptr(out), _BF16, 2, m, n, k, 1, _stream())
+    scratch, nscratch = _splitk_scratch(x, m, n)
+    _call("tp_linear", _ptr(x), _ptr(w), _BF16, _ptr(out), _BF16, 2, m, n, k, 1, _ptr(scratch),
+          ctypes.c_size_t(nscratch), _stream())
     return out
+
+
+def _splitk_scratch(x: torch.Tensor, m: int, n: int):
+    """Room for the partial sums of a bfloat16 product of 17..128 rows (its K is split over blocks)."""
+    if x.dtype != torch.bfloat16 or not (16 < m <= 128):
+        return None, 0
+    count = min(16, max(1, -(-512 // (-(-n // 128) * -(-m // 64))))) * m * n
+    return torch.empty((count,), dtype=torch.float32, device=x.device), count
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
@@ -183,7 +193,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
         out, acc = residual, 1
     else:
         out, acc = torch.empty((m, n), dtype=out_dtype, device=x.device), 0
-    _call("tp_linear", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _stream())
+    scratch, nscratch = _splitk_scratch(x, m, n) if allow_mfma else (None, 0)
+    _call("tp_linear", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
+          ctypes.c_size_t(nscratch), _stream())
     return out
 
 
