@@ -39,6 +39,7 @@ def parse_args():
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--point-steps", type=int, default=128)
+    ap.add_argument("--decode-target-blocks", type=int, default=None, help="tuning: blocks the split decode attention aims at")
     return ap.parse_args()
 
 
@@ -58,6 +59,8 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 3
     dev = torch.device("cuda:0")
+    if args.decode_target_blocks:
+        ops.decode_target_blocks = args.decode_target_blocks
     full = PRESETS[args.model_config]
     cfg = LlamaConfig.from_dict(full.to_dict())
     if args.layers is not None:

@@ -49,42 +49,56 @@ struct AttnArgs {
   float scale_log2;
 };
 
-// One step of 32 keys starting at j0 for NQ query tiles.  qpos[nq] is the absolute position
-// of this lane's query column (keys above it are masked); kvh the kv head; ctx the number
-// of keys that exist.  m/l/o are the running statistics and output of each tile.
-template <int D, int NQ>
-__device__ inline void attn_step(const AttnArgs& a, const int* __restrict__ table, int kvh, int ctx, int j0,
-                                 const bf16x8_t (&qf)[NQ][D / 32], const int (&qpos)[NQ], float (&m)[NQ],
-                                 float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+// The keys and values of one step of 32 keys, as MFMA operand fragments.
+template <int D>
+struct KvFrags {
+  bf16x8_t k[2][D / 32];
+  bf16x8_t v[D / 16];
+};
+
+// Fetch the fragments of the step starting at key j0 (kvh: kv head; ctx: keys that exist; keys
+// past the end are clamped to the last one and masked later).
+template <int D>
+__device__ inline void attn_load(const AttnArgs& a, const int* __restrict__ table, int kvh, int ctx, int j0,
+                                 KvFrags<D>& f) {
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4, c = lane & 15;
   const int ps = a.page_size;
-  // scores: two 16-key tiles
-  f32x4_t s[NQ][2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int key = min(j0 + 8 * (c >> 2) + 4 * t + (c & 3), ctx - 1);
     const int page = table[key / ps];
     const bf16_t* kr = a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + key % ps) * D + g * 8;
-    bf16x8_t kf[D / 32];
 #pragma unroll
-    for (int dk = 0; dk < D / 32; ++dk) kf[dk] = frag_of(*(const u32x4_t*)(kr + dk * 32));
-#pragma unroll
-    for (int nq = 0; nq < NQ; ++nq) {
-      s[nq][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int dk = 0; dk < D / 32; ++dk)
-        s[nq][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[dk], qf[nq][dk], s[nq][t], 0, 0, 0);
-    }
+    for (int dk = 0; dk < D / 32; ++dk) f.k[t][dk] = frag_of(*(const u32x4_t*)(kr + dk * 32));
   }
   // values: eight consecutive keys of element d per lane
   const int kb = min(j0 + 8 * g, (ctx - 1) & ~7);
   const int vpage = table[kb / ps];
   const bf16_t* vr = a.v_cache + ((size_t)(vpage * a.n_kv + kvh) * D + c) * ps + kb % ps;
-  bf16x8_t vf[D / 16];
 #pragma unroll
-  for (int dt = 0; dt < D / 16; ++dt) vf[dt] = frag_of(*(const u32x4_t*)(vr + (size_t)dt * 16 * ps));
+  for (int dt = 0; dt < D / 16; ++dt) f.v[dt] = frag_of(*(const u32x4_t*)(vr + (size_t)dt * 16 * ps));
+}
 
+// One step of 32 keys starting at j0 for NQ query tiles, on fetched fragments.  qpos[nq] is the
+// absolute position of this lane's query column (keys above it are masked).  m/l/o are the
+// running statistics and output of each tile.
+template <int D, int NQ>
+__device__ inline void attn_compute(const AttnArgs& a, int j0, const KvFrags<D>& f, const bf16x8_t (&qf)[NQ][D / 32],
+                                    const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+  // scores: two 16-key tiles
+  f32x4_t s[NQ][2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      s[nq][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dk = 0; dk < D / 32; ++dk)
+        s[nq][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[t][dk], qf[nq][dk], s[nq][t], 0, 0, 0);
+    }
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
     // this lane's keys: j0 + 8g + 4t + r
@@ -127,9 +141,18 @@ __device__ inline void attn_step(const AttnArgs& a, const int* __restrict__ tabl
       acc[1] *= alpha;
       acc[2] *= alpha;
       acc[3] *= alpha;
-      o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, acc, 0, 0, 0);
+      o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt], pf, acc, 0, 0, 0);
     }
   }
+}
+
+template <int D, int NQ>
+__device__ inline void attn_step(const AttnArgs& a, const int* __restrict__ table, int kvh, int ctx, int j0,
+                                 const bf16x8_t (&qf)[NQ][D / 32], const int (&qpos)[NQ], float (&m)[NQ],
+                                 float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+  KvFrags<D> f;
+  attn_load<D>(a, table, kvh, ctx, j0, f);
+  attn_compute<D, NQ>(a, j0, f, qf, qpos, m, l, o);
 }
 
 // ---- prefill ----------------------------------------------------------------------------
@@ -233,6 +256,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   const int steps = (ctx - first + 31) / 32;
   const int per_split = (steps + a.num_splits - 1) / a.num_splits;
   const int s_begin = blockIdx.z * per_split, s_end = min(steps, s_begin + per_split);
+  // (Fetching the next step's fragments while this one is computed was measured: the doubled
+  // fragment registers halve the occupancy and the kernel gets slower, not faster.)
   for (int s = s_begin + wave; s < s_end; s += 4) attn_step<D, 1>(a, table, kvh, ctx, first + s * 32, qf, qpos, m, l, o);
 
   // merge the four waves (fixed order), then write this split's partial

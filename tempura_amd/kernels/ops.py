@@ -236,6 +236,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[to
 
 #: bfloat16 attention may use the matrix-core kernels
 allow_fast_attention = True
+#: the split decode kernel aims at this many blocks (of four waves) in flight
+decode_target_blocks = 256
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
@@ -272,7 +274,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
         blocks_per_split = num_single * kvh * ((heads // kvh + 15) // 16)
-        splits = max(1, min(64, -(-1024 // blocks_per_split), max(1, max_context_len // 128)))
+        splits = max(1, min(64, -(-decode_target_blocks // blocks_per_split), max(1, max_context_len // 128)))
         if splits > 1:
             scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
     _call("tp_paged_attention", _ptr(q), _dt(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), width,
