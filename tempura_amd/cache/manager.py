@@ -101,12 +101,9 @@ class CacheManager:
         need = []
         for g in range(len(self.groups)):
             lo = max(self._first_needed(g, r.num_tokens), r.first_live[g])
-            table = r.tables[g]
-            cnt = 0
-            for lp in range(lo, last_page + 1):
-                if lp >= len(table) or table[lp] < 0:
-                    cnt += 1
-            need.append(cnt)
+            # every entry from first_live up to the table's end holds a page (pages are given back
+            # only below first_live), so what is missing is what lies beyond the table
+            need.append(max(0, last_page + 1 - max(lo, len(r.tables[g]))))
         return need
 
     def can_reserve(self, rid, n_new: int) -> bool:
@@ -127,11 +124,14 @@ class CacheManager:
         for g in range(len(self.groups)):
             lo = max(self._first_needed(g, r.num_tokens), r.first_live[g])
             table = r.tables[g]
+            have = len(table)
             while len(table) <= last_page:
                 table.append(-1)
-            for lp in range(lo, last_page + 1):
-                if table[lp] < 0:
-                    table[lp] = self.pools[g].alloc()
+            # pages that a window has already passed (below lo) stay unallocated
+            for lp in range(max(lo, have), last_page + 1):
+                table[lp] = self.pools[g].alloc()
+            if lo > have:
+                r.first_live[g] = max(r.first_live[g], min(lo, len(table)))
 
     def commit(self, rid, n_new: int) -> None:
         """``n_new`` tokens were written; give back pages a window has passed."""
@@ -161,6 +161,14 @@ class CacheManager:
 
     def table(self, rid, g: int) -> List[int]:
         return self._requests[rid].tables[g]
+
+    def slot(self, rid, g: int, pos: int) -> int:
+        """Physical cache row of one position (the single-token case of ``slots``)."""
+        table = self._requests[rid].tables[g]
+        lp = pos // self.page_size
+        if pos < 0 or lp >= len(table) or table[lp] < 0:
+            raise RuntimeError(f"request {rid!r}: position {pos} has no page reserved")
+        return table[lp] * self.page_size + pos % self.page_size
 
     def slots(self, rid, g: int, start: int, n: int) -> np.ndarray:
         """Physical cache rows (page * page_size + offset) of positions start..start+n-1."""

@@ -283,12 +283,13 @@ class ModelRunner:
             bt = h[offs[4 + gi]: offs[5 + gi]].reshape(g.rows, g.width)
             bt[:] = scratch
             for r, e in enumerate(entries):
-                t = np.asarray(self.cache.table(e.rid, gi), dtype=np.int32)
-                bt[r, : len(t)] = np.where(t >= 0, t, scratch)
+                t = self.cache.table(e.rid, gi)
+                bt[r, : len(t)] = t
+            if self.cache.groups[gi].kind != "full":
+                bt[bt < 0] = scratch       # pages a window has given back; no query reads them
             sl = h[offs[4 + n_groups + gi]: offs[5 + n_groups + gi]]
             sl[:] = scratch * self.page_size
-            for r, (e, s0) in enumerate(zip(entries, starts)):
-                sl[r] = self.cache.slots(e.rid, gi, s0, 1)[0]
+            sl[:n] = [self.cache.slot(e.rid, gi, s0) for e, s0 in zip(entries, starts)]
         g.packed.copy_(g.host, non_blocking=True)
         g.copied.record()
 
