@@ -26,7 +26,7 @@ MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=512, help="timed decode steps")
+    ap.add_argument("--steps", type=int, default=2000, help="timed decode steps (KV grows from 2,048 towards 4,096)")
     ap.add_argument("--warmup", type=int, default=16, help="untimed decode steps")
     ap.add_argument("--model-config", default="llama-3.1-8b")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
-    ap.add_argument("--point-steps", type=int, default=128)
+    ap.add_argument("--point-steps", type=int, default=1000, help="timed steps of the batch-1 and batch-64 points")
     ap.add_argument("--decode-target-blocks", type=int, default=None, help="tuning: blocks the split decode attention aims at")
     return ap.parse_args()
 
@@ -149,7 +149,7 @@ def main() -> int:
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            ps = min(args.point_steps, args.context - args.prompt_len - 8)
+            ps = min(args.point_steps, steps, args.context - args.prompt_len - 8)
             p_tps, p_ms, _ = decode_run(b, 8, ps)
             points[f"decode_b{b}"] = round(p_tps, 1)
             print(f"[bench] decode b{b}: {p_tps:.1f} tok/s, {p_ms:.3f} ms/step", file=sys.stderr, flush=True)

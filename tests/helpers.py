@@ -31,6 +31,13 @@ CONFIGS: Dict[str, LlamaConfig] = {
                      rope_scaling=RopeScaling("llama3", 4.0, 1.0, 2.0, 32), tie_word_embeddings=False,
                      sliding_window=24,
                      layer_types=["sliding_attention", "full_attention", "sliding_attention", "full_attention"]),
+    # D: sizes the matrix-core kernels take (head size 64, widths that are multiples of 32, gate/up rows
+    #    in eights): in bfloat16 every fast path runs end to end (skinny, mid and tiled products, fused
+    #    SwiGLU, MFMA attention for portions and for single tokens with a split context)
+    "D": LlamaConfig(hidden_size=128, intermediate_size=320, num_hidden_layers=2, num_attention_heads=4,
+                     num_key_value_heads=2, head_dim=64, vocab_size=512, max_position_embeddings=2048,
+                     rms_norm_eps=1e-5, rope_theta=500000.0,
+                     rope_scaling=RopeScaling("llama3", 8.0, 1.0, 4.0, 128), tie_word_embeddings=False),
 }
 #: weights are N(0, STD): large enough that attention is peaked and faults show
 STD = 0.15
@@ -46,7 +53,7 @@ class TinyModels:
         if key not in self._made:
             d = os.path.join(self.root, f"{name}_{dtype}")
             cfg = LlamaConfig.from_dict(CONFIGS[name].to_dict())
-            write_random_model(cfg, d, seed={"A": 11, "B": 23, "C": 37}[name], std=STD, norm_jitter=0.2, dtype=dtype)
+            write_random_model(cfg, d, seed={"A": 11, "B": 23, "C": 37, "D": 41}[name], std=STD, norm_jitter=0.2, dtype=dtype)
             self._made[key] = d
         return self._made[key]
 
@@ -143,8 +150,9 @@ def schedule_mixed(lengths: Dict[str, int], max_tokens: int, seed: int, max_live
 # ---- replaying a schedule through a runner -----------------------------------------------------
 LENGTHS = {"A": {"a0": 5, "a1": 17, "a2": 33, "a3": 150, "a4": 97, "a5": 64},
            "B": {"b0": 1, "b1": 9, "b2": 40, "b3": 63, "b4": 120, "b5": 201},
-           "C": {"c0": 3, "c1": 49, "c2": 130, "c3": 75, "c4": 25, "c5": 88}}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 32}
+           "C": {"c0": 3, "c1": 49, "c2": 130, "c3": 75, "c4": 25, "c5": 88},
+           "D": {"d0": 7, "d1": 300, "d2": 41, "d3": 170, "d4": 96, "d5": 33}}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 32, "D": 16}
 
 
 def requests_for(name: str) -> Dict[str, List[int]]:

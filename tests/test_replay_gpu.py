@@ -46,7 +46,7 @@ def _compare(got, ref, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_replay_modes(tiny_dirs, name, dtype, mode):
     requests = helpers.requests_for(name)
@@ -59,7 +59,7 @@ def test_replay_modes(tiny_dirs, name, dtype, mode):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("name", ["A", "C", "D"])
 def test_graph_replays_match_eager(tiny_dirs, name, dtype):
     """Decode steps replayed as a captured graph give the eager steps' logits, replay after replay, with
     eager steps (prompt portions of other requests) and synchronisations between the replays."""
@@ -71,7 +71,14 @@ def test_graph_replays_match_eager(tiny_dirs, name, dtype):
     graphed = helpers.run_schedule(runner, requests, steps)
     assert runner.graph_steps >= 32, "decode-only steps went through the graph"
     for rid in eager:
-        assert torch.equal(graphed[rid], eager[rid]), f"request {rid}: graph replay differs from the eager step"
+        if dtype == "float32" or name != "D":
+            assert torch.equal(graphed[rid], eager[rid]), f"request {rid}: graph replay differs from the eager step"
+        else:
+            # the captured step splits the context by its bound, the eager one by the actual length: the
+            # probabilities are rounded to bfloat16 against another running maximum.  Both stay within
+            # the tolerance of the plain implementation (checked below); against each other a third of it.
+            assert helpers.rel_err(graphed[rid], eager[rid]) < helpers.TOL[dtype] / 3, \
+                f"request {rid}: graph replay differs from the eager step"
     _compare(graphed, _reference(tiny_dirs, name, dtype), dtype, f"{name}/{dtype}/graph")
 
 
@@ -88,7 +95,7 @@ def test_long_decoding(tiny_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_first_tokens(tiny_dirs, name, dtype):
     """The first tokens of a sequence, one by one from position 0 (one key, then two, ...)."""
     cfg, W = tiny_dirs.plain_model(name, dtype)
@@ -153,3 +160,17 @@ def test_trace_run_program(tiny_dirs, tmp_path, dtype):
             checked += c
         assert row == arr.shape[0]
     assert checked > 200
+
+
+def test_long_context_decoding_bfloat16_fast_paths(tiny_dirs):
+    """Config D in bfloat16: 1,500 tokens in three portions (the tiled product and the MFMA prefill attention,
+    with and without a cached prefix), then 40 tokens one by one over a context long enough that the decode
+    attention splits it (graph replays)."""
+    cfg, W = tiny_dirs.plain_model("D", "bfloat16")
+    toks = helpers.random_tokens(cfg["vocab_size"], 1540, seed=81)
+    ref = plain.forward(cfg, W, toks)
+    runner = _runner(tiny_dirs, "D", "bfloat16", 1600, 16, use_graph=True)
+    steps = [([("x", 0, 700)], []), ([("x", 700, 90)], []), ([("x", 790, 710)], [])] + [([("x", i, 1)], []) for i in range(1500, 1540)]
+    got = helpers.run_schedule(runner, {"x": toks}, steps)
+    assert runner.graph_steps == 40
+    _compare(got, {"x": ref}, "bfloat16", "long context D")
