@@ -244,7 +244,7 @@ template <int BK, int WMT, int WNT>
 __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __restrict__ x,
                                                               const bf16_t* __restrict__ w, void* __restrict__ out,
                                                               float* __restrict__ partial, int mode, int M, int N,
-                                                              int K) {
+                                                              int K, int xcd_order) {
   constexpr int BM = 32 * WMT, BN = 32 * WNT;
   constexpr int LD = BK + 8;            // padded row, in bf16 elements (conflict-free 16-byte reads)
   constexpr int CPR = BK / 8;           // 16-byte chunks per tile row
@@ -254,7 +254,21 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(const bf16_t* __re
   __shared__ __attribute__((aligned(16))) uint16_t ws[BN * LD];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  int bm = blockIdx.y, bn = blockIdx.x;
+  if (xcd_order) {
+    // Blocks go to the eight XCDs round robin by launch order, and each XCD has an L2 of its own.
+    // XCD c takes the column blocks c, c + 8, ...; the blocks it runs at the same time form an
+    // 8 x 8 patch of (row block, column block), so that every weight tile and every activation
+    // tile it fetches is used by eight blocks while it is still in that L2.
+    const int MB = (M + BM - 1) / BM, NB = (N + BN - 1) / BN;
+    const int Q = (NB + 7) / 8, MS = (MB + 7) / 8;
+    const int c = blockIdx.x % 8, j = blockIdx.x / 8;
+    const int t = j / 64, r = j % 64;
+    bm = (t % MS) * 8 + r % 8;
+    bn = c + 8 * ((t / MS) * 8 + r / 8);
+    if (bm >= MB || bn >= NB || (t / MS) * 8 + r / 8 >= Q) return;
+  }
+  const int m0 = bm * BM, n0 = bn * BN;
   // this block's share of K, in tiles
   const int KT_all = K / BK;
   const int per = (KT_all + gridDim.z - 1) / gridDim.z;
@@ -372,6 +386,12 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
 // Tuning knobs of the skinny kernel (0 = choose by shape); set through tp_linear_tune.
 static int g_tune_waves = 0, g_tune_nt = 0, g_tune_depth = 0;   // depth 9 selects the LDS kernel
 static int g_tune_splits = 0, g_tune_mid = 0;                    // mid = 1: 17..64 rows stay on the skinny kernel
+static int g_tune_order = 0;   // large products: 1 tiled kernel, plain block order; 2 tiled, XCD patches; 3 pipelined kernel
+
+// Defined in gemm_pipe.hip; 0 when it took the product, -1 when the sizes are not its own.
+int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s);
+
+extern "C" void tp_linear_tune_tile(int order) { g_tune_order = order; }
 
 extern "C" void tp_linear_tune_mid(int mid, int splits) {
   g_tune_mid = mid;
@@ -469,13 +489,23 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   } else {
     // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
     // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.
-    if (M > 128 || scratch == nullptr) {
-      const dim3 grid((N + 127) / 128, (M + 127) / 128);
+    const bool pipe = g_tune_order ? g_tune_order == 3 : M > 256;
+    if (pipe && M > 128 && tp_linear_pipe(xb, wb, out, mode, M, N, K, s) == 0) {
+      // taken by the pipelined kernel
+    } else if (M > 128 || scratch == nullptr) {
+      dim3 grid((N + 127) / 128, (M + 127) / 128);
       if (grid.y > 65535) return -1;
+      const int xcd_order = g_tune_order != 1;
+      if (xcd_order) {  // one-dimensional grid: 8 XCDs x patches of 64 blocks
+        const int Q = ((int)grid.x + 7) / 8, MS = ((int)grid.y + 7) / 8, QS = (Q + 7) / 8;
+        grid = dim3(8 * QS * MS * 64, 1);
+      }
       if (K % 64 == 0)
-        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K);
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K,
+                           xcd_order);
       else
-        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K);
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 4, 4>), grid, dim3(256), 0, s, xb, wb, out, nullptr, mode, M, N, K,
+                           xcd_order);
     } else {
       const int nb = (N + 127) / 128, mb = (M + 63) / 64;
       int splits = g_tune_splits ? g_tune_splits : (512 + nb * mb - 1) / (nb * mb);
@@ -484,9 +514,9 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
       while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
       const dim3 grid(nb, mb, splits);
       if (K % 64 == 0)
-        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K);
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0);
       else
-        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K);
+        hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0);
       if (splits > 1) {
         const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out,

@@ -1,0 +1,321 @@
+// Large bfloat16 products (prefill): out[M, N] (+)= x[M, K] * w[N, K]^T on the gfx950 matrix cores,
+// software-pipelined by hand.
+//
+// A block of four waves (2 x 2) owns a 256 x 128 result tile, a wave 128 x 64 of it (8 x 4 tiles of
+// v_mfma_f32_16x16x32_bf16, 128 accumulator registers).  K moves in steps of 64.  Three stages of
+// (256 + 128) rows x 128 bytes live in LDS (144 KB, one block per CU); global memory is copied into
+// them by the direct global-to-LDS load, so the operands never pass through registers on their way
+// in.  What the measurements on MI355X asked for, in order of weight:
+//  * every instruction that is not an MFMA sits between two MFMAs.  One wave per SIMD issues in
+//    order, so a run of address arithmetic, loads or LDS reads is time in which the matrix core
+//    idles; spread out one at a time they cost nothing.  The LDS reads of the next half step (32 of
+//    K) and the global loads of the stage after next are therefore interleaved with the MFMAs of the
+//    current half step, and the operand fragments are double-buffered in registers.
+//  * LDS reads are inline assembly: the compiler would otherwise wait for every outstanding
+//    global-to-LDS load before each of them.  The waits are written by hand (vmcnt for the stage
+//    that must have landed, lgkmcnt for the fragments).
+//  * a 128-byte LDS row holds eight 16-byte chunks, chunk c of row r at position c ^ ((r >> 1) & 7):
+//    the 16 rows x 16 bytes that a quarter wave reads then fall into 16 different bank groups.
+//  * blocks go to the eight XCDs round robin; the blocks that one XCD runs at a time form a patch of
+//    (row blocks x column blocks) that share their operand tiles through that XCD's L2.
+//  * the result leaves through LDS, so that every store covers whole cache lines.
+// One barrier per 64 of K.  Sizes: K % 64 == 0; any M and N (loads clamp to the last row, stores are
+// masked).  The sum over K runs in ascending order for every output element.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+
+// the same codes as in gemm_mfma.hip
+enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_ACC_F32 = 2, OUT_SWIGLU = 3 };
+
+#define GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+namespace {
+
+constexpr int BM = 256, BN = 128, BK = 64, ROWB = 128;
+constexpr int STAGE_BYTES = (BM + BN) * ROWB;
+constexpr int NS = 3;
+constexpr int LPW = 12;        // direct loads per wave and stage: eight of x rows, four of w rows
+constexpr int CLD = 64 + 4;    // padded row of a wave's result tile in LDS, in floats
+
+__device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
+__device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+// vmcnt(n) alone: bits [3:0] and [15:14] hold n, the other counters stay at their maxima
+#define WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+// load I (0..11) of this wave into stage `buf`: 0..7 are x rows, 8..11 w rows; one load covers 8 rows
+template <int I>
+__device__ inline void issue_one(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                 const unsigned (&voff)[LPW], int wave) {
+  const int t = I < 8 ? wave * 8 + I : 32 + wave * 4 + (I - 8);
+  const unsigned char* src = (I < 8 ? xk : wk) + voff[I];
+  __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+}
+
+__device__ inline void issue_stage(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                   const unsigned (&voff)[LPW], int wave) {
+  issue_one<0>(buf, xk, wk, voff, wave);
+  issue_one<1>(buf, xk, wk, voff, wave);
+  issue_one<2>(buf, xk, wk, voff, wave);
+  issue_one<3>(buf, xk, wk, voff, wave);
+  issue_one<4>(buf, xk, wk, voff, wave);
+  issue_one<5>(buf, xk, wk, voff, wave);
+  issue_one<6>(buf, xk, wk, voff, wave);
+  issue_one<7>(buf, xk, wk, voff, wave);
+  issue_one<8>(buf, xk, wk, voff, wave);
+  issue_one<9>(buf, xk, wk, voff, wave);
+  issue_one<10>(buf, xk, wk, voff, wave);
+  issue_one<11>(buf, xk, wk, voff, wave);
+}
+
+template <int OFF>
+__device__ inline u32x4_t lds_read16(unsigned addr) {
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+
+// operand fragments of one half step (32 of K): eight 16-row tiles of x, four of w
+struct Frags {
+  u32x4_t a[8], b[4];
+};
+
+__device__ inline void wait_frags(Frags& f) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), "+v"(f.a[5]), "+v"(f.a[6]),
+                 "+v"(f.a[7]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3]));
+}
+
+// read R (0..11) of a half step: b0..b3, then a0..a7
+template <int R>
+__device__ inline void read_one(Frags& f, unsigned aaddr, unsigned baddr) {
+  if constexpr (R < 4)
+    f.b[R] = lds_read16<R * 16 * ROWB>(baddr);
+  else
+    f.a[R - 4] = lds_read16<(R - 4) * 16 * ROWB>(aaddr);
+}
+
+template <int I, int J>
+__device__ inline void mfma_one(f32x4_t (&acc)[8][4], const Frags& f) {
+  acc[I][J] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(f.a[I]), as_frag(f.b[J]), acc[I][J], 0, 0, 0);
+}
+
+// The 32 MFMAs of `cur`; between them, one at a time, the LDS reads into `nxt` (READ) and the global
+// loads of a stage (LOAD).
+template <bool READ, bool LOAD>
+__device__ inline void half_step(f32x4_t (&acc)[8][4], const Frags& cur, Frags& nxt, unsigned aaddr, unsigned baddr,
+                                 unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                 const unsigned (&voff)[LPW], int wave) {
+#define SB() __builtin_amdgcn_sched_barrier(0)
+#define RD(R) \
+  if (READ) read_one<R>(nxt, aaddr, baddr); \
+  SB()
+#define LD(I) \
+  if (LOAD) issue_one<I>(buf, xk, wk, voff, wave); \
+  SB()
+#define M1(I, J) \
+  mfma_one<I, J>(acc, cur); \
+  SB()
+  RD(0); M1(0, 0); LD(0); M1(0, 1); RD(1); M1(0, 2); LD(1); M1(0, 3);
+  RD(2); M1(1, 0); LD(2); M1(1, 1); RD(3); M1(1, 2); LD(3); M1(1, 3);
+  RD(4); M1(2, 0); LD(4); M1(2, 1); RD(5); M1(2, 2); LD(5); M1(2, 3);
+  RD(6); M1(3, 0); LD(6); M1(3, 1); RD(7); M1(3, 2); LD(7); M1(3, 3);
+  RD(8); M1(4, 0); LD(8); M1(4, 1); RD(9); M1(4, 2); LD(9); M1(4, 3);
+  RD(10); M1(5, 0); LD(10); M1(5, 1); RD(11); M1(5, 2); LD(11); M1(5, 3);
+  M1(6, 0); M1(6, 1); M1(6, 2); M1(6, 3); M1(7, 0); M1(7, 1); M1(7, 2); M1(7, 3);
+#undef RD
+#undef LD
+#undef M1
+#undef SB
+}
+
+#define READ_ALL(f, aaddr, baddr)                                                                                  \
+  read_one<0>(f, aaddr, baddr); read_one<1>(f, aaddr, baddr); read_one<2>(f, aaddr, baddr); read_one<3>(f, aaddr, baddr); \
+  read_one<4>(f, aaddr, baddr); read_one<5>(f, aaddr, baddr); read_one<6>(f, aaddr, baddr); read_one<7>(f, aaddr, baddr); \
+  read_one<8>(f, aaddr, baddr); read_one<9>(f, aaddr, baddr); read_one<10>(f, aaddr, baddr); read_one<11>(f, aaddr, baddr)
+
+// pm: row blocks of a patch (a power of two up to 8); a patch holds 32 blocks
+__global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                        void* __restrict__ out, int mode, int M, int N, int K, int pm) {
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE_BYTES];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  int bm, bn;
+  {
+    // XCD c takes the column blocks c, c + 8, ...; its blocks j = 0, 1, ... walk patches of pm row
+    // blocks x (32 / pm) of its column blocks, row blocks fastest
+    const int MB = (M + BM - 1) / BM, NB = (N + BN - 1) / BN;
+    const int pq = 32 / pm;
+    const int MS = (MB + pm - 1) / pm;
+    const int c = blockIdx.x % 8, j = blockIdx.x / 8;
+    const int t = j / 32, r = j % 32;
+    bm = (t % MS) * pm + r % pm;
+    bn = c + 8 * ((t / MS) * pq + r / pm);
+    if (bm >= MB || bn >= NB) return;
+  }
+  const int m0 = bm * BM, n0 = bn * BN;
+  f32x4_t acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const int KT = K / BK;
+  const int g = lane >> 4, c = lane & 15;
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
+  // this lane's byte offset inside a 16-row group of a stage, for the first and second 32 of K
+  const unsigned off0 = c * ROWB + (((0 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned off1 = c * ROWB + (((1 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned arow = wm * 128 * ROWB, brow = (BM + wn * 64) * ROWB;
+  // this lane's source of each of its loads, relative to the block's first row at the stage's k
+  unsigned voff[LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int row = (i < 8 ? (wave * 8 + i) * 8 : (wave * 4 + i - 8) * 8) + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    const int grow = i < 8 ? min(row, M - 1 - m0) : min(row, N - 1 - n0);
+    voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
+  }
+  const unsigned char* xk = (const unsigned char*)x + (size_t)m0 * K * 2;
+  const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2;
+#pragma unroll
+  for (int p = 0; p < NS; ++p)
+    if (p < KT) issue_stage(stages + p * STAGE_BYTES, xk + p * BK * 2, wk + p * BK * 2, voff, wave);
+  xk += NS * BK * 2;  // the next stage to load is that of tile NS
+  wk += NS * BK * 2;
+  Frags fa, fb;
+  if (KT > 2) WAIT_VM(2 * LPW); else WAIT_VM(0);
+  __builtin_amdgcn_s_barrier();
+  READ_ALL(fa, lds0 + arow + off0, lds0 + brow + off0);
+  wait_frags(fa);
+  // Tile kt: the first half step multiplies fa and reads the second half's fragments; then tile kt + 1
+  // must have landed for every wave (barrier), which also means that every wave is done reading tile
+  // kt's stage: the second half step refills it with tile kt + NS while it multiplies fb and reads the
+  // first fragments of tile kt + 1.
+  int st = 0, kt = 0;
+  for (; kt + NS < KT; ++kt) {
+    const int sn = st + 1 == NS ? 0 : st + 1;
+    const unsigned cur = lds0 + st * STAGE_BYTES, nxt = lds0 + sn * STAGE_BYTES;
+    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fb);
+    WAIT_VM(LPW);  // tile kt + 2 may stay in flight
+    __builtin_amdgcn_s_barrier();
+    half_step<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, stages + st * STAGE_BYTES, xk, wk, voff, wave);
+    wait_frags(fa);
+    xk += BK * 2;
+    wk += BK * 2;
+    st = sn;
+  }
+  for (; kt + 1 < KT; ++kt) {  // nothing left to load
+    const int sn = st + 1 == NS ? 0 : st + 1;
+    const unsigned cur = lds0 + st * STAGE_BYTES, nxt = lds0 + sn * STAGE_BYTES;
+    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fb);
+    WAIT_VM(0);
+    __builtin_amdgcn_s_barrier();
+    half_step<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fa);
+    st = sn;
+  }
+  {
+    const unsigned cur = lds0 + st * STAGE_BYTES;
+    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fb);
+    half_step<false, false>(acc, fb, fa, 0, 0, nullptr, nullptr, nullptr, voff, wave);
+  }
+
+  // ---- the result leaves through LDS: each wave lays its 128 x 64 tile out row by row -----------------
+  __syncthreads();  // every wave is done with the stages
+  float* ct = (float*)stages + wave * (128 * CLD);
+  // result lane l of tile (i, j): rows i * 16 + (l / 16) * 4 + r, column j * 16 + l % 16
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int mw = m0 + wm * 128, nw = n0 + wn * 64;
+  if (mode == OUT_SWIGLU) {
+    // the weight rows alternate eight gate rows and eight up rows: output column 8 b + i pairs
+    // columns 16 b + i and 16 b + 8 + i; 32 outputs per row, four per lane, eight rows per pass
+    const int o = (lane & 7) * 4, rr = lane >> 3;
+    const int cg = (o / 8) * 16 + o % 8;
+    bf16_t* ob = (bf16_t*)out;
+    const int half = N / 2;
+#pragma unroll 4
+    for (int p = 0; p < 16; ++p) {
+      const int row = p * 8 + rr, m = mw + row;
+      const f32x4_t gt = *(const f32x4_t*)(ct + row * CLD + cg);
+      const f32x4_t up = *(const f32x4_t*)(ct + row * CLD + cg + 8);
+      if (m >= M || nw + cg >= N) continue;   // N is a multiple of 16: the whole group is inside or outside
+      union {
+        bf16_t h[4];
+        u32x2_t v;
+      } pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(silu_mul(gt[e], up[e]));
+      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk.v;
+    }
+    return;
+  }
+  const int col = (lane & 15) * 4, rr = lane >> 4;
+  const bool vec = (N % 4 == 0) && nw + col + 3 < N;
+#pragma unroll 4
+  for (int p = 0; p < 32; ++p) {
+    const int row = p * 4 + rr, m = mw + row;
+    const f32x4_t v = *(const f32x4_t*)(ct + row * CLD + col);
+    if (m >= M) continue;
+    const size_t idx = (size_t)m * N + nw + col;
+    if (vec) {
+      if (mode == OUT_BF16) {
+        union {
+          bf16_t h[4];
+          u32x2_t v;
+        } pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(v[e]);
+        *(u32x2_t*)((bf16_t*)out + idx) = pk.v;
+      } else if (mode == OUT_F32) {
+        *(f32x4_t*)((float*)out + idx) = v;
+      } else {
+        f32x4_t* o = (f32x4_t*)((float*)out + idx);
+        *o = *o + v;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (nw + col + e >= N) break;
+        if (mode == OUT_BF16)
+          ((bf16_t*)out)[idx + e] = float_to_bf16(v[e]);
+        else if (mode == OUT_F32)
+          ((float*)out)[idx + e] = v[e];
+        else
+          ((float*)out)[idx + e] += v[e];
+      }
+    }
+  }
+}
+
+}  // namespace
+
+// Returns 0 when launched, -1 when the sizes are not this kernel's.
+int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s) {
+  if (K % BK != 0 || K < BK) return -1;
+  if ((size_t)(BM - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;  // a lane's source offset is 32 bits
+  if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
+  const int MB = (M + BM - 1) / BM, NB = (N + BN - 1) / BN;
+  const int pm = MB >= 5 ? 8 : (MB >= 3 ? 4 : MB);
+  const int pq = 32 / pm;
+  const long Q = (NB + 7) / 8, MS = (MB + pm - 1) / pm, QS = (Q + pq - 1) / pq;
+  const long blocks = 8 * QS * MS * 32;
+  if (blocks > 0x7fffffffL) return -1;
+  hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, w, out, mode, M, N, K, pm);
+  return 0;
+}
