@@ -142,25 +142,45 @@ static void launch_generic(const void* x, const void* w, void* out, int M, int N
 // Defined in gemm_mfma.hip; returns 0 when it took the product, -1 when the sizes are
 // not its own (the general kernel then runs), >0 on error.
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
-                   float* scratch, size_t scratch_floats, hipStream_t s);
+                   float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
+                   const void* post_w, void* post_xg, float* post_ss, hipStream_t s);
 
 // `scratch` (optional, `scratch_floats` float32): room for split-K partial sums of mid-sized products.
-extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
-                         int N, int K, int allow_mfma, float* scratch, size_t scratch_floats, hipStream_t s) {
+//
+// The split norm (bfloat16, at most 16 rows, K % 32 == 0): with `post_w` (a float32 norm weight [N]; accumulate
+// must be 1) the product also writes post_xg [M, N] = bfloat16(out * post_w) and post_ss
+// [ceil(N / 16), 16], per block of 16 columns and row the sum of squares of `out`.  With `pre_ss`
+// ([pre_count, 16], as written by such a product whose N is this product's K) the result rows are
+// multiplied by rsqrt(sum of squares / K + pre_eps): x is then that product's post_xg.
+extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
+                               int N, int K, int allow_mfma, float* scratch, size_t scratch_floats,
+                               const float* pre_ss, int pre_count, float pre_eps, const void* post_w, void* post_xg,
+                               float* post_ss, hipStream_t s) {
   TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(accumulate != 1 || out_dt == TP_F32, "linear: accumulating output must be float32");
+  const bool split_norm = pre_ss != nullptr || post_w != nullptr;
+  if (split_norm) {
+    TP_REQUIRE(in_dt == TP_BF16 && allow_mfma && M <= 16 && K % 32 == 0,
+               "linear: the split norm needs bfloat16 operands, at most 16 rows and K %% 32 == 0 (M=%d K=%d)", M, K);
+    TP_REQUIRE(post_w == nullptr || (accumulate == 1 && post_xg != nullptr && post_ss != nullptr),
+               "linear: the norm preparation belongs to a product that adds into the residual stream");
+    TP_REQUIRE(pre_ss == nullptr || pre_count == (K + 15) / 16, "linear: %d partial sums for K=%d", pre_count, K);
+  }
   if (accumulate == 2) {  // gated-SiLU epilogue: only the matrix-core kernels have it
     TP_REQUIRE(in_dt == TP_BF16 && allow_mfma, "linear: the gated epilogue needs bfloat16 operands");
-    const int r = tp_linear_mfma(x, w, out, out_dt, 2, M, N, K, scratch, scratch_floats, s);
+    const int r = tp_linear_mfma(x, w, out, out_dt, 2, M, N, K, scratch, scratch_floats, pre_ss, pre_count, pre_eps,
+                                 nullptr, nullptr, nullptr, s);
     TP_REQUIRE(r >= 0, "linear: sizes M=%d N=%d K=%d do not fit the gated epilogue", M, N, K);
     return r;
   }
   TP_REQUIRE((size_t)M * N < ((size_t)1 << 40), "linear: output too large");
   if (M == 0) return 0;
   if (in_dt == TP_BF16 && allow_mfma) {
-    const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, scratch, scratch_floats, s);
+    const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, scratch, scratch_floats, pre_ss, pre_count,
+                                 pre_eps, post_w, post_xg, post_ss, s);
     if (r >= 0) return r;
   }
+  TP_REQUIRE(!split_norm, "linear: sizes M=%d N=%d K=%d do not fit the split norm", M, N, K);
   if (in_dt == TP_F32 && out_dt == TP_F32) {
     if (accumulate)
       launch_generic<float, float, true>(x, w, out, M, N, K, s);
@@ -178,4 +198,10 @@ extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int
   }
   TP_CHECK_LAUNCH("linear");
   return 0;
+}
+
+extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
+                         int N, int K, int allow_mfma, float* scratch, size_t scratch_floats, hipStream_t s) {
+  return tp_linear_fused(x, w, in_dt, out, out_dt, accumulate, M, N, K, allow_mfma, scratch, scratch_floats, nullptr, 0,
+                         0.f, nullptr, nullptr, nullptr, s);
 }

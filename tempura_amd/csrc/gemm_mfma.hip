@@ -38,6 +38,68 @@ __device__ inline void store_out(void* out, int mode, size_t idx, float v) {
     ((float*)out)[idx] += v;
 }
 
+// A root-mean-square norm split over two products (rows of at most 16 tokens).  The product that
+// adds into the residual stream h also writes xg = bfloat16(h * norm weight) and, per block and row,
+// the sum of squares of the columns it owns (NormPrep).  The product that consumes xg adds those
+// partial sums in a fixed order and multiplies its float32 result rows by rsqrt(mean square + eps)
+// (RowScale): the norm kernel between the two products is gone, and the scale is applied in float32
+// after the sum instead of before the rounding to bfloat16.
+struct NormPrep {
+  const float* w;    // norm weight [N]; nullptr: no preparation
+  bf16_t* xg;        // [M, N]
+  float* ss;         // [blocks, 16]
+};
+struct RowScale {
+  const float* ss;   // [count, 16] partial sums of squares; nullptr: no scaling
+  int count;
+  float inv_k, eps;
+};
+
+// RowScale, first half: every thread fetches its share of the partial sums of one row.  The loads are
+// issued together, early (before the main loop), and nothing waits for them until the second half.
+struct RowScaleLoads {
+  float v[8];
+};
+__device__ inline RowScaleLoads row_scale_begin(const RowScale& pre, int nthreads) {
+  RowScaleLoads ld;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ld.v[i] = 0.f;
+  if (pre.ss == nullptr) return ld;
+  const int t = threadIdx.x, nparts = min(nthreads / 16, 32);
+  if (t < nparts * 16) {
+    const int m = t & 15, p = t >> 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int b = p + i * nparts;
+      if (b < pre.count) ld.v[i] = pre.ss[b * 16 + m];
+    }
+  }
+  return ld;
+}
+// Second half: call after a barrier and follow with one; afterwards rstd[m] is valid for every thread.
+__device__ inline void row_scale_finish(const RowScale& pre, const RowScaleLoads& ld, float (*part)[16], float* rstd,
+                                        int nthreads) {
+  const int t = threadIdx.x, nparts = min(nthreads / 16, 32);
+  if (pre.ss == nullptr) {
+    if (t < 16) rstd[t] = 1.0f;
+    return;
+  }
+  if (t < nparts * 16) {
+    const int m = t & 15, p = t >> 4;
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += ld.v[i];
+    for (int b = p + 8 * nparts; b < pre.count; b += nparts) sum += pre.ss[b * 16 + m];   // more than 8 each: rare
+    part[p][m] = sum;
+  }
+  __syncthreads();
+  if (t < 16) {
+    float sum = 0.f;
+    for (int p = 0; p < nparts; ++p) sum += part[p][t];
+    rstd[t] = rsqrtf(sum * pre.inv_k + pre.eps);
+  }
+}
+
 // ---- skinny ---------------------------------------------------------------------------
 // MT: 16-row tiles of activations; NT: 16-row tiles of weights per block; WAVES: waves that
 // split K.  A wave takes K in runs of four consecutive 32-wide steps (256 contiguous bytes of
@@ -46,8 +108,9 @@ template <int MT, int NT, int WAVES, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16_t* __restrict__ x,
                                                                       const bf16_t* __restrict__ w,
                                                                       void* __restrict__ out, int mode, int M,
-                                                                      int N, int K) {
+                                                                      int N, int K, RowScale pre, NormPrep post) {
   __shared__ float red[WAVES][NT * MT][256];
+  __shared__ float rs_part[32][16], rstd[16], ss_lds[NT][4][16];
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   const int n0 = blockIdx.x * 16 * NT;
   const int kofs = (lane >> 4) * 8;
@@ -69,6 +132,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[j][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
+  const RowScaleLoads rs_loads = row_scale_begin(pre, WAVES * 64);
   const int steps = K / 32;  // a step is 32 k = 4 u32x4 per row
   // DEPTH runs of four steps are fetched before any of them is multiplied: 4 * DEPTH * NT loads
   // of 16 bytes per lane are in flight, which is what keeps the memory system busy.
@@ -107,6 +171,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[wave][j * MT + t][lane * 4 + r] = acc[j][t][r];
   __syncthreads();
+  row_scale_finish(pre, rs_loads, rs_part, rstd, WAVES * 64);
+  __syncthreads();
   for (int e = threadIdx.x; e < NT * MT * 256; e += WAVES * 64) {
     const int jt = e / 256, q = e % 256;
     const int j = jt / MT, t = jt % MT;
@@ -116,15 +182,41 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
     const int l = q / 4, r = q % 4;
     const int n = n0 + j * 16 + (l >> 4) * 4 + r;   // weight row = output column
     const int m = t * 16 + (l & 15);
+    if (MT == 1) v *= rstd[l & 15];
     if (mode == OUT_SWIGLU) {
       if ((l >> 4) < 2 && n + 8 < N && m < M) {       // a gate row: its up row is eight further on
         float u = 0.f;
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) u += red[i][jt][q + 128];
+        if (MT == 1) u *= rstd[l & 15];
         ((bf16_t*)out)[(size_t)m * (N / 2) + (n0 + j * 16) / 2 + (l >> 4) * 4 + r] = float_to_bf16(silu_mul(v, u));
       }
+    } else if (MT == 1 && post.w != nullptr) {
+      // residual add, and the next norm's preparation (mode is OUT_ACC_F32)
+      float sq = 0.f;
+      if (n < N && m < M) {
+        float* o = (float*)out + (size_t)m * N + n;
+        const float h = *o + v;
+        *o = h;
+        post.xg[(size_t)m * N + n] = float_to_bf16(h * post.w[n]);
+        sq = h * h;
+      }
+      sq += __shfl_xor(sq, 1, 64);      // the four columns r = 0..3 of this row
+      sq += __shfl_xor(sq, 2, 64);
+      if (r == 0) ss_lds[j][l >> 4][l & 15] = sq;
     } else if (n < N && m < M) {
       store_out(out, mode, (size_t)m * N + n, v);
+    }
+  }
+  if (MT == 1 && post.w != nullptr) {
+    __syncthreads();
+    if (threadIdx.x < 16) {
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) sum += ss_lds[j][c][threadIdx.x];
+      post.ss[blockIdx.x * 16 + threadIdx.x] = sum;
     }
   }
 }
@@ -141,10 +233,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 
 template <int NT>
 __global__ __launch_bounds__(512) void gemm_skinny_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                              void* __restrict__ out, int mode, int M, int N, int K) {
+                                                              void* __restrict__ out, int mode, int M, int N, int K,
+                                                              RowScale pre, NormPrep post) {
   constexpr int WAVES = 8;
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][16 * LLD];
   __shared__ float red[WAVES][NT][256];
+  __shared__ float rs_part[32][16], rstd[16], ss_lds[NT][4][16];
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int n0 = blockIdx.x * 16 * NT;
   const int kofs = (lane >> 4) * 8;
@@ -183,6 +277,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_lds_kernel(const bf16_t* __re
     }
   };
   load_chunk(0);
+  const RowScaleLoads rs_loads = row_scale_begin(pre, 512);
   for (int ch = 0; ch < chunks; ++ch) {
     const int buf = ch & 1;
     if (xload) {
@@ -212,6 +307,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_lds_kernel(const bf16_t* __re
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][j][lane * 4 + r] = acc[j][r];
   __syncthreads();
+  row_scale_finish(pre, rs_loads, rs_part, rstd, 512);
+  __syncthreads();
   for (int e = tid; e < NT * 256; e += 512) {
     const int j = e / 256, q = e % 256;
     float v = 0.f;
@@ -220,15 +317,40 @@ __global__ __launch_bounds__(512) void gemm_skinny_lds_kernel(const bf16_t* __re
     const int l = q / 4, r = q % 4;
     const int n = n0 + j * 16 + (l >> 4) * 4 + r;
     const int m = l & 15;
+    v *= rstd[m];
     if (mode == OUT_SWIGLU) {
       if ((l >> 4) < 2 && n + 8 < N && m < M) {
         float u = 0.f;
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) u += red[i][j][q + 128];
+        u *= rstd[m];
         ((bf16_t*)out)[(size_t)m * (N / 2) + (n0 + j * 16) / 2 + (l >> 4) * 4 + r] = float_to_bf16(silu_mul(v, u));
       }
+    } else if (post.w != nullptr) {
+      float sq = 0.f;
+      if (n < N && m < M) {
+        float* o = (float*)out + (size_t)m * N + n;
+        const float h = *o + v;
+        *o = h;
+        post.xg[(size_t)m * N + n] = float_to_bf16(h * post.w[n]);
+        sq = h * h;
+      }
+      sq += __shfl_xor(sq, 1, 64);
+      sq += __shfl_xor(sq, 2, 64);
+      if (r == 0) ss_lds[j][l >> 4][m] = sq;
     } else if (n < N && m < M) {
       store_out(out, mode, (size_t)m * N + n, v);
+    }
+  }
+  if (post.w != nullptr) {
+    __syncthreads();
+    if (tid < 16) {
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) sum += ss_lds[j][c][tid];
+      post.ss[blockIdx.x * 16 + tid] = sum;
     }
   }
 }
@@ -405,14 +527,16 @@ extern "C" void tp_linear_tune(int waves, int nt, int depth) {
 }
 
 template <int MT, int NT, int WAVES, int DEPTH>
-static void launch_skinny4(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s) {
+static void launch_skinny4(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, RowScale pre,
+                           NormPrep post, hipStream_t s) {
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, NT, WAVES, DEPTH>), dim3(blocks), dim3(WAVES * 64), 0, s, x, w, out,
-                     mode, M, N, K);
+                     mode, M, N, K, pre, post);
 }
 
 template <int MT>
-static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s) {
+static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, RowScale pre,
+                          NormPrep post, hipStream_t s) {
   // every wave should get at least one run of four steps; small N wants many waves per block
   // (one block per 16 columns is all the parallelism there is), large N fewer and two row tiles
   // Measured on MI355X at Llama-8B shapes: eight waves with two runs in flight each stream
@@ -424,6 +548,7 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
   if (g_tune_waves) waves = g_tune_waves;
   if (g_tune_nt) nt = g_tune_nt;
   if (g_tune_depth) depth = g_tune_depth;
+  if (post.w != nullptr) nt = 1;   // the consumer counts one partial sum per 16 columns
   if constexpr (MT == 1) {
     // several activation rows: feed them through LDS, unless K is so long that the barrier per
     // chunk costs more than the gather (measured: K = 14336 is faster without)
@@ -433,9 +558,9 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
       if (nt > 2) nt = 2;
       const int blocks = (N + 16 * nt - 1) / (16 * nt);
       if (nt == 2)
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K);
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, pre, post);
       else
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K);
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, pre, post);
       return;
     }
   }
@@ -443,7 +568,7 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
   if (MT > 1) nt = 1;
   if (MT > 2 || nt > 2) depth = 1;           // registers
 #define CASE(NT_, W_, D_) \
-  if (nt == NT_ && waves == W_ && depth == D_) return launch_skinny4<MT, NT_, W_, D_>(x, w, out, mode, M, N, K, s)
+  if (nt == NT_ && waves == W_ && depth == D_) return launch_skinny4<MT, NT_, W_, D_>(x, w, out, mode, M, N, K, pre, post, s)
   CASE(1, 16, 1);
   CASE(1, 8, 1);
   CASE(1, 4, 1);
@@ -464,13 +589,19 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
     CASE(4, 4, 1);
   }
 #undef CASE
-  launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, s);
+  launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, pre, post, s);
 }
 
-// accumulate: 0 store, 1 add into the float32 output, 2 gated-SiLU epilogue (see OUT_SWIGLU)
+// accumulate: 0 store, 1 add into the float32 output, 2 gated-SiLU epilogue (see OUT_SWIGLU).
+// pre_ss / post_w: the split norm (RowScale / NormPrep above), at most 16 rows; nullptr without.
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
-                   float* scratch, size_t scratch_floats, hipStream_t s) {
+                   float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
+                   const void* post_w, void* post_xg, float* post_ss, hipStream_t s) {
   if (K % 32 != 0) return -1;
+  if ((pre_ss != nullptr || post_w != nullptr) && M > 16) return -1;
+  if (post_w != nullptr && accumulate != 1) return -1;
+  const RowScale pre = {pre_ss, pre_count, 1.0f / (float)K, pre_eps};
+  const NormPrep post = {(const float*)post_w, (bf16_t*)post_xg, post_ss};
   if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return -1;
   if (accumulate == 2 && (N % 16 != 0 || out_dt != TP_BF16)) return -1;
   const int mode = accumulate == 2 ? OUT_SWIGLU : (accumulate ? OUT_ACC_F32 : (out_dt == TP_F32 ? OUT_F32 : OUT_BF16));
@@ -479,13 +610,13 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   const bool mid_ok = scratch != nullptr && g_tune_mid != 1;
   if (M <= 16 || (M <= 64 && !mid_ok)) {
     if (M <= 16)
-      launch_skinny<1>(xb, wb, out, mode, M, N, K, s);
+      launch_skinny<1>(xb, wb, out, mode, M, N, K, pre, post, s);
     else if (M <= 32)
-      launch_skinny<2>(xb, wb, out, mode, M, N, K, s);
+      launch_skinny<2>(xb, wb, out, mode, M, N, K, pre, post, s);
     else if (M <= 48)
-      launch_skinny<3>(xb, wb, out, mode, M, N, K, s);
+      launch_skinny<3>(xb, wb, out, mode, M, N, K, pre, post, s);
     else
-      launch_skinny<4>(xb, wb, out, mode, M, N, K, s);
+      launch_skinny<4>(xb, wb, out, mode, M, N, K, pre, post, s);
   } else {
     // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
     // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.

@@ -106,7 +106,16 @@ class CausalLM:
         """``tokens`` int32 [n]; ``caches[i]`` is the ``LayerCache`` of run-order entry i.
         Returns float32 logits [len(ctx.logit_rows), vocab]."""
         h = self.embedding.forward(tokens)
+        m = h.shape[0]
+        x = None      # rows handed from one block to the next (a norm carried by the products around it)
         for i, call in enumerate(self.order):
-            self.layers[call.layer].forward(h, ctx, caches[i])
+            layer = self.layers[call.layer]
+            if not hasattr(layer, "entry_norm"):
+                layer.forward(h, ctx, caches[i])
+                x = None
+                continue
+            after = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else None
+            next_norm = after.entry_norm(m) if hasattr(after, "entry_norm") else None
+            x = layer.forward(h, ctx, caches[i], x, next_norm)
         x = self.final_norm.forward(h, ctx.logit_rows)
         return self.lm_head.forward(x)

@@ -151,11 +151,43 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.stack([gate.reshape(i // 8, 8, k), up.reshape(i // 8, 8, k)], dim=1).reshape(2 * i, k).contiguous()
 
 
-def linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """bfloat16 x [m, k], interleaved gate/up weight [2i, k] -> bfloat16 [m, i] = silu(x g^T) * (x u^T),
-    the gate applied to the float32 accumulators (no rounding in between)."""
+class Prenormed:
+    """Rows whose root-mean-square norm is finished by the product that consumes them: ``x`` is
+    bfloat16(h * norm weight) [m, k]; ``ss`` [ceil(k / 16), 16] float32 holds, per block of 16 columns
+    and row, the sum of squares of h; the consumer multiplies its float32 result rows by
+    rsqrt(sum(ss) / k + eps).  Made by ``linear(..., residual=h, next_norm=(weight, eps))``."""
+    __slots__ = ("x", "ss", "eps")
+
+    def __init__(self, x, ss, eps):
+        self.x, self.ss, self.eps = x, ss, float(eps)
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+
+def split_norm_ok(m: int, width: int, dtype: torch.dtype) -> bool:
+    """Whether a norm over ``width`` columns of ``m`` rows can be split over the two products around it."""
+    if _backend is not None:
+        return _backend.split_norm_ok(m, width, dtype)
+    return allow_mfma and dtype == torch.bfloat16 and 0 < m <= 16 and width % 32 == 0
+
+
+def _pre_args(x):
+    if isinstance(x, Prenormed):
+        _dev_ok(x.x, x.ss)
+        _need(x.x.dtype == torch.bfloat16 and x.ss.dtype == torch.float32 and
+              tuple(x.ss.shape) == ((x.x.shape[1] + 15) // 16, 16), "linear: malformed handed-over rows")
+        return x.x, (_ptr(x.ss), x.ss.shape[0], ctypes.c_float(x.eps))
+    return x, (_ptr(None), 0, ctypes.c_float(0.0))
+
+
+def linear_swiglu(x, w: torch.Tensor) -> torch.Tensor:
+    """bfloat16 x [m, k] (or ``Prenormed``), interleaved gate/up weight [2i, k] -> bfloat16 [m, i] =
+    silu(x g^T) * (x u^T), the gate applied to the float32 accumulators (no rounding in between)."""
     if _backend is not None:
         return _backend.linear_swiglu(x, w)
+    x, pre = _pre_args(x)
     _dev_ok(x, w)
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_swiglu: shapes {tuple(x.shape)} x {tuple(w.shape)}")
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "linear_swiglu: operands must be bfloat16")
@@ -164,8 +196,8 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     _need(n % 16 == 0 and k % 32 == 0, "linear_swiglu: needs 2i % 16 == 0 and k % 32 == 0")
     out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     scratch, nscratch = _splitk_scratch(x, m, n)
-    _call("tp_linear", _ptr(x), _ptr(w), _BF16, _ptr(out), _BF16, 2, m, n, k, 1, _ptr(scratch),
-          ctypes.c_size_t(nscratch), _stream())
+    _call("tp_linear_fused", _ptr(x), _ptr(w), _BF16, _ptr(out), _BF16, 2, m, n, k, 1, _ptr(scratch),
+          ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), _stream())
     return out
 
 
@@ -177,12 +209,16 @@ def _splitk_scratch(x: torch.Tensor, m: int, n: int):
     return torch.empty((count,), dtype=torch.float32, device=x.device), count
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
-           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x [m, k] @ w[n, k]^T -> out_dtype [m, n]; with ``residual`` (float32 [m, n]) the product is
-    added into it in place and it is returned."""
+def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.Tensor] = None, next_norm=None):
+    """x [m, k] (or ``Prenormed``) @ w[n, k]^T -> out_dtype [m, n]; with ``residual`` (float32 [m, n]) the
+    product is added into it in place and it is returned.  With ``next_norm`` = (float32 weight [n], eps)
+    (needs ``residual``) the result is the pair (residual, ``Prenormed`` rows of the updated residual), or
+    (residual, None) when the sizes do not allow it and the norm has to run on its own."""
     if _backend is not None:
+        if next_norm is not None:
+            return _backend.linear(x, w, out_dtype, residual, next_norm)
         return _backend.linear(x, w, out_dtype, residual)
+    x, pre = _pre_args(x)
     _dev_ok(x, w, residual)
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
     _need(x.dtype == w.dtype, f"linear: operand dtypes differ ({x.dtype}, {w.dtype})")
@@ -193,10 +229,19 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype,
         out, acc = residual, 1
     else:
         out, acc = torch.empty((m, n), dtype=out_dtype, device=x.device), 0
+    post, handed = (_ptr(None), _ptr(None), _ptr(None)), None
+    if next_norm is not None and split_norm_ok(m, n, x.dtype) and k % 32 == 0:
+        weight, eps = next_norm
+        _dev_ok(weight)
+        _need(residual is not None, "linear: next_norm needs a residual")
+        _need(weight.dtype == torch.float32 and weight.numel() == n, "linear: norm weight must be float32 [n]")
+        handed = Prenormed(torch.empty((m, n), dtype=torch.bfloat16, device=x.device),
+                           torch.empty(((n + 15) // 16, 16), dtype=torch.float32, device=x.device), eps)
+        post = (_ptr(weight), _ptr(handed.x), _ptr(handed.ss))
     scratch, nscratch = _splitk_scratch(x, m, n) if allow_mfma else (None, 0)
-    _call("tp_linear", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
-          ctypes.c_size_t(nscratch), _stream())
-    return out
+    _call("tp_linear_fused", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
+          ctypes.c_size_t(nscratch), *pre, *post, _stream())
+    return out if next_norm is None else (out, handed)
 
 
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],

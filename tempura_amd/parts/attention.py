@@ -19,6 +19,7 @@ from .base import CacheSpec, Mixer, WeightInfo, build_part, register_part
 
 class PagedAttention(Mixer):
     graph_safe = True      # only kernels on device-resident step data: may be captured in a graph
+    split_norm = True      # takes rows whose norm its first product finishes; prepares the next norm in its last
 
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
@@ -59,7 +60,7 @@ class PagedAttention(Mixer):
         kind = "window" if self.window is not None else "full"
         return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x, ctx, cache, residual):
+    def forward(self, x, ctx, cache, residual, next_norm=None):
         rot = self.position.rotary()
         if cache.writes:
             qkv = ops.linear(x, self.wqkv, torch.float32)
@@ -85,7 +86,10 @@ class PagedAttention(Mixer):
             q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
             ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
             ctx.num_single)
-        ops.linear(a, self.wo, torch.float32, residual=residual)
+        if next_norm is None:
+            ops.linear(a, self.wo, torch.float32, residual=residual)
+            return None
+        return ops.linear(a, self.wo, torch.float32, residual=residual, next_norm=next_norm)[1]
 
 
 register_part("mixer", "attention", PagedAttention)

@@ -4,6 +4,11 @@
 residual adds (/root/reference/engine/src/model.rs:952-1314; declared as
 [PreNormAttention, PreNormFfn], /root/reference/engine/src/architecture.rs:56-65).
 The residual stream ``h`` is float32 in every dtype.
+
+A norm may be carried by the two products around it instead of running as a kernel of its own
+(``Norm.deferred``, ``ops.Prenormed``): the part before it prepares the rows in the epilogue of its last
+product, the part after it finishes them in its first.  The block arranges that for parts that declare
+``split_norm``; any other part gets plain normed rows and returns nothing.
 """
 from __future__ import annotations
 
@@ -35,11 +40,31 @@ class PreNormBlock:
         for p in self.parts():
             p.load_weights(get)
 
-    def forward(self, h, ctx, cache):
-        x = self.mixer_norm.forward(h)
-        self.mixer.forward(x, ctx, cache, h)
-        x = self.ffn_norm.forward(h)
-        self.ffn.forward(x, ctx, h)
+    def entry_norm(self, m):
+        """What the part before this block needs to prepare this block's first norm for ``m`` rows, or None."""
+        if getattr(self.mixer, "split_norm", False) and hasattr(self.mixer_norm, "deferred"):
+            return self.mixer_norm.deferred(m)
+        return None
+
+    def forward(self, h, ctx, cache, x=None, next_norm=None):
+        """``x``: rows handed over by the block before (its last product prepared ``mixer_norm``);
+        ``next_norm``: the ``entry_norm`` of the block after.  Returns the rows handed to that block, or None."""
+        if x is None:
+            x = self.mixer_norm.forward(h)
+        x2 = None
+        if getattr(self.mixer, "split_norm", False):
+            mid = None
+            if getattr(self.ffn, "split_norm", False) and hasattr(self.ffn_norm, "deferred"):
+                mid = self.ffn_norm.deferred(h.shape[0])
+            x2 = self.mixer.forward(x, ctx, cache, h, next_norm=mid)
+        else:
+            self.mixer.forward(x, ctx, cache, h)
+        if x2 is None:
+            x2 = self.ffn_norm.forward(h)
+        if next_norm is not None and getattr(self.ffn, "split_norm", False):
+            return self.ffn.forward(x2, ctx, h, next_norm=next_norm)
+        self.ffn.forward(x2, ctx, h)
+        return None
 
 
 register_part("block", "prenorm", PreNormBlock)

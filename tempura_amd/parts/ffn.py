@@ -12,6 +12,7 @@ from .base import FeedForward, WeightInfo, register_part
 
 class SwiGLU(FeedForward):
     graph_safe = True      # only kernels on device-resident step data: may be captured in a graph
+    split_norm = True      # takes rows whose norm its first product finishes; prepares the next norm in its last
 
     def __init__(self, spec, hidden_size, dtype, device):
         super().__init__(spec, hidden_size, dtype, device)
@@ -40,13 +41,16 @@ class SwiGLU(FeedForward):
             self.w13 = torch.cat([gate, up], dim=0).contiguous()
         self.w2 = self._to_device(get(w["down"]))
 
-    def forward(self, x, ctx, residual):
+    def forward(self, x, ctx, residual, next_norm=None):
         if self.fused:
             a = ops.linear_swiglu(x, self.w13)
         else:
             gu = ops.linear(x, self.w13, torch.float32)
             a = ops.swiglu(gu, self.dtype)
-        ops.linear(a, self.w2, torch.float32, residual=residual)
+        if next_norm is None:
+            ops.linear(a, self.w2, torch.float32, residual=residual)
+            return None
+        return ops.linear(a, self.w2, torch.float32, residual=residual, next_norm=next_norm)[1]
 
 
 register_part("ffn", "swiglu", SwiGLU)

@@ -31,5 +31,12 @@ class RMSNorm(Norm):
     def forward(self, h, rows=None):
         return ops.rmsnorm(h, self.weight, self.eps, self.dtype, rows)
 
+    def deferred(self, m):
+        """(weight, eps) when the two products around this norm can carry it for ``m`` rows (the one
+        before prepares, the one after applies the scale), else None."""
+        if ops.split_norm_ok(m, self.hidden_size, self.dtype):
+            return self.weight, self.eps
+        return None
+
 
 register_part("norm", "rmsnorm", RMSNorm)

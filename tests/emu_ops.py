@@ -21,15 +21,41 @@ class EmuOps:
         y = x * (1.0 / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)) * weight.double()
         return y.to(out_dtype)
 
-    def linear(self, x, w, out_dtype, residual=None):
-        y = x.double() @ w.double().T
+    def split_norm_ok(self, m, width, dtype):
+        return dtype == torch.bfloat16 and 0 < m <= 16 and width % 32 == 0
+
+    @staticmethod
+    def _rows(x):
+        """Plain rows, or handed-over rows (x = bfloat16(h * weight), ss = sums of squares per 16 columns)
+        with the factor that finishes their norm."""
+        from tempura_amd.kernels.ops import Prenormed
+        if isinstance(x, Prenormed):
+            rstd = torch.rsqrt(x.ss.double().sum(0)[: x.x.shape[0]] / x.x.shape[1] + x.eps)
+            return x.x.double(), rstd[:, None]
+        return x.double(), 1.0
+
+    def linear(self, x, w, out_dtype, residual=None, next_norm=None):
+        from tempura_amd.kernels.ops import Prenormed
+        xd, scale = self._rows(x)
+        y = (xd @ w.double().T) * scale
         if residual is not None:
             residual.copy_((residual.double() + y).to(torch.float32))
-            return residual
+            if next_norm is None:
+                return residual
+            m, n = residual.shape
+            if not (self.split_norm_ok(m, n, x.dtype if torch.is_tensor(x) else torch.bfloat16) and xd.shape[1] % 32 == 0):
+                return residual, None
+            weight, eps = next_norm
+            ss = torch.zeros(((n + 15) // 16, 16), dtype=torch.float32)
+            sq = torch.nn.functional.pad(residual.double() ** 2, (0, ss.shape[0] * 16 - n))
+            ss[:, :m] = sq.reshape(m, -1, 16).sum(2).T.to(torch.float32)
+            return residual, Prenormed((residual * weight).to(torch.bfloat16), ss, eps)
         return y.to(out_dtype)
 
     def linear_swiglu(self, x, w):
-        y = (x.double() @ w.double().T).reshape(x.shape[0], -1, 2, 8)      # eight gate rows, eight up rows in turn
+        xd, scale = self._rows(x)
+        x = xd
+        y = ((x @ w.double().T) * scale).reshape(x.shape[0], -1, 2, 8)      # eight gate rows, eight up rows in turn
         g, u = y[:, :, 0].reshape(x.shape[0], -1), y[:, :, 1].reshape(x.shape[0], -1)
         return (g / (1.0 + torch.exp(-g)) * u).to(torch.bfloat16)
 

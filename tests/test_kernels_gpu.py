@@ -218,6 +218,49 @@ def test_linear_mfma(m, n, k):
         assert torch.equal(again, got), "the same call must give the same bits"
 
 
+@pytest.mark.parametrize("m,hidden,kp,nc", [(1, 64, 32, 48), (8, 4096, 4096, 6144), (16, 160, 96, 272), (5, 4096, 14336, 1024),
+                                             (3, 96, 2048, 40)])
+def test_linear_split_norm(m, hidden, kp, nc):
+    """A norm carried by the products around it: the product that adds into the residual stream prepares
+    (rows times norm weight in bfloat16, sums of squares per 16 columns), the next product applies the
+    scale to its float32 sums.  Against float64, and against the norm kernel followed by the plain product."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(30)
+    eps = 1e-5
+    h = torch.randn(m, hidden, generator=g) * 3
+    a = torch.randn(m, kp, generator=g).to(torch.bfloat16)
+    wo = (torch.randn(hidden, kp, generator=g) * 0.05).to(torch.bfloat16)
+    nw = (1 + 0.3 * torch.randn(hidden, generator=g)).float()
+    wc = (torch.randn(nc, hidden, generator=g) * 0.1).to(torch.bfloat16)
+    assert ops.split_norm_ok(m, hidden, torch.bfloat16)
+    h2_ref = h.double() + a.double() @ wo.double().T
+    hd = h.clone().to(DEV)
+    out, pre = ops.linear(a.to(DEV), wo.to(DEV), torch.float32, residual=hd, next_norm=(nw.to(DEV), eps))
+    assert out is hd and pre is not None
+    _close(hd, h2_ref, 2e-5, "residual")
+    assert torch.equal(pre.x.cpu(), (hd.cpu() * nw).to(torch.bfloat16)), "rows times norm weight, rounded once"
+    ss = pre.ss.cpu().double().sum(0)[:m]
+    assert float(((ss - (hd.cpu().double() ** 2).sum(1)).abs() / ss).max()) < 1e-5
+    normed = h2_ref * torch.rsqrt((h2_ref ** 2).mean(1, keepdim=True) + eps) * nw.double()
+    ref = normed @ wc.double().T
+    got = ops.linear(pre, wc.to(DEV), torch.float32)
+    _close(got, ref, 6e-3, "consumer of the handed-over rows")
+    plain = ops.linear(ops.rmsnorm(hd, nw.to(DEV), eps, torch.bfloat16), wc.to(DEV), torch.float32)
+    _close(got, plain.double().cpu(), 6e-3, "split norm vs norm kernel + product")
+    if nc % 16 == 0:
+        gu = ref.reshape(m, -1, 2, 8)
+        gt, up = gu[:, :, 0].reshape(m, -1), gu[:, :, 1].reshape(m, -1)
+        _close(ops.linear_swiglu(pre, wc.to(DEV)), gt / (1 + torch.exp(-gt)) * up, 1e-2, "gated consumer")
+    # sizes that do not allow it: the product still adds, and says that the norm has to run on its own
+    if hidden % 32 == 0:
+        a2 = torch.randn(m, 24, generator=g).to(torch.bfloat16)
+        w2 = torch.randn(hidden, 24, generator=g).to(torch.bfloat16)
+        h3 = hd.clone()
+        out, none = ops.linear(a2.to(DEV), w2.to(DEV), torch.float32, residual=h3, next_norm=(nw.to(DEV), eps))
+        assert none is None
+        _close(h3, hd.double().cpu() + a2.double() @ w2.double().T, 2e-5, "fallback product")
+
+
 @pytest.mark.parametrize("heads,kv,d,page", [(4, 2, 32, 8), (8, 2, 64, 16), (6, 3, 96, 32), (32, 8, 128, 16), (8, 8, 128, 64),
                                              (20, 1, 64, 16), (5, 1, 128, 8)])
 def test_attention_mfma(heads, kv, d, page):
