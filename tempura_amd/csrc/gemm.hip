@@ -143,7 +143,7 @@ static void launch_generic(const void* x, const void* w, void* out, int M, int N
 // not its own (the general kernel then runs), >0 on error.
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
                    float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
-                   const void* post_w, void* post_xg, float* post_ss, hipStream_t s);
+                   const void* post_w, void* post_xg, float* post_ss, int layout, hipStream_t s);
 
 // `scratch` (optional, `scratch_floats` float32): room for split-K partial sums of mid-sized products.
 //
@@ -152,16 +152,21 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
 // [ceil(N / 16), 16], per block of 16 columns and row the sum of squares of `out`.  With `pre_ss`
 // ([pre_count, 16], as written by such a product whose N is this product's K) the result rows are
 // multiplied by rsqrt(sum of squares / K + pre_eps): x is then that product's post_xg.
+//
+// `layout` (bfloat16, at most 16 rows): bit 0, x is k-blocked [K / 8, M, 8] instead of [M, K]; bit 1, the
+// gated output (accumulate == 2) is written k-blocked [N / 16, M, 8] for a product that reads it so.
 extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
                                int N, int K, int allow_mfma, float* scratch, size_t scratch_floats,
                                const float* pre_ss, int pre_count, float pre_eps, const void* post_w, void* post_xg,
-                               float* post_ss, hipStream_t s) {
+                               float* post_ss, int layout, hipStream_t s) {
   TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(accumulate != 1 || out_dt == TP_F32, "linear: accumulating output must be float32");
-  const bool split_norm = pre_ss != nullptr || post_w != nullptr;
+  const bool split_norm = pre_ss != nullptr || post_w != nullptr || layout != 0;
+  TP_REQUIRE((layout & ~3) == 0 && (!(layout & 2) || accumulate == 2) && (!(layout & 1) || pre_ss == nullptr),
+             "linear: bad layout flags %d", layout);
   if (split_norm) {
     TP_REQUIRE(in_dt == TP_BF16 && allow_mfma && M <= 16 && K % 32 == 0,
-               "linear: the split norm needs bfloat16 operands, at most 16 rows and K %% 32 == 0 (M=%d K=%d)", M, K);
+               "linear: the split norm and the k-blocked layout need bfloat16 operands, at most 16 rows and K %% 32 == 0 (M=%d K=%d)", M, K);
     TP_REQUIRE(post_w == nullptr || (accumulate == 1 && post_xg != nullptr && post_ss != nullptr),
                "linear: the norm preparation belongs to a product that adds into the residual stream");
     TP_REQUIRE(pre_ss == nullptr || pre_count == (K + 15) / 16, "linear: %d partial sums for K=%d", pre_count, K);
@@ -169,7 +174,7 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   if (accumulate == 2) {  // gated-SiLU epilogue: only the matrix-core kernels have it
     TP_REQUIRE(in_dt == TP_BF16 && allow_mfma, "linear: the gated epilogue needs bfloat16 operands");
     const int r = tp_linear_mfma(x, w, out, out_dt, 2, M, N, K, scratch, scratch_floats, pre_ss, pre_count, pre_eps,
-                                 nullptr, nullptr, nullptr, s);
+                                 nullptr, nullptr, nullptr, layout, s);
     TP_REQUIRE(r >= 0, "linear: sizes M=%d N=%d K=%d do not fit the gated epilogue", M, N, K);
     return r;
   }
@@ -177,10 +182,10 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   if (M == 0) return 0;
   if (in_dt == TP_BF16 && allow_mfma) {
     const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, scratch, scratch_floats, pre_ss, pre_count,
-                                 pre_eps, post_w, post_xg, post_ss, s);
+                                 pre_eps, post_w, post_xg, post_ss, layout, s);
     if (r >= 0) return r;
   }
-  TP_REQUIRE(!split_norm, "linear: sizes M=%d N=%d K=%d do not fit the split norm", M, N, K);
+  TP_REQUIRE(!split_norm, "linear: sizes M=%d N=%d K=%d do not fit the split norm or the k-blocked layout", M, N, K);
   if (in_dt == TP_F32 && out_dt == TP_F32) {
     if (accumulate)
       launch_generic<float, float, true>(x, w, out, M, N, K, s);
@@ -203,5 +208,5 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
 extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
                          int N, int K, int allow_mfma, float* scratch, size_t scratch_floats, hipStream_t s) {
   return tp_linear_fused(x, w, in_dt, out, out_dt, accumulate, M, N, K, allow_mfma, scratch, scratch_floats, nullptr, 0,
-                         0.f, nullptr, nullptr, nullptr, s);
+                         0.f, nullptr, nullptr, nullptr, 0, s);
 }

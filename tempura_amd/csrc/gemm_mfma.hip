@@ -29,6 +29,16 @@ __device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)
 
 __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 
+// Layouts of bfloat16 activations of at most 16 rows.  Row-major [M, K], or k-blocked [K / 8, M, 8]:
+// eight consecutive k of all rows side by side, so that the operand fragments that the lanes of a
+// wave fetch straight from global memory (16 bytes per row and k group) lie next to each other.
+enum { X_KBLOCKED = 1, OUT_KBLOCKED = 2 };
+
+__device__ inline void store_gated(void* out, int layout, int M, int width, int m, int col, float v) {
+  const size_t idx = (layout & OUT_KBLOCKED) ? ((size_t)(col >> 3) * M + m) * 8 + (col & 7) : (size_t)m * width + col;
+  ((bf16_t*)out)[idx] = float_to_bf16(v);
+}
+
 __device__ inline void store_out(void* out, int mode, size_t idx, float v) {
   if (mode == OUT_F32)
     ((float*)out)[idx] = v;
@@ -108,7 +118,8 @@ template <int MT, int NT, int WAVES, int DEPTH>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16_t* __restrict__ x,
                                                                       const bf16_t* __restrict__ w,
                                                                       void* __restrict__ out, int mode, int M,
-                                                                      int N, int K, RowScale pre, NormPrep post) {
+                                                                      int N, int K, int layout, RowScale pre,
+                                                                      NormPrep post) {
   __shared__ float red[WAVES][NT * MT][256];
   __shared__ float rs_part[32][16], rstd[16], ss_lds[NT][4][16];
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
@@ -120,11 +131,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
     const int wrow = min(n0 + j * 16 + (lane & 15), N - 1);
     wp[j] = (const u32x4_t*)(w + (size_t)wrow * K + kofs);
   }
+  // x is [M, K] row-major, or (xblocked, M <= 16) [K / 8, M, 8]: eight consecutive k of all rows side by
+  // side, so that the 16 bytes the lanes of a wave fetch lie next to each other
   const u32x4_t* xp[MT];
+  const bool xblocked = (layout & X_KBLOCKED) != 0;
+  const int xstep = xblocked ? 4 * M : 4;   // u32x4 units per 32 of k
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int xrow = min(t * 16 + (lane & 15), M - 1);
-    xp[t] = (const u32x4_t*)(x + (size_t)xrow * K + kofs);
+    xp[t] = xblocked ? (const u32x4_t*)(x + ((size_t)(lane >> 4) * M + xrow) * 8) : (const u32x4_t*)(x + (size_t)xrow * K + kofs);
   }
   f32x4_t acc[NT][MT];
 #pragma unroll
@@ -148,7 +163,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 #pragma unroll
         for (int j = 0; j < NT; ++j) a[d][j][u] = wp[j][(size_t)sidx * 4];
 #pragma unroll
-        for (int t = 0; t < MT; ++t) b[d][t][u] = xp[t][(size_t)sidx * 4];
+        for (int t = 0; t < MT; ++t) b[d][t][u] = xp[t][(size_t)sidx * xstep];
       }
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d)
@@ -189,7 +204,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) u += red[i][jt][q + 128];
         if (MT == 1) u *= rstd[l & 15];
-        ((bf16_t*)out)[(size_t)m * (N / 2) + (n0 + j * 16) / 2 + (l >> 4) * 4 + r] = float_to_bf16(silu_mul(v, u));
+        store_gated(out, layout, M, N / 2, m, (n0 + j * 16) / 2 + (l >> 4) * 4 + r, silu_mul(v, u));
       }
     } else if (MT == 1 && post.w != nullptr) {
       // residual add, and the next norm's preparation (mode is OUT_ACC_F32)
@@ -238,7 +253,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 template <int NT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                void* __restrict__ out, int mode, int M, int N, int K,
-                                                               RowScale pre, NormPrep post) {
+                                                               int layout, RowScale pre, NormPrep post) {
   constexpr int THREADS = WAVES * 64, G = 1;
   constexpr int KC = WAVES * 128;        // K elements per chunk: one run of four steps per wave
   constexpr int LD = KC + 8;             // padded LDS row
@@ -340,7 +355,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_
 #pragma unroll
         for (int i = 0; i < WAVES; ++i) u += red[ge * WAVES + i][j][q + 128];
         u *= rstd[m];
-        ((bf16_t*)out)[(size_t)m * (N / 2) + nt0 / 2 + (l >> 4) * 4 + r] = float_to_bf16(silu_mul(v, u));
+        store_gated(out, layout, M, N / 2, m, nt0 / 2 + (l >> 4) * 4 + r, silu_mul(v, u));
       }
     } else if (post.w != nullptr) {
       float sq = 0.f;
@@ -543,16 +558,16 @@ extern "C" void tp_linear_tune(int waves, int nt, int depth) {
 }
 
 template <int MT, int NT, int WAVES, int DEPTH>
-static void launch_skinny4(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, RowScale pre,
-                           NormPrep post, hipStream_t s) {
+static void launch_skinny4(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, int layout,
+                           RowScale pre, NormPrep post, hipStream_t s) {
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, NT, WAVES, DEPTH>), dim3(blocks), dim3(WAVES * 64), 0, s, x, w, out,
-                     mode, M, N, K, pre, post);
+                     mode, M, N, K, layout, pre, post);
 }
 
 template <int MT>
-static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, RowScale pre,
-                          NormPrep post, hipStream_t s) {
+static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, int layout,
+                          RowScale pre, NormPrep post, hipStream_t s) {
   // every wave should get at least one run of four steps; small N wants many waves per block
   // (one block per 16 columns is all the parallelism there is), large N fewer and two row tiles
   // Measured on MI355X at Llama-8B shapes: eight waves with two runs in flight each stream
@@ -568,15 +583,15 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
   if constexpr (MT == 1) {
     // several activation rows: feed them through LDS, unless K is so long that the barrier per
     // chunk costs more than the gather (measured: K = 14336 is faster without)
-    bool lds = M > 1 && K >= 2 * LKC && K <= 8 * LKC;
-    if (g_tune_depth) lds = g_tune_depth == 9;
+    bool lds = M > 1 && K >= 2 * LKC && K <= 8 * LKC && !(layout & X_KBLOCKED);
+    if (g_tune_depth && !(layout & X_KBLOCKED)) lds = g_tune_depth == 9;
     if (lds) {
       if (nt > 2) nt = 2;
       const int blocks = (N + 16 * nt - 1) / (16 * nt);
       if (nt == 2)
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, pre, post);
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post);
       else
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, pre, post);
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post);
       return;
     }
   }
@@ -584,7 +599,7 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
   if (MT > 1) nt = 1;
   if (MT > 2 || nt > 2) depth = 1;           // registers
 #define CASE(NT_, W_, D_) \
-  if (nt == NT_ && waves == W_ && depth == D_) return launch_skinny4<MT, NT_, W_, D_>(x, w, out, mode, M, N, K, pre, post, s)
+  if (nt == NT_ && waves == W_ && depth == D_) return launch_skinny4<MT, NT_, W_, D_>(x, w, out, mode, M, N, K, layout, pre, post, s)
   CASE(1, 16, 1);
   CASE(1, 8, 1);
   CASE(1, 4, 1);
@@ -605,15 +620,17 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
     CASE(4, 4, 1);
   }
 #undef CASE
-  launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, pre, post, s);
+  launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, layout, pre, post, s);
 }
 
 // accumulate: 0 store, 1 add into the float32 output, 2 gated-SiLU epilogue (see OUT_SWIGLU).
 // pre_ss / post_w: the split norm (RowScale / NormPrep above), at most 16 rows; nullptr without.
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
                    float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
-                   const void* post_w, void* post_xg, float* post_ss, hipStream_t s) {
+                   const void* post_w, void* post_xg, float* post_ss, int layout, hipStream_t s) {
   if (K % 32 != 0) return -1;
+  if (layout != 0 && M > 16) return -1;
+  if ((layout & OUT_KBLOCKED) && accumulate != 2) return -1;
   if ((pre_ss != nullptr || post_w != nullptr) && M > 16) return -1;
   if (post_w != nullptr && accumulate != 1) return -1;
   const RowScale pre = {pre_ss, pre_count, 1.0f / (float)K, pre_eps};
@@ -626,13 +643,13 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   const bool mid_ok = scratch != nullptr && g_tune_mid != 1;
   if (M <= 16 || (M <= 64 && !mid_ok)) {
     if (M <= 16)
-      launch_skinny<1>(xb, wb, out, mode, M, N, K, pre, post, s);
+      launch_skinny<1>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
     else if (M <= 32)
-      launch_skinny<2>(xb, wb, out, mode, M, N, K, pre, post, s);
+      launch_skinny<2>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
     else if (M <= 48)
-      launch_skinny<3>(xb, wb, out, mode, M, N, K, pre, post, s);
+      launch_skinny<3>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
     else
-      launch_skinny<4>(xb, wb, out, mode, M, N, K, pre, post, s);
+      launch_skinny<4>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
   } else {
     // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
     // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.

@@ -166,6 +166,24 @@ class Prenormed:
         return self.x.shape
 
 
+class KBlocked:
+    """bfloat16 activations of at most 16 rows stored k-blocked, ``data`` [k / 8, m, 8]: eight consecutive
+    columns of all rows side by side.  A product of a few rows that reads its activations straight from
+    global memory then fetches neighbouring bytes instead of short pieces of several rows.  Made by
+    ``linear_swiglu(..., blocked_out=True)``, taken by ``linear``."""
+    __slots__ = ("data", "rows", "width")
+
+    def __init__(self, data, rows, width):
+        self.data, self.rows, self.width = data, rows, width
+
+    @property
+    def shape(self):
+        return (self.rows, self.width)
+
+    def row_major(self) -> torch.Tensor:
+        return self.data.permute(1, 0, 2).reshape(self.rows, self.width).contiguous()
+
+
 def split_norm_ok(m: int, width: int, dtype: torch.dtype) -> bool:
     """Whether a norm over ``width`` columns of ``m`` rows can be split over the two products around it."""
     if _backend is not None:
@@ -182,11 +200,12 @@ def _pre_args(x):
     return x, (_ptr(None), 0, ctypes.c_float(0.0))
 
 
-def linear_swiglu(x, w: torch.Tensor) -> torch.Tensor:
+def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     """bfloat16 x [m, k] (or ``Prenormed``), interleaved gate/up weight [2i, k] -> bfloat16 [m, i] =
-    silu(x g^T) * (x u^T), the gate applied to the float32 accumulators (no rounding in between)."""
+    silu(x g^T) * (x u^T), the gate applied to the float32 accumulators (no rounding in between).
+    With ``blocked_out`` the result comes as ``KBlocked`` when there are at most 16 rows (else as a tensor)."""
     if _backend is not None:
-        return _backend.linear_swiglu(x, w)
+        return _backend.linear_swiglu(x, w, blocked_out) if blocked_out else _backend.linear_swiglu(x, w)
     x, pre = _pre_args(x)
     _dev_ok(x, w)
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_swiglu: shapes {tuple(x.shape)} x {tuple(w.shape)}")
@@ -194,10 +213,15 @@ def linear_swiglu(x, w: torch.Tensor) -> torch.Tensor:
     m, k = x.shape
     n = w.shape[0]
     _need(n % 16 == 0 and k % 32 == 0, "linear_swiglu: needs 2i % 16 == 0 and k % 32 == 0")
-    out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    blocked_out = blocked_out and 0 < m <= 16
+    if blocked_out:
+        out = KBlocked(torch.empty((n // 16, m, 8), dtype=torch.bfloat16, device=x.device), m, n // 2)
+    else:
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     scratch, nscratch = _splitk_scratch(x, m, n)
-    _call("tp_linear_fused", _ptr(x), _ptr(w), _BF16, _ptr(out), _BF16, 2, m, n, k, 1, _ptr(scratch),
-          ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), _stream())
+    _call("tp_linear_fused", _ptr(x), _ptr(w), _BF16, _ptr(out.data if blocked_out else out), _BF16, 2, m, n, k, 1,
+          _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), 2 if blocked_out else 0,
+          _stream())
     return out
 
 
@@ -218,11 +242,21 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
         if next_norm is not None:
             return _backend.linear(x, w, out_dtype, residual, next_norm)
         return _backend.linear(x, w, out_dtype, residual)
-    x, pre = _pre_args(x)
-    _dev_ok(x, w, residual)
-    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
-    _need(x.dtype == w.dtype, f"linear: operand dtypes differ ({x.dtype}, {w.dtype})")
-    m, k = x.shape
+    layout = 0
+    if isinstance(x, KBlocked):
+        _need(allow_mfma and x.data.dtype == torch.bfloat16 and tuple(x.data.shape) == (x.width // 8, x.rows, 8)
+              and x.width % 32 == 0, "linear: malformed k-blocked rows")
+        kb, layout = x, 1
+        x, pre = x.data, (_ptr(None), 0, ctypes.c_float(0.0))
+        m, k = kb.rows, kb.width
+        _dev_ok(x, w, residual)
+        _need(w.dim() == 2 and w.shape[1] == k and w.dtype == torch.bfloat16, f"linear: shapes {(m, k)} x {tuple(w.shape)}")
+    else:
+        x, pre = _pre_args(x)
+        _dev_ok(x, w, residual)
+        _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
+        _need(x.dtype == w.dtype, f"linear: operand dtypes differ ({x.dtype}, {w.dtype})")
+        m, k = x.shape
     n = w.shape[0]
     if residual is not None:
         _need(residual.dtype == torch.float32 and tuple(residual.shape) == (m, n), "linear: residual must be float32 [m, n]")
@@ -240,7 +274,7 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
         post = (_ptr(weight), _ptr(handed.x), _ptr(handed.ss))
     scratch, nscratch = _splitk_scratch(x, m, n) if allow_mfma else (None, 0)
     _call("tp_linear_fused", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
-          ctypes.c_size_t(nscratch), *pre, *post, _stream())
+          ctypes.c_size_t(nscratch), *pre, *post, layout, _stream())
     return out if next_norm is None else (out, handed)
 
 

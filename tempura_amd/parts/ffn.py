@@ -43,7 +43,8 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, ctx, residual, next_norm=None):
         if self.fused:
-            a = ops.linear_swiglu(x, self.w13)
+            # (a few rows go to the next product k-blocked: it reads them straight from global memory)
+            a = ops.linear_swiglu(x, self.w13, blocked_out=True)
         else:
             gu = ops.linear(x, self.w13, torch.float32)
             a = ops.swiglu(gu, self.dtype)

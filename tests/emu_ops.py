@@ -28,7 +28,9 @@ class EmuOps:
     def _rows(x):
         """Plain rows, or handed-over rows (x = bfloat16(h * weight), ss = sums of squares per 16 columns)
         with the factor that finishes their norm."""
-        from tempura_amd.kernels.ops import Prenormed
+        from tempura_amd.kernels.ops import KBlocked, Prenormed
+        if isinstance(x, KBlocked):
+            return x.row_major().double(), 1.0
         if isinstance(x, Prenormed):
             rstd = torch.rsqrt(x.ss.double().sum(0)[: x.x.shape[0]] / x.x.shape[1] + x.eps)
             return x.x.double(), rstd[:, None]
@@ -52,12 +54,17 @@ class EmuOps:
             return residual, Prenormed((residual * weight).to(torch.bfloat16), ss, eps)
         return y.to(out_dtype)
 
-    def linear_swiglu(self, x, w):
+    def linear_swiglu(self, x, w, blocked_out=False):
+        from tempura_amd.kernels.ops import KBlocked
         xd, scale = self._rows(x)
         x = xd
         y = ((x @ w.double().T) * scale).reshape(x.shape[0], -1, 2, 8)      # eight gate rows, eight up rows in turn
         g, u = y[:, :, 0].reshape(x.shape[0], -1), y[:, :, 1].reshape(x.shape[0], -1)
-        return (g / (1.0 + torch.exp(-g)) * u).to(torch.bfloat16)
+        out = (g / (1.0 + torch.exp(-g)) * u).to(torch.bfloat16)
+        m, i = out.shape
+        if blocked_out and 0 < m <= 16:
+            return KBlocked(out.reshape(m, i // 8, 8).permute(1, 0, 2).contiguous(), m, i)
+        return out
 
     def rope_kv_write(self, qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads, num_kv_heads,
                       head_dim, k_cache, v_cache, q_dtype):

@@ -323,3 +323,18 @@ def test_linear_swiglu(m, inter, k):
     assert got.shape == (m, inter)
     _close(got, ref, 6e-3, "linear_swiglu")
     assert torch.equal(emu.linear_swiglu(x, w), ref.to(torch.bfloat16))
+    # k-blocked output for a few rows: the same numbers in the other layout, and the product that takes them
+    blk = ops.linear_swiglu(x.to(DEV), w.to(DEV), blocked_out=True)
+    if m > 16:
+        assert torch.is_tensor(blk) and torch.equal(blk, got)
+    else:
+        assert tuple(blk.data.shape) == (inter // 8, m, 8) and blk.shape == (m, inter)
+        assert torch.equal(blk.row_major(), got)
+        assert torch.equal(emu.linear_swiglu(x, w, True).data, ref.to(torch.bfloat16).reshape(m, inter // 8, 8).permute(1, 0, 2))
+        if inter % 32 == 0:
+            w2 = (torch.randn(72, inter, generator=g) * 0.2).to(torch.bfloat16)
+            res = torch.randn(m, 72, generator=g)
+            want = res.double() + got.double().cpu() @ w2.double().T
+            r1 = res.clone().to(DEV)
+            ops.linear(blk, w2.to(DEV), torch.float32, residual=r1)
+            _close(r1, want, 2e-5, "product of k-blocked rows")
