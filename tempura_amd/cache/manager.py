@@ -8,32 +8,42 @@ group keeps every page until the request ends; a ``window`` group gives a page
 back as soon as no later query can see any key in it.  Pages return to the free
 list at once and are handed out again (most recently freed first).
 
-This module is host bookkeeping only: it never touches device memory.  The
-reference keeps one table per layer with ``u32::MAX`` for an empty entry and
-grows by ``ceil(n / block) - have`` pages
-(/root/reference/engine/src/kv_cache.rs:836-893,975-984); here a table is per
-request and group, empty entries are -1, and growth reports need/free without
-side effects when it cannot be met
-(/root/reference/engine/src/cutile_kv_cache.rs:31-44).
+This is host bookkeeping only: it never touches device memory.  The bookkeeping
+itself is native code (csrc/host/cache_core.cpp, as the reference's is:
+/root/reference/engine/src/kv_cache.rs:836-893,975-984); this class maps request
+names to the core's request slots and turns its error codes into exceptions.  Empty
+table entries are -1, and growth reports need/free without side effects when it
+cannot be met (/root/reference/engine/src/cutile_kv_cache.rs:31-44).
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence
+import ctypes
+from typing import Dict, Hashable, List, Sequence
 
 import numpy as np
 
 from ..parts.base import CacheSpec
-from .pages import PagePool, PagesExhausted
+from . import native
+from .pages import PagesExhausted
 
 
-@dataclass
-class _Request:
-    rid: Hashable
-    num_tokens: int = 0                      # tokens whose keys/values are in the cache
-    tables: List[List[int]] = field(default_factory=list)   # per group: logical page -> physical, -1 = none
-    first_live: List[int] = field(default_factory=list)     # per group: first logical page still held
-    state_slot: int = -1
+class _PoolView:
+    """Counts of one group's page pool."""
+
+    def __init__(self, manager: "CacheManager", g: int, num_pages: int):
+        self._m, self._g, self.num_pages = manager, g, num_pages
+
+    @property
+    def num_free(self) -> int:
+        return self._m.free_pages()[self._g]
+
+    @property
+    def num_held(self) -> int:
+        return self.num_pages - self.num_free
+
+
+def _ints(values) -> ctypes.Array:
+    return (ctypes.c_int * len(values))(*values)
 
 
 class CacheManager:
@@ -46,171 +56,152 @@ class CacheManager:
             num_pages = [num_pages] * len(self.groups)
         if len(num_pages) != len(self.groups):
             raise ValueError("num_pages must give one count per cache group")
-        self.pools = [PagePool(int(n)) for n in num_pages]
+        if any(int(n) < 0 for n in num_pages):
+            raise ValueError("num_pages must be >= 0")
         self.max_requests = int(max_requests)
-        self._free_state = list(range(self.max_requests - 1, -1, -1))
-        self._requests: Dict[Hashable, _Request] = {}
+        self._lib = native.lib()
+        kinds = [1 if (s.kind == "window" and s.window is not None) else 0 for s in self.groups]
+        windows = [int(s.window) if s.window is not None else 0 for s in self.groups]
+        self._h = ctypes.c_void_p(self._lib.cc_create(len(self.groups), _ints(kinds), _ints(windows), self.page_size,
+                                                      _ints([int(n) for n in num_pages]), self.max_requests))
+        if not self._h:
+            raise ValueError(native.last_error())
+        self.pools = [_PoolView(self, g, int(n)) for g, n in enumerate(num_pages)]
+        self._slot_of: Dict[Hashable, int] = {}
+        self._g_buf = (ctypes.c_int * max(1, len(self.groups)))()
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.cc_destroy(self._h)
+            self._h = None
+
+    def _slot(self, rid) -> int:
+        try:
+            return self._slot_of[rid]
+        except KeyError:
+            raise KeyError(f"request {rid!r} is not live") from None
 
     # ---- requests ------------------------------------------------------
     def has(self, rid) -> bool:
-        return rid in self._requests
+        return rid in self._slot_of
 
     def live_requests(self):
-        return list(self._requests)
+        return list(self._slot_of)
 
     def add(self, rid) -> int:
         """Start tracking ``rid``; returns its state slot."""
-        if rid in self._requests:
+        if rid in self._slot_of:
             raise ValueError(f"request {rid!r} is already live")
-        if not self._free_state:
-            raise RuntimeError(f"no free state slot: {self.max_requests} requests are live")
-        r = _Request(rid, 0, [[] for _ in self.groups], [0] * len(self.groups), self._free_state.pop())
-        self._requests[rid] = r
-        return r.state_slot
+        s = self._lib.cc_add(self._h)
+        if s < 0:
+            raise RuntimeError(native.last_error())
+        self._slot_of[rid] = s
+        return s
 
     def release(self, rid) -> None:
         """The request has ended: every page and its state slot go back."""
-        r = self._requests.pop(rid, None)
-        if r is None:
+        s = self._slot_of.pop(rid, None)
+        if s is None:
             raise ValueError(f"request {rid!r} is not live (released twice?)")
-        for g, table in enumerate(r.tables):
-            for p in table:
-                if p >= 0:
-                    self.pools[g].free(p)
-        self._free_state.append(r.state_slot)
+        if self._lib.cc_release(self._h, s) != 0:
+            raise RuntimeError(native.last_error())
 
     def num_tokens(self, rid) -> int:
-        return self._requests[rid].num_tokens
+        return self._lib.cc_num_tokens(self._h, self._slot(rid))
+
+    def max_num_tokens(self, rids: Sequence) -> int:
+        """The largest token count among ``rids``."""
+        m = self._lib.cc_max_tokens(self._h, len(rids), _ints([self._slot(r) for r in rids]))
+        if m < 0:
+            raise RuntimeError(native.last_error())
+        return m
 
     def state_slot(self, rid) -> int:
-        return self._requests[rid].state_slot
+        return self._slot(rid)
 
     # ---- pages ---------------------------------------------------------
-    def _first_needed(self, g: int, start: int) -> int:
-        """First logical page a query at position ``start`` can still see."""
-        spec = self.groups[g]
-        if spec.kind == "window" and spec.window is not None:
-            return max(0, start - spec.window + 1) // self.page_size
-        return 0
-
     def pages_needed(self, rid, n_new: int) -> List[int]:
         """Pages each group must allocate so that ``rid`` can take ``n_new`` more tokens."""
-        r = self._requests[rid]
-        end = r.num_tokens + n_new
-        last_page = (end - 1) // self.page_size if end > 0 else -1
-        need = []
-        for g in range(len(self.groups)):
-            lo = max(self._first_needed(g, r.num_tokens), r.first_live[g])
-            # every entry from first_live up to the table's end holds a page (pages are given back
-            # only below first_live), so what is missing is what lies beyond the table
-            need.append(max(0, last_page + 1 - max(lo, len(r.tables[g]))))
-        return need
+        self._lib.cc_pages_needed(self._h, self._slot(rid), int(n_new), self._g_buf)
+        return list(self._g_buf[: len(self.groups)])
 
     def can_reserve(self, rid, n_new: int) -> bool:
-        return all(n <= pool.num_free for n, pool in zip(self.pages_needed(rid, n_new), self.pools))
+        return all(n <= f for n, f in zip(self.pages_needed(rid, n_new), self.free_pages()))
 
     def reserve(self, rid, n_new: int) -> None:
         """Allocate the pages for ``n_new`` more tokens, or raise ``PagesExhausted``
         leaving everything as it was."""
-        if n_new <= 0:
+        self.reserve_many([rid], [n_new])
+
+    def reserve_many(self, rids: Sequence, n_new: Sequence[int]) -> None:
+        """Pages for every request of a step, or ``PagesExhausted`` with nothing changed."""
+        if any(int(n) <= 0 for n in n_new):
             raise ValueError("reserve needs at least one token")
-        r = self._requests[rid]
-        need = self.pages_needed(rid, n_new)
-        for g, n in enumerate(need):
-            if n > self.pools[g].num_free:
-                raise PagesExhausted(n, self.pools[g].num_free, g)
-        end = r.num_tokens + n_new
-        last_page = (end - 1) // self.page_size
-        for g in range(len(self.groups)):
-            lo = max(self._first_needed(g, r.num_tokens), r.first_live[g])
-            table = r.tables[g]
-            have = len(table)
-            while len(table) <= last_page:
-                table.append(-1)
-            # pages that a window has already passed (below lo) stay unallocated
-            for lp in range(max(lo, have), last_page + 1):
-                table[lp] = self.pools[g].alloc()
-            if lo > have:
-                r.first_live[g] = max(r.first_live[g], min(lo, len(table)))
+        info = (ctypes.c_int * 3)()
+        rc = self._lib.cc_reserve(self._h, len(rids), _ints([self._slot(r) for r in rids]), _ints([int(n) for n in n_new]),
+                                  info)
+        if rc == 1:
+            raise PagesExhausted(info[0], info[1], info[2])
+        if rc != 0:
+            raise RuntimeError(native.last_error())
 
     def commit(self, rid, n_new: int) -> None:
         """``n_new`` tokens were written; give back pages a window has passed."""
-        r = self._requests[rid]
-        r.num_tokens += n_new
-        for g in range(len(self.groups)):
-            keep_from = self._first_needed(g, r.num_tokens)
-            table = r.tables[g]
-            for lp in range(r.first_live[g], min(keep_from, len(table))):
-                if table[lp] >= 0:
-                    self.pools[g].free(table[lp])
-                    table[lp] = -1
-            r.first_live[g] = max(r.first_live[g], min(keep_from, len(table)))
+        self.commit_many([rid], [n_new])
+
+    def commit_many(self, rids: Sequence, n_new: Sequence[int]) -> None:
+        if self._lib.cc_commit(self._h, len(rids), _ints([self._slot(r) for r in rids]), _ints([int(n) for n in n_new])) != 0:
+            raise RuntimeError(native.last_error())
 
     def truncate(self, rid, num_tokens: int) -> None:
         """Forget tokens past ``num_tokens`` and return whole pages beyond them."""
-        r = self._requests[rid]
-        if num_tokens > r.num_tokens or num_tokens < 0:
-            raise ValueError("truncate beyond what is cached")
-        keep_pages = (num_tokens + self.page_size - 1) // self.page_size
-        for g, table in enumerate(r.tables):
-            for lp in range(keep_pages, len(table)):
-                if table[lp] >= 0:
-                    self.pools[g].free(table[lp])
-            del table[keep_pages:]
-        r.num_tokens = num_tokens
+        if self._lib.cc_truncate(self._h, self._slot(rid), int(num_tokens)) != 0:
+            raise ValueError(native.last_error())
 
     def table(self, rid, g: int) -> List[int]:
-        return self._requests[rid].tables[g]
+        s = self._slot(rid)
+        n = self._lib.cc_table_len(self._h, s, g)
+        buf = (ctypes.c_int * max(1, n))()
+        self._lib.cc_table(self._h, s, g, buf)
+        return list(buf[:n])
 
     def slot(self, rid, g: int, pos: int) -> int:
         """Physical cache row of one position (the single-token case of ``slots``)."""
-        table = self._requests[rid].tables[g]
-        lp = pos // self.page_size
-        if pos < 0 or lp >= len(table) or table[lp] < 0:
-            raise RuntimeError(f"request {rid!r}: position {pos} has no page reserved")
-        return table[lp] * self.page_size + pos % self.page_size
+        return int(self.slots(rid, g, pos, 1)[0])
 
     def slots(self, rid, g: int, start: int, n: int) -> np.ndarray:
         """Physical cache rows (page * page_size + offset) of positions start..start+n-1."""
-        table = self._requests[rid].tables[g]
-        pos = np.arange(start, start + n, dtype=np.int64)
-        if start < 0 or (start + n - 1) // self.page_size >= len(table):
-            raise RuntimeError(f"request {rid!r}: positions {start}..{start + n - 1} have no page reserved")
-        pages = np.asarray(table, dtype=np.int64)[pos // self.page_size]
-        if (pages < 0).any():
-            raise RuntimeError(f"request {rid!r}: positions {start}..{start + n - 1} have no page reserved")
-        return pages * self.page_size + pos % self.page_size
+        out = np.empty(n, dtype=np.int32)
+        if self._lib.cc_slots(self._h, self._slot(rid), g, int(start), int(n), out.ctypes.data_as(ctypes.c_void_p)) != 0:
+            raise RuntimeError(f"request {rid!r}: {native.last_error()}")
+        return out
+
+    def fill_decode(self, rids: Sequence, tokens: Sequence[int], rows: int, width: int, scratch_pages: Sequence[int],
+                    out: np.ndarray) -> None:
+        """Pack the device inputs of a decode step (one new token per request, pages reserved) into ``out``
+        (int32): tokens, positions, context lengths and state slots of ``rows`` rows, then per group the block
+        tables [rows, width], then per group the cache rows of the new tokens.  Rows past ``len(rids)`` are
+        padding that reads and writes the scratch page."""
+        need = 4 * rows + len(self.groups) * rows * (width + 1)
+        if out.dtype != np.int32 or out.size < need or not out.flags["C_CONTIGUOUS"]:
+            raise ValueError("fill_decode: the buffer must be contiguous int32 of the packed size")
+        rc = self._lib.cc_fill_decode(self._h, len(rids), _ints([self._slot(r) for r in rids]), _ints([int(t) for t in tokens]),
+                                      int(rows), int(width), _ints([int(p) for p in scratch_pages]),
+                                      out.ctypes.data_as(ctypes.c_void_p))
+        if rc != 0:
+            raise RuntimeError(native.last_error())
 
     # ---- statistics and invariants -------------------------------------
     def free_pages(self) -> List[int]:
-        return [p.num_free for p in self.pools]
+        self._lib.cc_free_pages(self._h, self._g_buf)
+        return list(self._g_buf[: len(self.groups)])
 
     def waste_ratio(self) -> float:
         """Share of held token places that hold no token
         (/root/reference/engine/src/kv_cache.rs:1066-1074)."""
-        held = sum(p.num_held for p in self.pools) * self.page_size
-        if held == 0:
-            return 0.0
-        used = 0
-        for r in self._requests.values():
-            for g in range(len(self.groups)):
-                live_from = r.first_live[g] * self.page_size
-                used += max(0, r.num_tokens - live_from)
-        return max(0.0, 1.0 - used / held)
+        return float(self._lib.cc_waste_ratio(self._h))
 
     def check(self) -> None:
         """No page lost, held twice or free while in a table; state slots likewise."""
-        for g, pool in enumerate(self.pools):
-            pool.check()
-            seen = set()
-            for r in self._requests.values():
-                for p in r.tables[g]:
-                    if p >= 0:
-                        assert p not in seen, f"group {g}: page {p} is in two tables"
-                        assert pool.is_held(p), f"group {g}: page {p} is in a table but free"
-                        seen.add(p)
-            assert len(seen) == pool.num_held, f"group {g}: {pool.num_held - len(seen)} pages held by no request"
-        slots = [r.state_slot for r in self._requests.values()]
-        assert len(set(slots)) == len(slots), "a state slot is held twice"
-        assert len(slots) + len(self._free_state) == self.max_requests, "a state slot was lost"
-        assert not (set(slots) & set(self._free_state)), "a held state slot is on the free list"
+        assert self._lib.cc_check(self._h) == 0, native.last_error()
+        assert self._lib.cc_num_live(self._h) == len(self._slot_of), "the core and the name table disagree"

@@ -3,11 +3,14 @@
 The reference's CPU allocator is a LIFO free list whose invariant is
 ``available + in_use == total`` (/root/reference/engine/src/kv_cache.rs:762-795,
 /root/reference/kernel-api/src/lib.rs:604-618).  A page id addresses the same
-page in the key and value pool of every cache slot of its group.
+page in the key and value pool of every cache slot of its group.  The list itself
+lives in the compiled host library (csrc/host/cache_core.cpp); this is its Python face.
 """
 from __future__ import annotations
 
-from typing import List
+import ctypes
+
+from . import native
 
 
 class PagesExhausted(RuntimeError):
@@ -25,40 +28,36 @@ class PagePool:
     def __init__(self, num_pages: int):
         if num_pages < 0:
             raise ValueError("num_pages must be >= 0")
-        self.num_pages = num_pages
-        # LIFO: the most recently freed page is handed out first, so reuse is prompt.
-        self._free: List[int] = list(range(num_pages - 1, -1, -1))
-        self._held = [False] * num_pages
+        self.num_pages = int(num_pages)
+        self._lib = native.lib()
+        self._h = ctypes.c_void_p(self._lib.pp_create(self.num_pages))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.pp_destroy(self._h)
+            self._h = None
 
     @property
     def num_free(self) -> int:
-        return len(self._free)
+        return self._lib.pp_num_free(self._h)
 
     @property
     def num_held(self) -> int:
-        return self.num_pages - len(self._free)
+        return self.num_pages - self.num_free
 
     def alloc(self) -> int:
-        if not self._free:
+        p = self._lib.pp_alloc(self._h)
+        if p < 0:
             raise PagesExhausted(1, 0)
-        p = self._free.pop()
-        assert not self._held[p], f"page {p} handed out twice"
-        self._held[p] = True
         return p
 
     def free(self, page: int) -> None:
-        if page < 0 or page >= self.num_pages:
-            raise ValueError(f"page {page} out of range")
-        if not self._held[page]:
-            raise ValueError(f"page {page} freed twice (or never allocated)")
-        self._held[page] = False
-        self._free.append(page)
+        if self._lib.pp_free(self._h, int(page)) != 0:
+            raise ValueError(native.last_error())
 
     def is_held(self, page: int) -> bool:
-        return self._held[page]
+        return bool(self._lib.pp_is_held(self._h, int(page)))
 
     def check(self) -> None:
         """Conservation: every page is either free or held, exactly once."""
-        assert len(set(self._free)) == len(self._free), "a page is on the free list twice"
-        assert all(not self._held[p] for p in self._free), "a free page is marked held"
-        assert sum(self._held) + len(self._free) == self.num_pages, "a page was lost"
+        assert self._lib.pp_check(self._h) == 0, native.last_error()

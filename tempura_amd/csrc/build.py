@@ -150,5 +150,60 @@ def ensure_built(verbose: bool = True) -> str:
     return library_path() or build(verbose)
 
 
+# ---- the host library: plain C++ (no GPU code), needed on machines without a GPU too ------------
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+
+def host_sources() -> List[str]:
+    return sorted(glob.glob(os.path.join(HERE, "host", "*.cpp")))
+
+
+def _host_lib_name() -> str:
+    h = hashlib.sha256()
+    for p in host_sources():
+        h.update(os.path.basename(p).encode())
+        with open(p, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return f"libtempura_host_{h.hexdigest()[:16]}.so"
+
+
+def host_library_path() -> Optional[str]:
+    name = _host_lib_name()
+    for d in _build_dirs():
+        p = os.path.join(d, name)
+        if os.path.exists(p):
+            return p
+    return None
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compile the host library (always); returns its path."""
+    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++") or shutil.which("clang++")
+    if not cxx:
+        raise RuntimeError("no C++ compiler found (looked at $CXX, g++, c++, clang++): the host library cannot be built")
+    out_dir = _writable_build_dir()
+    name = _host_lib_name()
+    t0 = time.time()
+    tmp = os.path.join(out_dir, name + f".{os.getpid()}.tmp")
+    _run([cxx, *HOST_FLAGS, *host_sources(), "-o", tmp], "compiling the host library")
+    final = os.path.join(out_dir, name)
+    os.replace(tmp, final)
+    for old in glob.glob(os.path.join(out_dir, "libtempura_host_*.so")):
+        if os.path.basename(old) != name:
+            try:
+                os.remove(old)
+            except OSError:
+                pass
+    if verbose:
+        print(f"[tempura_amd] host library built in {time.time() - t0:.0f} s: {final}", file=sys.stderr, flush=True)
+    return final
+
+
+def ensure_host_built(verbose: bool = True) -> str:
+    return host_library_path() or build_host(verbose)
+
+
 if __name__ == "__main__":
+    print(build_host())
     print(build())

@@ -183,17 +183,7 @@ class ModelRunner:
 
     def reserve(self, entries: Sequence[StepEntry]) -> None:
         """Pages for every entry, or ``PagesExhausted`` with nothing changed."""
-        n_groups = len(self.cache.groups)
-        total = [0] * n_groups
-        for e in entries:
-            for g, n in enumerate(self.cache.pages_needed(e.rid, len(e.tokens))):
-                total[g] += n
-        free = self.cache.free_pages()
-        for g in range(n_groups):
-            if total[g] > free[g]:
-                raise PagesExhausted(total[g], free[g], g)
-        for e in entries:
-            self.cache.reserve(e.rid, len(e.tokens))
+        self.cache.reserve_many([e.rid for e in entries], [len(e.tokens) for e in entries])
 
     def build_context(self, entries: Sequence[StepEntry]):
         """Host side of a step: flatten the batch and describe it (pages must be reserved)."""
@@ -264,37 +254,14 @@ class ModelRunner:
         return g
 
     def _fill_graph_inputs(self, g: _DecodeGraph, entries: Sequence[StepEntry]) -> None:
-        n_groups = len(self.cache.groups)
         g.copied.synchronize()                     # the last copy out of the pinned buffer has finished
-        h, offs = g.host_np, g.offs
-        n = len(entries)
-        starts = [self.cache.num_tokens(e.rid) for e in entries]
-        tok, pos, ctxl, slot = (h[offs[i]: offs[i + 1]] for i in range(4))
-        tok[:] = 0
-        pos[:] = 0
-        ctxl[:] = 1                                 # padded rows: one key, in the scratch page
-        slot[:] = self.cache.max_requests
-        tok[:n] = [e.tokens[0] for e in entries]
-        pos[:n] = starts
-        ctxl[:n] = [s + 1 for s in starts]
-        slot[:n] = [self.cache.state_slot(e.rid) for e in entries]
-        for gi in range(n_groups):
-            scratch = self.pools.scratch_page(gi)
-            bt = h[offs[4 + gi]: offs[5 + gi]].reshape(g.rows, g.width)
-            bt[:] = scratch
-            for r, e in enumerate(entries):
-                t = self.cache.table(e.rid, gi)
-                bt[r, : len(t)] = t
-            if self.cache.groups[gi].kind != "full":
-                bt[bt < 0] = scratch       # pages a window has given back; no query reads them
-            sl = h[offs[4 + n_groups + gi]: offs[5 + n_groups + gi]]
-            sl[:] = scratch * self.page_size
-            sl[:n] = [self.cache.slot(e.rid, gi, s0) for e, s0 in zip(entries, starts)]
+        self.cache.fill_decode([e.rid for e in entries], [e.tokens[0] for e in entries], g.rows, g.width,
+                               [self.pools.scratch_page(gi) for gi in range(len(self.cache.groups))], g.host_np)
         g.packed.copy_(g.host, non_blocking=True)
         g.copied.record()
 
     def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        ctx_len = max(self.cache.num_tokens(e.rid) for e in entries) + 1
+        ctx_len = self.cache.max_num_tokens([e.rid for e in entries]) + 1
         g = self._graph_for(len(entries), ctx_len)
         self._fill_graph_inputs(g, entries)
         if g.graph is None:
@@ -325,8 +292,7 @@ class ModelRunner:
         self.reserve(entries)
         if self.use_graph and all(len(e.tokens) == 1 for e in entries):
             logits = self._graph_step(entries)
-            for e in entries:
-                self.cache.commit(e.rid, 1)
+            self.cache.commit_many([e.rid for e in entries], [1] * len(entries))
             self.steps_run += 1
             self.tokens_run += len(entries)
             return logits

@@ -129,11 +129,11 @@ def test_random_orders_of_requests(seed):
         elif op < 0.85 and live:
             rid = g.choice(list(live))
             n = g.choice([1, 1, 1, 2, 3, 7, 16, 33])
-            before = (m.free_pages(), [list(t) for t in m._requests[rid].tables])
+            before = (m.free_pages(), [m.table(rid, gi) for gi in range(len(groups))])
             try:
                 m.reserve(rid, n)
             except PagesExhausted:
-                assert (m.free_pages(), [list(t) for t in m._requests[rid].tables]) == before
+                assert (m.free_pages(), [m.table(rid, gi) for gi in range(len(groups))]) == before
                 victim = g.choice(list(live))
                 m.release(victim)
                 del live[victim]
@@ -150,3 +150,43 @@ def test_random_orders_of_requests(seed):
         m.release(rid)
     m.check()
     assert m.free_pages() == [40] * len(groups)
+
+
+def test_fill_decode_packs_what_the_tables_say():
+    """The packed inputs of a decode step: tokens, positions, lengths, state slots, block tables with
+    given-back pages and padding pointed at the scratch page, and the cache row of every new token."""
+    import numpy as np
+    groups = [FULL, WIN]
+    ps = 8
+    m = CacheManager(groups, page_size=ps, num_pages=[20, 9], max_requests=4)
+    lens = {"a": 45, "b": 3, "c": 16}
+    for rid, n in lens.items():
+        m.add(rid)
+        m.reserve(rid, n)
+        m.commit(rid, n)
+    rids = ["c", "a", "b"]
+    m.reserve_many(rids, [1, 1, 1])
+    rows, width, scratch = 4, 8, [20, 9]
+    out = np.full(4 * rows + 2 * rows * (width + 1), -7, dtype=np.int32)
+    m.fill_decode(rids, [11, 12, 13], rows, width, scratch, out)
+    tok, pos, ctxl, slot = (out[i * rows:(i + 1) * rows] for i in range(4))
+    assert list(tok) == [11, 12, 13, 0] and list(pos) == [16, 45, 3, 0]
+    assert list(ctxl) == [17, 46, 4, 1] and list(slot) == [m.state_slot(r) for r in rids] + [4]
+    for g in range(2):
+        bt = out[4 * rows + g * rows * width: 4 * rows + (g + 1) * rows * width].reshape(rows, width)
+        sl = out[4 * rows + 2 * rows * width + g * rows: 4 * rows + 2 * rows * width + (g + 1) * rows]
+        for r, rid in enumerate(rids):
+            t = m.table(rid, g)
+            want = [p if p >= 0 else scratch[g] for p in t] + [scratch[g]] * (width - len(t))
+            assert list(bt[r]) == want
+            assert sl[r] == m.slots(rid, g, lens[rid], 1)[0] == m.slot(rid, g, lens[rid])
+        assert list(bt[3]) == [scratch[g]] * width and sl[3] == scratch[g] * ps
+    assert any(p < 0 for p in m.table("a", 1)), "the window group gave pages of the long request back"
+    assert m.max_num_tokens(rids) == 45
+    m.commit_many(rids, [1, 1, 1])
+    assert [m.num_tokens(r) for r in rids] == [17, 46, 4]
+    m.check()
+    with pytest.raises(RuntimeError):
+        m.fill_decode(["a"], [1], rows, 3, scratch, out)          # a table of six pages does not fit three columns
+    with pytest.raises(RuntimeError):
+        m.fill_decode(["c", "a", "b", "c", "a"], [1] * 5, rows, width, scratch, out)   # more requests than rows
