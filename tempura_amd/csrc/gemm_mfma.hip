@@ -542,7 +542,8 @@ static int g_tune_splits = 0, g_tune_mid = 0;                    // mid = 1: 17.
 static int g_tune_order = 0;   // large products: 1 tiled kernel, plain block order; 2 tiled, XCD patches; 3 pipelined kernel
 
 // Defined in gemm_pipe.hip; 0 when it took the product, -1 when the sizes are not its own.
-int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s);
+int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+                   size_t scratch_floats, int tune_splits, hipStream_t s);
 
 extern "C" void tp_linear_tune_tile(int order) { g_tune_order = order; }
 
@@ -653,8 +654,8 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   } else {
     // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
     // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.
-    const bool pipe = g_tune_order ? g_tune_order == 3 : M > 256;
-    if (pipe && M > 128 && tp_linear_pipe(xb, wb, out, mode, M, N, K, s) == 0) {
+    const bool pipe = g_tune_order ? g_tune_order == 3 : M > 128;
+    if (pipe && M > 128 && tp_linear_pipe(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, s) == 0) {
       // taken by the pipelined kernel
     } else if (M > 128 || scratch == nullptr) {
       dim3 grid((N + 127) / 128, (M + 127) / 128);

@@ -21,6 +21,8 @@
 //  * the result leaves through LDS, so that every store covers whole cache lines.
 // One barrier per 64 of K.  Sizes: K % 64 == 0; any M and N (loads clamp to the last row, stores are
 // masked).  The sum over K runs in ascending order for every output element.
+#include <algorithm>
+
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -139,9 +141,12 @@ __device__ inline void half_step(f32x4_t (&acc)[8][4], const Frags& cur, Frags& 
   read_one<4>(f, aaddr, baddr); read_one<5>(f, aaddr, baddr); read_one<6>(f, aaddr, baddr); read_one<7>(f, aaddr, baddr); \
   read_one<8>(f, aaddr, baddr); read_one<9>(f, aaddr, baddr); read_one<10>(f, aaddr, baddr); read_one<11>(f, aaddr, baddr)
 
-// pm: row blocks of a patch (a power of two up to 8); a patch holds 32 blocks
+// pm: row blocks of a patch (a power of two up to 8); a patch holds 32 blocks.  blockIdx.y splits K:
+// with more than one split every block writes its float32 partial tile to `partial` [split, M, N]
+// and a second kernel adds the splits in ascending order and applies the epilogue.
 __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                        void* __restrict__ out, int mode, int M, int N, int K, int pm) {
+                                                        void* __restrict__ out, float* __restrict__ partial, int mode,
+                                                        int M, int N, int K, int pm) {
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE_BYTES];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -164,7 +169,14 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
   for (int i = 0; i < 8; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  const int KT = K / BK;
+  // this block's share of K, in tiles
+  const int kt_per = (K / BK + gridDim.y - 1) / gridDim.y;
+  const int kt_first = blockIdx.y * kt_per;
+  const int KT = min(K / BK, kt_first + kt_per) - kt_first;
+  if (gridDim.y > 1) {
+    mode = OUT_F32;
+    out = partial + (size_t)blockIdx.y * M * N;
+  }
   const int g = lane >> 4, c = lane & 15;
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
   // this lane's byte offset inside a 16-row group of a stage, for the first and second 32 of K
@@ -180,8 +192,8 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
     const int grow = i < 8 ? min(row, M - 1 - m0) : min(row, N - 1 - n0);
     voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
   }
-  const unsigned char* xk = (const unsigned char*)x + (size_t)m0 * K * 2;
-  const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2;
+  const unsigned char* xk = (const unsigned char*)x + ((size_t)m0 * K + (size_t)kt_first * BK) * 2;
+  const unsigned char* wk = (const unsigned char*)w + ((size_t)n0 * K + (size_t)kt_first * BK) * 2;
 #pragma unroll
   for (int p = 0; p < NS; ++p)
     if (p < KT) issue_stage(stages + p * STAGE_BYTES, xk + p * BK * 2, wk + p * BK * 2, voff, wave);
@@ -305,8 +317,14 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
 
 }  // namespace
 
-// Returns 0 when launched, -1 when the sizes are not this kernel's.
-int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, hipStream_t s) {
+// Defined in gemm_mfma.hip.
+__global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out, int mode,
+                                          int splits, int M, int N);
+
+// Returns 0 when launched, -1 when the sizes are not this kernel's.  `scratch` (optional) is room for
+// float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
+int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+                   size_t scratch_floats, int tune_splits, hipStream_t s) {
   if (K % BK != 0 || K < BK) return -1;
   if ((size_t)(BM - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;  // a lane's source offset is 32 bits
   if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
@@ -316,6 +334,23 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
   const long Q = (NB + 7) / 8, MS = (MB + pm - 1) / pm, QS = (Q + pq - 1) / pq;
   const long blocks = 8 * QS * MS * 32;
   if (blocks > 0x7fffffffL) return -1;
-  hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, w, out, mode, M, N, K, pm);
+  // splits: enough blocks for the 256 CUs, at least sixteen tiles of K each (measured: more splits than
+  // that cost more in partial sums than they gain)
+  int splits = 1;
+  if (scratch != nullptr) {
+    const int tiles = MB * NB, KT = K / BK;
+    splits = tune_splits > 0 ? tune_splits : (tiles >= 128 ? 1 : (256 + tiles - 1) / tiles);
+    splits = std::max(1, std::min(splits, std::min(16, KT / 16)));
+    while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
+    const int per = (KT + splits - 1) / splits;
+    splits = (KT + per - 1) / per;   // no split without a tile
+  }
+  hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks, splits), dim3(256), 0, s, x, w, out, scratch, mode, M, N, K,
+                     pm);
+  if (splits > 1) {
+    const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
+                       splits, M, N);
+  }
   return 0;
 }

@@ -226,10 +226,18 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
 
 
 def _splitk_scratch(x: torch.Tensor, m: int, n: int):
-    """Room for the partial sums of a bfloat16 product of 17..128 rows (its K is split over blocks)."""
-    if x.dtype != torch.bfloat16 or not (16 < m <= 128):
+    """Room for the partial sums of a bfloat16 product whose K is split over blocks: products of 17..128
+    rows, and larger ones with too few result tiles (256 x 128) to give every CU work."""
+    if x.dtype != torch.bfloat16 or m <= 16:
         return None, 0
-    count = min(16, max(1, -(-512 // (-(-n // 128) * -(-m // 64))))) * m * n
+    if m <= 128:
+        splits = min(16, max(1, -(-512 // (-(-n // 128) * -(-m // 64)))))
+    else:
+        tiles = -(-m // 256) * -(-n // 128)
+        if tiles >= 128:
+            return None, 0
+        splits = min(16, -(-256 // tiles))
+    count = splits * m * n
     return torch.empty((count,), dtype=torch.float32, device=x.device), count
 
 

@@ -189,7 +189,8 @@ def test_argmax_last_max_wins(m, vocab):
 @pytest.mark.parametrize("m,n,k", [(1, 16, 32), (1, 4096, 4096), (8, 200, 96), (16, 6144, 4096), (17, 48, 64),
                                    (33, 1000, 320), (48, 130, 2048), (64, 4096, 1024), (65, 128, 64),
                                    (200, 300, 96), (257, 384, 160), (512, 1024, 4096),
-                                   (300, 333, 192), (513, 130, 64), (700, 1024, 448), (1030, 264, 128), (2048, 128, 320)])
+                                   (300, 333, 192), (513, 130, 64), (700, 1024, 448), (1030, 264, 128), (2048, 128, 320),
+                                   (129, 256, 2048), (200, 4096, 4096), (260, 136, 3072)])
 def test_linear_mfma(m, n, k):
     """The matrix-core kernels (decode and prefill shapes) against float64, and against the general kernel."""
     ops = _ops()
@@ -307,7 +308,7 @@ def test_attention_window_edge(dtype, fast):
     _close(got, ref, 2e-5 if dtype == torch.float32 else 1.2e-2, "window edge")
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 192, 64), (8, 14336, 4096), (16, 320, 96), (40, 136, 160), (64, 1024, 2048), (300, 200, 128), (2048, 512, 256), (515, 328, 64)])
+@pytest.mark.parametrize("m,inter,k", [(1, 192, 64), (8, 14336, 4096), (16, 320, 96), (40, 136, 160), (64, 1024, 2048), (300, 200, 128), (2048, 512, 256), (515, 328, 64), (160, 256, 2048)])
 def test_linear_swiglu(m, inter, k):
     """The gated epilogue of the matrix-core products, on the interleaved gate/up layout."""
     ops = _ops()
