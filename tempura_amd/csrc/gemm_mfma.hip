@@ -654,8 +654,10 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   } else {
     // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
     // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.
-    const bool pipe = g_tune_order ? g_tune_order == 3 : M > 128;
-    if (pipe && M > 128 && tp_linear_pipe(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, s) == 0) {
+    // the pipelined kernel: from 129 rows on, and from 65 rows on when there are many column blocks
+    // (measured at 128 rows: N = 28,672 59 us against 77 us, the narrow products a few us slower)
+    const bool pipe = g_tune_order ? g_tune_order == 3 : (M > 128 || (M > 64 && N >= 16384));
+    if (pipe && tp_linear_pipe(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, s) == 0) {
       // taken by the pipelined kernel
     } else if (M > 128 || scratch == nullptr) {
       dim3 grid((N + 127) / 128, (M + 127) / 128);

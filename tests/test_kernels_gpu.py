@@ -190,7 +190,7 @@ def test_argmax_last_max_wins(m, vocab):
                                    (33, 1000, 320), (48, 130, 2048), (64, 4096, 1024), (65, 128, 64),
                                    (200, 300, 96), (257, 384, 160), (512, 1024, 4096),
                                    (300, 333, 192), (513, 130, 64), (700, 1024, 448), (1030, 264, 128), (2048, 128, 320),
-                                   (129, 256, 2048), (200, 4096, 4096), (260, 136, 3072)])
+                                   (129, 256, 2048), (200, 4096, 4096), (260, 136, 3072), (100, 16400, 128)])
 def test_linear_mfma(m, n, k):
     """The matrix-core kernels (decode and prefill shapes) against float64, and against the general kernel."""
     ops = _ops()
