@@ -31,8 +31,34 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ inline bf16x8_t frag_of(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// two floats to two bfloat16 (round to nearest even) with the hardware's packed conversion
 __device__ inline unsigned int pack_bf16(float a, float b) {
-  return (unsigned int)float_to_bf16(a).bits | ((unsigned int)float_to_bf16(b).bits << 16);
+  const f32x2_t f = {a, b};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(f, bf16x2_t));
+}
+
+// Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 with the row-swap instructions of gfx950
+// (no trip through LDS): v_permlane16_swap exchanges the odd 16-lane rows of its first operand with
+// the even rows of its second, v_permlane32_swap the upper half of the first with the lower half of
+// the second; with both operands equal beforehand, the two registers afterwards hold each lane's own
+// value and its partner's.  Written as assembly, with the wait states the instruction needs after a
+// vector write, because the compiler's builtin folds the following max/add of the two results away.
+__device__ inline void rows16_swap(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ inline void rows32_swap(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ inline float quad_rows_max(float x) {
+  float y = x;
+  rows16_swap(x, y);
+  x = fmaxf(x, y);
+  y = x;
+  rows32_swap(x, y);
+  return fmaxf(x, y);
 }
 
 struct AttnArgs {
@@ -46,6 +72,7 @@ struct AttnArgs {
   bf16_t* out;
   float* scratch;
   int n_heads, n_kv, page_size, window, num_splits;
+  int page_shift;   // log2(page_size), or -1
   float scale_log2;
 };
 
@@ -82,14 +109,13 @@ __device__ inline void attn_load(const AttnArgs& a, const int* __restrict__ tabl
 
 // One step of 32 keys starting at j0 for NQ query tiles, on fetched fragments.  qpos[nq] is the
 // absolute position of this lane's query column (keys above it are masked).  m/l/o are the
-// running statistics and output of each tile.
+// running statistics and output of each tile.  MASK false: the caller knows that every key of the
+// step is visible to every query of the wave (no comparison needed).
+// The softmax arithmetic, not the matrix core, bounds this step, so it is kept short: the scale is
+// folded into the exponent's FMA, and the running output is rescaled only when a maximum moved
+// (when none did the factor is exactly 1).
 template <int D, int NQ>
-__device__ inline void attn_compute(const AttnArgs& a, int j0, const KvFrags<D>& f, const bf16x8_t (&qf)[NQ][D / 32],
-                                    const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
-  const int lane = threadIdx.x & 63;
-  const int g = lane >> 4;
-  // scores: two 16-key tiles
-  f32x4_t s[NQ][2];
+__device__ inline void attn_scores(const bf16x8_t (&k)[2][D / 32], const bf16x8_t (&qf)[NQ][D / 32], f32x4_t (&s)[NQ][2]) {
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -97,53 +123,105 @@ __device__ inline void attn_compute(const AttnArgs& a, int j0, const KvFrags<D>&
       s[nq][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int dk = 0; dk < D / 32; ++dk)
-        s[nq][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[t][dk], qf[nq][dk], s[nq][t], 0, 0, 0);
+        s[nq][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k[t][dk], qf[nq][dk], s[nq][t], 0, 0, 0);
     }
+}
+
+// Softmax of one step's scores: probabilities as the next product's operand (pf), and the factor by
+// which the running sums shrink (alpha; `moved` false when no maximum of the wave moved: alpha is 1).
+template <int NQ, bool MASK>
+__device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const int (&qpos)[NQ],
+                                    float (&m)[NQ], float (&l)[NQ], bf16x8_t (&pf)[NQ], float (&alpha)[NQ], bool (&moved)[NQ]) {
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
     // this lane's keys: j0 + 8g + 4t + r
     float v[8];
     float mx = -INFINITY;
-    const int hi = qpos[nq];
-    const int lo = a.window > 0 ? hi - a.window + 1 : 0;
+    if (MASK) {
+      const int hi = qpos[nq];
+      const int lo = a.window > 0 ? hi - a.window + 1 : 0;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = j0 + 8 * g + 4 * t + r;
-        const float x = (key <= hi && key >= lo) ? s[nq][t][r] * a.scale_log2 : -INFINITY;
-        v[t * 4 + r] = x;
-        mx = fmaxf(mx, x);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m[nq], mx);
+        for (int r = 0; r < 4; ++r) {
+          const int key = j0 + 8 * g + 4 * t + r;
+          v[t * 4 + r] = (key <= hi && key >= lo) ? s[nq][t][r] : -INFINITY;
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[t * 4 + r] = s[nq][t][r];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mx = fmaxf(mx, v[i]);
+    mx = quad_rows_max(mx);
+    const float m_new = fmaxf(m[nq], mx * a.scale_log2);    // the scale is positive
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column with nothing visible yet
-    const float alpha = __builtin_amdgcn_exp2f(m[nq] - m_use);
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      v[i] = __builtin_amdgcn_exp2f(v[i] - m_use);
+      v[i] = __builtin_amdgcn_exp2f(fmaf(v[i], a.scale_log2, -m_use));
       sum += v[i];
     }
-    l[nq] = l[nq] * alpha + sum;  // per-lane partial sum; lanes of a column are added at the end
-    m[nq] = m_new;
     u32x4_t pk;
     pk[0] = pack_bf16(v[0], v[1]);
     pk[1] = pack_bf16(v[2], v[3]);
     pk[2] = pack_bf16(v[4], v[5]);
     pk[3] = pack_bf16(v[6], v[7]);
-    const bf16x8_t pf = frag_of(pk);
-#pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt) {
-      f32x4_t acc = o[nq][dt];
-      acc[0] *= alpha;
-      acc[1] *= alpha;
-      acc[2] *= alpha;
-      acc[3] *= alpha;
-      o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt], pf, acc, 0, 0, 0);
+    pf[nq] = frag_of(pk);
+    moved[nq] = __builtin_amdgcn_ballot_w64(m_new != m[nq]) != 0;
+    if (moved[nq]) {
+      alpha[nq] = __builtin_amdgcn_exp2f(m[nq] - m_use);
+      l[nq] = l[nq] * alpha[nq] + sum;  // per-lane partial sum; lanes of a column are added at the end
+      m[nq] = m_new;
+    } else {
+      alpha[nq] = 1.0f;
+      l[nq] += sum;
     }
   }
+}
+
+template <int D, int NQ>
+__device__ inline void attn_pv(const bf16x8_t (&vf)[D / 16], const bf16x8_t (&pf)[NQ], const float (&alpha)[NQ],
+                               const bool (&moved)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    if (moved[nq]) {
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) {
+        f32x4_t acc = o[nq][dt];
+        acc[0] *= alpha[nq];
+        acc[1] *= alpha[nq];
+        acc[2] *= alpha[nq];
+        acc[3] *= alpha[nq];
+        o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf[nq], acc, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf[nq], o[nq][dt], 0, 0, 0);
+    }
+  }
+}
+
+template <int D, int NQ, bool MASK>
+__device__ inline void attn_softmax_pv(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const bf16x8_t (&vf)[D / 16],
+                                       const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+  bf16x8_t pf[NQ];
+  float alpha[NQ];
+  bool moved[NQ];
+  attn_softmax<NQ, MASK>(a, j0, s, qpos, m, l, pf, alpha, moved);
+  attn_pv<D, NQ>(vf, pf, alpha, moved, o);
+}
+
+template <int D, int NQ, bool MASK = true>
+__device__ inline void attn_compute(const AttnArgs& a, int j0, const KvFrags<D>& f, const bf16x8_t (&qf)[NQ][D / 32],
+                                    const int (&qpos)[NQ], float (&m)[NQ], float (&l)[NQ], f32x4_t (&o)[NQ][D / 16]) {
+  f32x4_t s[NQ][2];
+  attn_scores<D, NQ>(f.k, qf, s);
+  attn_softmax_pv<D, NQ, MASK>(a, j0, s, f.v, qpos, m, l, o);
 }
 
 template <int D, int NQ>
@@ -210,6 +288,246 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int skip_
 #pragma unroll
       for (int dt = 0; dt < D / 16; ++dt) {
         // O^T tile: rows d = dt*16 + 4g + r
+        uint2 w;
+        w.x = pack_bf16(o[nq][dt][0] * inv, o[nq][dt][1] * inv);
+        w.y = pack_bf16(o[nq][dt][2] * inv, o[nq][dt][3] * inv);
+        *(uint2*)(orow + dt * 16 + 4 * g) = w;
+      }
+    }
+  }
+}
+
+// ---- prefill, keys and values through LDS ---------------------------------------------------
+// The four waves of a block (four heads of one kv group) need the same keys and values.  Here a
+// step's 32 keys and values are copied once per block into LDS by the direct global-to-LDS load,
+// three steps ahead of their use (a ring of four stages, one barrier per step), and every wave reads
+// its operand fragments from there: a quarter of the global load instructions, and none of their
+// latency in the way.  Head sizes 32, 64, 128 (a power-of-two number of 16-byte chunks per key row).
+// LDS layout of a stage: the key tile as 32 rows of D elements, chunk c of row r stored at
+// (c + f(r)) mod (D / 8) so that the 16 rows a quarter wave reads fall into different banks; the
+// value tile as D rows of 32 keys (64 bytes), chunk g of row d at g ^ ((d >> 2) & 3).
+#define GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define ATTN_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+template <int OFF>
+__device__ inline u32x4_t attn_lds_read(unsigned addr) {
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+
+template <int D, int NQ>
+__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, int skip_single) {
+  constexpr int C = D / 8;             // 16-byte chunks per key row
+  constexpr int SH = C == 16 ? 0 : (C == 8 ? 1 : 2);
+  constexpr int KI = D / 16;           // 1 KB loads per key tile (32 rows of 2 D bytes), and per value tile
+  constexpr int LP = 2 * KI / 4;       // loads per wave and step
+  constexpr int STAGE = 2 * KI * 1024;
+  constexpr int NS = 4;
+  static_assert(D == 32 || D == 64 || D == 128, "head size");
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = lane >> 4, c = lane & 15;
+  const int r = blockIdx.z;
+  const int q_start = a.cu_seqlens[r];
+  const int q_len = a.cu_seqlens[r + 1] - q_start;
+  if (q_len <= 0 || (skip_single && q_len == 1)) return;
+  const int q0 = blockIdx.x * 16 * NQ;
+  if (q0 >= q_len) return;
+  const int group = a.n_heads / a.n_kv;
+  const int hblocks = (group + 3) / 4;
+  const int kvh = blockIdx.y / hblocks;
+  const int hin = (blockIdx.y % hblocks) * 4 + wave;
+  const bool active = hin < group;     // a wave without a head still loads and waits with the others
+  const int head = kvh * group + min(hin, group - 1);
+  const int ctx = a.context_lens[r];
+  const int pos0 = ctx - q_len;
+  const int* table = a.block_tables + (size_t)r * a.table_width;
+  const int ps = a.page_size;
+
+  bf16x8_t qf[NQ][D / 32];
+  int qpos[NQ];
+  float m[NQ], l[NQ];
+  f32x4_t o[NQ][D / 16];
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    const int qi = min(q0 + nq * 16 + c, q_len - 1);
+    qpos[nq] = pos0 + qi;
+    const bf16_t* qr = a.q + ((size_t)(q_start + qi) * a.n_heads + head) * D + g * 8;
+#pragma unroll
+    for (int dk = 0; dk < D / 32; ++dk) qf[nq][dk] = frag_of(*(const u32x4_t*)(qr + dk * 32));
+    m[nq] = -INFINITY;
+    l[nq] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt) o[nq][dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  }
+  const int last_pos = pos0 + min(q0 + 16 * NQ, q_len) - 1;
+  int first = 0;
+  if (a.window > 0) first = max(0, pos0 + q0 - a.window + 1) & ~31;
+  const int nsteps = (last_pos - first) / 32 + 1;
+  const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this block
+
+  // what this lane fetches in each of its loads of a step: load t = wave + 4 i; t < KI is a piece of
+  // the key tile (64 chunk slots: 64 / C whole rows, all in one page), else of the value tile (16 rows
+  // of four chunks of eight keys, up to four pages).  Page numbers are read with wave-uniform (scalar)
+  // loads: a vector load here would have to wait for every outstanding copy into LDS.
+  const int psh = a.page_shift, pmask = ps - 1;
+  // the block table through the constant address space: uniform loads from it are scalar loads
+  const __attribute__((address_space(4))) int* ctab = (const __attribute__((address_space(4))) int*)(uintptr_t)table;
+  int koff_row[LP], boff[LP];
+#pragma unroll
+  for (int i = 0; i < LP; ++i) {
+    const int t = wave + 4 * i;
+    if (t < KI) {
+      const int slot = 64 * t + lane;
+      const int row = slot / C, pc = slot % C;
+      const int f = ((((row >> 3) << 2) | (row & 3)) >> SH);
+      koff_row[i] = row;
+      boff[i] = ((pc - f) & (C - 1)) * 16;
+    } else {
+      const int d = 16 * (t - KI) + (lane >> 2);
+      koff_row[i] = (lane & 3) ^ ((d >> 2) & 3);   // which group of eight keys
+      boff[i] = d;                                  // the value row
+    }
+  }
+  // the pages of the four groups of eight keys of a step (clamped to the last key that exists); a key
+  // load's rows lie in one of these groups, or past the end in the last key's page
+  auto pages_of = [&](int step, int (&pg)[4]) {
+    const int j0 = first + step * 32;
+#pragma unroll
+    for (int gg = 0; gg < 4; ++gg) pg[gg] = ctab[min(j0 + 8 * gg, (ctx - 1) & ~7) >> psh];
+  };
+  auto issue = [&](int step, int stage, const int (&pg)[4]) {
+    const int j0 = first + step * 32;
+    unsigned char* buf = stages + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < LP; ++i) {
+      const int t = wave + 4 * i;
+      const unsigned char* src;
+      if (t < KI) {
+        const int gr = ((64 * t) / C) >> 3;                  // the group of eight keys this load lies in
+        const int page = gr == 0 ? pg[0] : (gr == 1 ? pg[1] : (gr == 2 ? pg[2] : pg[3]));
+        const int key = min(j0 + koff_row[i], ctx - 1);
+        src = (const unsigned char*)(a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + (key & pmask)) * D) + boff[i];
+      } else {
+        const int gg = koff_row[i];
+        const int kb = min(j0 + 8 * gg, (ctx - 1) & ~7);
+        const int page = gg == 0 ? pg[0] : (gg == 1 ? pg[1] : (gg == 2 ? pg[2] : pg[3]));
+        src = (const unsigned char*)(a.v_cache + ((size_t)(page * a.n_kv + kvh) * D + boff[i]) * ps + (kb & pmask));
+      }
+      __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+    }
+  };
+  // this lane's read addresses inside a stage
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
+  unsigned kaddr[2][D / 32];
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2) {
+    const int row = 8 * (c >> 2) + 4 * t2 + (c & 3);
+#pragma unroll
+    for (int dk = 0; dk < D / 32; ++dk) kaddr[t2][dk] = (row * C + ((dk * 4 + g + (c >> SH)) & (C - 1))) * 16;
+  }
+  const unsigned vaddr = KI * 1024 + (c * 4 + (g ^ ((c >> 2) & 3))) * 16;
+
+  int pg[4];          // page numbers of the step that is issued next, fetched one step ahead (scalar loads)
+#pragma unroll
+  for (int p = 0; p < NS; ++p)
+    if (p < nsteps) {
+      pages_of(p, pg);
+      issue(p, p, pg);
+    }
+  if (NS < nsteps) pages_of(NS, pg);
+  // The scores of step s + 1 are multiplied while the softmax of step s runs on the vector ALU (two
+  // independent instruction streams for the scheduler to interleave); so step s reads the values of
+  // stage s and the keys of stage s + 1, and a stage is free again one step later than it would be.
+  auto read_keys = [&](unsigned base, bf16x8_t (&kf)[2][D / 32]) {
+    u32x4_t kk[2][D / 32];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int dk = 0; dk < D / 32; ++dk) kk[t2][dk] = attn_lds_read<0>(base + kaddr[t2][dk]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int dk = 0; dk < D / 32; ++dk) {
+        asm volatile("" : "+v"(kk[t2][dk]));
+        kf[t2][dk] = frag_of(kk[t2][dk]);
+      }
+  };
+  f32x4_t sc[NQ][2];
+  {
+    const int behind = min(NS - 1, nsteps - 1);   // steps in flight behind the first
+    if (behind >= 3) ATTN_WAIT_VM(3 * LP); else if (behind == 2) ATTN_WAIT_VM(2 * LP); else if (behind == 1) ATTN_WAIT_VM(LP); else ATTN_WAIT_VM(0);
+    __builtin_amdgcn_s_barrier();
+    bf16x8_t kf[2][D / 32];
+    read_keys(lds0, kf);
+    attn_scores<D, NQ>(kf, qf, sc);
+  }
+  int stage = 0;
+  for (int s = 0; s < nsteps; ++s) {
+    const int nstage = stage + 1 == NS ? 0 : stage + 1;
+    // step s + 1 has landed for this wave (later steps may stay in flight), then for all; every wave
+    // is done with the stage of step s - 1
+    const int ahead = min(NS - 3, nsteps - 2 - s);
+    if (ahead >= 1) ATTN_WAIT_VM(LP); else ATTN_WAIT_VM(0);
+    __builtin_amdgcn_s_barrier();
+    if (s >= 1 && s + NS - 1 < nsteps) {
+      issue(s + NS - 1, stage == 0 ? NS - 1 : stage - 1, pg);
+      if (s + NS < nsteps) pages_of(s + NS, pg);
+    }
+    const unsigned base = lds0 + stage * STAGE;
+    // the keys of the following stage are multiplied into the next step's scores before this step's
+    // softmax runs on the vector ALU
+    f32x4_t sn[NQ][2];
+    if (s + 1 < nsteps) {
+      bf16x8_t kf[2][D / 32];
+      read_keys(lds0 + nstage * STAGE, kf);
+      attn_scores<D, NQ>(kf, qf, sn);
+    }
+    // the value fragments travel while the softmax runs
+    u32x4_t vv[D / 16];
+#define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<dt * 1024>(base + vaddr)
+    ATTN_RV(0); ATTN_RV(1); ATTN_RV(2); ATTN_RV(3); ATTN_RV(4); ATTN_RV(5); ATTN_RV(6); ATTN_RV(7);
+#undef ATTN_RV
+    bf16x8_t pf[NQ];
+    float alpha[NQ];
+    bool moved[NQ];
+    const int j0 = first + s * 32;
+    if (j0 + 31 <= qpos_min && (a.window <= 0 || j0 >= last_pos - a.window + 1))
+      attn_softmax<NQ, false>(a, j0, sc, qpos, m, l, pf, alpha, moved);
+    else
+      attn_softmax<NQ, true>(a, j0, sc, qpos, m, l, pf, alpha, moved);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    bf16x8_t vf[D / 16];
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt) {
+      asm volatile("" : "+v"(vv[dt]));
+      vf[dt] = frag_of(vv[dt]);
+    }
+    attn_pv<D, NQ>(vf, pf, alpha, moved, o);
+    if (s + 1 < nsteps) {
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq) {
+        sc[nq][0] = sn[nq][0];
+        sc[nq][1] = sn[nq][1];
+      }
+    }
+    stage = nstage;
+  }
+  if (!active) return;
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    float lt = l[nq];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    const float inv = 1.0f / lt;
+    const int qi = q0 + nq * 16 + c;
+    if (qi < q_len) {
+      bf16_t* orow = a.out + ((size_t)(q_start + qi) * a.n_heads + head) * D;
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) {
         uint2 w;
         w.x = pack_bf16(o[nq][dt][0] * inv, o[nq][dt][1] * inv);
         w.y = pack_bf16(o[nq][dt][2] * inv, o[nq][dt][3] * inv);
@@ -338,6 +656,9 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 }
 
 // ---- dispatch ------------------------------------------------------------------------------
+static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave
+extern "C" void tp_attention_tune(int v) { g_attn_tune = v; }
+
 template <int D>
 static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_single, hipStream_t s) {
   const int group = a.n_heads / a.n_kv;
@@ -354,6 +675,13 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
   if (has_multi) {
     constexpr int NQ = (D <= 128) ? 2 : 1;
     const dim3 grid((max_q_len + 16 * NQ - 1) / (16 * NQ), a.n_kv * ((group + 3) / 4), n_req);
+    if constexpr (D == 32 || D == 64 || D == 128) {
+      // (a key load covers 512 / D rows, which must lie in one page)
+      if (g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<D, NQ>), grid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0);
+        return 0;
+      }
+    }
     hipLaunchKernelGGL((attn_prefill_kernel<D, NQ>), grid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0);
   }
   return 0;
@@ -380,6 +708,9 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
   a.n_heads = n_heads;
   a.n_kv = n_kv;
   a.page_size = page_size;
+  a.page_shift = -1;
+  for (int b = 0; b < 30; ++b)
+    if ((1 << b) == page_size) a.page_shift = b;
   a.window = window;
   a.num_splits = num_splits;
   a.scale_log2 = scale * 1.4426950408889634f;
