@@ -141,6 +141,8 @@ __device__ inline void half_step(f32x4_t (&acc)[8][4], const Frags& cur, Frags& 
   read_one<4>(f, aaddr, baddr); read_one<5>(f, aaddr, baddr); read_one<6>(f, aaddr, baddr); read_one<7>(f, aaddr, baddr); \
   read_one<8>(f, aaddr, baddr); read_one<9>(f, aaddr, baddr); read_one<10>(f, aaddr, baddr); read_one<11>(f, aaddr, baddr)
 
+}  // namespace
+
 // pm: row blocks of a patch (a power of two up to 8); a patch holds 32 blocks.  blockIdx.y splits K:
 // with more than one split every block writes its float32 partial tile to `partial` [split, M, N]
 // and a second kernel adds the splits in ascending order and applies the epilogue.
@@ -314,8 +316,6 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
     }
   }
 }
-
-}  // namespace
 
 // Defined in gemm_mfma.hip.
 __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out, int mode,
