@@ -288,6 +288,10 @@ int cc_truncate(void* h, int req, int num_tokens) {
   Request* r = c->live(req);
   if (!r) return -1;
   if (num_tokens > r->num_tokens || num_tokens < 0) return fail("truncate beyond what is cached");
+  // a window group has given pages back for good: it cannot go back to where a query would need them
+  for (int g = 0; g < c->n_groups(); ++g)
+    if (num_tokens < r->num_tokens && c->first_needed(g, num_tokens) < r->first_live[g])
+      return fail("group %d has given back pages that the truncated request would need", g);
   const int keep = (num_tokens + c->page_size - 1) / c->page_size;
   for (int g = 0; g < c->n_groups(); ++g) {
     std::vector<int>& table = r->tables[g];
