@@ -112,7 +112,7 @@ extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void*
 // each q and k head turns by the angle pos * inv_freq[d]: the product is formed in float64 and
 // reduced to [0, 2 pi) there, sine and cosine of the small rest are float32.  q goes to
 // q_out, rotated k and raw v go to the cache place `slots[t]` (page * page_size + offset) of
-// the paged pools: keys as [page, kv_head, page_size, head_dim], values TRANSPOSED as
+// the paged pools (qkv may be [splits, n, row] partial sums of the projection, added here): keys as [page, kv_head, page_size, head_dim], values TRANSPOSED as
 // [page, kv_head, head_dim, page_size] so that the attention kernels read eight consecutive
 // keys of one value element with one 16-byte load.  With slots == nullptr only q is produced
 // (the row then holds q heads only).
@@ -124,7 +124,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
                                      const double* __restrict__ inv_freq, int rotary_dim, float factor,
                                      int n_heads, int n_kv, int head_dim, TQ* __restrict__ q_out,
                                      TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size,
-                                     int pairs, int heads_per_block) {
+                                     int pairs, int heads_per_block, int splits, size_t split_stride) {
   const int t = blockIdx.x;
   const int hl = threadIdx.x / pairs, d = threadIdx.x % pairs;   // pairs = head_dim / 2
   const int h = blockIdx.y * heads_per_block + hl;
@@ -141,7 +141,23 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
     i0 = rotary_dim + 2 * (d - half);
     i1 = i0 + 1;
   }
-  float y0 = row[i0], y1 = row[i1];
+  // (splits > 1: the rows are the partial sums of a product whose K was split; added in ascending order)
+  float y0 = 0.f, y1 = 0.f;
+  {
+    float p0[16], p1[16];   // (all loads in flight before the first sum; splits <= 16)
+#pragma unroll
+    for (int sp = 0; sp < 16; ++sp)
+      if (sp < splits) {
+        p0[sp] = row[(size_t)sp * split_stride + i0];
+        p1[sp] = row[(size_t)sp * split_stride + i1];
+      }
+#pragma unroll
+    for (int sp = 0; sp < 16; ++sp)
+      if (sp < splits) {
+        y0 += p0[sp];
+        y1 += p1[sp];
+      }
+  }
   size_t page = 0, off = 0;
   if (slots) {
     const int slot = slots[t];
@@ -177,8 +193,10 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
 extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* positions, const int* slots,
                                 const double* inv_freq, int rotary_dim, float factor, int n, int n_heads,
                                 int n_kv, int head_dim, void* q_out, int q_dt, void* k_cache, void* v_cache,
-                                int cache_dt, int page_size, hipStream_t s) {
+                                int cache_dt, int page_size, int splits, hipStream_t s) {
   TP_REQUIRE(n >= 0 && n_heads > 0 && n_kv >= 0 && head_dim > 0, "rope_kv_write: bad sizes");
+  TP_REQUIRE(splits >= 1 && splits <= 16, "rope_kv_write: bad number of partial sums");
+  const size_t split_stride = (size_t)n * row_stride;   // qkv is [splits, n, row_stride]
   TP_REQUIRE(head_dim % 2 == 0 && head_dim <= 1024, "rope_kv_write: head_dim %d must be even and <= 1024", head_dim);
   TP_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim,
              "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, head_dim);
@@ -195,7 +213,7 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
 #define LAUNCH(TQ, TC)                                                                                    \
   hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), grid, dim3(threads), 0, s, qkv, row_stride, positions, \
                      slots, inv_freq, rotary_dim, factor, n_heads, n_kv, head_dim, (TQ*)q_out, (TC*)k_cache, \
-                     (TC*)v_cache, page_size, pairs, hpb)
+                     (TC*)v_cache, page_size, pairs, hpb, splits, split_stride)
   if (q_dt == TP_F32 && cache_dt == TP_F32)
     LAUNCH(float, float);
   else if (q_dt == TP_BF16 && cache_dt == TP_BF16)

@@ -143,7 +143,8 @@ static void launch_generic(const void* x, const void* w, void* out, int M, int N
 // not its own (the general kernel then runs), >0 on error.
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
                    float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
-                   const void* post_w, void* post_xg, float* post_ss, int layout, hipStream_t s);
+                   const void* post_w, void* post_xg, float* post_ss, int layout, int defer_reduce, int* splits_out,
+                   hipStream_t s);
 
 // `scratch` (optional, `scratch_floats` float32): room for split-K partial sums of mid-sized products.
 //
@@ -155,10 +156,15 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
 //
 // `layout` (bfloat16, at most 16 rows): bit 0, x is k-blocked [K / 8, M, 8] instead of [M, K]; bit 1, the
 // gated output (accumulate == 2) is written k-blocked [N / 16, M, 8] for a product that reads it so.
+//
+// `defer_reduce` (products of 17..128 rows whose K is split over blocks): the partial sums stay in `scratch`
+// as [*splits_out, M, N] float32 and `out` is not touched; the caller's next kernel adds them (ascending).
+// *splits_out == 1 means that the product wrote `out` itself.
 extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
                                int N, int K, int allow_mfma, float* scratch, size_t scratch_floats,
                                const float* pre_ss, int pre_count, float pre_eps, const void* post_w, void* post_xg,
-                               float* post_ss, int layout, hipStream_t s) {
+                               float* post_ss, int layout, int defer_reduce, int* splits_out, hipStream_t s) {
+  if (splits_out) *splits_out = 1;
   TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(accumulate != 1 || out_dt == TP_F32, "linear: accumulating output must be float32");
   const bool split_norm = pre_ss != nullptr || post_w != nullptr || layout != 0;
@@ -174,7 +180,7 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   if (accumulate == 2) {  // gated-SiLU epilogue: only the matrix-core kernels have it
     TP_REQUIRE(in_dt == TP_BF16 && allow_mfma, "linear: the gated epilogue needs bfloat16 operands");
     const int r = tp_linear_mfma(x, w, out, out_dt, 2, M, N, K, scratch, scratch_floats, pre_ss, pre_count, pre_eps,
-                                 nullptr, nullptr, nullptr, layout, s);
+                                 nullptr, nullptr, nullptr, layout, 0, nullptr, s);
     TP_REQUIRE(r >= 0, "linear: sizes M=%d N=%d K=%d do not fit the gated epilogue", M, N, K);
     return r;
   }
@@ -182,7 +188,7 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   if (M == 0) return 0;
   if (in_dt == TP_BF16 && allow_mfma) {
     const int r = tp_linear_mfma(x, w, out, out_dt, accumulate, M, N, K, scratch, scratch_floats, pre_ss, pre_count,
-                                 pre_eps, post_w, post_xg, post_ss, layout, s);
+                                 pre_eps, post_w, post_xg, post_ss, layout, defer_reduce, splits_out, s);
     if (r >= 0) return r;
   }
   TP_REQUIRE(!split_norm, "linear: sizes M=%d N=%d K=%d do not fit the split norm or the k-blocked layout", M, N, K);
@@ -208,5 +214,5 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
 extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
                          int N, int K, int allow_mfma, float* scratch, size_t scratch_floats, hipStream_t s) {
   return tp_linear_fused(x, w, in_dt, out, out_dt, accumulate, M, N, K, allow_mfma, scratch, scratch_floats, nullptr, 0,
-                         0.f, nullptr, nullptr, nullptr, 0, s);
+                         0.f, nullptr, nullptr, nullptr, 0, 0, nullptr, s);
 }

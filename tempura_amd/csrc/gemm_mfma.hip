@@ -533,6 +533,67 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
   store_out(out, mode, idx, v);
 }
 
+// Adds the K splits of `partial` [splits, M, N] (ascending) into the float32 residual rows h [M, N] and
+// writes the root-mean-square norm of the updated rows: out = h / sqrt(mean(h^2) + eps) * w.  One block
+// per row; takes the place of the reduction kernel and the norm kernel that would follow it.
+// Each thread owns four neighbouring columns (N % 4 == 0); all its loads are issued before the first sum.
+template <typename TO>
+__global__ __launch_bounds__(1024) void splitk_add_rmsnorm_kernel(const float* __restrict__ partial, int splits,
+                                                                   float* __restrict__ h, const float* __restrict__ w,
+                                                                   float eps, TO* __restrict__ out, int M, int N) {
+  __shared__ float red[32];
+  const int m = blockIdx.x;
+  const size_t total = (size_t)M * N;
+  float* hr = h + (size_t)m * N;
+  constexpr int MAXC = 4;                       // column groups per thread: N <= 4 * 1024 * MAXC
+  f32x4_t acc[MAXC];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int n = (threadIdx.x + i * 1024) * 4;
+    acc[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    if (n < N) {
+      f32x4_t p[16];
+#pragma unroll
+      for (int s = 0; s < 16; ++s)
+        if (s < splits) p[s] = *(const f32x4_t*)(partial + (size_t)s * total + (size_t)m * N + n);
+      const f32x4_t base = *(const f32x4_t*)(hr + n);
+      f32x4_t add = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 16; ++s)
+        if (s < splits) add += p[s];
+      acc[i] = base + add;
+      *(f32x4_t*)(hr + n) = acc[i];
+      ss += acc[i][0] * acc[i][0] + acc[i][1] * acc[i][1] + acc[i][2] * acc[i][2] + acc[i][3] * acc[i][3];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float scale = rsqrtf(ss / (float)N + eps);
+#pragma unroll
+  for (int i = 0; i < MAXC; ++i) {
+    const int n = (threadIdx.x + i * 1024) * 4;
+    if (n < N) {
+      const f32x4_t wv = *(const f32x4_t*)(w + n);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) from_float(out + (size_t)m * N + n + e, acc[i][e] * scale * wv[e]);
+    }
+  }
+}
+
+extern "C" int tp_splitk_add_rmsnorm(const float* partial, int splits, float* h, const float* w, float eps, void* out,
+                                     int out_dt, int M, int N, hipStream_t s) {
+  TP_REQUIRE(M > 0 && N > 0 && splits >= 1 && splits <= 16, "splitk_add_rmsnorm: bad sizes");
+  TP_REQUIRE(N % 4 == 0 && N <= 16384, "splitk_add_rmsnorm: width %d must be a multiple of 4, at most 16384", N);
+  if (out_dt == TP_BF16)
+    hipLaunchKernelGGL(splitk_add_rmsnorm_kernel<bf16_t>, dim3(M), dim3(1024), 0, s, partial, splits, h, w, eps, (bf16_t*)out, M, N);
+  else if (out_dt == TP_F32)
+    hipLaunchKernelGGL(splitk_add_rmsnorm_kernel<float>, dim3(M), dim3(1024), 0, s, partial, splits, h, w, eps, (float*)out, M, N);
+  else
+    TP_REQUIRE(false, "splitk_add_rmsnorm: unknown dtype %d", out_dt);
+  TP_CHECK_LAUNCH("splitk_add_rmsnorm");
+  return 0;
+}
+
 // In the skinny kernel x is the second operand, so the result lane holds weight rows
 // (l / 16) * 4 + r and activation row l % 16; see the index arithmetic there.
 
@@ -628,7 +689,9 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
 // pre_ss / post_w: the split norm (RowScale / NormPrep above), at most 16 rows; nullptr without.
 int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accumulate, int M, int N, int K,
                    float* scratch, size_t scratch_floats, const float* pre_ss, int pre_count, float pre_eps,
-                   const void* post_w, void* post_xg, float* post_ss, int layout, hipStream_t s) {
+                   const void* post_w, void* post_xg, float* post_ss, int layout, int defer_reduce, int* splits_out,
+                   hipStream_t s) {
+  if (splits_out) *splits_out = 1;
   if (K % 32 != 0) return -1;
   if (layout != 0 && M > 16) return -1;
   if ((layout & OUT_KBLOCKED) && accumulate != 2) return -1;
@@ -684,7 +747,9 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
         hipLaunchKernelGGL((gemm_tiled_mfma_kernel<64, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0);
       else
         hipLaunchKernelGGL((gemm_tiled_mfma_kernel<32, 2, 4>), grid, dim3(256), 0, s, xb, wb, out, scratch, mode, M, N, K, 0);
-      if (splits > 1) {
+      if (splits > 1 && defer_reduce && splits_out != nullptr && mode != OUT_SWIGLU) {
+        *splits_out = splits;   // the caller's next kernel adds the partial sums [splits, M, N] in `scratch`
+      } else if (splits > 1) {
         const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out,
                            mode, splits, M, N);

@@ -184,11 +184,27 @@ class KBlocked:
         return self.data.permute(1, 0, 2).reshape(self.rows, self.width).contiguous()
 
 
+class Partials:
+    """The float32 partial sums [splits, m, n] of a product whose K was split over blocks, not yet added:
+    the kernel that consumes the rows adds them (in ascending order), which saves the reduction kernel.
+    Made by ``linear(..., partial_ok=True)``, taken by ``rope_kv_write``."""
+    __slots__ = ("data",)
+
+    def __init__(self, data):
+        self.data = data
+
+    @property
+    def shape(self):
+        return tuple(self.data.shape[1:])
+
+
 def split_norm_ok(m: int, width: int, dtype: torch.dtype) -> bool:
-    """Whether a norm over ``width`` columns of ``m`` rows can be split over the two products around it."""
+    """Whether the product before a norm over ``width`` columns of ``m`` rows can carry it (``linear`` with
+    ``next_norm``): up to 16 rows the two products around the norm share it, up to 128 rows the kernel
+    that adds the product's partial sums into the residual stream also norms the rows."""
     if _backend is not None:
         return _backend.split_norm_ok(m, width, dtype)
-    return allow_mfma and dtype == torch.bfloat16 and 0 < m <= 16 and width % 32 == 0
+    return allow_mfma and dtype == torch.bfloat16 and 0 < m <= 128 and width % 32 == 0
 
 
 def _pre_args(x):
@@ -221,7 +237,7 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     scratch, nscratch = _splitk_scratch(x, m, n)
     _call("tp_linear_fused", _ptr(x), _ptr(w), _BF16, _ptr(out.data if blocked_out else out), _BF16, 2, m, n, k, 1,
           _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), 2 if blocked_out else 0,
-          _stream())
+          0, _ptr(None), _stream())
     return out
 
 
@@ -241,11 +257,15 @@ def _splitk_scratch(x: torch.Tensor, m: int, n: int):
     return torch.empty((count,), dtype=torch.float32, device=x.device), count
 
 
-def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.Tensor] = None, next_norm=None):
-    """x [m, k] (or ``Prenormed``) @ w[n, k]^T -> out_dtype [m, n]; with ``residual`` (float32 [m, n]) the
-    product is added into it in place and it is returned.  With ``next_norm`` = (float32 weight [n], eps)
-    (needs ``residual``) the result is the pair (residual, ``Prenormed`` rows of the updated residual), or
-    (residual, None) when the sizes do not allow it and the norm has to run on its own."""
+def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.Tensor] = None, next_norm=None,
+           partial_ok: bool = False):
+    """x [m, k] (or ``Prenormed`` / ``KBlocked``) @ w[n, k]^T -> out_dtype [m, n]; with ``residual`` (float32
+    [m, n]) the product is added into it in place and it is returned.
+    With ``next_norm`` = (float32 weight [n], eps) (needs ``residual``) the result is the pair (residual, rows
+    for the part behind that norm): ``Prenormed`` rows up to 16 rows of bfloat16, the normed rows themselves
+    up to 128 rows when the product's K was split (one kernel adds the partial sums into the residual and norms
+    it), or None when the norm has to run on its own.
+    With ``partial_ok`` (float32 output, no residual) the result may be ``Partials``."""
     if _backend is not None:
         if next_norm is not None:
             return _backend.linear(x, w, out_dtype, residual, next_norm)
@@ -272,7 +292,7 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
     else:
         out, acc = torch.empty((m, n), dtype=out_dtype, device=x.device), 0
     post, handed = (_ptr(None), _ptr(None), _ptr(None)), None
-    if next_norm is not None and split_norm_ok(m, n, x.dtype) and k % 32 == 0:
+    if next_norm is not None and split_norm_ok(m, n, x.dtype) and k % 32 == 0 and m <= 16:
         weight, eps = next_norm
         _dev_ok(weight)
         _need(residual is not None, "linear: next_norm needs a residual")
@@ -281,22 +301,42 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
                            torch.empty(((n + 15) // 16, 16), dtype=torch.float32, device=x.device), eps)
         post = (_ptr(weight), _ptr(handed.x), _ptr(handed.ss))
     scratch, nscratch = _splitk_scratch(x, m, n) if allow_mfma else (None, 0)
+    # 17..128 rows: the partial sums of a split K may stay unadded for the kernel that consumes the rows
+    defer = scratch is not None and 16 < m <= 128 and layout == 0 and \
+        ((next_norm is not None and residual is not None and split_norm_ok(m, n, x.dtype) and n % 4 == 0 and n <= 16384) or
+         (partial_ok and residual is None and out_dtype == torch.float32))
+    splits = ctypes.c_int(1)
     _call("tp_linear_fused", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
-          ctypes.c_size_t(nscratch), *pre, *post, layout, _stream())
+          ctypes.c_size_t(nscratch), *pre, *post, layout, int(defer), ctypes.byref(splits), _stream())
+    if defer and splits.value > 1:
+        if next_norm is None:
+            return Partials(scratch[: splits.value * m * n].view(splits.value, m, n))
+        weight, eps = next_norm
+        _dev_ok(weight)
+        _need(weight.dtype == torch.float32 and weight.numel() == n, "linear: norm weight must be float32 [n]")
+        normed = torch.empty((m, n), dtype=x.dtype, device=x.device)
+        _call("tp_splitk_add_rmsnorm", _ptr(scratch), splits.value, _ptr(residual), _ptr(weight), ctypes.c_float(eps),
+              _ptr(normed), _dt(normed), m, n, _stream())
+        return out, normed
     return out if next_norm is None else (out, handed)
 
 
-def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
+def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
                   inv_freq: Optional[torch.Tensor], rotary_dim: int, factor: float, num_heads: int,
                   num_kv_heads: int, head_dim: int, k_cache: Optional[torch.Tensor],
                   v_cache: Optional[torch.Tensor], q_dtype: torch.dtype) -> torch.Tensor:
-    """Rotate q and k of float32 rows [n, (heads + 2 kv_heads) * head_dim], store k and v into the
-    cache rows ``slots`` and return q as q_dtype [n, heads, head_dim].  With ``slots`` None the rows
-    hold q only and nothing is stored."""
+    """Rotate q and k of float32 rows [n, (heads + 2 kv_heads) * head_dim] (or the ``Partials`` of the
+    projection that makes them), store k and v into the cache rows ``slots`` and return q as q_dtype
+    [n, heads, head_dim].  With ``slots`` None the rows hold q only and nothing is stored."""
     if _backend is not None:
         return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,
                                       num_kv_heads, head_dim, k_cache, v_cache, q_dtype)
-    _dev_ok(qkv, positions, slots, inv_freq, k_cache, v_cache)
+    splits = 1
+    if isinstance(qkv, Partials):
+        splits, qkv = qkv.data.shape[0], qkv.data.view(-1, qkv.data.shape[2])[: qkv.data.shape[1]]
+        _need(qkv.is_contiguous() or splits == 1, "rope_kv_write: malformed partial sums")
+    _dev_ok(positions, slots, inv_freq, k_cache, v_cache)
+    _need(qkv.is_cuda, "operand is not on the GPU")
     _need(qkv.dtype == torch.float32 and qkv.dim() == 2, "rope_kv_write: rows must be float32 [n, width]")
     n = qkv.shape[0]
     width = (num_heads + (2 * num_kv_heads if slots is not None else 0)) * head_dim
@@ -317,7 +357,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[to
     q = torch.empty((n, num_heads, head_dim), dtype=q_dtype, device=qkv.device)
     _call("tp_rope_kv_write", _ptr(qkv), qkv.shape[1], _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
           ctypes.c_float(factor), n, num_heads, num_kv_heads, head_dim, _ptr(q), _dtcode(q_dtype),
-          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, _stream())
+          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, splits, _stream())
     return q
 
 

@@ -62,11 +62,12 @@ class PagedAttention(Mixer):
 
     def forward(self, x, ctx, cache, residual, next_norm=None):
         rot = self.position.rotary()
+        # (with a rotary position the next kernel may add the projection's partial sums itself)
         if cache.writes:
-            qkv = ops.linear(x, self.wqkv, torch.float32)
+            qkv = ops.linear(x, self.wqkv, torch.float32, partial_ok=rot is not None)
         else:
             # A call that reads another call's cache needs queries only.
-            qkv = ops.linear(x, self.wqkv[: self.q_dim], torch.float32)
+            qkv = ops.linear(x, self.wqkv[: self.q_dim], torch.float32, partial_ok=rot is not None)
         if rot is None:
             q = qkv[:, : self.q_dim]
             k = qkv[:, self.q_dim: self.q_dim + self.kv_dim] if cache.writes else None

@@ -22,7 +22,7 @@ class EmuOps:
         return y.to(out_dtype)
 
     def split_norm_ok(self, m, width, dtype):
-        return dtype == torch.bfloat16 and 0 < m <= 16 and width % 32 == 0
+        return dtype == torch.bfloat16 and 0 < m <= 128 and width % 32 == 0
 
     @staticmethod
     def _rows(x):
@@ -48,6 +48,8 @@ class EmuOps:
             if not (self.split_norm_ok(m, n, x.dtype if torch.is_tensor(x) else torch.bfloat16) and xd.shape[1] % 32 == 0):
                 return residual, None
             weight, eps = next_norm
+            if m > 16:       # the kernel that adds the product into the residual norms the rows as well
+                return residual, self.rmsnorm(residual, weight, eps, torch.bfloat16)
             ss = torch.zeros(((n + 15) // 16, 16), dtype=torch.float32)
             sq = torch.nn.functional.pad(residual.double() ** 2, (0, ss.shape[0] * 16 - n))
             ss[:, :m] = sq.reshape(m, -1, 16).sum(2).T.to(torch.float32)

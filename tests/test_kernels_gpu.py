@@ -262,6 +262,56 @@ def test_linear_split_norm(m, hidden, kp, nc):
         _close(h3, hd.double().cpu() + a2.double() @ w2.double().T, 2e-5, "fallback product")
 
 
+@pytest.mark.parametrize("m,hidden,kp", [(17, 256, 1024), (64, 4096, 4096), (100, 160, 2048), (128, 512, 256)])
+def test_linear_deferred_reduction(m, hidden, kp):
+    """Products of 17..128 rows split K over blocks; the partial sums may stay unadded for the next kernel:
+    the one that adds them into the residual stream and norms it, or the rotation and cache write."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(31)
+    eps = 1e-5
+    h = torch.randn(m, hidden, generator=g) * 3
+    a = torch.randn(m, kp, generator=g).to(torch.bfloat16)
+    wo = (torch.randn(hidden, kp, generator=g) * 0.05).to(torch.bfloat16)
+    nw = (1 + 0.3 * torch.randn(hidden, generator=g)).float()
+    assert ops.split_norm_ok(m, hidden, torch.bfloat16)
+    # residual product + norm in one go, against the three kernels it replaces
+    h_plain = ops.linear(a.to(DEV), wo.to(DEV), torch.float32, residual=h.clone().to(DEV))
+    x_plain = ops.rmsnorm(h_plain, nw.to(DEV), eps, torch.bfloat16)
+    hd = h.clone().to(DEV)
+    out, x = ops.linear(a.to(DEV), wo.to(DEV), torch.float32, residual=hd, next_norm=(nw.to(DEV), eps))
+    assert out is hd
+    _close(hd, h.double() + a.double() @ wo.double().T, 2e-5, "residual")
+    if x is None:                      # K too short to be split: the product wrote the residual itself
+        assert torch.equal(hd, h_plain)
+    else:
+        assert torch.equal(hd, h_plain), "the same sums in the same order"
+        h64 = hd.double().cpu()
+        want = h64 * torch.rsqrt((h64 ** 2).mean(1, keepdim=True) + eps) * nw.double()
+        assert x.dtype == torch.bfloat16
+        _close(x, want, 5e-3, "normed rows")            # (the sum of squares runs in another order than the norm kernel's)
+        _close(x, x_plain.double().cpu(), 1e-2, "fused against the norm kernel")
+    # projection whose partial sums the rotation adds
+    heads, kvh, d, ps = 4, 2, 32, 16
+    width = (heads + 2 * kvh) * d
+    xin = torch.randn(m, hidden, generator=g).to(torch.bfloat16)
+    wqkv = (torch.randn(width, hidden, generator=g) * 0.05).to(torch.bfloat16)
+    pos = torch.arange(3, 3 + m, dtype=torch.int32)
+    slots = torch.randperm(m * 2, generator=g)[:m].to(torch.int32)
+    inv_freq = (1.0 / 10000.0 ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
+    pages = (m * 2 + ps - 1) // ps
+    results = []
+    for partial_ok in (False, True):
+        kc = torch.zeros(pages, kvh, ps, d, dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros(pages, kvh, d, ps, dtype=torch.bfloat16, device=DEV)
+        qkv = ops.linear(xin.to(DEV), wqkv.to(DEV), torch.float32, partial_ok=partial_ok)
+        if partial_ok and hidden >= 1024:
+            assert isinstance(qkv, ops.Partials) and qkv.shape == (m, width)
+        q = ops.rope_kv_write(qkv, pos.to(DEV), slots.to(DEV), inv_freq.to(DEV), d, 1.0, heads, kvh, d, kc, vc, torch.bfloat16)
+        results.append((q, kc, vc))
+    for u, v in zip(results[0], results[1]):
+        assert torch.equal(u, v), "adding the partial sums in the next kernel changes nothing"
+
+
 @pytest.mark.parametrize("heads,kv,d,page", [(4, 2, 32, 8), (8, 2, 64, 16), (6, 3, 96, 32), (32, 8, 128, 16), (8, 8, 128, 64),
                                              (20, 1, 64, 16), (5, 1, 128, 8)])
 def test_attention_mfma(heads, kv, d, page):
