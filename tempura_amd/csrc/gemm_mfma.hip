@@ -606,6 +606,9 @@ static int g_tune_order = 0;   // large products: 1 tiled kernel, plain block or
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
                    size_t scratch_floats, int tune_splits, hipStream_t s);
 
+int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+                     size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s);
+
 extern "C" void tp_linear_tune_tile(int order) { g_tune_order = order; }
 
 extern "C" void tp_linear_tune_mid(int mid, int splits) {
@@ -720,8 +723,12 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
     // the pipelined kernel: from 129 rows on, and from 65 rows on when there are many column blocks
     // (measured at 128 rows: N = 28,672 59 us against 77 us, the narrow products a few us slower)
     const bool pipe = g_tune_order ? g_tune_order == 3 : (M > 128 || (M > 64 && N >= 16384));
+    const bool pipe64 = !pipe && M <= 128 && scratch != nullptr && g_tune_mid != 2;
     if (pipe && tp_linear_pipe(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, s) == 0) {
       // taken by the pipelined kernel
+    } else if (pipe64 && tp_linear_pipe64(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, defer_reduce,
+                                          splits_out, s) == 0) {
+      // taken by the 64-row pipelined kernel
     } else if (M > 128 || scratch == nullptr) {
       dim3 grid((N + 127) / 128, (M + 127) / 128);
       if (grid.y > 65535) return -1;

@@ -317,6 +317,219 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
   }
 }
 
+// ---- the same pipeline for 17..128 rows -----------------------------------------------------------
+// Here the weights are the traffic and the matrix core has little to do: a block owns 64 x 128 of the
+// result (a wave 32 x 64), three stages of (64 + 128) rows (72 KB: two blocks per CU), K split over
+// blockIdx.y until there are about two blocks for every CU.  Loads, LDS reads and MFMAs interleave as above.
+namespace {
+
+constexpr int BM64 = 64, STAGE64 = (BM64 + BN) * ROWB, LPW64 = 6;
+
+struct Frags64 {
+  u32x4_t a[2], b[4];
+};
+__device__ inline void wait_frags(Frags64& f) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3]));
+}
+template <int R>
+__device__ inline void read_one(Frags64& f, unsigned aaddr, unsigned baddr) {
+  if constexpr (R < 4)
+    f.b[R] = lds_read16<R * 16 * ROWB>(baddr);
+  else
+    f.a[R - 4] = lds_read16<(R - 4) * 16 * ROWB>(aaddr);
+}
+// load I (0..5) of this wave: 0..1 are x rows, 2..5 w rows
+template <int I>
+__device__ inline void issue_one64(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                   const unsigned (&voff)[LPW64], int wave) {
+  const int t = I < 2 ? wave * 2 + I : 8 + wave * 4 + (I - 2);
+  const unsigned char* src = (I < 2 ? xk : wk) + voff[I];
+  __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+}
+template <bool READ, bool LOAD>
+__device__ inline void half_step64(f32x4_t (&acc)[2][4], const Frags64& cur, Frags64& nxt, unsigned aaddr, unsigned baddr,
+                                   unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                   const unsigned (&voff)[LPW64], int wave) {
+#define SB() __builtin_amdgcn_sched_barrier(0)
+#define RD(R) \
+  if (READ) read_one<R>(nxt, aaddr, baddr); \
+  SB()
+#define LD(I) \
+  if (LOAD) issue_one64<I>(buf, xk, wk, voff, wave); \
+  SB()
+#define M1(I, J) \
+  acc[I][J] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(cur.a[I]), as_frag(cur.b[J]), acc[I][J], 0, 0, 0); \
+  SB()
+  RD(0); M1(0, 0); LD(0); RD(1); M1(0, 1); LD(1); RD(2); M1(0, 2); LD(2); RD(3); M1(0, 3); LD(3);
+  RD(4); M1(1, 0); LD(4); RD(5); M1(1, 1); LD(5); M1(1, 2); M1(1, 3);
+#undef RD
+#undef LD
+#undef M1
+#undef SB
+}
+
+}  // namespace
+
+__global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                             void* __restrict__ out, float* __restrict__ partial,
+                                                             int mode, int M, int N, int K) {
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int MB = (M + BM64 - 1) / BM64;
+  const int bm = blockIdx.x % MB, bn = blockIdx.x / MB;     // the row blocks of a column block run side by side
+  const int m0 = bm * BM64, n0 = bn * BN;
+  f32x4_t acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const int kt_per = (K / BK + gridDim.y - 1) / gridDim.y;
+  const int kt_first = blockIdx.y * kt_per;
+  const int KT = min(K / BK, kt_first + kt_per) - kt_first;
+  if (partial != nullptr) {   // K is split, or the caller adds the (single) partial sum itself
+    mode = OUT_F32;
+    out = partial + (size_t)blockIdx.y * M * N;
+  }
+  const int g = lane >> 4, c = lane & 15;
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
+  const unsigned off0 = c * ROWB + (((0 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned off1 = c * ROWB + (((1 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned arow = wm * 32 * ROWB, brow = (BM64 + wn * 64) * ROWB;
+  unsigned voff[LPW64];
+#pragma unroll
+  for (int i = 0; i < LPW64; ++i) {
+    const int row = (i < 2 ? (wave * 2 + i) * 8 : (wave * 4 + i - 2) * 8) + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    const int grow = i < 2 ? min(row, M - 1 - m0) : min(row, N - 1 - n0);
+    voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
+  }
+  const unsigned char* xk = (const unsigned char*)x + ((size_t)m0 * K + (size_t)kt_first * BK) * 2;
+  const unsigned char* wk = (const unsigned char*)w + ((size_t)n0 * K + (size_t)kt_first * BK) * 2;
+  auto issue_stage64 = [&](unsigned char* buf, const unsigned char* xs, const unsigned char* ws) {
+    issue_one64<0>(buf, xs, ws, voff, wave);
+    issue_one64<1>(buf, xs, ws, voff, wave);
+    issue_one64<2>(buf, xs, ws, voff, wave);
+    issue_one64<3>(buf, xs, ws, voff, wave);
+    issue_one64<4>(buf, xs, ws, voff, wave);
+    issue_one64<5>(buf, xs, ws, voff, wave);
+  };
+#pragma unroll
+  for (int p = 0; p < NS; ++p)
+    if (p < KT) issue_stage64(stages + p * STAGE64, xk + p * BK * 2, wk + p * BK * 2);
+  xk += NS * BK * 2;
+  wk += NS * BK * 2;
+  Frags64 fa, fb;
+  if (KT > 2) WAIT_VM(2 * LPW64); else WAIT_VM(0);
+  __builtin_amdgcn_s_barrier();
+#define READ_ALL64(f, aaddr, baddr) \
+  read_one<0>(f, aaddr, baddr); read_one<1>(f, aaddr, baddr); read_one<2>(f, aaddr, baddr); \
+  read_one<3>(f, aaddr, baddr); read_one<4>(f, aaddr, baddr); read_one<5>(f, aaddr, baddr)
+  READ_ALL64(fa, lds0 + arow + off0, lds0 + brow + off0);
+  wait_frags(fa);
+  int st = 0, kt = 0;
+  for (; kt + NS < KT; ++kt) {
+    const int sn = st + 1 == NS ? 0 : st + 1;
+    const unsigned cur = lds0 + st * STAGE64, nxt = lds0 + sn * STAGE64;
+    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fb);
+    WAIT_VM(LPW64);
+    __builtin_amdgcn_s_barrier();
+    half_step64<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, stages + st * STAGE64, xk, wk, voff, wave);
+    wait_frags(fa);
+    xk += BK * 2;
+    wk += BK * 2;
+    st = sn;
+  }
+  for (; kt + 1 < KT; ++kt) {
+    const int sn = st + 1 == NS ? 0 : st + 1;
+    const unsigned cur = lds0 + st * STAGE64, nxt = lds0 + sn * STAGE64;
+    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fb);
+    WAIT_VM(0);
+    __builtin_amdgcn_s_barrier();
+    half_step64<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fa);
+    st = sn;
+  }
+  {
+    const unsigned cur = lds0 + st * STAGE64;
+    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags(fb);
+    half_step64<false, false>(acc, fb, fa, 0, 0, nullptr, nullptr, nullptr, voff, wave);
+  }
+  // the result leaves through LDS, as above: 32 x 64 per wave
+  __syncthreads();
+  float* ct = (float*)stages + wave * (32 * CLD);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int mw = m0 + wm * 32, nw = n0 + wn * 64;
+  if (mode == OUT_SWIGLU) {
+    const int o = (lane & 7) * 4, rr = lane >> 3;
+    const int cg = (o / 8) * 16 + o % 8;
+    bf16_t* ob = (bf16_t*)out;
+    const int half = N / 2;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int row = p * 8 + rr, m = mw + row;
+      const f32x4_t gt = *(const f32x4_t*)(ct + row * CLD + cg);
+      const f32x4_t up = *(const f32x4_t*)(ct + row * CLD + cg + 8);
+      if (m >= M || nw + cg >= N) continue;
+      union {
+        bf16_t h[4];
+        u32x2_t v;
+      } pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(silu_mul(gt[e], up[e]));
+      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk.v;
+    }
+    return;
+  }
+  const int col = (lane & 15) * 4, rr = lane >> 4;
+  const bool vec = (N % 4 == 0) && nw + col + 3 < N;
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const int row = p * 4 + rr, m = mw + row;
+    const f32x4_t v = *(const f32x4_t*)(ct + row * CLD + col);
+    if (m >= M) continue;
+    const size_t idx = (size_t)m * N + nw + col;
+    if (vec) {
+      if (mode == OUT_BF16) {
+        union {
+          bf16_t h[4];
+          u32x2_t v;
+        } pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(v[e]);
+        *(u32x2_t*)((bf16_t*)out + idx) = pk.v;
+      } else if (mode == OUT_F32) {
+        *(f32x4_t*)((float*)out + idx) = v;
+      } else {
+        f32x4_t* o = (f32x4_t*)((float*)out + idx);
+        *o = *o + v;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (nw + col + e >= N) break;
+        if (mode == OUT_BF16)
+          ((bf16_t*)out)[idx + e] = float_to_bf16(v[e]);
+        else if (mode == OUT_F32)
+          ((float*)out)[idx + e] = v[e];
+        else
+          ((float*)out)[idx + e] += v[e];
+      }
+    }
+  }
+}
+
 // Defined in gemm_mfma.hip.
 __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out, int mode,
                                           int splits, int M, int N);
@@ -348,6 +561,40 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
   hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks, splits), dim3(256), 0, s, x, w, out, scratch, mode, M, N, K,
                      pm);
   if (splits > 1) {
+    const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
+                       splits, M, N);
+  }
+  return 0;
+}
+
+// The 64-row pipeline (17..128 rows).  `defer`: when K is split, leave the partial sums in `scratch` for the
+// caller's next kernel and report their number through *splits_out.
+int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+                     size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s) {
+  if (K % BK != 0 || K < BK || M > 128) return -1;
+  if ((size_t)(BM64 - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;
+  if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
+  const int MB = (M + BM64 - 1) / BM64, NB = (N + BN - 1) / BN;
+  const long tiles = (long)MB * NB;
+  if (tiles > 0x7fffffffL) return -1;
+  // a block for every CU, at least sixteen tiles of K each (measured at 24, 64 and 128 rows of the 8B
+  // shapes: more splits than that cost more in partial sums than they gain)
+  int splits = 1;
+  const int KT = K / BK;
+  if (scratch != nullptr) {
+    splits = tune_splits > 0 ? tune_splits : (int)(256 / tiles);
+    splits = std::max(1, std::min(splits, std::min(16, KT / 16)));
+    while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
+    const int per = (KT + splits - 1) / splits;
+    splits = (KT + per - 1) / per;
+  }
+  const bool leave = defer && splits > 1 && splits_out != nullptr && mode != OUT_SWIGLU;
+  hipLaunchKernelGGL(gemm_pipe64_kernel, dim3((unsigned)tiles, splits), dim3(256), 0, s, x, w, out,
+                     splits > 1 ? scratch : nullptr, mode, M, N, K);
+  if (leave) {
+    *splits_out = splits;
+  } else if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
                        splits, M, N);
