@@ -32,11 +32,12 @@ def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> CausalLM:
 
 
 def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: float = 0.02,
-                 norm_jitter: float = 0.0, on_device: bool = None) -> CausalLM:
+                 norm_jitter: float = 0.0, on_device: bool = None, values_as=None) -> CausalLM:
     """A model with seeded random weights made tensor by tensor, never written to disk
     (for sizes whose folder would be tens of gigabytes).  With ``on_device`` (the default on a
     GPU) each tensor is filled by a kernel in device memory; its values then differ from the
-    host generator's that ``write_random_model`` uses."""
+    host generator's that ``write_random_model`` uses.  ``values_as`` (a dtype name) rounds the matrix
+    values to that type first, so that a float32 model can hold exactly a bfloat16 model's weights."""
     from ..kernels import ops
     from ..weights.random_init import _tensor_seed
     td = parse_dtype(dtype)
@@ -59,8 +60,8 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
             if norm_jitter:
                 ops.fill_normal(t, _tensor_seed(seed, name), 1.0, norm_jitter)
             return t
-        t = torch.empty(info.shape, dtype=store, device=dev)
-        return ops.fill_normal(t, _tensor_seed(seed, name), 0.0, std)
+        t = torch.empty(info.shape, dtype=parse_dtype(values_as) if values_as else store, device=dev)
+        return ops.fill_normal(t, _tensor_seed(seed, name), 0.0, std).to(store)
 
     model.load_weights(get)
     return model

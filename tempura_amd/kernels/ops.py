@@ -229,7 +229,7 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     m, k = x.shape
     n = w.shape[0]
     _need(n % 16 == 0 and k % 32 == 0, "linear_swiglu: needs 2i % 16 == 0 and k % 32 == 0")
-    blocked_out = blocked_out and 0 < m <= 16
+    blocked_out = blocked_out and allow_mfma and 0 < m <= 16   # (the product that takes such rows is an MFMA kernel)
     if blocked_out:
         out = KBlocked(torch.empty((n // 16, m, 8), dtype=torch.bfloat16, device=x.device), m, n // 2)
     else:
