@@ -14,7 +14,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import CacheSpec, Mixer, WeightInfo, build_part, register_part
+from .base import CacheSpec, Mixer, WeightInfo, build_part, part_class, register_part
 
 
 class PagedAttention(Mixer):
@@ -42,12 +42,15 @@ class PagedAttention(Mixer):
         p, w = spec.params, spec.weights
         q_dim = p["num_heads"] * p["head_dim"]
         kv_dim = p["num_kv_heads"] * p["head_dim"]
-        return {
+        out = {
             w["q"]: WeightInfo((q_dim, hidden_size)),
             w["k"]: WeightInfo((kv_dim, hidden_size)),
             w["v"]: WeightInfo((kv_dim, hidden_size)),
             w["o"]: WeightInfo((hidden_size, q_dim)),
         }
+        # a position encoding may have tensors of its own (a rotary one has none)
+        out.update(part_class("position", p["position"].kind).expected_weights(p["position"], hidden_size))
+        return out
 
     def load_weights(self, get):
         w = self.spec.weights
@@ -55,6 +58,7 @@ class PagedAttention(Mixer):
         parts = [get(w["q"]), get(w["k"]), get(w["v"])]
         self.wqkv = torch.cat([self._to_device(t) for t in parts], dim=0).contiguous()
         self.wo = self._to_device(get(w["o"]))
+        self.position.load_weights(get)
 
     def cache_spec(self):
         kind = "window" if self.window is not None else "full"

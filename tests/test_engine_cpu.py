@@ -169,3 +169,30 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
     runner.add_request("again")
     lg = runner.step([StepEntry("again", reqs["q"], list(range(9)))])
     assert helpers.rel_err(lg, ref["q"]) < 1e-6
+
+
+def test_toy_routed_ffn_and_learned_position_register_build_and_step(tmp_path):
+    """A feed-forward with routing and a position encoding that is not rotary (with a tensor of its own),
+    defined in the tests, in layers beside the library's rotary attention (windowed: a second cache group)
+    and SwiGLU."""
+    import toy_parts
+    from tempura_amd.config import load_config
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.weights import write_random_model
+    cfg = toy_parts.ToyRoutedConfig()
+    d = write_random_model(cfg, str(tmp_path / "routed"), seed=6, std=0.25, norm_jitter=0.1, dtype="float32")
+    assert type(load_config(d)) is toy_parts.ToyRoutedConfig
+    model = load_model(d, "float32", "cpu")
+    assert sorted(g.kind for g in model.cache_groups) == ["full", "window"] and not model.state_specs
+    _, W = plain.read_model_dir(d)
+    assert {"r.0.pos", "r.2.pos", "r.0.router", "r.1.gate"} <= set(W)
+    runner = ModelRunner(model, 8, [12, 8], max_requests=3)
+    reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=10 + i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30}.items())}
+    ref = {r: toy_parts.plain_routed_forward(cfg, W, t) for r, t in reqs.items()}
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
+             ([("p", 10, 11), ("r", 17, 13)], ["p", "r"])]
+    got = helpers.run_schedule(runner, reqs, steps)
+    for r in reqs:
+        assert helpers.first_difference(got[r], ref[r], 1e-6) is None, r
+    assert runner.cache.free_pages() == [12, 8]

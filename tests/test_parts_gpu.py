@@ -191,3 +191,27 @@ def test_toy_mixer_with_state_on_the_gpu(tmp_path, dtype):
     for r, t in reqs.items():
         ref = toy_parts.plain_toy_forward(cfg, W, t)
         assert helpers.rel_err(got[r], ref) < helpers.TOL[dtype], r
+
+
+def test_toy_routed_ffn_and_learned_position_on_the_gpu(tmp_path):
+    """Registered, built and stepped without a change to the framework: a feed-forward with routing and a
+    learned position encoding from the tests, beside the library's kernels (rotary windowed attention, SwiGLU),
+    portions and single tokens of three requests mixed.  In float32 only: rounding to bfloat16 may send a token
+    whose two best experts score alike to the other one, which no tolerance covers."""
+    dtype = "float32"
+    import toy_parts
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.weights import write_random_model
+    cfg = toy_parts.ToyRoutedConfig()
+    d = write_random_model(cfg, str(tmp_path / "routed"), seed=6, std=0.25, norm_jitter=0.1, dtype=dtype)
+    model = load_model(d, dtype, "cuda:0")
+    _, W = plain.read_model_dir(d)
+    runner = ModelRunner(model, 8, [12, 8], max_requests=3)
+    reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=10 + i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30}.items())}
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
+             ([("p", 10, 11), ("r", 17, 13)], ["p", "r"])]
+    got = helpers.run_schedule(runner, reqs, steps)
+    for r, t in reqs.items():
+        ref = toy_parts.plain_routed_forward(cfg, W, t)
+        assert helpers.rel_err(got[r], ref) < helpers.TOL[dtype], r

@@ -1,6 +1,10 @@
-"""A toy architecture defined entirely in the tests: a mixer with per-request state of its own (a decaying
-running sum, no paged cache), used in some layers beside attention in others, registered through the public
-registries.  Nothing under tempura_amd/ knows about it."""
+"""Toy parts and toy architectures defined entirely in the tests and registered through the public registries;
+nothing under tempura_amd/ knows about them.
+* a mixer with per-request state of its own (a decaying running sum, no paged cache), used in some layers
+  beside attention in others (``ToyForCausalLM``);
+* a feed-forward with routing (each token goes to the expert its router scores highest) and a position
+  encoding that is not rotary (a learned vector per position, added to queries and keys), in layers beside
+  the library's own parts (``ToyRoutedForCausalLM``)."""
 from __future__ import annotations
 
 import json
@@ -10,7 +14,7 @@ from typing import Dict, List
 import torch
 
 from tempura_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, register_architecture
-from tempura_amd.parts import Mixer, StateSpec, WeightInfo, register_part
+from tempura_amd.parts import FeedForward, Mixer, PositionEncoding, StateSpec, WeightInfo, register_part
 
 
 class DecaySumMixer(Mixer):
@@ -46,6 +50,65 @@ class DecaySumMixer(Mixer):
 
 
 register_part("mixer", "decay_sum", DecaySumMixer)
+
+
+class TopOneRoutedFFN(FeedForward):
+    """Router logits in float32; each token's output is its best expert's two-layer ReLU network times the
+    softmax weight of that expert.  Tokens are grouped by expert on the host; a token's result does not
+    depend on which other tokens are in the batch."""
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        self.experts = int(spec.params["experts"])
+        self.inner = int(spec.params["inner"])
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        e, i, w = spec.params["experts"], spec.params["inner"], spec.weights
+        return {w["router"]: WeightInfo((e, hidden_size)), w["up"]: WeightInfo((e * i, hidden_size)),
+                w["down"]: WeightInfo((e * hidden_size, i))}
+
+    def load_weights(self, get):
+        w = self.spec.weights
+        self.router = self._to_device(get(w["router"]), torch.float32)
+        self.up = self._to_device(get(w["up"]), torch.float32).view(self.experts, self.inner, self.hidden_size)
+        self.down = self._to_device(get(w["down"]), torch.float32).view(self.experts, self.hidden_size, self.inner)
+
+    def forward(self, x, ctx, residual):
+        xf = x.float()
+        probs = torch.softmax(xf @ self.router.T, dim=-1)
+        weight, choice = probs.max(dim=-1)
+        for e in range(self.experts):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                y = torch.relu(xf[rows] @ self.up[e].T) @ self.down[e].T
+                residual[rows] += y * weight[rows, None]
+
+
+class LearnedPosition(PositionEncoding):
+    """A learned vector per position, added to every query and key head before the scores."""
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        self.table = None
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        return {spec.weights["table"]: WeightInfo((spec.params["max_positions"], spec.params["head_dim"]))}
+
+    def load_weights(self, get):
+        self.table = self._to_device(get(self.spec.weights["table"]), torch.float32)
+
+    def apply(self, q, k, positions):
+        d = self.table.shape[1]
+        add = self.table[positions.long()]                                # [tokens, head_dim]
+        q2 = (q.reshape(q.shape[0], -1, d) + add[:, None, :]).reshape(q.shape)
+        k2 = None if k is None else (k.reshape(k.shape[0], -1, d) + add[:, None, :]).reshape(k.shape)
+        return q2, k2
+
+
+register_part("ffn", "toy_routed", TopOneRoutedFFN)
+register_part("position", "toy_learned", LearnedPosition)
 
 
 @dataclass
@@ -97,6 +160,96 @@ class ToyConfig:
 
 
 register_architecture("ToyForCausalLM", ToyConfig)
+
+
+@dataclass
+class ToyRoutedConfig:
+    """Three layers: attention with a learned position and a routed feed-forward; attention with rotary
+    position (window 12) and the library's SwiGLU; again a learned position and a routed feed-forward."""
+    hidden_size: int = 64
+    vocab_size: int = 90
+    num_attention_heads: int = 4
+    num_key_value_heads: int = 2
+    head_dim: int = 16
+    experts: int = 3
+    inner: int = 40
+    intermediate_size: int = 96
+    max_position_embeddings: int = 128
+    architecture: str = "ToyRoutedForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        keys = cls.__dataclass_fields__
+        return cls(**{k: v for k, v in d.items() if k in keys})
+
+    def to_json(self):
+        d = {k: getattr(self, k) for k in self.__dataclass_fields__}
+        d["architectures"] = [self.architecture]
+        return json.dumps(d)
+
+    def _attention(self, p, position, window):
+        return PartSpec("attention", {"num_heads": self.num_attention_heads, "num_kv_heads": self.num_key_value_heads,
+                                      "head_dim": self.head_dim, "scale": self.head_dim ** -0.5, "window": window,
+                                      "position": position},
+                        {"q": f"{p}.q", "k": f"{p}.k", "v": f"{p}.v", "o": f"{p}.o"})
+
+    def build_spec(self) -> ModelSpec:
+        learned = lambda p: PartSpec("toy_learned", {"max_positions": self.max_position_embeddings, "head_dim": self.head_dim},
+                                     {"table": f"{p}.pos"})
+        rope = PartSpec("rope", {"head_dim": self.head_dim, "theta": 1e4, "scaling": None})
+        routed = lambda p: PartSpec("toy_routed", {"experts": self.experts, "inner": self.inner},
+                                    {"router": f"{p}.router", "up": f"{p}.up", "down": f"{p}.down"})
+        swiglu = lambda p: PartSpec("swiglu", {"intermediate_size": self.intermediate_size},
+                                    {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"})
+        norm = lambda n: PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": n})
+        layers = [
+            LayerSpec("prenorm", self._attention("r.0", learned("r.0"), None), routed("r.0"), norm("r.0.n1"), norm("r.0.n2")),
+            LayerSpec("prenorm", self._attention("r.1", rope, 12), swiglu("r.1"), norm("r.1.n1"), norm("r.1.n2")),
+            LayerSpec("prenorm", self._attention("r.2", learned("r.2"), None), routed("r.2"), norm("r.2.n1"), norm("r.2.n2")),
+        ]
+        return ModelSpec(self.architecture, self.hidden_size, self.vocab_size, self.max_position_embeddings, layers,
+                         [LayerCall(0), LayerCall(1), LayerCall(2)],
+                         norm("r.norm"), PartSpec("embedding", {}, {"weight": "r.embed"}),
+                         PartSpec("lm_head", {"tied": False}, {"weight": "r.head"}))
+
+
+register_architecture("ToyRoutedForCausalLM", ToyRoutedConfig)
+
+
+def plain_routed_forward(cfg: ToyRoutedConfig, W: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
+    """Whole sequence, no cache, float64: the routed toy model written out plainly."""
+    import plain
+    W = {k: v.double() for k, v in W.items()}
+    T = len(tokens)
+    H, KV, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    h = W["r.embed"][torch.tensor(tokens)]
+    inv = plain.rope_inv_freq(D, 1e4, None)
+    pos = torch.arange(T)
+    for l in range(3):
+        p = f"r.{l}"
+        x = plain.rmsnorm(h, W[f"{p}.n1"], 1e-5)
+        q = (x @ W[f"{p}.q"].T).reshape(T, H, D)
+        k = (x @ W[f"{p}.k"].T).reshape(T, KV, D)
+        v = (x @ W[f"{p}.v"].T).reshape(T, KV, D)
+        if l == 1:
+            q, k = plain.rope(q, pos, inv), plain.rope(k, pos, inv)
+            a = plain.attention(q, k, v, D ** -0.5, window=12)
+        else:
+            add = W[f"{p}.pos"][:T]
+            q, k = q + add[:, None, :], k + add[:, None, :]
+            a = plain.attention(q, k, v, D ** -0.5)
+        h = h + a @ W[f"{p}.o"].T
+        x = plain.rmsnorm(h, W[f"{p}.n2"], 1e-5)
+        if l == 1:
+            h = h + plain.swiglu_ffn(x, W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
+        else:
+            probs = torch.softmax(x @ W[f"{p}.router"].T, dim=-1)
+            weight, choice = probs.max(dim=-1)
+            up = W[f"{p}.up"].view(cfg.experts, cfg.inner, cfg.hidden_size)
+            down = W[f"{p}.down"].view(cfg.experts, cfg.hidden_size, cfg.inner)
+            y = torch.stack([torch.relu(x[t] @ up[choice[t]].T) @ down[choice[t]].T * weight[t] for t in range(T)])
+            h = h + y
+    return plain.rmsnorm(h, W["r.norm"], 1e-5) @ W["r.head"].T
 
 
 def plain_toy_forward(cfg: ToyConfig, W: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
