@@ -318,7 +318,7 @@ __device__ inline u32x4_t attn_lds_read(unsigned addr) {
 }
 
 template <int D, int NQ>
-__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, int skip_single) {
+__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, int skip_single, int pair) {
   constexpr int C = D / 8;             // 16-byte chunks per key row
   constexpr int SH = C == 16 ? 0 : (C == 8 ? 1 : 2);
   constexpr int KI = D / 16;           // 1 KB loads per key tile (32 rows of 2 D bytes), and per value tile
@@ -333,8 +333,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   const int q_start = a.cu_seqlens[r];
   const int q_len = a.cu_seqlens[r + 1] - q_start;
   if (q_len <= 0 || (skip_single && q_len == 1)) return;
-  const int q0 = blockIdx.x * 16 * NQ;
-  if (q0 >= q_len) return;
+  // pair: a block takes query block x and then query block (last - x): under the causal mask the two
+  // together see about as many keys as any other pair, so every block runs equally long
+  const int nqb = (q_len + 16 * NQ - 1) / (16 * NQ);
+  if (pair ? (int)blockIdx.x >= (nqb + 1) / 2 : (int)blockIdx.x >= nqb) return;
   const int group = a.n_heads / a.n_kv;
   const int hblocks = (group + 3) / 4;
   const int kvh = blockIdx.y / hblocks;
@@ -346,6 +348,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   const int* table = a.block_tables + (size_t)r * a.table_width;
   const int ps = a.page_size;
 
+  for (int turn = 0; turn < (pair ? 2 : 1); ++turn) {
+  const int qb = turn == 0 ? (int)blockIdx.x : nqb - 1 - (int)blockIdx.x;
+  if (turn == 1) {
+    if (qb == (int)blockIdx.x) break;     // the middle block of an odd count has no partner
+    __syncthreads();                      // every wave is done with the stages of the first turn
+  }
+  const int q0 = qb * 16 * NQ;
   bf16x8_t qf[NQ][D / 32];
   int qpos[NQ];
   float m[NQ], l[NQ];
@@ -516,7 +525,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     }
     stage = nstage;
   }
-  if (!active) return;
+  if (active) {
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
     float lt = l[nq];
@@ -534,6 +543,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
         *(uint2*)(orow + dt * 16 + 4 * g) = w;
       }
     }
+  }
+  }
   }
 }
 
@@ -656,7 +667,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 }
 
 // ---- dispatch ------------------------------------------------------------------------------
-static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave
+static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave; 2 / 3: query blocks never / always in pairs
 extern "C" void tp_attention_tune(int v) { g_attn_tune = v; }
 
 template <int D>
@@ -678,7 +689,11 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
       if (g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
-        hipLaunchKernelGGL((attn_prefill_lds_kernel<D, NQ>), grid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0);
+        // pairs of query blocks once the pairs alone fill the CUs twice over (each block then runs equally long)
+        const long pairs = (long)((grid.x + 1) / 2) * grid.y * grid.z;
+        const int pair = g_attn_tune == 2 ? 0 : (g_attn_tune == 3 ? 1 : (pairs >= 256 ? 1 : 0));
+        const dim3 pgrid(pair ? (grid.x + 1) / 2 : grid.x, grid.y, grid.z);
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<D, NQ>), pgrid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0, pair);
         return 0;
       }
     }
