@@ -192,17 +192,14 @@ __device__ inline void attn_pv(const bf16x8_t (&vf)[D / 16], const bf16x8_t (&pf
     if (moved[nq]) {
 #pragma unroll
       for (int dt = 0; dt < D / 16; ++dt) {
-        f32x4_t acc = o[nq][dt];
-        acc[0] *= alpha[nq];
-        acc[1] *= alpha[nq];
-        acc[2] *= alpha[nq];
-        acc[3] *= alpha[nq];
-        o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf[nq], acc, 0, 0, 0);
+        o[nq][dt][0] *= alpha[nq];
+        o[nq][dt][1] *= alpha[nq];
+        o[nq][dt][2] *= alpha[nq];
+        o[nq][dt][3] *= alpha[nq];
       }
-    } else {
-#pragma unroll
-      for (int dt = 0; dt < D / 16; ++dt) o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf[nq], o[nq][dt], 0, 0, 0);
     }
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt) o[nq][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf[nq], o[nq][dt], 0, 0, 0);
   }
 }
 
@@ -318,7 +315,7 @@ __device__ inline u32x4_t attn_lds_read(unsigned addr) {
 }
 
 template <int D, int NQ>
-__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, int skip_single, int pair) {
+__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, int skip_single) {
   constexpr int C = D / 8;             // 16-byte chunks per key row
   constexpr int SH = C == 16 ? 0 : (C == 8 ? 1 : 2);
   constexpr int KI = D / 16;           // 1 KB loads per key tile (32 rows of 2 D bytes), and per value tile
@@ -329,18 +326,20 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g = lane >> 4, c = lane & 15;
-  const int r = blockIdx.z;
+  // Blocks go to the eight XCDs in turn, each with an L2 of its own: neighbouring blocks take different
+  // kv heads (fastest index), so that one L2 holds the keys and values of few heads, read by all their
+  // query blocks; the longest query blocks come first.
+  const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int by = lin % gridDim.y, bx = (lin / gridDim.y) % gridDim.x;
+  const int r = lin / (gridDim.x * gridDim.y);
   const int q_start = a.cu_seqlens[r];
   const int q_len = a.cu_seqlens[r + 1] - q_start;
   if (q_len <= 0 || (skip_single && q_len == 1)) return;
-  // pair: a block takes query block x and then query block (last - x): under the causal mask the two
-  // together see about as many keys as any other pair, so every block runs equally long
   const int nqb = (q_len + 16 * NQ - 1) / (16 * NQ);
-  if (pair ? (int)blockIdx.x >= (nqb + 1) / 2 : (int)blockIdx.x >= nqb) return;
+  if (bx >= nqb) return;
   const int group = a.n_heads / a.n_kv;
-  const int hblocks = (group + 3) / 4;
-  const int kvh = blockIdx.y / hblocks;
-  const int hin = (blockIdx.y % hblocks) * 4 + wave;
+  const int kvh = by % a.n_kv;
+  const int hin = (by / a.n_kv) * 4 + wave;
   const bool active = hin < group;     // a wave without a head still loads and waits with the others
   const int head = kvh * group + min(hin, group - 1);
   const int ctx = a.context_lens[r];
@@ -348,13 +347,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   const int* table = a.block_tables + (size_t)r * a.table_width;
   const int ps = a.page_size;
 
-  for (int turn = 0; turn < (pair ? 2 : 1); ++turn) {
-  const int qb = turn == 0 ? (int)blockIdx.x : nqb - 1 - (int)blockIdx.x;
-  if (turn == 1) {
-    if (qb == (int)blockIdx.x) break;     // the middle block of an odd count has no partner
-    __syncthreads();                      // every wave is done with the stages of the first turn
-  }
-  const int q0 = qb * 16 * NQ;
+  const int q0 = (nqb - 1 - bx) * 16 * NQ;
   bf16x8_t qf[NQ][D / 32];
   int qpos[NQ];
   float m[NQ], l[NQ];
@@ -384,22 +377,26 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   const int psh = a.page_shift, pmask = ps - 1;
   // the block table through the constant address space: uniform loads from it are scalar loads
   const __attribute__((address_space(4))) int* ctab = (const __attribute__((address_space(4))) int*)(uintptr_t)table;
-  int koff_row[LP], boff[LP];
+  // (load t = wave + 4 i; t < KI: slot 64 t + lane of the key tile, row = slot / C, chunk slot % C rotated
+  // by the row; else value row d = 16 (t - KI) + lane / 4 and the group of eight keys vgroup)
+  const int vgroup = (lane & 3) ^ ((lane >> 4) & 3);
+  auto key_row = [&](int t) { return (64 * t + lane) / C; };
+  auto key_byte = [&](int t) {
+    const int row = (64 * t + lane) / C, pc = (64 * t + lane) % C;
+    const int f = ((((row >> 3) << 2) | (row & 3)) >> SH);
+    return ((pc - f) & (C - 1)) * 16;
+  };
+  auto value_row = [&](int t) { return 16 * (t - KI) + (lane >> 2); };
+  unsigned lane_off[LP];   // byte offset of this lane's 16 bytes from the uniform part of a load's address
 #pragma unroll
   for (int i = 0; i < LP; ++i) {
     const int t = wave + 4 * i;
-    if (t < KI) {
-      const int slot = 64 * t + lane;
-      const int row = slot / C, pc = slot % C;
-      const int f = ((((row >> 3) << 2) | (row & 3)) >> SH);
-      koff_row[i] = row;
-      boff[i] = ((pc - f) & (C - 1)) * 16;
-    } else {
-      const int d = 16 * (t - KI) + (lane >> 2);
-      koff_row[i] = (lane & 3) ^ ((d >> 2) & 3);   // which group of eight keys
-      boff[i] = d;                                  // the value row
-    }
+    if (t < KI)
+      lane_off[i] = (unsigned)((key_row(t) - 8 * (((64 * t) / C) >> 3)) * D * 2 + key_byte(t));
+    else
+      lane_off[i] = (unsigned)(((kvh * D + value_row(t)) * ps + ((8 * vgroup) & pmask)) * 2);
   }
+  const unsigned vpage_bytes = (unsigned)(a.n_kv * D * ps * 2);
   // the pages of the four groups of eight keys of a step (clamped to the last key that exists); a key
   // load's rows lie in one of these groups, or past the end in the last key's page
   auto pages_of = [&](int step, int (&pg)[4]) {
@@ -410,6 +407,32 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   auto issue = [&](int step, int stage, const int (&pg)[4]) {
     const int j0 = first + step * 32;
     unsigned char* buf = stages + stage * STAGE;
+    if (j0 + 32 <= ctx) {
+      // all 32 keys exist: a load's address is a uniform part (page, kv head, place in the page; scalar
+      // arithmetic) plus the lane's constant offset; only the page of a value load differs by lane
+      const unsigned in_page = (unsigned)(j0 & pmask);
+      // (opaque copies: the compiler otherwise turns the selection by lane into an indexed load from a
+      // copy of pg in scratch memory)
+      int p0 = pg[0], p1 = pg[1], p2 = pg[2], p3 = pg[3];
+      asm volatile("" : "+s"(p0), "+s"(p1), "+s"(p2), "+s"(p3));
+      const int vpage = vgroup == 0 ? p0 : (vgroup == 1 ? p1 : (vgroup == 2 ? p2 : p3));
+      const unsigned char* vsrc = (const unsigned char*)a.v_cache + (size_t)(unsigned)vpage * vpage_bytes + in_page * 2;
+#pragma unroll
+      for (int i = 0; i < LP; ++i) {
+        const int t = wave + 4 * i;
+        const unsigned char* src;
+        if (t < KI) {
+          const int gr = ((64 * t) / C) >> 3;
+          const int page = gr == 0 ? pg[0] : (gr == 1 ? pg[1] : (gr == 2 ? pg[2] : pg[3]));
+          const unsigned char* kb = (const unsigned char*)(a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + ((j0 + 8 * gr) & pmask)) * D);
+          src = kb + lane_off[i];
+        } else {
+          src = vsrc + lane_off[i];
+        }
+        __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < LP; ++i) {
       const int t = wave + 4 * i;
@@ -417,13 +440,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
       if (t < KI) {
         const int gr = ((64 * t) / C) >> 3;                  // the group of eight keys this load lies in
         const int page = gr == 0 ? pg[0] : (gr == 1 ? pg[1] : (gr == 2 ? pg[2] : pg[3]));
-        const int key = min(j0 + koff_row[i], ctx - 1);
-        src = (const unsigned char*)(a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + (key & pmask)) * D) + boff[i];
+        const int key = min(j0 + key_row(t), ctx - 1);
+        src = (const unsigned char*)(a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + (key & pmask)) * D) + key_byte(t);
       } else {
-        const int gg = koff_row[i];
+        const int gg = vgroup;
         const int kb = min(j0 + 8 * gg, (ctx - 1) & ~7);
         const int page = gg == 0 ? pg[0] : (gg == 1 ? pg[1] : (gg == 2 ? pg[2] : pg[3]));
-        src = (const unsigned char*)(a.v_cache + ((size_t)(page * a.n_kv + kvh) * D + boff[i]) * ps + (kb & pmask));
+        src = (const unsigned char*)(a.v_cache + ((size_t)(page * a.n_kv + kvh) * D + value_row(t)) * ps + (kb & pmask));
       }
       __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
     }
@@ -543,7 +566,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
         *(uint2*)(orow + dt * 16 + 4 * g) = w;
       }
     }
-  }
   }
   }
 }
@@ -667,7 +689,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 }
 
 // ---- dispatch ------------------------------------------------------------------------------
-static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave; 2 / 3: query blocks never / always in pairs
+static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave
 extern "C" void tp_attention_tune(int v) { g_attn_tune = v; }
 
 template <int D>
@@ -689,11 +711,7 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
       if (g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
-        // pairs of query blocks once the pairs alone fill the CUs twice over (each block then runs equally long)
-        const long pairs = (long)((grid.x + 1) / 2) * grid.y * grid.z;
-        const int pair = g_attn_tune == 2 ? 0 : (g_attn_tune == 3 ? 1 : (pairs >= 256 ? 1 : 0));
-        const dim3 pgrid(pair ? (grid.x + 1) / 2 : grid.x, grid.y, grid.z);
-        hipLaunchKernelGGL((attn_prefill_lds_kernel<D, NQ>), pgrid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0, pair);
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<D, NQ>), grid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0);
         return 0;
       }
     }
