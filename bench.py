@@ -155,7 +155,8 @@ def main() -> int:
             print(f"[bench] decode b{b}: {p_tps:.1f} tok/s, {p_ms:.3f} ms/step", file=sys.stderr, flush=True)
 
     out = {
-        "metric": f"decode tok/s at batch {args.batch}, Llama-3.1-8B shape bf16, KV {args.prompt_len}->{args.context}",
+        "metric": f"decode tok/s at batch {args.batch}, {args.model_config} shape {'bf16' if args.dtype == 'bfloat16' else 'fp32'}, "
+                  f"KV {args.prompt_len}->{args.context}",
         "value": round(tps, 1),
         "unit": "tok/s",
         "n_gpus": 1,
