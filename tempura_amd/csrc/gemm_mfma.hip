@@ -25,7 +25,11 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 // 8*b + i is silu(row 16*b + i) * (row 16*b + 8 + i), stored as bfloat16 [M, N / 2].
 enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_ACC_F32 = 2, OUT_SWIGLU = 3 };
 
-__device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+// g * sigmoid(g) * u with the hardware's exp2 and reciprocal (one ulp each; the result is rounded to bfloat16),
+// the same arithmetic in every bfloat16 product, whatever the number of rows
+__device__ inline float silu_mul(float g, float u) {
+  return g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+}
 
 __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
 

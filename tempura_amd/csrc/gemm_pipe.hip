@@ -45,7 +45,17 @@ constexpr int LPW = 12;        // direct loads per wave and stage: eight of x ro
 constexpr int CLD = 64 + 4;    // padded row of a wave's result tile in LDS, in floats
 
 __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8_t, v); }
-__device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+// g * sigmoid(g) * u with the hardware's exp2 and reciprocal (one ulp each; the result is rounded to bfloat16)
+__device__ inline float silu_mul(float g, float u) {
+  return g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+}
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// two floats to two bfloat16 (round to nearest even) in one instruction
+__device__ inline unsigned pack_bf16(float a, float b) {
+  const f32x2_t f = {a, b};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2_t));
+}
 
 // vmcnt(n) alone: bits [3:0] and [15:14] hold n, the other counters stay at their maxima
 #define WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
@@ -269,13 +279,10 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
       const f32x4_t gt = *(const f32x4_t*)(ct + row * CLD + cg);
       const f32x4_t up = *(const f32x4_t*)(ct + row * CLD + cg + 8);
       if (m >= M || nw + cg >= N) continue;   // N is a multiple of 16: the whole group is inside or outside
-      union {
-        bf16_t h[4];
-        u32x2_t v;
-      } pk;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(silu_mul(gt[e], up[e]));
-      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk.v;
+      u32x2_t pk;
+      pk[0] = pack_bf16(silu_mul(gt[0], up[0]), silu_mul(gt[1], up[1]));
+      pk[1] = pack_bf16(silu_mul(gt[2], up[2]), silu_mul(gt[3], up[3]));
+      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk;
     }
     return;
   }
@@ -289,13 +296,10 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
     const size_t idx = (size_t)m * N + nw + col;
     if (vec) {
       if (mode == OUT_BF16) {
-        union {
-          bf16_t h[4];
-          u32x2_t v;
-        } pk;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(v[e]);
-        *(u32x2_t*)((bf16_t*)out + idx) = pk.v;
+        u32x2_t pk;
+        pk[0] = pack_bf16(v[0], v[1]);
+        pk[1] = pack_bf16(v[2], v[3]);
+        *(u32x2_t*)((bf16_t*)out + idx) = pk;
       } else if (mode == OUT_F32) {
         *(f32x4_t*)((float*)out + idx) = v;
       } else {
@@ -482,13 +486,10 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
       const f32x4_t gt = *(const f32x4_t*)(ct + row * CLD + cg);
       const f32x4_t up = *(const f32x4_t*)(ct + row * CLD + cg + 8);
       if (m >= M || nw + cg >= N) continue;
-      union {
-        bf16_t h[4];
-        u32x2_t v;
-      } pk;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(silu_mul(gt[e], up[e]));
-      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk.v;
+      u32x2_t pk;
+      pk[0] = pack_bf16(silu_mul(gt[0], up[0]), silu_mul(gt[1], up[1]));
+      pk[1] = pack_bf16(silu_mul(gt[2], up[2]), silu_mul(gt[3], up[3]));
+      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk;
     }
     return;
   }
@@ -502,13 +503,10 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
     const size_t idx = (size_t)m * N + nw + col;
     if (vec) {
       if (mode == OUT_BF16) {
-        union {
-          bf16_t h[4];
-          u32x2_t v;
-        } pk;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(v[e]);
-        *(u32x2_t*)((bf16_t*)out + idx) = pk.v;
+        u32x2_t pk;
+        pk[0] = pack_bf16(v[0], v[1]);
+        pk[1] = pack_bf16(v[2], v[3]);
+        *(u32x2_t*)((bf16_t*)out + idx) = pk;
       } else if (mode == OUT_F32) {
         *(f32x4_t*)((float*)out + idx) = v;
       } else {
