@@ -613,7 +613,12 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
 int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
                      size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s);
 
-extern "C" void tp_linear_tune_tile(int order) { g_tune_order = order; }
+extern int g_pipe_big;
+// order: 1 tiled plain, 2 tiled XCD-aware, 3 pipelined; 5 / 6: pipelined with 256 x 256 tiles always / never
+extern "C" void tp_linear_tune_tile(int order) {
+  g_pipe_big = order == 5 ? 1 : (order == 6 ? 2 : 0);
+  g_tune_order = order >= 5 ? 0 : order;
+}
 
 extern "C" void tp_linear_tune_mid(int mid, int splits) {
   g_tune_mid = mid;

@@ -153,12 +153,14 @@ __device__ inline void half_step(f32x4_t (&acc)[8][4], const Frags& cur, Frags& 
 
 }  // namespace
 
+// ldo: row stride of `out` in elements (N, or N / 2 for the gated mode, when the launch covers all columns;
+// a launch may cover a range of columns with `w` and `out` pointing at its first).
 // pm: row blocks of a patch (a power of two up to 8); a patch holds 32 blocks.  blockIdx.y splits K:
 // with more than one split every block writes its float32 partial tile to `partial` [split, M, N]
 // and a second kernel adds the splits in ascending order and applies the epilogue.
 __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                         void* __restrict__ out, float* __restrict__ partial, int mode,
-                                                        int M, int N, int K, int pm) {
+                                                        int M, int N, int K, int pm, int ldo) {
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE_BYTES];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -188,6 +190,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
   if (gridDim.y > 1) {
     mode = OUT_F32;
     out = partial + (size_t)blockIdx.y * M * N;
+    ldo = N;
   }
   const int g = lane >> 4, c = lane & 15;
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
@@ -272,7 +275,6 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
     const int o = (lane & 7) * 4, rr = lane >> 3;
     const int cg = (o / 8) * 16 + o % 8;
     bf16_t* ob = (bf16_t*)out;
-    const int half = N / 2;
 #pragma unroll 4
     for (int p = 0; p < 16; ++p) {
       const int row = p * 8 + rr, m = mw + row;
@@ -282,18 +284,18 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
       u32x2_t pk;
       pk[0] = pack_bf16(silu_mul(gt[0], up[0]), silu_mul(gt[1], up[1]));
       pk[1] = pack_bf16(silu_mul(gt[2], up[2]), silu_mul(gt[3], up[3]));
-      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk;
+      *(u32x2_t*)(ob + (size_t)m * ldo + nw / 2 + o) = pk;
     }
     return;
   }
   const int col = (lane & 15) * 4, rr = lane >> 4;
-  const bool vec = (N % 4 == 0) && nw + col + 3 < N;
+  const bool vec = (ldo % 4 == 0) && nw + col + 3 < N;
 #pragma unroll 4
   for (int p = 0; p < 32; ++p) {
     const int row = p * 4 + rr, m = mw + row;
     const f32x4_t v = *(const f32x4_t*)(ct + row * CLD + col);
     if (m >= M) continue;
-    const size_t idx = (size_t)m * N + nw + col;
+    const size_t idx = (size_t)m * ldo + nw + col;
     if (vec) {
       if (mode == OUT_BF16) {
         u32x2_t pk;
@@ -318,6 +320,253 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
           ((float*)out)[idx + e] += v[e];
       }
     }
+  }
+}
+
+// ---- 256 x 256 block tiles ---------------------------------------------------------------------------
+// What bounds the kernel above is the operand traffic from L2 into LDS (48 KB per 64 of K and CU, three
+// quarters of what the path delivers at the full MFMA rate).  A 256 x 256 block tile (a wave owns 128 x 128,
+// 256 accumulator registers) needs 64 KB for twice the work.  Two stages of (256 + 256) rows x 128 bytes
+// (128 KB); the pipeline is the same: fragments of the next half step and the loads of the tile after next
+// between the MFMAs of this half step, one barrier per 64 of K.  Used where whole rounds of such tiles fill
+// the CUs; the columns that are left go to the kernel above.
+namespace {
+
+constexpr int BNB = 256, STAGE_BIG = (BM + BNB) * ROWB, NSB = 2, LPWB = 16;
+constexpr int CLDB = 128 + 4;   // padded row of a quarter (32 rows) of a wave's result tile in LDS, in floats
+
+// Operand fragments of a half step (32 of K): eight 16-row tiles of x, eight of w.  The w fragments are
+// double-buffered, and so are the last two x fragments; x fragments 0..5 are used by one row of MFMAs each,
+// so the next half step's takes the register as soon as that row has been issued (the LDS read takes far
+// longer than an MFMA needs to fetch its operands).
+struct FragsBig {
+  u32x4_t a[6], a6[2], a7[2], b[2][8];
+};
+#define TIE_FRAGS(f, p)                                                                                                  \
+  asm volatile("s_waitcnt lgkmcnt(0)"                                                                                   \
+               : "+v"(f.b[p][0]), "+v"(f.b[p][1]), "+v"(f.b[p][2]), "+v"(f.b[p][3]), "+v"(f.b[p][4]), "+v"(f.b[p][5]),    \
+                 "+v"(f.b[p][6]), "+v"(f.b[p][7]), "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), \
+                 "+v"(f.a[5]), "+v"(f.a6[p]), "+v"(f.a7[p]))
+// load I (0..15) of this wave into stage `buf`: 0..7 are x rows, 8..15 w rows; one load covers 8 rows
+template <int I>
+__device__ inline void issue_big(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                 const unsigned (&voff)[LPWB], int wave) {
+  const int t = I < 8 ? wave * 8 + I : 32 + wave * 8 + (I - 8);
+  const unsigned char* src = (I < 8 ? xk : wk) + voff[I];
+  __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+}
+__device__ inline void issue_stage_big(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                       const unsigned (&voff)[LPWB], int wave) {
+  issue_big<0>(buf, xk, wk, voff, wave); issue_big<1>(buf, xk, wk, voff, wave); issue_big<2>(buf, xk, wk, voff, wave);
+  issue_big<3>(buf, xk, wk, voff, wave); issue_big<4>(buf, xk, wk, voff, wave); issue_big<5>(buf, xk, wk, voff, wave);
+  issue_big<6>(buf, xk, wk, voff, wave); issue_big<7>(buf, xk, wk, voff, wave); issue_big<8>(buf, xk, wk, voff, wave);
+  issue_big<9>(buf, xk, wk, voff, wave); issue_big<10>(buf, xk, wk, voff, wave); issue_big<11>(buf, xk, wk, voff, wave);
+  issue_big<12>(buf, xk, wk, voff, wave); issue_big<13>(buf, xk, wk, voff, wave); issue_big<14>(buf, xk, wk, voff, wave);
+  issue_big<15>(buf, xk, wk, voff, wave);
+}
+// The 64 MFMAs of a half step with the fragments of parity P, row by row.  READ: the next half step's
+// fragments are requested between them (w and the last two x fragments into the other set, x fragment i into
+// a[i] after row i).  LOAD: one global load per group of four MFMAs.
+template <int P, bool READ, bool LOAD>
+__device__ inline void half_step_big(f32x4_t (&acc)[8][8], FragsBig& f, unsigned aaddr, unsigned baddr, unsigned char* buf,
+                                     const unsigned char* xk, const unsigned char* wk, const unsigned (&voff)[LPWB],
+                                     int wave) {
+#define SB() __builtin_amdgcn_sched_barrier(0)
+#define AF(I) (I < 6 ? f.a[I < 6 ? I : 0] : (I == 6 ? f.a6[P] : f.a7[P]))
+// (written as assembly with the accumulator tied to an AGPR: left to itself the register allocator keeps
+// part of the 256 accumulator registers in VGPRs and copies them back and forth inside the loop)
+#define M1(I, J) \
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[I][J]) : "v"(AF(I)), "v"(f.b[P][J])); \
+  SB()
+#define RB(J) \
+  if (READ) f.b[P ^ 1][J] = lds_read16<(J) * 16 * ROWB>(baddr); \
+  SB()
+#define RA(I) \
+  if (READ) f.a[I] = lds_read16<(I) * 16 * ROWB>(aaddr); \
+  SB()
+#define R67()                                                  \
+  if (READ) f.a6[P ^ 1] = lds_read16<6 * 16 * ROWB>(aaddr);    \
+  SB();                                                        \
+  if (READ) f.a7[P ^ 1] = lds_read16<7 * 16 * ROWB>(aaddr);    \
+  SB()
+#define LD(G) \
+  if (LOAD) issue_big<G>(buf, xk, wk, voff, wave); \
+  SB()
+#define ROW(I, PRE0, PRE1)                             \
+  PRE0;                                                \
+  M1(I, 0); M1(I, 1); LD(2 * (I)); M1(I, 2); M1(I, 3); \
+  PRE1;                                                \
+  M1(I, 4); M1(I, 5); LD(2 * (I) + 1); M1(I, 6); M1(I, 7)
+  ROW(0, RB(0), RB(1));
+  ROW(1, RB(2); RA(0), RB(3));
+  ROW(2, RB(4); RA(1), RB(5));
+  ROW(3, RB(6); RA(2), RB(7));
+  ROW(4, RA(3), R67());
+  ROW(5, RA(4), (void)0);
+  ROW(6, RA(5), (void)0);
+  ROW(7, (void)0, (void)0);
+  if (READ) {
+    TIE_FRAGS(f, P ^ 1);
+    SB();
+  }
+#undef ROW
+#undef LD
+#undef R67
+#undef RA
+#undef RB
+#undef M1
+#undef AF
+#undef SB
+}
+__device__ inline void read_all_big(FragsBig& f, unsigned aaddr, unsigned baddr) {
+#define RB0(J) f.b[0][J] = lds_read16<(J) * 16 * ROWB>(baddr)
+#define RA0(I) f.a[I] = lds_read16<(I) * 16 * ROWB>(aaddr)
+  RB0(0); RB0(1); RB0(2); RB0(3); RB0(4); RB0(5); RB0(6); RB0(7);
+  RA0(0); RA0(1); RA0(2); RA0(3); RA0(4); RA0(5);
+  f.a6[0] = lds_read16<6 * 16 * ROWB>(aaddr);
+  f.a7[0] = lds_read16<7 * 16 * ROWB>(aaddr);
+#undef RB0
+#undef RA0
+  TIE_FRAGS(f, 0);
+}
+
+}  // namespace
+
+// No split of K here.  N: the columns of this launch (a multiple of 256); ldo as above.
+__global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                            void* __restrict__ out, int mode, int M, int N, int K,
+                                                            int pm, int ldo) {
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[NSB * STAGE_BIG];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  int bm, bn;
+  {
+    const int MB = (M + BM - 1) / BM, NB = N / BNB;
+    const int pq = 32 / pm;
+    const int MS = (MB + pm - 1) / pm;
+    const int c = blockIdx.x % 8, j = blockIdx.x / 8;
+    const int t = j / 32, r = j % 32;
+    bm = (t % MS) * pm + r % pm;
+    bn = c + 8 * ((t / MS) * pq + r / pm);
+    if (bm >= MB || bn >= NB) return;
+  }
+  const int m0 = bm * BM, n0 = bn * BNB;
+  f32x4_t acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const int KT = K / BK;
+  const int g = lane >> 4, c = lane & 15;
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
+  const unsigned off0 = c * ROWB + (((0 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned off1 = c * ROWB + (((1 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned arow = wm * 128 * ROWB, brow = (BM + wn * 128) * ROWB;
+  unsigned voff[LPWB];
+#pragma unroll
+  for (int i = 0; i < LPWB; ++i) {
+    const int row = (wave * 8 + (i & 7)) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    const int grow = i < 8 ? min(row, M - 1 - m0) : row;   // (every w row of the launch exists)
+    voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
+  }
+  const unsigned char* xk = (const unsigned char*)x + (size_t)m0 * K * 2;
+  const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2;
+#pragma unroll
+  for (int p = 0; p < NSB; ++p)
+    if (p < KT) issue_stage_big(stages + p * STAGE_BIG, xk + p * BK * 2, wk + p * BK * 2, voff, wave);
+  xk += NSB * BK * 2;
+  wk += NSB * BK * 2;
+  FragsBig f;
+  if (KT > 1) WAIT_VM(LPWB); else WAIT_VM(0);
+  __builtin_amdgcn_s_barrier();
+  read_all_big(f, lds0 + arow + off0, lds0 + brow + off0);
+  // Tile kt: the first half step multiplies the fragments of its first 32 of K and reads those of the second;
+  // then tile kt + 1 must have landed for every wave (barrier), which also means that every wave is done
+  // reading tile kt's stage: the second half step refills it with tile kt + 2 while it multiplies and reads
+  // the first fragments of tile kt + 1.
+  int st = 0, kt = 0;
+  for (; kt + NSB < KT; ++kt) {
+    const unsigned cur = lds0 + st * STAGE_BIG, nxt = lds0 + (st ^ 1) * STAGE_BIG;
+    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    WAIT_VM(0);
+    __builtin_amdgcn_s_barrier();
+    half_step_big<1, true, true>(acc, f, nxt + arow + off0, nxt + brow + off0, stages + st * STAGE_BIG, xk, wk, voff, wave);
+    xk += BK * 2;
+    wk += BK * 2;
+    st ^= 1;
+  }
+  for (; kt + 1 < KT; ++kt) {  // nothing left to load
+    const unsigned cur = lds0 + st * STAGE_BIG, nxt = lds0 + (st ^ 1) * STAGE_BIG;
+    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    WAIT_VM(0);
+    __builtin_amdgcn_s_barrier();
+    half_step_big<1, true, false>(acc, f, nxt + arow + off0, nxt + brow + off0, nullptr, nullptr, nullptr, voff, wave);
+    st ^= 1;
+  }
+  {
+    const unsigned cur = lds0 + st * STAGE_BIG;
+    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step_big<1, false, false>(acc, f, 0, 0, nullptr, nullptr, nullptr, voff, wave);
+  }
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs' results, before they are read below
+
+  // ---- the result leaves through LDS, 32 rows of the wave's 128 x 128 at a time ---------------------------
+  __syncthreads();
+  float* ct = (float*)stages + wave * (32 * CLDB);
+  const int mw = m0 + wm * 128, nw = n0 + wn * 128;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLDB + j * 16 + c] = acc[q * 2 + i][j][r];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int mq = mw + q * 32;
+    if (mode == OUT_SWIGLU) {
+      // 64 outputs per row, four per lane, four rows per pass
+      const int o = (lane & 15) * 4, rr = lane >> 4;
+      const int cg = (o / 8) * 16 + o % 8;
+      bf16_t* ob = (bf16_t*)out;
+#pragma unroll 4
+      for (int p = 0; p < 8; ++p) {
+        const int row = p * 4 + rr, m = mq + row;
+        const f32x4_t gt = *(const f32x4_t*)(ct + row * CLDB + cg);
+        const f32x4_t up = *(const f32x4_t*)(ct + row * CLDB + cg + 8);
+        if (m >= M) continue;
+        u32x2_t pk;
+        pk[0] = pack_bf16(silu_mul(gt[0], up[0]), silu_mul(gt[1], up[1]));
+        pk[1] = pack_bf16(silu_mul(gt[2], up[2]), silu_mul(gt[3], up[3]));
+        *(u32x2_t*)(ob + (size_t)m * ldo + nw / 2 + o) = pk;
+      }
+    } else {
+      const int col = (lane & 31) * 4, rr = lane >> 5;
+#pragma unroll 4
+      for (int p = 0; p < 16; ++p) {
+        const int row = p * 2 + rr, m = mq + row;
+        const f32x4_t v = *(const f32x4_t*)(ct + row * CLDB + col);
+        if (m >= M) continue;
+        const size_t idx = (size_t)m * ldo + nw + col;
+        if (mode == OUT_BF16) {
+          u32x2_t pk;
+          pk[0] = pack_bf16(v[0], v[1]);
+          pk[1] = pack_bf16(v[2], v[3]);
+          *(u32x2_t*)((bf16_t*)out + idx) = pk;
+        } else if (mode == OUT_F32) {
+          *(f32x4_t*)((float*)out + idx) = v;
+        } else {
+          f32x4_t* o = (f32x4_t*)((float*)out + idx);
+          *o = *o + v;
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
@@ -534,6 +783,7 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
 
 // Returns 0 when launched, -1 when the sizes are not this kernel's.  `scratch` (optional) is room for
 // float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
+int g_pipe_big = 0;   // tuning: 1 = 256 x 256 tiles for every whole block of 256 columns, 2 = never
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
                    size_t scratch_floats, int tune_splits, hipStream_t s) {
   if (K % BK != 0 || K < BK) return -1;
@@ -556,8 +806,47 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
     const int per = (KT + splits - 1) / splits;
     splits = (KT + per - 1) / per;   // no split without a tile
   }
+  const int ldo = mode == OUT_SWIGLU ? N / 2 : N;
+  // Whole rounds of 256 x 256 tiles first (see gemm_pipe_big_kernel), the columns that are left as above.
+  // How many blocks of 256 columns take the big tiles: all, none, or whole rounds of 256 tiles, whichever
+  // needs the fewest rounds when a big tile is priced at 1.72 small ones (measured: 113 against 65 us at
+  // K = 4096).
+  int nb_big = 0;
+  if (splits == 1 && g_pipe_big != 2 && ldo % 4 == 0) {
+    const long NB2 = N / BNB;
+    auto rounds = [&](long nb) {
+      const long rest = (N - nb * BNB + BN - 1) / BN;
+      return 1.72 * (double)((MB * nb + 255) / 256) + (double)((MB * rest + 255) / 256);
+    };
+    const long whole = ((long)MB * NB2 / 256) * 256 / MB;
+    double best = rounds(0);
+    for (long cand : {NB2, whole})
+      if (cand > 0 && rounds(cand) < best - 1e-9) {
+        best = rounds(cand);
+        nb_big = (int)cand;
+      }
+    if (g_pipe_big == 1) nb_big = (int)NB2;
+  }
+  if (nb_big > 0) {
+    const long Q2 = (nb_big + 7) / 8, QS2 = (Q2 + pq - 1) / pq;
+    const long blocks2 = 8 * QS2 * MS * 32;
+    hipLaunchKernelGGL(gemm_pipe_big_kernel, dim3((unsigned)blocks2), dim3(256), 0, s, x, w, out, mode, M, nb_big * BNB, K,
+                       pm, ldo);
+    const int n_done = nb_big * BNB;
+    if (n_done == N) return 0;
+    // the rest of the columns
+    const int N2 = N - n_done;
+    const int NBr = (N2 + BN - 1) / BN;
+    const long Qr = (NBr + 7) / 8, QSr = (Qr + pq - 1) / pq;
+    const long blocksr = 8 * QSr * MS * 32;
+    const size_t esz = mode == OUT_BF16 || mode == OUT_SWIGLU ? 2 : 4;
+    void* out2 = (char*)out + (size_t)(mode == OUT_SWIGLU ? n_done / 2 : n_done) * esz;
+    hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocksr, 1), dim3(256), 0, s, x, w + (size_t)n_done * K, out2, scratch,
+                       mode, M, N2, K, pm, ldo);
+    return 0;
+  }
   hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks, splits), dim3(256), 0, s, x, w, out, scratch, mode, M, N, K,
-                     pm);
+                     pm, ldo);
   if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,

@@ -219,6 +219,33 @@ def test_linear_mfma(m, n, k):
         assert torch.equal(again, got), "the same call must give the same bits"
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 512, 128), (1000, 816, 192), (257, 256, 64), (2048, 8448, 128)])
+def test_linear_big_tiles(m, n, k):
+    """The 256 x 256 block tiles, forced for every whole block of 256 columns (the columns that are left take
+    the 256 x 128 tiles in a second launch): every output mode against float64, with rows and columns that
+    fill no whole tile; and the choice the library makes by itself at a size where it mixes both."""
+    ops = _ops()
+    lib = ops.library()
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    ref = x.double() @ w.double().T
+    res = torch.randn(m, n, generator=g)
+    xd, wd = x.to(DEV), w.to(DEV)
+    gate_up = ref.view(m, n // 16, 2, 8)
+    gated = (torch.nn.functional.silu(gate_up[:, :, 0]) * gate_up[:, :, 1]).reshape(m, n // 2)
+    for mode in (5, 0):
+        lib.tp_linear_tune_tile(mode)
+        try:
+            _close(ops.linear(xd, wd, torch.float32), ref, 2e-5, f"f32 out, tile mode {mode}")
+            _close(ops.linear(xd, wd, torch.bfloat16), ref, 1e-2, f"bf16 out, tile mode {mode}")
+            _close(ops.linear(xd, wd, torch.float32, residual=res.clone().to(DEV)), ref + res.double(), 2e-5,
+                   f"residual, tile mode {mode}")
+            _close(ops.linear_swiglu(xd, wd), gated, 1e-2, f"gated, tile mode {mode}")
+        finally:
+            lib.tp_linear_tune_tile(0)
+
+
 @pytest.mark.parametrize("m,hidden,kp,nc", [(1, 64, 32, 48), (8, 4096, 4096, 6144), (16, 160, 96, 272), (5, 4096, 14336, 1024),
                                              (3, 96, 2048, 40)])
 def test_linear_split_norm(m, hidden, kp, nc):
