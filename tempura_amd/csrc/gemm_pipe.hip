@@ -151,6 +151,93 @@ __device__ inline void half_step(f32x4_t (&acc)[8][4], const Frags& cur, Frags& 
   read_one<4>(f, aaddr, baddr); read_one<5>(f, aaddr, baddr); read_one<6>(f, aaddr, baddr); read_one<7>(f, aaddr, baddr); \
   read_one<8>(f, aaddr, baddr); read_one<9>(f, aaddr, baddr); read_one<10>(f, aaddr, baddr); read_one<11>(f, aaddr, baddr)
 
+
+// A wave's result rows [0, ROWS) x COLS columns, laid out in LDS with rows of LD floats, to memory: rows mrow0..,
+// columns ncol0.. of the launch's N (row stride ldo).  Four rows are read from LDS before the first of them is
+// stored, so that the reads (and, when adding into `out`, the loads) overlap.
+template <int ROWS, int COLS, int LD>
+__device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0, void* out, int mode, int M, int N, int ldo) {
+  if (mode == OUT_SWIGLU) {
+    // the weight rows alternate eight gate rows and eight up rows: output column 8 b + i pairs columns
+    // 16 b + i and 16 b + 8 + i; COLS / 2 outputs per row, four per lane
+    constexpr int LPR = COLS / 8, RPP = 64 / LPR, PASSES = ROWS / RPP;
+    const int o = (lane % LPR) * 4, rr = lane / LPR;
+    const int cg = (o / 8) * 16 + o % 8;
+    bf16_t* ob = (bf16_t*)out;
+    if (ncol0 + cg >= N) return;   // N is a multiple of 16: the whole group is inside or outside
+#pragma unroll
+    for (int p0 = 0; p0 < PASSES; p0 += 4) {
+      f32x4_t gt[4], up[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int row = (p0 + u) * RPP + rr;
+        gt[u] = *(const f32x4_t*)(ct + row * LD + cg);
+        up[u] = *(const f32x4_t*)(ct + row * LD + cg + 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int m = mrow0 + (p0 + u) * RPP + rr;
+        u32x2_t pk;
+        pk[0] = pack_bf16(silu_mul(gt[u][0], up[u][0]), silu_mul(gt[u][1], up[u][1]));
+        pk[1] = pack_bf16(silu_mul(gt[u][2], up[u][2]), silu_mul(gt[u][3], up[u][3]));
+        if (m < M) *(u32x2_t*)(ob + (size_t)m * ldo + ncol0 / 2 + o) = pk;
+      }
+    }
+    return;
+  }
+  constexpr int LPR = COLS / 4, RPP = 64 / LPR, PASSES = ROWS / RPP;
+  const int col = (lane % LPR) * 4, rr = lane / LPR;
+  if (ldo % 4 == 0 && ncol0 + col + 3 < N) {
+#pragma unroll
+    for (int p0 = 0; p0 < PASSES; p0 += 4) {
+      f32x4_t v[4], old[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = *(const f32x4_t*)(ct + ((p0 + u) * RPP + rr) * LD + col);
+      if (mode == OUT_ACC_F32) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int m = mrow0 + (p0 + u) * RPP + rr;
+          old[u] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+          if (m < M) old[u] = *(const f32x4_t*)((const float*)out + (size_t)m * ldo + ncol0 + col);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int m = mrow0 + (p0 + u) * RPP + rr;
+        if (m >= M) continue;
+        const size_t idx = (size_t)m * ldo + ncol0 + col;
+        if (mode == OUT_BF16) {
+          u32x2_t pk;
+          pk[0] = pack_bf16(v[u][0], v[u][1]);
+          pk[1] = pack_bf16(v[u][2], v[u][3]);
+          *(u32x2_t*)((bf16_t*)out + idx) = pk;
+        } else if (mode == OUT_F32) {
+          *(f32x4_t*)((float*)out + idx) = v[u];
+        } else {
+          *(f32x4_t*)((float*)out + idx) = old[u] + v[u];
+        }
+      }
+    }
+    return;
+  }
+  // the last columns of an N that is no multiple of four, or a row stride that is none: element by element
+  for (int p = 0; p < PASSES; ++p) {
+    const int row = p * RPP + rr, m = mrow0 + row;
+    if (m >= M) continue;
+    const size_t idx = (size_t)m * ldo + ncol0 + col;
+    for (int e = 0; e < 4; ++e) {
+      if (ncol0 + col + e >= N) break;
+      const float v = ct[row * LD + col + e];
+      if (mode == OUT_BF16)
+        ((bf16_t*)out)[idx + e] = float_to_bf16(v);
+      else if (mode == OUT_F32)
+        ((float*)out)[idx + e] = v;
+      else
+        ((float*)out)[idx + e] += v;
+    }
+  }
+}
+
 }  // namespace
 
 // ldo: row stride of `out` in elements (N, or N / 2 for the gated mode, when the launch covers all columns;
@@ -265,62 +352,8 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  const int mw = m0 + wm * 128, nw = n0 + wn * 64;
-  if (mode == OUT_SWIGLU) {
-    // the weight rows alternate eight gate rows and eight up rows: output column 8 b + i pairs
-    // columns 16 b + i and 16 b + 8 + i; 32 outputs per row, four per lane, eight rows per pass
-    const int o = (lane & 7) * 4, rr = lane >> 3;
-    const int cg = (o / 8) * 16 + o % 8;
-    bf16_t* ob = (bf16_t*)out;
-#pragma unroll 4
-    for (int p = 0; p < 16; ++p) {
-      const int row = p * 8 + rr, m = mw + row;
-      const f32x4_t gt = *(const f32x4_t*)(ct + row * CLD + cg);
-      const f32x4_t up = *(const f32x4_t*)(ct + row * CLD + cg + 8);
-      if (m >= M || nw + cg >= N) continue;   // N is a multiple of 16: the whole group is inside or outside
-      u32x2_t pk;
-      pk[0] = pack_bf16(silu_mul(gt[0], up[0]), silu_mul(gt[1], up[1]));
-      pk[1] = pack_bf16(silu_mul(gt[2], up[2]), silu_mul(gt[3], up[3]));
-      *(u32x2_t*)(ob + (size_t)m * ldo + nw / 2 + o) = pk;
-    }
-    return;
-  }
-  const int col = (lane & 15) * 4, rr = lane >> 4;
-  const bool vec = (ldo % 4 == 0) && nw + col + 3 < N;
-#pragma unroll 4
-  for (int p = 0; p < 32; ++p) {
-    const int row = p * 4 + rr, m = mw + row;
-    const f32x4_t v = *(const f32x4_t*)(ct + row * CLD + col);
-    if (m >= M) continue;
-    const size_t idx = (size_t)m * ldo + nw + col;
-    if (vec) {
-      if (mode == OUT_BF16) {
-        u32x2_t pk;
-        pk[0] = pack_bf16(v[0], v[1]);
-        pk[1] = pack_bf16(v[2], v[3]);
-        *(u32x2_t*)((bf16_t*)out + idx) = pk;
-      } else if (mode == OUT_F32) {
-        *(f32x4_t*)((float*)out + idx) = v;
-      } else {
-        f32x4_t* o = (f32x4_t*)((float*)out + idx);
-        *o = *o + v;
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (nw + col + e >= N) break;
-        if (mode == OUT_BF16)
-          ((bf16_t*)out)[idx + e] = float_to_bf16(v[e]);
-        else if (mode == OUT_F32)
-          ((float*)out)[idx + e] = v[e];
-        else
-          ((float*)out)[idx + e] += v[e];
-      }
-    }
-  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's LDS writes before its reads
+  emit_tile<128, 64, CLD>(ct, lane, m0 + wm * 128, n0 + wn * 64, out, mode, M, N, ldo);
 }
 
 // ---- 256 x 256 block tiles ---------------------------------------------------------------------------
@@ -523,50 +556,10 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
       for (int j = 0; j < 8; ++j)
 #pragma unroll
         for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLDB + j * 16 + c] = acc[q * 2 + i][j][r];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int mq = mw + q * 32;
-    if (mode == OUT_SWIGLU) {
-      // 64 outputs per row, four per lane, four rows per pass
-      const int o = (lane & 15) * 4, rr = lane >> 4;
-      const int cg = (o / 8) * 16 + o % 8;
-      bf16_t* ob = (bf16_t*)out;
-#pragma unroll 4
-      for (int p = 0; p < 8; ++p) {
-        const int row = p * 4 + rr, m = mq + row;
-        const f32x4_t gt = *(const f32x4_t*)(ct + row * CLDB + cg);
-        const f32x4_t up = *(const f32x4_t*)(ct + row * CLDB + cg + 8);
-        if (m >= M) continue;
-        u32x2_t pk;
-        pk[0] = pack_bf16(silu_mul(gt[0], up[0]), silu_mul(gt[1], up[1]));
-        pk[1] = pack_bf16(silu_mul(gt[2], up[2]), silu_mul(gt[3], up[3]));
-        *(u32x2_t*)(ob + (size_t)m * ldo + nw / 2 + o) = pk;
-      }
-    } else {
-      const int col = (lane & 31) * 4, rr = lane >> 5;
-#pragma unroll 4
-      for (int p = 0; p < 16; ++p) {
-        const int row = p * 2 + rr, m = mq + row;
-        const f32x4_t v = *(const f32x4_t*)(ct + row * CLDB + col);
-        if (m >= M) continue;
-        const size_t idx = (size_t)m * ldo + nw + col;
-        if (mode == OUT_BF16) {
-          u32x2_t pk;
-          pk[0] = pack_bf16(v[0], v[1]);
-          pk[1] = pack_bf16(v[2], v[3]);
-          *(u32x2_t*)((bf16_t*)out + idx) = pk;
-        } else if (mode == OUT_F32) {
-          *(f32x4_t*)((float*)out + idx) = v;
-        } else {
-          f32x4_t* o = (f32x4_t*)((float*)out + idx);
-          *o = *o + v;
-        }
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // (this wave's LDS writes before its reads, and the reverse below)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    emit_tile<32, 128, CLDB>(ct, lane, mw + q * 32, nw, out, mode, M, N, ldo);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
 }
 
@@ -720,61 +713,8 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  const int mw = m0 + wm * 32, nw = n0 + wn * 64;
-  if (mode == OUT_SWIGLU) {
-    const int o = (lane & 7) * 4, rr = lane >> 3;
-    const int cg = (o / 8) * 16 + o % 8;
-    bf16_t* ob = (bf16_t*)out;
-    const int half = N / 2;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int row = p * 8 + rr, m = mw + row;
-      const f32x4_t gt = *(const f32x4_t*)(ct + row * CLD + cg);
-      const f32x4_t up = *(const f32x4_t*)(ct + row * CLD + cg + 8);
-      if (m >= M || nw + cg >= N) continue;
-      u32x2_t pk;
-      pk[0] = pack_bf16(silu_mul(gt[0], up[0]), silu_mul(gt[1], up[1]));
-      pk[1] = pack_bf16(silu_mul(gt[2], up[2]), silu_mul(gt[3], up[3]));
-      *(u32x2_t*)(ob + (size_t)m * half + nw / 2 + o) = pk;
-    }
-    return;
-  }
-  const int col = (lane & 15) * 4, rr = lane >> 4;
-  const bool vec = (N % 4 == 0) && nw + col + 3 < N;
-#pragma unroll
-  for (int p = 0; p < 8; ++p) {
-    const int row = p * 4 + rr, m = mw + row;
-    const f32x4_t v = *(const f32x4_t*)(ct + row * CLD + col);
-    if (m >= M) continue;
-    const size_t idx = (size_t)m * N + nw + col;
-    if (vec) {
-      if (mode == OUT_BF16) {
-        u32x2_t pk;
-        pk[0] = pack_bf16(v[0], v[1]);
-        pk[1] = pack_bf16(v[2], v[3]);
-        *(u32x2_t*)((bf16_t*)out + idx) = pk;
-      } else if (mode == OUT_F32) {
-        *(f32x4_t*)((float*)out + idx) = v;
-      } else {
-        f32x4_t* o = (f32x4_t*)((float*)out + idx);
-        *o = *o + v;
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (nw + col + e >= N) break;
-        if (mode == OUT_BF16)
-          ((bf16_t*)out)[idx + e] = float_to_bf16(v[e]);
-        else if (mode == OUT_F32)
-          ((float*)out)[idx + e] = v[e];
-        else
-          ((float*)out)[idx + e] += v[e];
-      }
-    }
-  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  emit_tile<32, 64, CLD>(ct, lane, m0 + wm * 32, n0 + wn * 64, out, mode, M, N, mode == OUT_SWIGLU ? N / 2 : N);
 }
 
 // Defined in gemm_mfma.hip.
