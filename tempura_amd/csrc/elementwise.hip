@@ -118,17 +118,50 @@ extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void*
 // (the row then holds q heads only).
 // grid: (tokens, head blocks); a thread owns one pair (or two plain elements) of one head, so
 // every load of the row is in flight at once.
+// cosine and sine (times factor) of pos * inv_freq: the product in float64, reduced to [0, 2 pi) there
+__device__ inline void rope_cos_sin(int pos, double inv_freq, float factor, float& c, float& sn) {
+  const double turns = (double)pos * inv_freq * 0.15915494309189535;
+  const float rest = (float)((turns - floor(turns)) * 6.283185307179586);
+  sincosf(rest, &sn, &c);
+  c *= factor;
+  sn *= factor;
+}
+
+// table[t, d] = (cos, sin) of token t's position times inv_freq[d]: long steps compute it once and every
+// layer's rotation reads it
+__global__ void rope_table_kernel(const int* __restrict__ positions, const double* __restrict__ inv_freq, int half,
+                                  float factor, size_t total, float2* __restrict__ table) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float c, sn;
+  rope_cos_sin(positions[i / half], inv_freq[i % half], factor, c, sn);
+  table[i] = make_float2(c, sn);
+}
+
+extern "C" int tp_rope_table(const int* positions, const double* inv_freq, int rotary_dim, float factor, int n,
+                             float* table, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && rotary_dim > 0 && rotary_dim % 2 == 0 && inv_freq != nullptr, "rope_table: bad sizes");
+  const size_t total = (size_t)n * (rotary_dim / 2);
+  if (total == 0) return 0;
+  TP_REQUIRE((total + 255) / 256 < ((size_t)1 << 31), "rope_table: too many tokens");
+  hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, positions, inv_freq,
+                     rotary_dim / 2, factor, total, (float2*)table);
+  TP_CHECK_LAUNCH("rope_table");
+  return 0;
+}
+
 template <typename TQ, typename TC>
 __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stride,
                                      const int* __restrict__ positions, const int* __restrict__ slots,
                                      const double* __restrict__ inv_freq, int rotary_dim, float factor,
                                      int n_heads, int n_kv, int head_dim, TQ* __restrict__ q_out,
                                      TC* __restrict__ k_cache, TC* __restrict__ v_cache, int page_size,
-                                     int pairs, int heads_per_block, int splits, size_t split_stride) {
+                                     int pairs, int heads_per_block, int splits, size_t split_stride,
+                                     const float2* __restrict__ cos_sin, int with_values) {
   const int t = blockIdx.x;
   const int hl = threadIdx.x / pairs, d = threadIdx.x % pairs;   // pairs = head_dim / 2
   const int h = blockIdx.y * heads_per_block + hl;
-  const int total_heads = n_heads + (slots ? 2 * n_kv : 0);
+  const int total_heads = n_heads + (slots ? (with_values ? 2 : 1) * n_kv : 0);
   if (hl >= heads_per_block || h >= total_heads) return;
   const int half = rotary_dim / 2;
   const float* row = qkv + (size_t)t * row_stride + (size_t)h * head_dim;
@@ -165,12 +198,14 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
     off = (size_t)(slot % page_size);
   }
   if (h < n_heads + n_kv && d < half) {  // q and k heads rotate
-    const double turns = (double)positions[t] * inv_freq[d] * 0.15915494309189535;
-    const float rest = (float)((turns - floor(turns)) * 6.283185307179586);
     float sn, c;
-    sincosf(rest, &sn, &c);
-    c *= factor;
-    sn *= factor;
+    if (cos_sin != nullptr) {   // this step's table (rope_table_kernel: the same arithmetic, once for all layers)
+      const float2 cs = cos_sin[(size_t)t * half + d];
+      c = cs.x;
+      sn = cs.y;
+    } else {
+      rope_cos_sin(positions[t], inv_freq[d], factor, c, sn);
+    }
     const float x0 = y0, x1 = y1;
     y0 = x0 * c - x1 * sn;
     y1 = x0 * sn + x1 * c;
@@ -190,10 +225,148 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
   }
 }
 
+// The same rotation for the q and k heads of long steps, four pairs per thread (16-byte loads, 8-byte
+// stores of bfloat16): needs head_dim, rotary_dim and the row stride to be multiples of eight.
+// grid: (tokens, blocks of 256 threads over heads x head_dim / 8).
+template <typename T>
+__device__ inline void store4(T* p, const float (&v)[4]) {
+  if constexpr (sizeof(T) == 2) {
+    union {
+      bf16_t h[4];
+      uint2 u;
+    } pk;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pk.h[e] = float_to_bf16(v[e]);
+    *(uint2*)p = pk.u;
+  } else {
+    *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+  }
+}
+
+template <typename TQ, typename TC>
+__global__ void rope_qk4_kernel(const float* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
+                                const int* __restrict__ slots, const double* __restrict__ inv_freq, int rotary_dim,
+                                float factor, int n_heads, int n_rot_heads, int n_kv, int head_dim,
+                                TQ* __restrict__ q_out, TC* __restrict__ k_cache, int page_size, int splits,
+                                size_t split_stride, const float2* __restrict__ cos_sin) {
+  const int t = blockIdx.x;
+  const int tph = head_dim / 8;                       // threads per head
+  const int idx = blockIdx.y * blockDim.x + threadIdx.x;
+  const int h = idx / tph, j = idx % tph;
+  if (h >= n_rot_heads) return;
+  const int half = rotary_dim / 2;
+  // the eight elements this thread moves: four rotary pairs (d, d + half), or eight plain elements
+  const bool rot = 4 * j < half;
+  const int i0 = rot ? 4 * j : rotary_dim + 8 * (j - half / 4);
+  const int i1 = rot ? i0 + half : i0 + 4;
+  const float* row = qkv + (size_t)t * row_stride + (size_t)h * head_dim;
+  float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+  {
+    float4 pa[16], pb[16];   // all loads in flight before the first sum; splits <= 16, added in ascending order
+#pragma unroll
+    for (int sp = 0; sp < 16; ++sp)
+      if (sp < splits) {
+        pa[sp] = *(const float4*)(row + (size_t)sp * split_stride + i0);
+        pb[sp] = *(const float4*)(row + (size_t)sp * split_stride + i1);
+      }
+#pragma unroll
+    for (int sp = 0; sp < 16; ++sp)
+      if (sp < splits) {
+        a[0] += pa[sp].x; a[1] += pa[sp].y; a[2] += pa[sp].z; a[3] += pa[sp].w;
+        b[0] += pb[sp].x; b[1] += pb[sp].y; b[2] += pb[sp].z; b[3] += pb[sp].w;
+      }
+  }
+  if (rot) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float sn, c;
+      if (cos_sin != nullptr) {
+        const float2 cs = cos_sin[(size_t)t * half + i0 + e];
+        c = cs.x;
+        sn = cs.y;
+      } else {
+        rope_cos_sin(positions[t], inv_freq[i0 + e], factor, c, sn);
+      }
+      const float x0 = a[e], x1 = b[e];
+      a[e] = x0 * c - x1 * sn;
+      b[e] = x0 * sn + x1 * c;
+    }
+  }
+  if (h < n_heads) {
+    TQ* o = q_out + ((size_t)t * n_heads + h) * head_dim;
+    store4(o + i0, a);
+    store4(o + i1, b);
+  } else {
+    const int slot = slots[t];
+    const size_t page = (size_t)(slot / page_size), off = (size_t)(slot % page_size);
+    TC* o = k_cache + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+    store4(o + i0, a);
+    store4(o + i1, b);
+  }
+}
+
+// The values of long steps: a thread takes one element of one kv head for sixteen consecutive tokens and
+// stores each run of eight whose cache places follow one another from a multiple of eight (always so inside
+// a prompt portion) as one 16-byte piece of the transposed layout, instead of eight scattered elements.
+// grid: (ceil(n / 16), kv heads); block: head_dim threads.
+template <typename TC>
+__global__ void value_write_kernel(const float* __restrict__ qkv, int row_stride, const int* __restrict__ slots,
+                                   int n, int v_col0, int n_kv, int head_dim, TC* __restrict__ v_cache,
+                                   int page_size, int splits, size_t split_stride) {
+  const int t0 = blockIdx.x * 16, kh = blockIdx.y, d = threadIdx.x;
+  if (d >= head_dim) return;
+  const float* col = qkv + (size_t)v_col0 + (size_t)kh * head_dim + d;
+  float y[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) y[i] = 0.f;
+  for (int sp = 0; sp < splits; ++sp) {   // ascending order, all sixteen loads of a split in flight
+    float p[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) p[i] = t0 + i < n ? col[(size_t)sp * split_stride + (size_t)(t0 + i) * row_stride] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) y[i] += p[i];
+  }
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    const int tg = t0 + 8 * g;
+    if (tg >= n) break;
+    const int s0 = slots[tg];
+    bool run = tg + 8 <= n && (s0 & 7) == 0 && page_size % 8 == 0;
+    if (run) {
+#pragma unroll
+      for (int i = 1; i < 8; ++i) run = run && slots[tg + i] == s0 + i;
+    }
+    if (run) {
+      const size_t page = (size_t)(s0 / page_size), off = (size_t)(s0 % page_size);
+      TC* o = v_cache + ((page * n_kv + kh) * head_dim + d) * page_size + off;
+      if constexpr (sizeof(TC) == 2) {
+        union {
+          bf16_t h[8];
+          uint4 v;
+        } pk;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pk.h[i] = float_to_bf16(y[8 * g + i]);
+        *(uint4*)o = pk.v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) from_float(o + i, y[8 * g + i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (tg + i >= n) break;
+        const int sl = slots[tg + i];
+        const size_t page = (size_t)(sl / page_size), off = (size_t)(sl % page_size);
+        from_float(v_cache + ((page * n_kv + kh) * head_dim + d) * page_size + off, y[8 * g + i]);
+      }
+    }
+  }
+}
+
 extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* positions, const int* slots,
                                 const double* inv_freq, int rotary_dim, float factor, int n, int n_heads,
                                 int n_kv, int head_dim, void* q_out, int q_dt, void* k_cache, void* v_cache,
-                                int cache_dt, int page_size, int splits, hipStream_t s) {
+                                int cache_dt, int page_size, int splits, const float* cos_sin, hipStream_t s) {
   TP_REQUIRE(n >= 0 && n_heads > 0 && n_kv >= 0 && head_dim > 0, "rope_kv_write: bad sizes");
   TP_REQUIRE(splits >= 1 && splits <= 16, "rope_kv_write: bad number of partial sums");
   const size_t split_stride = (size_t)n * row_stride;   // qkv is [splits, n, row_stride]
@@ -207,13 +380,38 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
   const int pairs = head_dim / 2;
   const int threads = pairs <= 256 ? 256 : 512;
   const int hpb = threads / pairs;
-  const int total_heads = n_heads + (slots ? 2 * n_kv : 0);
+  // long steps write their values sixteen tokens at a time (value_write_kernel)
+  const bool grouped_values = slots != nullptr && n >= 64 && n_kv <= 65535;
+  const int total_heads = n_heads + (slots ? (grouped_values ? 1 : 2) * n_kv : 0);
   const dim3 grid(n, (total_heads + hpb - 1) / hpb);
   TP_REQUIRE(grid.y <= 65535, "rope_kv_write: too many heads");
+  // long steps: q and k four pairs per thread, v sixteen tokens per thread
+  if (n >= 64 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 4 == 0 && (slots == nullptr || grouped_values) &&
+      ((uintptr_t)qkv % 16) == 0 && (split_stride % 4) == 0) {
+    const int n_rot_heads = n_heads + (slots ? n_kv : 0);
+    const int work = n_rot_heads * (head_dim / 8);
+    const dim3 g4(n, (work + 255) / 256);
+    TP_REQUIRE(g4.y <= 65535, "rope_kv_write: too many heads");
+#define LAUNCH4(TQ, TC)                                                                                               \
+  hipLaunchKernelGGL((rope_qk4_kernel<TQ, TC>), g4, dim3(256), 0, s, qkv, row_stride, positions, slots, inv_freq,      \
+                     rotary_dim, factor, n_heads, n_rot_heads, n_kv, head_dim, (TQ*)q_out, (TC*)k_cache, page_size, \
+                     splits, split_stride, (const float2*)cos_sin)
+    if (q_dt == TP_F32 && cache_dt == TP_F32)
+      LAUNCH4(float, float);
+    else if (q_dt == TP_BF16 && cache_dt == TP_BF16)
+      LAUNCH4(bf16_t, bf16_t);
+    else if (q_dt == TP_F32 && cache_dt == TP_BF16)
+      LAUNCH4(float, bf16_t);
+    else if (q_dt == TP_BF16 && cache_dt == TP_F32)
+      LAUNCH4(bf16_t, float);
+    else
+      TP_REQUIRE(false, "rope_kv_write: unknown dtypes %d %d", q_dt, cache_dt);
+#undef LAUNCH4
+  } else {
 #define LAUNCH(TQ, TC)                                                                                    \
   hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), grid, dim3(threads), 0, s, qkv, row_stride, positions, \
                      slots, inv_freq, rotary_dim, factor, n_heads, n_kv, head_dim, (TQ*)q_out, (TC*)k_cache, \
-                     (TC*)v_cache, page_size, pairs, hpb, splits, split_stride)
+                     (TC*)v_cache, page_size, pairs, hpb, splits, split_stride, (const float2*)cos_sin, grouped_values ? 0 : 1)
   if (q_dt == TP_F32 && cache_dt == TP_F32)
     LAUNCH(float, float);
   else if (q_dt == TP_BF16 && cache_dt == TP_BF16)
@@ -225,6 +423,17 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
   else
     TP_REQUIRE(false, "rope_kv_write: unknown dtypes %d %d", q_dt, cache_dt);
 #undef LAUNCH
+  }
+  if (grouped_values) {
+    const dim3 vgrid((n + 15) / 16, n_kv);
+    const int v_col0 = (n_heads + n_kv) * head_dim;
+    if (cache_dt == TP_BF16)
+      hipLaunchKernelGGL((value_write_kernel<bf16_t>), vgrid, dim3((head_dim + 63) / 64 * 64), 0, s, qkv, row_stride, slots, n,
+                         v_col0, n_kv, head_dim, (bf16_t*)v_cache, page_size, splits, split_stride);
+    else
+      hipLaunchKernelGGL((value_write_kernel<float>), vgrid, dim3((head_dim + 63) / 64 * 64), 0, s, qkv, row_stride, slots, n,
+                         v_col0, n_kv, head_dim, (float*)v_cache, page_size, splits, split_stride);
+  }
   TP_CHECK_LAUNCH("rope_kv_write");
   return 0;
 }

@@ -42,6 +42,8 @@ class StepContext:
     logit_rows[m]     flattened token indices whose logits are returned
     Host copies (``q_starts``, ``q_lens``, ``ctx_lens``, ``state_slot_list``) serve parts
     that loop over requests on the host.
+    ``shared``: what the parts of several layers compute once per step and keep under a key of
+    their own (a rotation table, for instance); empty when the step begins.
     """
 
     def __init__(self):
@@ -63,6 +65,7 @@ class StepContext:
         self.q_lens: List[int] = []
         self.ctx_lens: List[int] = []
         self.state_slot_list: List[int] = []
+        self.shared: dict = {}
 
 
 class _DecodeGraph:

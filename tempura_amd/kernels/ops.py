@@ -324,10 +324,12 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
 def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
                   inv_freq: Optional[torch.Tensor], rotary_dim: int, factor: float, num_heads: int,
                   num_kv_heads: int, head_dim: int, k_cache: Optional[torch.Tensor],
-                  v_cache: Optional[torch.Tensor], q_dtype: torch.dtype) -> torch.Tensor:
+                  v_cache: Optional[torch.Tensor], q_dtype: torch.dtype,
+                  cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotate q and k of float32 rows [n, (heads + 2 kv_heads) * head_dim] (or the ``Partials`` of the
     projection that makes them), store k and v into the cache rows ``slots`` and return q as q_dtype
-    [n, heads, head_dim].  With ``slots`` None the rows hold q only and nothing is stored."""
+    [n, heads, head_dim].  With ``slots`` None the rows hold q only and nothing is stored.
+    ``cos_sin``: this step's table from ``rope_table`` (the same values, computed once for all layers)."""
     if _backend is not None:
         return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,
                                       num_kv_heads, head_dim, k_cache, v_cache, q_dtype)
@@ -354,11 +356,29 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
     if rotary_dim:
         _need(inv_freq is not None and inv_freq.dtype == torch.float64 and inv_freq.numel() == rotary_dim // 2,
               "rope_kv_write: inv_freq must be float64 [rotary_dim / 2]")
+    if cos_sin is not None:
+        _need(cos_sin.is_cuda and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
+              and tuple(cos_sin.shape) == (n, rotary_dim // 2, 2), "rope_kv_write: table must be float32 [n, rotary_dim / 2, 2]")
     q = torch.empty((n, num_heads, head_dim), dtype=q_dtype, device=qkv.device)
     _call("tp_rope_kv_write", _ptr(qkv), qkv.shape[1], _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
           ctypes.c_float(factor), n, num_heads, num_kv_heads, head_dim, _ptr(q), _dtcode(q_dtype),
-          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, splits, _stream())
+          _ptr(k_cache), _ptr(v_cache), cache_dt, page_size, splits, _ptr(cos_sin), _stream())
     return q
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int, factor: float) -> torch.Tensor:
+    """float32 [n, rotary_dim / 2, 2]: cosine and sine (times factor) of every token's angles, as
+    ``rope_kv_write`` would compute them itself."""
+    if _backend is not None:
+        return None
+    _dev_ok(positions, inv_freq)
+    n = positions.numel()
+    _i32(positions, n, "positions") if n else None
+    _need(rotary_dim > 0 and inv_freq.dtype == torch.float64 and inv_freq.numel() == rotary_dim // 2,
+          "rope_table: inv_freq must be float64 [rotary_dim / 2]")
+    table = torch.empty((n, rotary_dim // 2, 2), dtype=torch.float32, device=positions.device)
+    _call("tp_rope_table", _ptr(positions), _ptr(inv_freq), rotary_dim, ctypes.c_float(factor), n, _ptr(table), _stream())
+    return table
 
 
 #: bfloat16 attention may use the matrix-core kernels

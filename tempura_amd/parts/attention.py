@@ -80,13 +80,14 @@ class PagedAttention(Mixer):
                 qkv = torch.cat([q2, k2, qkv[:, self.q_dim + self.kv_dim:]], dim=1).contiguous()
             else:
                 qkv = q2.contiguous()
-            inv_freq, rotary_dim, factor = None, 0, 1.0
+            inv_freq, rotary_dim, factor, table = None, 0, 1.0, None
         else:
             inv_freq, rotary_dim, factor = rot
+            table = self.position.table(ctx) if hasattr(self.position, "table") else None
         q = ops.rope_kv_write(
             qkv, ctx.positions, ctx.slot_mapping[cache.group] if cache.writes else None,
             inv_freq, rotary_dim, factor, self.num_heads, self.num_kv_heads, self.head_dim,
-            cache.k if cache.writes else None, cache.v if cache.writes else None, self.dtype)
+            cache.k if cache.writes else None, cache.v if cache.writes else None, self.dtype, table)
         a = ops.paged_attention(
             q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
             ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,

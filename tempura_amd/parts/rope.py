@@ -13,6 +13,7 @@ import math
 
 import torch
 
+from ..kernels import ops
 from .base import PositionEncoding, register_part
 
 
@@ -56,11 +57,25 @@ class RotaryPosition(PositionEncoding):
         self.head_dim = int(p["head_dim"])
         self.rotary_dim = int(p.get("rotary_dim") or self.head_dim)
         self.factor = float(p.get("attn_factor", 1.0))
-        self.inv_freq = rotary_inv_freq(self.head_dim, float(p["theta"]), p.get("scaling"),
-                                        self.rotary_dim).to(device)
+        inv_freq = rotary_inv_freq(self.head_dim, float(p["theta"]), p.get("scaling"), self.rotary_dim)
+        self.inv_freq = inv_freq.to(device)
+        # layers whose rotations have the same frequencies share one table per step
+        self._table_key = ("rope", self.rotary_dim, self.factor, hash(tuple(inv_freq.tolist())))
+
+    #: steps with at least this many tokens compute cosines and sines once for all layers
+    TABLE_FROM = 256
 
     def rotary(self):
         return self.inv_freq, self.rotary_dim, self.factor
+
+    def table(self, ctx):
+        """This step's [tokens, rotary_dim / 2, 2] cosines and sines, shared by every layer whose rotation has
+        the same frequencies; None for short steps (the rotation kernel then computes them itself)."""
+        if ctx.num_tokens < self.TABLE_FROM or self.rotary_dim == 0:
+            return None
+        if self._table_key not in ctx.shared:
+            ctx.shared[self._table_key] = ops.rope_table(ctx.positions, self.inv_freq, self.rotary_dim, self.factor)
+        return ctx.shared[self._table_key]
 
 
 class NoPosition(PositionEncoding):

@@ -98,6 +98,53 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
     q2 = ops.rope_kv_write(qkv[:, : heads * d].contiguous().to(DEV), pos.to(DEV), None, inv.to(DEV), rot, 1.0,
                            heads, kv, d, None, None, dtype)
     assert torch.equal(q2, q)
+    # cosines and sines from the step's table: the same bits as when the kernel computes them itself
+    if rot:
+        table = ops.rope_table(pos.to(DEV), inv.to(DEV), rot, 1.0)
+        k3, v3 = kc.to(DEV), vc.to(DEV)
+        q3 = ops.rope_kv_write(qkv.to(DEV), pos.to(DEV), slots.to(DEV), inv.to(DEV), rot, 1.0, heads, kv, d, k3, v3,
+                               dtype, table)
+        assert torch.equal(q3, q) and torch.equal(k3, kd) and torch.equal(v3, vd)
+        ang = pos.double()[:, None] * inv.double()[None, :]
+        _close(table[..., 0], torch.cos(ang), 2e-6, "table cosines")
+        _close(table[..., 1], torch.sin(ang), 2e-6, "table sines")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv,d,page,n", [(4, 2, 64, 16, 150), (3, 1, 48, 8, 77), (8, 2, 128, 32, 300)])
+def test_rope_kv_write_long_step(dtype, heads, kv, d, page, n):
+    """Long steps store their values in runs of eight tokens where the cache places allow it: a prompt portion
+    that starts in the middle of a page, single tokens scattered between, a tail that fills no run."""
+    ops = _ops()
+    from tempura_amd.parts.rope import rotary_inv_freq
+    g = torch.Generator().manual_seed(5)
+    pages = (n + page - 1) // page + 6
+    qkv = torch.randn(n, (heads + 2 * kv) * d, generator=g)
+    pos = torch.randint(0, 5000, (n,), generator=g, dtype=torch.int32)
+    order = torch.randperm(pages, generator=g).tolist()
+    first = n * 2 // 3
+    # a portion of `first` tokens that starts five tokens into its first page and walks shuffled pages
+    slots = [order[(5 + i) // page] * page + (5 + i) % page for i in range(first)]
+    used = set(slots)
+    rest = [s for s in torch.randperm(pages * page, generator=g).tolist() if s not in used][: n - first]
+    slots = torch.tensor(slots + rest, dtype=torch.int32)
+    inv = rotary_inv_freq(d, 10000.0, None, d)
+    kc = torch.zeros(pages, kv, page, d, dtype=dtype)
+    vc = torch.zeros(pages, kv, d, page, dtype=dtype)
+    kr, vr = kc.clone(), vc.clone()
+    qr = emu.rope_kv_write(qkv, pos, slots, inv, d, 1.0, heads, kv, d, kr, vr, torch.float64)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    q = ops.rope_kv_write(qkv.to(DEV), pos.to(DEV), slots.to(DEV), inv.to(DEV), d, 1.0, heads, kv, d, kd, vd, dtype)
+    tol = 2e-6 if dtype == torch.float32 else 8e-3
+    _close(q, qr, tol, "q")
+    _close(kd, kr, tol, "k cache")
+    _close(vd, vr, tol, "v cache")
+    # token by token (the short-step kernel) gives the same bits
+    k1, v1 = kc.to(DEV), vc.to(DEV)
+    for i in range(0, n, 40):
+        ops.rope_kv_write(qkv[i: i + 40].to(DEV), pos[i: i + 40].to(DEV), slots[i: i + 40].to(DEV), inv.to(DEV), d, 1.0,
+                          heads, kv, d, k1, v1, dtype)
+    assert torch.equal(k1, kd) and torch.equal(v1, vd)
 
 
 def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, allow_fast=True):
