@@ -380,13 +380,14 @@ extern "C" int tp_rope_kv_write(const float* qkv, int row_stride, const int* pos
   const int pairs = head_dim / 2;
   const int threads = pairs <= 256 ? 256 : 512;
   const int hpb = threads / pairs;
-  // long steps write their values sixteen tokens at a time (value_write_kernel)
-  const bool grouped_values = slots != nullptr && n >= 64 && n_kv <= 65535;
+  // long steps (prompt portions, mostly) write their values sixteen tokens at a time (value_write_kernel);
+  // a batch of single decoded tokens has no runs, and a second kernel would only cost it a launch
+  const bool grouped_values = slots != nullptr && n >= 256 && n_kv <= 65535;
   const int total_heads = n_heads + (slots ? (grouped_values ? 1 : 2) * n_kv : 0);
   const dim3 grid(n, (total_heads + hpb - 1) / hpb);
   TP_REQUIRE(grid.y <= 65535, "rope_kv_write: too many heads");
   // long steps: q and k four pairs per thread, v sixteen tokens per thread
-  if (n >= 64 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 4 == 0 && (slots == nullptr || grouped_values) &&
+  if (n >= 256 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 4 == 0 && (slots == nullptr || grouped_values) &&
       ((uintptr_t)qkv % 16) == 0 && (split_stride % 4) == 0) {
     const int n_rot_heads = n_heads + (slots ? n_kv : 0);
     const int work = n_rot_heads * (head_dim / 8);

@@ -111,7 +111,7 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,kv,d,page,n", [(4, 2, 64, 16, 150), (3, 1, 48, 8, 77), (8, 2, 128, 32, 300)])
+@pytest.mark.parametrize("heads,kv,d,page,n", [(4, 2, 64, 16, 300), (3, 1, 48, 8, 277), (8, 2, 128, 32, 600), (2, 2, 12, 16, 260)])
 def test_rope_kv_write_long_step(dtype, heads, kv, d, page, n):
     """Long steps store their values in runs of eight tokens where the cache places allow it: a prompt portion
     that starts in the middle of a page, single tokens scattered between, a tail that fills no run."""
