@@ -152,11 +152,100 @@ __device__ inline void half_step(f32x4_t (&acc)[8][4], const Frags& cur, Frags& 
   read_one<8>(f, aaddr, baddr); read_one<9>(f, aaddr, baddr); read_one<10>(f, aaddr, baddr); read_one<11>(f, aaddr, baddr)
 
 
+// The epilogue's fast path, for a wave tile that lies inside the result with rows of `out` aligned to 16 bytes:
+// a lane moves 16 bytes per row (eight bfloat16 or four float32 columns), the output pointer steps by a uniform
+// stride from pass to pass, and nothing is compared.  (Measured on 256 x 256 tiles: per row and lane a 64-bit
+// multiply for the address, a row check and a branch took as long as the store itself, and stores of 8 bytes
+// per lane twice as long as stores of 16.)
+template <int ROWS, int COLS, int LD>
+__device__ inline void emit_tile_fast(const float* ct, int lane, int mrow0, int ncol0, void* out, int mode, int ldo) {
+  if (mode == OUT_SWIGLU) {
+    // eight outputs per lane: the eight gate columns of a group of sixteen and the eight up columns after them
+    constexpr int LPR = COLS / 16, RPP = 64 / LPR, PASSES = ROWS / RPP, B = PASSES < 4 ? PASSES : 4;
+    const int o = (lane % LPR) * 8, rr = lane / LPR;
+    const float* src = ct + rr * LD + (lane % LPR) * 16;
+    bf16_t* dst = (bf16_t*)out + (size_t)(mrow0 + rr) * ldo + ncol0 / 2 + o;
+    const size_t step = (size_t)RPP * ldo;
+#pragma unroll
+    for (int p0 = 0; p0 < PASSES; p0 += B) {
+      f32x4_t g0[B], g1[B], u0[B], u1[B];
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        const float* r = src + (p0 + u) * RPP * LD;
+        g0[u] = *(const f32x4_t*)(r);
+        g1[u] = *(const f32x4_t*)(r + 4);
+        u0[u] = *(const f32x4_t*)(r + 8);
+        u1[u] = *(const f32x4_t*)(r + 12);
+      }
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        u32x4_t pk;
+        pk[0] = pack_bf16(silu_mul(g0[u][0], u0[u][0]), silu_mul(g0[u][1], u0[u][1]));
+        pk[1] = pack_bf16(silu_mul(g0[u][2], u0[u][2]), silu_mul(g0[u][3], u0[u][3]));
+        pk[2] = pack_bf16(silu_mul(g1[u][0], u1[u][0]), silu_mul(g1[u][1], u1[u][1]));
+        pk[3] = pack_bf16(silu_mul(g1[u][2], u1[u][2]), silu_mul(g1[u][3], u1[u][3]));
+        *(u32x4_t*)(dst + (p0 + u) * step) = pk;
+      }
+    }
+    return;
+  }
+  if (mode == OUT_BF16) {
+    constexpr int LPR = COLS / 8, RPP = 64 / LPR, PASSES = ROWS / RPP, B = PASSES < 4 ? PASSES : 4;
+    const int col = (lane % LPR) * 8, rr = lane / LPR;
+    const float* src = ct + rr * LD + col;
+    bf16_t* dst = (bf16_t*)out + (size_t)(mrow0 + rr) * ldo + ncol0 + col;
+    const size_t step = (size_t)RPP * ldo;
+#pragma unroll
+    for (int p0 = 0; p0 < PASSES; p0 += B) {
+      f32x4_t a[B], b[B];
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        a[u] = *(const f32x4_t*)(src + (p0 + u) * RPP * LD);
+        b[u] = *(const f32x4_t*)(src + (p0 + u) * RPP * LD + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        u32x4_t pk;
+        pk[0] = pack_bf16(a[u][0], a[u][1]);
+        pk[1] = pack_bf16(a[u][2], a[u][3]);
+        pk[2] = pack_bf16(b[u][0], b[u][1]);
+        pk[3] = pack_bf16(b[u][2], b[u][3]);
+        *(u32x4_t*)(dst + (p0 + u) * step) = pk;
+      }
+    }
+    return;
+  }
+  constexpr int LPR = COLS / 4, RPP = 64 / LPR, PASSES = ROWS / RPP, B = PASSES < 4 ? PASSES : 4;
+  const int col = (lane % LPR) * 4, rr = lane / LPR;
+  const float* src = ct + rr * LD + col;
+  float* dst = (float*)out + (size_t)(mrow0 + rr) * ldo + ncol0 + col;
+  const size_t step = (size_t)RPP * ldo;
+#pragma unroll
+  for (int p0 = 0; p0 < PASSES; p0 += B) {
+    f32x4_t v[B], old[B];
+#pragma unroll
+    for (int u = 0; u < B; ++u) v[u] = *(const f32x4_t*)(src + (p0 + u) * RPP * LD);
+    if (mode == OUT_ACC_F32) {
+#pragma unroll
+      for (int u = 0; u < B; ++u) old[u] = *(const f32x4_t*)(dst + (p0 + u) * step);
+#pragma unroll
+      for (int u = 0; u < B; ++u) *(f32x4_t*)(dst + (p0 + u) * step) = old[u] + v[u];
+    } else {
+#pragma unroll
+      for (int u = 0; u < B; ++u) *(f32x4_t*)(dst + (p0 + u) * step) = v[u];
+    }
+  }
+}
+
 // A wave's result rows [0, ROWS) x COLS columns, laid out in LDS with rows of LD floats, to memory: rows mrow0..,
 // columns ncol0.. of the launch's N (row stride ldo).  Four rows are read from LDS before the first of them is
 // stored, so that the reads (and, when adding into `out`, the loads) overlap.
 template <int ROWS, int COLS, int LD>
 __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0, void* out, int mode, int M, int N, int ldo) {
+  if (mrow0 + ROWS <= M && ncol0 + COLS <= N && ldo % 8 == 0 && ((uintptr_t)out & 15) == 0) {
+    emit_tile_fast<ROWS, COLS, LD>(ct, lane, mrow0, ncol0, out, mode, ldo);
+    return;
+  }
   if (mode == OUT_SWIGLU) {
     // the weight rows alternate eight gate rows and eight up rows: output column 8 b + i pairs columns
     // 16 b + i and 16 b + 8 + i; COLS / 2 outputs per row, four per lane
