@@ -18,9 +18,11 @@
 //    the 16 rows x 16 bytes that a quarter wave reads then fall into 16 different bank groups.
 //  * blocks go to the eight XCDs round robin; the blocks that one XCD runs at a time form a patch of
 //    (row blocks x column blocks) that share their operand tiles through that XCD's L2.
-//  * the result leaves through LDS, so that every store covers whole cache lines.
+//  * the result leaves through LDS, so that every store covers whole cache lines (emit_tile).
 // One barrier per 64 of K.  Sizes: K % 64 == 0; any M and N (loads clamp to the last row, stores are
 // masked).  The sum over K runs in ascending order for every output element.
+// Further down: the same pipeline on 256 x 256 block tiles (gemm_pipe_big_kernel; the host mixes both tile
+// sizes so that whole rounds of tiles fill the CUs) and on 64 x 128 tiles for 17..128 rows (gemm_pipe64_kernel).
 #include <algorithm>
 
 #include "common.h"
