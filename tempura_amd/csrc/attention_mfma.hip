@@ -52,13 +52,20 @@ __device__ inline void rows16_swap(float& a, float& b) {
 __device__ inline void rows32_swap(float& a, float& b) {
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
 }
+// (v_max_f32 as assembly: behind the swaps the compiler cannot tell that its operands are no signalling NaNs
+// and would quiet each of them with an instruction of its own)
+__device__ inline float max_raw(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
 __device__ inline float quad_rows_max(float x) {
   float y = x;
   rows16_swap(x, y);
-  x = fmaxf(x, y);
+  x = max_raw(x, y);
   y = x;
   rows32_swap(x, y);
-  return fmaxf(x, y);
+  return max_raw(x, y);
 }
 
 struct AttnArgs {
@@ -498,7 +505,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     attn_scores<D, NQ>(kf, qf, sc);
   }
   int stage = 0;
-  for (int s = 0; s < nsteps; ++s) {
+  // one step: `cur` holds this step's scores, the next step's go to `nxt` (the loop below runs two steps per
+  // turn with the two sets swapping roles, so that no register is copied)
+  auto step = [&](int s, f32x4_t (&cur)[NQ][2], f32x4_t (&nxt)[NQ][2]) {
     const int nstage = stage + 1 == NS ? 0 : stage + 1;
     // step s + 1 has landed for this wave (later steps may stay in flight), then for all; every wave
     // is done with the stage of step s - 1
@@ -512,11 +521,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     const unsigned base = lds0 + stage * STAGE;
     // the keys of the following stage are multiplied into the next step's scores before this step's
     // softmax runs on the vector ALU
-    f32x4_t sn[NQ][2];
     if (s + 1 < nsteps) {
       bf16x8_t kf[2][D / 32];
       read_keys(lds0 + nstage * STAGE, kf);
-      attn_scores<D, NQ>(kf, qf, sn);
+      attn_scores<D, NQ>(kf, qf, nxt);
     }
     // the value fragments travel while the softmax runs
     u32x4_t vv[D / 16];
@@ -528,9 +536,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     bool moved[NQ];
     const int j0 = first + s * 32;
     if (j0 + 31 <= qpos_min && (a.window <= 0 || j0 >= last_pos - a.window + 1))
-      attn_softmax<NQ, false>(a, j0, sc, qpos, m, l, pf, alpha, moved);
+      attn_softmax<NQ, false>(a, j0, cur, qpos, m, l, pf, alpha, moved);
     else
-      attn_softmax<NQ, true>(a, j0, sc, qpos, m, l, pf, alpha, moved);
+      attn_softmax<NQ, true>(a, j0, cur, qpos, m, l, pf, alpha, moved);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     bf16x8_t vf[D / 16];
 #pragma unroll
@@ -539,14 +547,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
       vf[dt] = frag_of(vv[dt]);
     }
     attn_pv<D, NQ>(vf, pf, alpha, moved, o);
-    if (s + 1 < nsteps) {
-#pragma unroll
-      for (int nq = 0; nq < NQ; ++nq) {
-        sc[nq][0] = sn[nq][0];
-        sc[nq][1] = sn[nq][1];
-      }
-    }
     stage = nstage;
+  };
+  f32x4_t sd[NQ][2];
+  for (int s = 0; s < nsteps; s += 2) {
+    step(s, sc, sd);
+    if (s + 1 < nsteps) step(s + 1, sd, sc);
   }
   if (active) {
 #pragma unroll
