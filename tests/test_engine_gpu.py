@@ -116,8 +116,8 @@ def test_command_line(tiny_dirs, tmp_path):
 def test_model_sized_layers_bfloat16_against_float32():
     """Two layers with the sizes of Llama-3.1-8B (hidden 4096, 32 heads of 128 in 8 groups, intermediate 14336,
     vocabulary 128256) and the same weights in both precisions: the bfloat16 engine (pipelined products of
-    300 and 70 rows, split K with sums left to the next kernel, the decode products with the norm carried by
-    them, k-blocked rows, LDS attention, graphs) against the float32 engine's plain-FMA kernels, portion by
+    2,200 rows in one step: 256 x 256 and 256 x 128 tiles side by side, the long-step rotation kernels; the
+    decode products with the norm carried by them, k-blocked rows, LDS attention, graphs) against the float32 engine's plain-FMA kernels, portion by
     portion and token by token.  The weights have the scale of trained checkpoints (N(0, 0.02)); the rounding of
     bfloat16 operands then costs about 1e-2 of the largest logit at this width, with the matrix-core kernels
     and with the general ones alike (at N(0, 0.05) both reach 3.5e-2: the scores get ten times sharper)."""
@@ -129,12 +129,12 @@ def test_model_sized_layers_bfloat16_against_float32():
     cfg = LlamaConfig.from_dict(PRESETS["llama-3.1-8b"].to_dict())
     cfg.num_hidden_layers = 2
     cfg.validate()
-    prompts = {r: helpers.random_tokens(cfg.vocab_size, n, seed=500 + n) for r, n in (("a", 300), ("b", 70), ("c", 23), ("d", 5))}
+    prompts = {r: helpers.random_tokens(cfg.vocab_size, n, seed=500 + n) for r, n in (("a", 2100), ("b", 70), ("c", 23), ("d", 5))}
     tails = {r: helpers.random_tokens(cfg.vocab_size, 6, seed=600 + i) for i, r in enumerate(prompts)}
     logits = {}
     for dtype in ("float32", "bfloat16"):
         model = random_model(cfg, seed=3, dtype=dtype, device="cuda:0", std=0.02, values_as="bfloat16")
-        runner = ModelRunner(model, 16, 64, max_requests=4, use_graph=(dtype == "bfloat16"))
+        runner = ModelRunner(model, 16, 160, max_requests=4, use_graph=(dtype == "bfloat16"))
         got = {r: [] for r in prompts}
         for r, toks in prompts.items():
             runner.add_request(r)
