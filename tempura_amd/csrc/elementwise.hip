@@ -108,11 +108,15 @@ extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void*
 }
 
 // ---- rotary position encoding + cache write -----------------------------------------
-// qkv row: [q heads | k heads | v heads] x head_dim, float32.  Pair (d, d + rotary_dim/2) of
-// each q and k head turns by the angle pos * inv_freq[d]: the product is formed in float64 and
-// reduced to [0, 2 pi) there, sine and cosine of the small rest are float32.  q goes to
-// q_out, rotated k and raw v go to the cache place `slots[t]` (page * page_size + offset) of
-// the paged pools (qkv may be [splits, n, row] partial sums of the projection, added here): keys as [page, kv_head, page_size, head_dim], values TRANSPOSED as
+// qkv row: [q heads | k heads | v heads] x head_dim, float32.  The q and k heads come in PAIRED order: the two
+// elements that rotate together lie side by side, elements (2 d, 2 d + 1) of a head being elements
+// (d, d + rotary_dim / 2) of the reference's split-half order (the attention part lays the rows of its
+// projection out so; scores do not change when q and k are permuted alike, so the cache holds keys in this
+// order and nothing is ever permuted back).  Pair d of each q and k head turns by the angle
+// pos * inv_freq[d]: the product is formed in float64 and reduced to [0, 2 pi) there, sine and cosine of
+// the small rest are float32.  q goes to q_out, rotated k and raw v go to the cache place `slots[t]`
+// (page * page_size + offset) of the paged pools (qkv may be [splits, n, row] partial sums of the
+// projection, added here): keys as [page, kv_head, page_size, head_dim], values TRANSPOSED as
 // [page, kv_head, head_dim, page_size] so that the attention kernels read eight consecutive
 // keys of one value element with one 16-byte load.  With slots == nullptr only q is produced
 // (the row then holds q heads only).
@@ -165,15 +169,8 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
   if (hl >= heads_per_block || h >= total_heads) return;
   const int half = rotary_dim / 2;
   const float* row = qkv + (size_t)t * row_stride + (size_t)h * head_dim;
-  // the two elements this thread moves: a rotary pair, or two pass-through elements
-  int i0, i1;
-  if (d < half) {
-    i0 = d;
-    i1 = d + half;
-  } else {
-    i0 = rotary_dim + 2 * (d - half);
-    i1 = i0 + 1;
-  }
+  // the two elements this thread moves: a rotary pair (d < half), or two pass-through elements
+  const int i0 = 2 * d, i1 = 2 * d + 1;
   // (splits > 1: the rows are the partial sums of a product whose K was split; added in ascending order)
   float y0 = 0.f, y1 = 0.f;
   {
@@ -225,8 +222,8 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, int row_stri
   }
 }
 
-// The same rotation for the q and k heads of long steps, four pairs per thread (16-byte loads, 8-byte
-// stores of bfloat16): needs head_dim, rotary_dim and the row stride to be multiples of eight.
+// The same rotation for the q and k heads of long steps, four pairs (eight consecutive elements) per thread
+// (16-byte loads, 8-byte stores of bfloat16): needs head_dim, rotary_dim and the row stride to be multiples of eight.
 // grid: (tokens, blocks of 256 threads over heads x head_dim / 8).
 template <typename T>
 __device__ inline void store4(T* p, const float (&v)[4]) {
@@ -255,10 +252,9 @@ __global__ void rope_qk4_kernel(const float* __restrict__ qkv, int row_stride, c
   const int h = idx / tph, j = idx % tph;
   if (h >= n_rot_heads) return;
   const int half = rotary_dim / 2;
-  // the eight elements this thread moves: four rotary pairs (d, d + half), or eight plain elements
-  const bool rot = 4 * j < half;
-  const int i0 = rot ? 4 * j : rotary_dim + 8 * (j - half / 4);
-  const int i1 = rot ? i0 + half : i0 + 4;
+  // the eight elements this thread moves: four rotary pairs (side by side), or eight plain elements
+  const bool rot = 8 * j < rotary_dim;
+  const int i0 = 8 * j, i1 = 8 * j + 4;
   const float* row = qkv + (size_t)t * row_stride + (size_t)h * head_dim;
   float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
   {
@@ -278,18 +274,20 @@ __global__ void rope_qk4_kernel(const float* __restrict__ qkv, int row_stride, c
   }
   if (rot) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < 4; ++e) {   // pair 4 j + e: elements (a[0], a[1]), (a[2], a[3]), (b[0], b[1]), (b[2], b[3])
       float sn, c;
       if (cos_sin != nullptr) {
-        const float2 cs = cos_sin[(size_t)t * half + i0 + e];
+        const float2 cs = cos_sin[(size_t)t * half + 4 * j + e];
         c = cs.x;
         sn = cs.y;
       } else {
-        rope_cos_sin(positions[t], inv_freq[i0 + e], factor, c, sn);
+        rope_cos_sin(positions[t], inv_freq[4 * j + e], factor, c, sn);
       }
-      const float x0 = a[e], x1 = b[e];
-      a[e] = x0 * c - x1 * sn;
-      b[e] = x0 * sn + x1 * c;
+      float& r0 = e < 2 ? a[2 * e] : b[2 * e - 4];
+      float& r1 = e < 2 ? a[2 * e + 1] : b[2 * e - 3];
+      const float x0 = r0, x1 = r1;
+      r0 = x0 * c - x1 * sn;
+      r1 = x0 * sn + x1 * c;
     }
   }
   if (h < n_heads) {

@@ -329,6 +329,8 @@ def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
     """Rotate q and k of float32 rows [n, (heads + 2 kv_heads) * head_dim] (or the ``Partials`` of the
     projection that makes them), store k and v into the cache rows ``slots`` and return q as q_dtype
     [n, heads, head_dim].  With ``slots`` None the rows hold q only and nothing is stored.
+    The q and k heads are in PAIRED order: elements (2 d, 2 d + 1) of a head rotate together by the angle
+    of pair d (they are elements (d, d + rotary_dim / 2) of the split-half order).
     ``cos_sin``: this step's table from ``rope_table`` (the same values, computed once for all layers)."""
     if _backend is not None:
         return _backend.rope_kv_write(qkv, positions, slots, inv_freq, rotary_dim, factor, num_heads,

@@ -52,10 +52,26 @@ class PagedAttention(Mixer):
         out.update(part_class("position", p["position"].kind).expected_weights(p["position"], hidden_size))
         return out
 
+    def _paired(self, t: torch.Tensor) -> torch.Tensor:
+        """The rows of a q or k projection with every head's rotary elements in paired order: rows
+        (2 d, 2 d + 1) of a head are rows (d, d + rotary_dim / 2) of the checkpoint's split-half order, so
+        that the two elements that rotate together are neighbours (the rotation kernels expect that, and a
+        product's epilogue can rotate what it holds).  q and k are permuted alike, which leaves every score
+        as it was; the cache then holds keys in this order."""
+        rot = self.position.rotary()
+        if rot is None or rot[1] == 0:
+            return t
+        rd, half, d = rot[1], rot[1] // 2, self.head_dim
+        order = torch.arange(d)
+        order[0:rd:2] = torch.arange(half)
+        order[1:rd:2] = torch.arange(half) + half
+        heads = t.shape[0] // d
+        return t.view(heads, d, -1)[:, order.to(t.device), :].reshape(t.shape)
+
     def load_weights(self, get):
         w = self.spec.weights
         # One [q_dim + 2 kv_dim, hidden] matrix: one product instead of three.
-        parts = [get(w["q"]), get(w["k"]), get(w["v"])]
+        parts = [self._paired(get(w["q"])), self._paired(get(w["k"])), get(w["v"])]
         self.wqkv = torch.cat([self._to_device(t) for t in parts], dim=0).contiguous()
         self.wo = self._to_device(get(w["o"]))
         self.position.load_weights(get)

@@ -78,9 +78,10 @@ class EmuOps:
             ang = positions.double()[:, None] * inv_freq.double()[None, :]
             c = (torch.cos(ang) * factor)[:, None, :]
             s = (torch.sin(ang) * factor)[:, None, :]
-            x0, x1 = x[..., :half].clone(), x[..., half:rotary_dim].clone()
-            x[..., :half] = x0 * c - x1 * s
-            x[..., half:rotary_dim] = x0 * s + x1 * c
+            # paired order: elements (2 d, 2 d + 1) rotate together by the angle of pair d
+            x0, x1 = x[..., 0:rotary_dim:2].clone(), x[..., 1:rotary_dim:2].clone()
+            x[..., 0:rotary_dim:2] = x0 * c - x1 * s
+            x[..., 1:rotary_dim:2] = x0 * s + x1 * c
         q = x[:, :num_heads].to(q_dtype).contiguous()
         if slots is not None:
             k = x[:, num_heads:]

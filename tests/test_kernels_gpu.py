@@ -110,6 +110,29 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
         _close(table[..., 1], torch.sin(ang), 2e-6, "table sines")
 
 
+def test_rope_paired_order_is_the_split_half_rotation():
+    """The kernels rotate neighbours (2 d, 2 d + 1); the reference rotates (d, d + D / 2)
+    (/root/reference/kernels/src/rope.rs:18-53).  Laying a head out in paired order, rotating, and laying it
+    back must give the plain implementation's split-half rotation of the same head."""
+    ops = _ops()
+    import plain
+    g = torch.Generator().manual_seed(6)
+    n, heads, d = 9, 3, 32
+    half = d // 2
+    x = torch.randn(n, heads, d, generator=g)
+    pos = torch.tensor([0, 1, 2, 3, 50, 777, 4095, 131071, 5], dtype=torch.int32)
+    inv = plain.rope_inv_freq(d, 10000.0, None)
+    want = plain.rope(x.double(), pos, inv)                      # split-half order in and out
+    order = torch.arange(d)
+    order[0::2] = torch.arange(half)
+    order[1::2] = torch.arange(half) + half
+    paired = x[:, :, order].reshape(n, heads * d).contiguous()
+    got = ops.rope_kv_write(paired.to(DEV), pos.to(DEV), None, inv.to(DEV), d, 1.0, heads, 0, d, None, None, torch.float32)
+    back = torch.empty_like(got.cpu())
+    back[:, :, order] = got.cpu()
+    _close(back, want, 2e-6, "paired rotation against the split-half formula")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv,d,page,n", [(4, 2, 64, 16, 300), (3, 1, 48, 8, 277), (8, 2, 128, 32, 600), (2, 2, 12, 16, 260)])
 def test_rope_kv_write_long_step(dtype, heads, kv, d, page, n):
