@@ -46,6 +46,16 @@ __device__ inline float to_float(bf16_t v) { return bf16_to_float(v); }
 __device__ inline void from_float(float* p, float v) { *p = v; }
 __device__ inline void from_float(bf16_t* p, float v) { *p = float_to_bf16(v); }
 
+// cosine and sine (times factor) of pos * inv_freq: the product in float64, reduced to [0, 2 pi) there,
+// sine and cosine of the small rest in float32 (every kernel that rotates uses this one routine)
+__device__ inline void rope_cos_sin(int pos, double inv_freq, float factor, float& c, float& sn) {
+  const double turns = (double)pos * inv_freq * 0.15915494309189535;
+  const float rest = (float)((turns - floor(turns)) * 6.283185307179586);
+  sincosf(rest, &sn, &c);
+  c *= factor;
+  sn *= factor;
+}
+
 __device__ inline float wave_sum(float v) {
 #pragma unroll
   for (int o = TP_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TP_WAVE);

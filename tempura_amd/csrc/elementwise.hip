@@ -122,15 +122,6 @@ extern "C" int tp_rmsnorm(const float* x, const float* w, const int* rows, void*
 // (the row then holds q heads only).
 // grid: (tokens, head blocks); a thread owns one pair (or two plain elements) of one head, so
 // every load of the row is in flight at once.
-// cosine and sine (times factor) of pos * inv_freq: the product in float64, reduced to [0, 2 pi) there
-__device__ inline void rope_cos_sin(int pos, double inv_freq, float factor, float& c, float& sn) {
-  const double turns = (double)pos * inv_freq * 0.15915494309189535;
-  const float rest = (float)((turns - floor(turns)) * 6.283185307179586);
-  sincosf(rest, &sn, &c);
-  c *= factor;
-  sn *= factor;
-}
-
 // table[t, d] = (cos, sin) of token t's position times inv_freq[d]: long steps compute it once and every
 // layer's rotation reads it
 __global__ void rope_table_kernel(const int* __restrict__ positions, const double* __restrict__ inv_freq, int half,

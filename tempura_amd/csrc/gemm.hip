@@ -146,6 +146,31 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
                    const void* post_w, void* post_xg, float* post_ss, int layout, int defer_reduce, int* splits_out,
                    hipStream_t s);
 
+int tp_linear_rope_mfma(const void* x, const void* w, int M, int N, int K, const float* pre_ss, int pre_count,
+                        float pre_eps, const int* positions, const int* slots, const double* inv_freq, int rotary_dim,
+                        float factor, int n_heads, int n_kv, int head_dim, void* q_out, void* k_cache, void* v_cache,
+                        int page_size, const float* cos_sin, hipStream_t s);
+
+// The q/k/v projection of at most 16 bfloat16 rows that finishes its rows itself: x [M, K] (or the rows of a
+// split norm, see below) times w [(n_heads + 2 n_kv) * head_dim, K], the q and k heads in paired order; the
+// epilogue rotates q and k (pair d of a head by positions[m] * inv_freq[d]), writes q as bfloat16
+// [M, n_heads, head_dim], k into the cache place slots[m] and v into the transposed value cache (both
+// bfloat16), as tp_rope_kv_write does for the rows of a plain product.  cos_sin: the step's table from
+// tp_rope_table [M, rotary_dim / 2, 2], or nullptr (the epilogue then computes cosines and sines itself).
+extern "C" int tp_linear_rope(const void* x, const void* w, int M, int N, int K, const float* pre_ss, int pre_count,
+                              float pre_eps, const int* positions, const int* slots, const double* inv_freq,
+                              int rotary_dim, float factor, int n_heads, int n_kv, int head_dim, void* q_out,
+                              void* k_cache, void* v_cache, int page_size, const float* cos_sin, hipStream_t s) {
+  TP_REQUIRE(x && w && positions && slots && q_out && k_cache && v_cache, "linear_rope: missing operand");
+  TP_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "linear_rope: no frequency table");
+  const int r = tp_linear_rope_mfma(x, w, M, N, K, pre_ss, pre_count, pre_eps, positions, slots, inv_freq, rotary_dim,
+                                    factor, n_heads, n_kv, head_dim, q_out, k_cache, v_cache, page_size, cos_sin, s);
+  TP_REQUIRE(r == 0, "linear_rope: sizes M %d N %d K %d head_dim %d are not this product's (at most 16 rows, "
+             "K %% 32 == 0, head_dim %% 16 == 0)", M, N, K, head_dim);
+  TP_CHECK_LAUNCH("linear_rope");
+  return 0;
+}
+
 // `scratch` (optional, `scratch_floats` float32): room for split-K partial sums of mid-sized products.
 //
 // The split norm (bfloat16, at most 16 rows, K % 32 == 0): with `post_w` (a float32 norm weight [N]; accumulate

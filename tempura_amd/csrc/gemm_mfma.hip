@@ -52,6 +52,53 @@ __device__ inline void store_out(void* out, int mode, size_t idx, float v) {
     ((float*)out)[idx] += v;
 }
 
+// The q/k/v projection of at most 16 tokens can finish its rows itself (mode OUT_ROPE): the q and k heads
+// come in paired order (the two elements that rotate together are neighbouring columns, held by
+// neighbouring lanes of the epilogue), so a lane fetches its partner's sum, rotates, and stores q as
+// bfloat16 [M, heads, head_dim], k into the cache place slots[m] and v into the transposed value cache:
+// the rotation and cache-write kernel between the projection and the attention is gone.  The arithmetic is
+// that kernel's, on the same float32 sums.
+struct RopeOut {
+  const int* positions;      // [M]
+  const int* slots;          // [M] cache place (page * page_size + offset)
+  const double* inv_freq;    // [rotary_dim / 2]
+  const float2* cos_sin;     // [M, rotary_dim / 2] this step's table (rope_table_kernel), or nullptr
+  float factor;
+  int rotary_dim, n_heads, n_kv, head_dim, page_size;
+  bf16_t* q_out;
+  bf16_t* k_cache;           // [page, kv_head, page_size, head_dim]
+  bf16_t* v_cache;           // [page, kv_head, head_dim, page_size]
+};
+enum { OUT_ROPE = 4 };
+
+// v: this lane's sum of column n of row m; other: the sum of column n ^ 1 (the partner of a rotary pair)
+__device__ inline void rope_store(const RopeOut& rp, int m, int n, float v, float other) {
+  const int h = n / rp.head_dim, d = n % rp.head_dim;
+  float y = v;
+  if (h < rp.n_heads + rp.n_kv && d < rp.rotary_dim) {
+    float c, sn;
+    if (rp.cos_sin != nullptr) {
+      const float2 cs = rp.cos_sin[(size_t)m * (rp.rotary_dim >> 1) + (d >> 1)];
+      c = cs.x;
+      sn = cs.y;
+    } else {
+      rope_cos_sin(rp.positions[m], rp.inv_freq[d >> 1], rp.factor, c, sn);
+    }
+    // the pair is (x0, x1) = (even column, odd column): x0 c - x1 s and x0 s + x1 c
+    y = (d & 1) ? other * sn + v * c : v * c - other * sn;
+  }
+  if (h < rp.n_heads) {
+    rp.q_out[((size_t)m * rp.n_heads + h) * rp.head_dim + d] = float_to_bf16(y);
+    return;
+  }
+  const int slot = rp.slots[m];
+  const size_t page = (size_t)(slot / rp.page_size), off = (size_t)(slot % rp.page_size);
+  if (h < rp.n_heads + rp.n_kv)
+    rp.k_cache[((page * rp.n_kv + (h - rp.n_heads)) * rp.page_size + off) * rp.head_dim + d] = float_to_bf16(y);
+  else
+    rp.v_cache[((page * rp.n_kv + (h - rp.n_heads - rp.n_kv)) * rp.head_dim + d) * rp.page_size + off] = float_to_bf16(y);
+}
+
 // A root-mean-square norm split over two products (rows of at most 16 tokens).  The product that
 // adds into the residual stream h also writes xg = bfloat16(h * norm weight) and, per block and row,
 // the sum of squares of the columns it owns (NormPrep).  The product that consumes xg adds those
@@ -123,7 +170,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
                                                                       const bf16_t* __restrict__ w,
                                                                       void* __restrict__ out, int mode, int M,
                                                                       int N, int K, int layout, RowScale pre,
-                                                                      NormPrep post) {
+                                                                      NormPrep post, RopeOut rp) {
   __shared__ float red[WAVES][NT * MT][256];
   __shared__ float rs_part[32][16], rstd[16], ss_lds[NT][4][16];
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
@@ -223,6 +270,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
       sq += __shfl_xor(sq, 1, 64);      // the four columns r = 0..3 of this row
       sq += __shfl_xor(sq, 2, 64);
       if (r == 0) ss_lds[j][l >> 4][l & 15] = sq;
+    } else if (mode == OUT_ROPE) {
+      const float other = __shfl_xor(v, 1, 64);   // r and r ^ 1 are neighbouring lanes
+      if (n < N && m < M) rope_store(rp, m, n, v, other);
     } else if (n < N && m < M) {
       store_out(out, mode, (size_t)m * N + n, v);
     }
@@ -257,7 +307,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 template <int NT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                void* __restrict__ out, int mode, int M, int N, int K,
-                                                               int layout, RowScale pre, NormPrep post) {
+                                                               int layout, RowScale pre, NormPrep post, RopeOut rp) {
   constexpr int THREADS = WAVES * 64, G = 1;
   constexpr int KC = WAVES * 128;        // K elements per chunk: one run of four steps per wave
   constexpr int LD = KC + 8;             // padded LDS row
@@ -373,6 +423,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_
       sq += __shfl_xor(sq, 1, 64);
       sq += __shfl_xor(sq, 2, 64);
       if (r == 0) ss_lds[gj][l >> 4][m] = sq;
+    } else if (mode == OUT_ROPE) {
+      const float other = __shfl_xor(v, 1, 64);
+      if (n < N && m < M) rope_store(rp, m, n, v, other);
     } else if (n < N && m < M) {
       store_out(out, mode, (size_t)m * N + n, v);
     }
@@ -633,15 +686,15 @@ extern "C" void tp_linear_tune(int waves, int nt, int depth) {
 
 template <int MT, int NT, int WAVES, int DEPTH>
 static void launch_skinny4(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, int layout,
-                           RowScale pre, NormPrep post, hipStream_t s) {
+                           RowScale pre, NormPrep post, const RopeOut& rp, hipStream_t s) {
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
   hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, NT, WAVES, DEPTH>), dim3(blocks), dim3(WAVES * 64), 0, s, x, w, out,
-                     mode, M, N, K, layout, pre, post);
+                     mode, M, N, K, layout, pre, post, rp);
 }
 
 template <int MT>
 static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, int layout,
-                          RowScale pre, NormPrep post, hipStream_t s) {
+                          RowScale pre, NormPrep post, const RopeOut& rp, hipStream_t s) {
   // every wave should get at least one run of four steps; small N wants many waves per block
   // (one block per 16 columns is all the parallelism there is), large N fewer and two row tiles
   // Measured on MI355X at Llama-8B shapes: eight waves with two runs in flight each stream
@@ -663,9 +716,9 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
       if (nt > 2) nt = 2;
       const int blocks = (N + 16 * nt - 1) / (16 * nt);
       if (nt == 2)
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post);
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post, rp);
       else
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post);
+        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post, rp);
       return;
     }
   }
@@ -673,7 +726,7 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
   if (MT > 1) nt = 1;
   if (MT > 2 || nt > 2) depth = 1;           // registers
 #define CASE(NT_, W_, D_) \
-  if (nt == NT_ && waves == W_ && depth == D_) return launch_skinny4<MT, NT_, W_, D_>(x, w, out, mode, M, N, K, layout, pre, post, s)
+  if (nt == NT_ && waves == W_ && depth == D_) return launch_skinny4<MT, NT_, W_, D_>(x, w, out, mode, M, N, K, layout, pre, post, rp, s)
   CASE(1, 16, 1);
   CASE(1, 8, 1);
   CASE(1, 4, 1);
@@ -694,7 +747,24 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
     CASE(4, 4, 1);
   }
 #undef CASE
-  launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, layout, pre, post, s);
+  launch_skinny4<MT, 1, 8, 1>(x, w, out, mode, M, N, K, layout, pre, post, rp, s);
+}
+
+// The q/k/v projection of at most 16 rows with rotation and cache write in its epilogue (see RopeOut).
+// N = (n_heads + 2 n_kv) * head_dim.  Returns -1 for sizes this path does not take.
+int tp_linear_rope_mfma(const void* x, const void* w, int M, int N, int K, const float* pre_ss, int pre_count,
+                        float pre_eps, const int* positions, const int* slots, const double* inv_freq, int rotary_dim,
+                        float factor, int n_heads, int n_kv, int head_dim, void* q_out, void* k_cache, void* v_cache,
+                        int page_size, const float* cos_sin, hipStream_t s) {
+  if (M < 1 || M > 16 || K % 32 != 0 || head_dim % 16 != 0 || rotary_dim % 2 != 0 || rotary_dim > head_dim) return -1;
+  if (N != (n_heads + 2 * n_kv) * head_dim || page_size < 1) return -1;
+  if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return -1;
+  const RowScale pre = {pre_ss, pre_count, 1.0f / (float)K, pre_eps};
+  const NormPrep post = {nullptr, nullptr, nullptr};
+  const RopeOut rp = {positions, slots, inv_freq, (const float2*)cos_sin, factor, rotary_dim, n_heads, n_kv, head_dim, page_size,
+                      (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache};
+  launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, 0, pre, post, rp, s);
+  return 0;
 }
 
 // accumulate: 0 store, 1 add into the float32 output, 2 gated-SiLU epilogue (see OUT_SWIGLU).
@@ -717,15 +787,16 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   const bf16_t* xb = (const bf16_t*)x;
   const bf16_t* wb = (const bf16_t*)w;
   const bool mid_ok = scratch != nullptr && g_tune_mid != 1;
+  const RopeOut no_rope = {};
   if (M <= 16 || (M <= 64 && !mid_ok)) {
     if (M <= 16)
-      launch_skinny<1>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
+      launch_skinny<1>(xb, wb, out, mode, M, N, K, layout, pre, post, no_rope, s);
     else if (M <= 32)
-      launch_skinny<2>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
+      launch_skinny<2>(xb, wb, out, mode, M, N, K, layout, pre, post, no_rope, s);
     else if (M <= 48)
-      launch_skinny<3>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
+      launch_skinny<3>(xb, wb, out, mode, M, N, K, layout, pre, post, no_rope, s);
     else
-      launch_skinny<4>(xb, wb, out, mode, M, N, K, layout, pre, post, s);
+      launch_skinny<4>(xb, wb, out, mode, M, N, K, layout, pre, post, no_rope, s);
   } else {
     // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
     // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.

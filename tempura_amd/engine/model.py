@@ -105,6 +105,8 @@ class CausalLM:
     def forward(self, tokens: torch.Tensor, ctx, caches) -> torch.Tensor:
         """``tokens`` int32 [n]; ``caches[i]`` is the ``LayerCache`` of run-order entry i.
         Returns float32 logits [len(ctx.logit_rows), vocab]."""
+        if hasattr(ctx, "shared"):
+            ctx.shared.clear()      # what layers share is computed anew in every pass (also in one that is captured)
         h = self.embedding.forward(tokens)
         m = h.shape[0]
         x = None      # rows handed from one block to the next (a norm carried by the products around it)

@@ -321,6 +321,47 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
     return out if next_norm is None else (out, handed)
 
 
+def linear_rope_ok(m: int, k: int, head_dim: int, x_dtype: torch.dtype, cache_dtype: torch.dtype) -> bool:
+    """Whether ``linear_rope_kv`` takes a projection of m rows."""
+    return (_backend is None and allow_mfma and 0 < m <= 16 and k % 32 == 0 and head_dim % 16 == 0
+            and x_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16)
+
+
+def linear_rope_kv(x, w: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, inv_freq: Optional[torch.Tensor],
+                   rotary_dim: int, factor: float, num_heads: int, num_kv_heads: int, head_dim: int,
+                   k_cache: torch.Tensor, v_cache: torch.Tensor, cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The q/k/v projection of at most 16 bfloat16 rows (or ``Prenormed`` rows) with the rotation and the
+    cache write in its epilogue: the same result as ``linear`` to float32 followed by ``rope_kv_write``
+    (w's q and k heads in paired order), without the kernel and the rows in between.  Returns q as
+    bfloat16 [m, heads, head_dim]."""
+    x, pre = _pre_args(x)
+    _dev_ok(x, w, positions, slots, inv_freq, k_cache, v_cache)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_rope_kv: shapes {tuple(x.shape)} x {tuple(w.shape)}")
+    m, k = x.shape
+    n = w.shape[0]
+    _need(linear_rope_ok(m, k, head_dim, x.dtype, k_cache.dtype) and w.dtype == torch.bfloat16,
+          "linear_rope_kv: at most 16 bfloat16 rows, k % 32 == 0, head_dim % 16 == 0, a bfloat16 cache")
+    _need(n == (num_heads + 2 * num_kv_heads) * head_dim, f"linear_rope_kv: {n} weight rows for {num_heads} + 2 x {num_kv_heads} heads of {head_dim}")
+    _i32(positions, m, "positions")
+    _i32(slots, m, "slots")
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim
+          and tuple(v_cache.shape) == (k_cache.shape[0], k_cache.shape[1], k_cache.shape[3], k_cache.shape[2])
+          and v_cache.dtype == torch.bfloat16,
+          "linear_rope_kv: caches must be k [pages, kv_heads, page_size, head_dim], v [pages, kv_heads, head_dim, page_size]")
+    if rotary_dim:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float64 and inv_freq.numel() == rotary_dim // 2,
+              "linear_rope_kv: inv_freq must be float64 [rotary_dim / 2]")
+    if cos_sin is not None:
+        _dev_ok(cos_sin)
+        _need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and tuple(cos_sin.shape) == (m, rotary_dim // 2, 2),
+              "linear_rope_kv: table must be float32 [m, rotary_dim / 2, 2]")
+    q = torch.empty((m, num_heads, head_dim), dtype=torch.bfloat16, device=x.device)
+    _call("tp_linear_rope", _ptr(x), _ptr(w), m, n, k, *pre, _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
+          ctypes.c_float(factor), num_heads, num_kv_heads, head_dim, _ptr(q), _ptr(k_cache), _ptr(v_cache),
+          k_cache.shape[2], _ptr(cos_sin), _stream())
+    return q
+
+
 def rope_kv_write(qkv, positions: torch.Tensor, slots: Optional[torch.Tensor],
                   inv_freq: Optional[torch.Tensor], rotary_dim: int, factor: float, num_heads: int,
                   num_kv_heads: int, head_dim: int, k_cache: Optional[torch.Tensor],

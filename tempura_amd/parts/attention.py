@@ -82,6 +82,27 @@ class PagedAttention(Mixer):
 
     def forward(self, x, ctx, cache, residual, next_norm=None):
         rot = self.position.rotary()
+        q = None
+        if rot is not None and cache.writes:
+            rows = x.x if isinstance(x, ops.Prenormed) else x
+            if ops.linear_rope_ok(rows.shape[0], rows.shape[1], self.head_dim, rows.dtype, cache.k.dtype):
+                # a few rows (decoding): the projection rotates and stores its rows itself
+                table = self.position.table(ctx, always=True) if hasattr(self.position, "table") else None
+                q = ops.linear_rope_kv(x, self.wqkv, ctx.positions, ctx.slot_mapping[cache.group], rot[0], rot[1], rot[2],
+                                       self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v, table)
+        if q is None:
+            q = self._project_and_rotate(x, ctx, cache, rot)
+        a = ops.paged_attention(
+            q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
+            ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
+            ctx.num_single)
+        if next_norm is None:
+            ops.linear(a, self.wo, torch.float32, residual=residual)
+            return None
+        return ops.linear(a, self.wo, torch.float32, residual=residual, next_norm=next_norm)[1]
+
+    def _project_and_rotate(self, x, ctx, cache, rot):
+        """q (rotated, [n, heads, head_dim]) of the projection; k and v go to the cache."""
         # (with a rotary position the next kernel may add the projection's partial sums itself)
         if cache.writes:
             qkv = ops.linear(x, self.wqkv, torch.float32, partial_ok=rot is not None)
@@ -104,14 +125,7 @@ class PagedAttention(Mixer):
             qkv, ctx.positions, ctx.slot_mapping[cache.group] if cache.writes else None,
             inv_freq, rotary_dim, factor, self.num_heads, self.num_kv_heads, self.head_dim,
             cache.k if cache.writes else None, cache.v if cache.writes else None, self.dtype, table)
-        a = ops.paged_attention(
-            q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
-            ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
-            ctx.num_single)
-        if next_norm is None:
-            ops.linear(a, self.wo, torch.float32, residual=residual)
-            return None
-        return ops.linear(a, self.wo, torch.float32, residual=residual, next_norm=next_norm)[1]
+        return q
 
 
 register_part("mixer", "attention", PagedAttention)

@@ -68,10 +68,11 @@ class RotaryPosition(PositionEncoding):
     def rotary(self):
         return self.inv_freq, self.rotary_dim, self.factor
 
-    def table(self, ctx):
+    def table(self, ctx, always: bool = False):
         """This step's [tokens, rotary_dim / 2, 2] cosines and sines, shared by every layer whose rotation has
-        the same frequencies; None for short steps (the rotation kernel then computes them itself)."""
-        if ctx.num_tokens < self.TABLE_FROM or self.rotary_dim == 0:
+        the same frequencies; None for short steps (the rotation kernel then computes them itself) unless
+        ``always`` (a product that rotates in its epilogue wants the table at any size)."""
+        if self.rotary_dim == 0 or (ctx.num_tokens < self.TABLE_FROM and not always):
             return None
         if self._table_key not in ctx.shared:
             ctx.shared[self._table_key] = ops.rope_table(ctx.positions, self.inv_freq, self.rotary_dim, self.factor)

@@ -110,6 +110,40 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
         _close(table[..., 1], torch.sin(ang), 2e-6, "table sines")
 
 
+@pytest.mark.parametrize("m,heads,kv,d,rot,k,page", [(1, 4, 2, 64, 64, 256, 16), (8, 32, 8, 128, 128, 4096, 16),
+                                                    (16, 3, 1, 48, 32, 96, 8), (5, 6, 3, 16, 16, 2048, 32)])
+def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
+    """The projection of a few rows that rotates and stores its rows in its epilogue gives the bits of the
+    plain product followed by the rotation and cache-write kernel; and both agree with float64."""
+    ops = _ops()
+    from tempura_amd.parts.rope import rotary_inv_freq
+    g = torch.Generator().manual_seed(7)
+    n = (heads + 2 * kv) * d
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) * 0.1).to(torch.bfloat16)
+    pos = torch.randint(0, 100000, (m,), generator=g, dtype=torch.int32)
+    pages = 5
+    slots = torch.randperm(pages * page, generator=g)[:m].to(torch.int32)
+    inv = rotary_inv_freq(d, 500000.0, None, rot)
+    kc = torch.zeros(pages, kv, page, d, dtype=torch.bfloat16)
+    vc = torch.zeros(pages, kv, d, page, dtype=torch.bfloat16)
+    xd, wd, pd, sd, invd = x.to(DEV), w.to(DEV), pos.to(DEV), slots.to(DEV), inv.to(DEV)
+    k1, v1 = kc.to(DEV), vc.to(DEV)
+    q1 = ops.rope_kv_write(ops.linear(xd, wd, torch.float32), pd, sd, invd, rot, 1.0, heads, kv, d, k1, v1, torch.bfloat16)
+    k2, v2 = kc.to(DEV), vc.to(DEV)
+    q2 = ops.linear_rope_kv(xd, wd, pd, sd, invd, rot, 1.0, heads, kv, d, k2, v2)
+    assert torch.equal(q2, q1) and torch.equal(k2, k1) and torch.equal(v2, v1)
+    if rot:   # with the step's table of cosines and sines: the same bits again
+        k3, v3 = kc.to(DEV), vc.to(DEV)
+        q3 = ops.linear_rope_kv(xd, wd, pd, sd, invd, rot, 1.0, heads, kv, d, k3, v3, ops.rope_table(pd, invd, rot, 1.0))
+        assert torch.equal(q3, q1) and torch.equal(k3, k1) and torch.equal(v3, v1)
+    kr, vr = kc.clone(), vc.clone()
+    qr = emu.rope_kv_write(x.double() @ w.double().T, pos, slots, inv, rot, 1.0, heads, kv, d, kr, vr, torch.float64)
+    _close(q2, qr, 1e-2, "q")
+    _close(k2, kr, 1e-2, "k cache")
+    _close(v2, vr, 1e-2, "v cache")
+
+
 def test_rope_paired_order_is_the_split_half_rotation():
     """The kernels rotate neighbours (2 d, 2 d + 1); the reference rotates (d, d + D / 2)
     (/root/reference/kernels/src/rope.rs:18-53).  Laying a head out in paired order, rotating, and laying it
