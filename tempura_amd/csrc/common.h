@@ -56,6 +56,25 @@ __device__ inline void rope_cos_sin(int pos, double inv_freq, float factor, floa
   sn *= factor;
 }
 
+// The q/k/v projection can finish its rows itself (mode OUT_ROPE of the bfloat16 products): the q and k heads
+// come in paired order (the two elements that rotate together are neighbouring columns), so the epilogue
+// rotates what it holds and stores q as bfloat16 [M, heads, head_dim], k into the cache place slots[m] and v
+// into the transposed value cache: the rotation and cache-write kernel between the projection and the
+// attention is gone.  The arithmetic is that kernel's, on the same float32 sums.
+struct RopeOut {
+  const int* positions;      // [M]
+  const int* slots;          // [M] cache place (page * page_size + offset)
+  const double* inv_freq;    // [rotary_dim / 2]
+  const float2* cos_sin;     // [M, rotary_dim / 2] this step's table (rope_table_kernel), or nullptr
+  float factor;
+  int rotary_dim, n_heads, n_kv, head_dim, page_size;
+  int col0;                  // first column of this launch (a launch may cover a range of columns)
+  bf16_t* q_out;
+  bf16_t* k_cache;           // [page, kv_head, page_size, head_dim]
+  bf16_t* v_cache;           // [page, kv_head, head_dim, page_size]
+};
+enum { OUT_ROPE = 4 };
+
 __device__ inline float wave_sum(float v) {
 #pragma unroll
   for (int o = TP_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TP_WAVE);

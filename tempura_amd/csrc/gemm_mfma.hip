@@ -52,25 +52,6 @@ __device__ inline void store_out(void* out, int mode, size_t idx, float v) {
     ((float*)out)[idx] += v;
 }
 
-// The q/k/v projection of at most 16 tokens can finish its rows itself (mode OUT_ROPE): the q and k heads
-// come in paired order (the two elements that rotate together are neighbouring columns, held by
-// neighbouring lanes of the epilogue), so a lane fetches its partner's sum, rotates, and stores q as
-// bfloat16 [M, heads, head_dim], k into the cache place slots[m] and v into the transposed value cache:
-// the rotation and cache-write kernel between the projection and the attention is gone.  The arithmetic is
-// that kernel's, on the same float32 sums.
-struct RopeOut {
-  const int* positions;      // [M]
-  const int* slots;          // [M] cache place (page * page_size + offset)
-  const double* inv_freq;    // [rotary_dim / 2]
-  const float2* cos_sin;     // [M, rotary_dim / 2] this step's table (rope_table_kernel), or nullptr
-  float factor;
-  int rotary_dim, n_heads, n_kv, head_dim, page_size;
-  bf16_t* q_out;
-  bf16_t* k_cache;           // [page, kv_head, page_size, head_dim]
-  bf16_t* v_cache;           // [page, kv_head, head_dim, page_size]
-};
-enum { OUT_ROPE = 4 };
-
 // v: this lane's sum of column n of row m; other: the sum of column n ^ 1 (the partner of a rotary pair)
 __device__ inline void rope_store(const RopeOut& rp, int m, int n, float v, float other) {
   const int h = n / rp.head_dim, d = n % rp.head_dim;
@@ -661,7 +642,7 @@ static int g_tune_order = 0;   // large products: 1 tiled kernel, plain block or
 
 // Defined in gemm_pipe.hip; 0 when it took the product, -1 when the sizes are not its own.
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
-                   size_t scratch_floats, int tune_splits, hipStream_t s);
+                   size_t scratch_floats, int tune_splits, const RopeOut* rope, hipStream_t s);
 
 int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
                      size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s);
@@ -756,13 +737,19 @@ int tp_linear_rope_mfma(const void* x, const void* w, int M, int N, int K, const
                         float pre_eps, const int* positions, const int* slots, const double* inv_freq, int rotary_dim,
                         float factor, int n_heads, int n_kv, int head_dim, void* q_out, void* k_cache, void* v_cache,
                         int page_size, const float* cos_sin, hipStream_t s) {
-  if (M < 1 || M > 16 || K % 32 != 0 || head_dim % 16 != 0 || rotary_dim % 2 != 0 || rotary_dim > head_dim) return -1;
+  if (M < 1 || (M > 16 && M <= 128) || K % 32 != 0 || head_dim % 16 != 0 || rotary_dim % 2 != 0 || rotary_dim > head_dim) return -1;
   if (N != (n_heads + 2 * n_kv) * head_dim || page_size < 1) return -1;
   if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return -1;
   const RowScale pre = {pre_ss, pre_count, 1.0f / (float)K, pre_eps};
   const NormPrep post = {nullptr, nullptr, nullptr};
   const RopeOut rp = {positions, slots, inv_freq, (const float2*)cos_sin, factor, rotary_dim, n_heads, n_kv, head_dim, page_size,
-                      (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache};
+                      0, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache};
+  if (M > 16) {
+    // long steps: the pipelined kernels, whose wave tiles (64 or 128 columns) must lie inside one head, with the
+    // step's table of cosines and sines
+    if (head_dim != 128 || rotary_dim % 8 != 0 || cos_sin == nullptr || pre_ss != nullptr || page_size % 8 != 0) return -1;
+    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, s);
+  }
   launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, 0, pre, post, rp, s);
   return 0;
 }
@@ -804,7 +791,7 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
     // (measured at 128 rows: N = 28,672 59 us against 77 us, the narrow products a few us slower)
     const bool pipe = g_tune_order ? g_tune_order == 3 : (M > 128 || (M > 64 && N >= 16384));
     const bool pipe64 = !pipe && M <= 128 && scratch != nullptr && g_tune_mid != 2;
-    if (pipe && tp_linear_pipe(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, s) == 0) {
+    if (pipe && tp_linear_pipe(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, nullptr, s) == 0) {
       // taken by the pipelined kernel
     } else if (pipe64 && tp_linear_pipe64(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, defer_reduce,
                                           splits_out, s) == 0) {

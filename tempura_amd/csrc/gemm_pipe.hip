@@ -239,6 +239,147 @@ __device__ inline void emit_tile_fast(const float* ct, int lane, int mrow0, int 
   }
 }
 
+// The q/k/v projection's epilogue (see RopeOut): the wave tile lies inside one head (head_dim is 128, COLS 64 or
+// 128).  q and k: a lane takes eight neighbouring columns (four rotary pairs) of a row, rotates them with the
+// step's table of cosines and sines and stores 16 bytes of bfloat16, q into [M, heads, head_dim], k into the row
+// of its cache place.  v: a lane takes one column for eight consecutive tokens and stores them as one 16-byte
+// piece of the transposed value cache when their cache places follow one another from a multiple of eight
+// (inside a prompt portion they do), else one by one.
+// What the epilogue needs from global memory (cosines and sines, cache places) is fetched by rope_fetch before
+// the accumulators go to LDS, so that the loads travel meanwhile; a tile of eight passes at a time.
+template <int ROWS, int COLS>
+struct RopeFetch {
+  static constexpr int LPR = COLS / 8, RPP = 64 / LPR, PASSES = ROWS / RPP;
+  static_assert(PASSES == 8 && COLS * (ROWS / 8) == 8 * 64, "eight passes of q/k rows, eight value items per lane");
+  f32x4_t c0[8], c1[8];   // q/k: (cos, sin) of this lane's four pairs in the row of pass p
+  int slot[8];            // q/k: the row's cache place; v: the first place of item p's eight tokens, -1 when they
+                          // form no run, -2 when the item lies past the last row
+};
+
+template <int ROWS, int COLS>
+__device__ inline void rope_fetch(RopeFetch<ROWS, COLS>& f, int lane, int mrow0, int ncol0, const RopeOut& rp, int M) {
+  using F = RopeFetch<ROWS, COLS>;
+  const int n0 = rp.col0 + ncol0;
+  const int q_dim = rp.n_heads * rp.head_dim, kv_dim = rp.n_kv * rp.head_dim;
+  if (n0 < q_dim + kv_dim) {
+    const int col = (lane % F::LPR) * 8, rr = lane / F::LPR;
+    const int d = (n0 + col) % rp.head_dim;
+    const bool rotate = d < rp.rotary_dim, is_q = n0 < q_dim;
+    const int half = rp.rotary_dim >> 1;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int m = min(mrow0 + p * F::RPP + rr, M - 1);
+      if (rotate) {
+        const f32x4_t* cs = (const f32x4_t*)(rp.cos_sin + (size_t)m * half + (d >> 1));
+        f.c0[p] = cs[0];
+        f.c1[p] = cs[1];
+      }
+      f.slot[p] = is_q ? 0 : rp.slots[m];
+    }
+    return;
+  }
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const int rg = (lane + 64 * p) / COLS;
+    const int m0 = mrow0 + rg * 8;
+    int s0 = -2;
+    if (m0 < M) {
+      s0 = -1;
+      if (m0 + 8 <= M) {
+        int sl[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sl[i] = rp.slots[m0 + i];
+        bool run = (sl[0] & 7) == 0;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) run = run && sl[i] == sl[0] + i;
+        if (run) s0 = sl[0];
+      }
+    }
+    f.slot[p] = s0;
+  }
+}
+
+template <int ROWS, int COLS, int LD>
+__device__ inline void emit_tile_rope(const float* ct, int lane, int mrow0, int ncol0, const RopeOut& rp, int M,
+                                      const RopeFetch<ROWS, COLS>& f) {
+  using F = RopeFetch<ROWS, COLS>;
+  const int n0 = rp.col0 + ncol0;                       // first column of the wave tile in the whole projection
+  const int q_dim = rp.n_heads * rp.head_dim, kv_dim = rp.n_kv * rp.head_dim;
+  if (n0 < q_dim + kv_dim) {
+    const int col = (lane % F::LPR) * 8, rr = lane / F::LPR;
+    const bool is_q = n0 < q_dim;
+    const int d = (n0 + col) % rp.head_dim;             // first of this lane's eight elements within its head
+    const int kh = is_q ? 0 : (n0 - q_dim) / rp.head_dim;
+    const bool rotate = d < rp.rotary_dim;
+    const float* src = ct + rr * LD + col;
+#pragma unroll
+    for (int p0 = 0; p0 < 8; p0 += 4) {
+      f32x4_t a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = *(const f32x4_t*)(src + (p0 + u) * F::RPP * LD);
+        b[u] = *(const f32x4_t*)(src + (p0 + u) * F::RPP * LD + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int p = p0 + u;
+        const int m = mrow0 + p * F::RPP + rr;
+        if (rotate) {
+          const f32x4_t c0 = f.c0[p], c1 = f.c1[p];
+          float x0, x1;
+          x0 = a[u][0]; x1 = a[u][1]; a[u][0] = x0 * c0[0] - x1 * c0[1]; a[u][1] = x0 * c0[1] + x1 * c0[0];
+          x0 = a[u][2]; x1 = a[u][3]; a[u][2] = x0 * c0[2] - x1 * c0[3]; a[u][3] = x0 * c0[3] + x1 * c0[2];
+          x0 = b[u][0]; x1 = b[u][1]; b[u][0] = x0 * c1[0] - x1 * c1[1]; b[u][1] = x0 * c1[1] + x1 * c1[0];
+          x0 = b[u][2]; x1 = b[u][3]; b[u][2] = x0 * c1[2] - x1 * c1[3]; b[u][3] = x0 * c1[3] + x1 * c1[2];
+        }
+        u32x4_t pk;
+        pk[0] = pack_bf16(a[u][0], a[u][1]);
+        pk[1] = pack_bf16(a[u][2], a[u][3]);
+        pk[2] = pack_bf16(b[u][0], b[u][1]);
+        pk[3] = pack_bf16(b[u][2], b[u][3]);
+        if (m >= M) continue;
+        bf16_t* dst;
+        if (is_q) {
+          dst = rp.q_out + (size_t)m * q_dim + n0 + col;
+        } else {
+          const size_t page = (size_t)(f.slot[p] / rp.page_size), off = (size_t)(f.slot[p] % rp.page_size);
+          dst = rp.k_cache + ((page * rp.n_kv + kh) * rp.page_size + off) * rp.head_dim + d;
+        }
+        *(u32x4_t*)dst = pk;
+      }
+    }
+    return;
+  }
+  // values: COLS columns x ROWS / 8 groups of eight tokens, one (column, group) per lane and pass
+  const int kh = (n0 - q_dim - kv_dim) / rp.head_dim, d0 = (n0 - q_dim - kv_dim) % rp.head_dim;
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const int it = lane + 64 * p;
+    const int colv = it % COLS, rg = it / COLS;
+    const int m0 = mrow0 + rg * 8;
+    const int s0 = f.slot[p];
+    if (s0 == -2) continue;
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = ct[(rg * 8 + i) * LD + colv];
+    if (s0 >= 0) {
+      const size_t page = (size_t)(s0 / rp.page_size), off = (size_t)(s0 % rp.page_size);
+      u32x4_t pk;
+      pk[0] = pack_bf16(y[0], y[1]);
+      pk[1] = pack_bf16(y[2], y[3]);
+      pk[2] = pack_bf16(y[4], y[5]);
+      pk[3] = pack_bf16(y[6], y[7]);
+      *(u32x4_t*)(rp.v_cache + ((page * rp.n_kv + kh) * rp.head_dim + d0 + colv) * rp.page_size + off) = pk;
+    } else {
+      for (int i = 0; i < 8 && m0 + i < M; ++i) {
+        const int sl = rp.slots[m0 + i];
+        const size_t page = (size_t)(sl / rp.page_size), off = (size_t)(sl % rp.page_size);
+        rp.v_cache[((page * rp.n_kv + kh) * rp.head_dim + d0 + colv) * rp.page_size + off] = float_to_bf16(y[i]);
+      }
+    }
+  }
+}
+
 // A wave's result rows [0, ROWS) x COLS columns, laid out in LDS with rows of LD floats, to memory: rows mrow0..,
 // columns ncol0.. of the launch's N (row stride ldo).  Four rows are read from LDS before the first of them is
 // stored, so that the reads (and, when adding into `out`, the loads) overlap.
@@ -338,7 +479,7 @@ __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0
 // and a second kernel adds the splits in ascending order and applies the epilogue.
 __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                         void* __restrict__ out, float* __restrict__ partial, int mode,
-                                                        int M, int N, int K, int pm, int ldo) {
+                                                        int M, int N, int K, int pm, int ldo, RopeOut rp) {
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE_BYTES];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -436,6 +577,8 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
   // ---- the result leaves through LDS: each wave lays its 128 x 64 tile out row by row -----------------
   __syncthreads();  // every wave is done with the stages
   float* ct = (float*)stages + wave * (128 * CLD);
+  RopeFetch<64, 64> fetched;   // (the rotating epilogue's loads travel while the tile goes to LDS)
+  if (mode == OUT_ROPE) rope_fetch(fetched, lane, m0 + wm * 128, n0 + wn * 64, rp, M);
   // result lane l of tile (i, j): rows i * 16 + (l / 16) * 4 + r, column j * 16 + l % 16
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -444,7 +587,13 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
 #pragma unroll
       for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's LDS writes before its reads
-  emit_tile<128, 64, CLD>(ct, lane, m0 + wm * 128, n0 + wn * 64, out, mode, M, N, ldo);
+  if (mode == OUT_ROPE) {
+    emit_tile_rope<64, 64, CLD>(ct, lane, m0 + wm * 128, n0 + wn * 64, rp, M, fetched);
+    rope_fetch(fetched, lane, m0 + wm * 128 + 64, n0 + wn * 64, rp, M);
+    emit_tile_rope<64, 64, CLD>(ct + 64 * CLD, lane, m0 + wm * 128 + 64, n0 + wn * 64, rp, M, fetched);
+  } else {
+    emit_tile<128, 64, CLD>(ct, lane, m0 + wm * 128, n0 + wn * 64, out, mode, M, N, ldo);
+  }
 }
 
 // ---- 256 x 256 block tiles ---------------------------------------------------------------------------
@@ -559,7 +708,7 @@ __device__ inline void read_all_big(FragsBig& f, unsigned aaddr, unsigned baddr)
 // No split of K here.  N: the columns of this launch (a multiple of 256); ldo as above.
 __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                             void* __restrict__ out, int mode, int M, int N, int K,
-                                                            int pm, int ldo) {
+                                                            int pm, int ldo, RopeOut rp) {
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NSB * STAGE_BIG];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -633,25 +782,45 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
     half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
     half_step_big<1, false, false>(acc, f, 0, 0, nullptr, nullptr, nullptr, voff, wave);
   }
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs' results, before they are read below
+  // The MFMAs are assembly, so the compiler does not know that their results take time: wait out the last ones
+  // (eight passes of the matrix core and the write-back).  The wait is tied to their accumulators, or the
+  // compiler may read them (a register copy on the way into the epilogue) before it.
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15"
+               : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]), "+a"(acc[7][4]), "+a"(acc[7][5]),
+                 "+a"(acc[7][6]), "+a"(acc[7][7])
+               :
+               : "memory");
+  // (and every other accumulator passes through an ordered statement after it)
+#pragma unroll
+  for (int i = 0; i < 7; ++i)
+    asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]), "+a"(acc[i][5]),
+                 "+a"(acc[i][6]), "+a"(acc[i][7]));
 
   // ---- the result leaves through LDS, 32 rows of the wave's 128 x 128 at a time ---------------------------
   __syncthreads();
   float* ct = (float*)stages + wave * (32 * CLDB);
   const int mw = m0 + wm * 128, nw = n0 + wn * 128;
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLDB + j * 16 + c] = acc[q * 2 + i][j][r];
-    // (this wave's LDS writes before its reads, and the reverse below)
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    emit_tile<32, 128, CLDB>(ct, lane, mw + q * 32, nw, out, mode, M, N, ldo);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // (written out four times: were the loop over the quarters not unrolled, the accumulators would be indexed at
+  // run time and live in scratch memory)
+#define QUARTER(Q)                                                                                              \
+  {                                                                                                             \
+    RopeFetch<32, 128> fetched;   /* the rotating epilogue's loads travel while the quarter goes to LDS */       \
+    if (mode == OUT_ROPE) rope_fetch(fetched, lane, mw + (Q) * 32, nw, rp, M);                                  \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i) _Pragma("unroll") for (int j = 0; j < 8; ++j)                 \
+        _Pragma("unroll") for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLDB + j * 16 + c] = acc[(Q) * 2 + i][j][r]; \
+    /* this wave's LDS writes before its reads, and the reverse below */                                        \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
+    if (mode == OUT_ROPE)                                                                                       \
+      emit_tile_rope<32, 128, CLDB>(ct, lane, mw + (Q) * 32, nw, rp, M, fetched);                               \
+    else                                                                                                        \
+      emit_tile<32, 128, CLDB>(ct, lane, mw + (Q) * 32, nw, out, mode, M, N, ldo);                              \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
   }
+  QUARTER(0)
+  QUARTER(1)
+  QUARTER(2)
+  QUARTER(3)
+#undef QUARTER
 }
 
 // ---- the same pipeline for 17..128 rows -----------------------------------------------------------
@@ -816,7 +985,8 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
 // float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
 int g_pipe_big = 0;   // tuning: 1 = 256 x 256 tiles for every whole block of 256 columns, 2 = never
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
-                   size_t scratch_floats, int tune_splits, hipStream_t s) {
+                   size_t scratch_floats, int tune_splits, const RopeOut* rope, hipStream_t s) {
+  if ((mode == OUT_ROPE) != (rope != nullptr)) return -1;
   if (K % BK != 0 || K < BK) return -1;
   if ((size_t)(BM - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;  // a lane's source offset is 32 bits
   if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
@@ -838,6 +1008,8 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
     splits = (KT + per - 1) / per;   // no split without a tile
   }
   const int ldo = mode == OUT_SWIGLU ? N / 2 : N;
+  RopeOut rp = {};
+  if (rope != nullptr) rp = *rope;
   // Whole rounds of 256 x 256 tiles first (see gemm_pipe_big_kernel), the columns that are left as above.
   // How many blocks of 256 columns take the big tiles: all, none, or whole rounds of 256 tiles, whichever
   // needs the fewest rounds when a big tile is priced at 1.72 small ones (measured: 113 against 65 us at
@@ -862,7 +1034,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
     const long Q2 = (nb_big + 7) / 8, QS2 = (Q2 + pq - 1) / pq;
     const long blocks2 = 8 * QS2 * MS * 32;
     hipLaunchKernelGGL(gemm_pipe_big_kernel, dim3((unsigned)blocks2), dim3(256), 0, s, x, w, out, mode, M, nb_big * BNB, K,
-                       pm, ldo);
+                       pm, ldo, rp);
     const int n_done = nb_big * BNB;
     if (n_done == N) return 0;
     // the rest of the columns
@@ -871,13 +1043,14 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
     const long Qr = (NBr + 7) / 8, QSr = (Qr + pq - 1) / pq;
     const long blocksr = 8 * QSr * MS * 32;
     const size_t esz = mode == OUT_BF16 || mode == OUT_SWIGLU ? 2 : 4;
-    void* out2 = (char*)out + (size_t)(mode == OUT_SWIGLU ? n_done / 2 : n_done) * esz;
+    void* out2 = out == nullptr ? nullptr : (char*)out + (size_t)(mode == OUT_SWIGLU ? n_done / 2 : n_done) * esz;
+    rp.col0 = n_done;
     hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocksr, 1), dim3(256), 0, s, x, w + (size_t)n_done * K, out2, scratch,
-                       mode, M, N2, K, pm, ldo);
+                       mode, M, N2, K, pm, ldo, rp);
     return 0;
   }
   hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks, splits), dim3(256), 0, s, x, w, out, scratch, mode, M, N, K,
-                     pm, ldo);
+                     pm, ldo, rp);
   if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,

@@ -321,26 +321,39 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
     return out if next_norm is None else (out, handed)
 
 
-def linear_rope_ok(m: int, k: int, head_dim: int, x_dtype: torch.dtype, cache_dtype: torch.dtype) -> bool:
-    """Whether ``linear_rope_kv`` takes a projection of m rows."""
-    return (_backend is None and allow_mfma and 0 < m <= 16 and k % 32 == 0 and head_dim % 16 == 0
-            and x_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16)
+#: long steps may rotate and store in the projection's epilogue too (False: only the few rows of decoding)
+rope_in_long_products = True
+
+
+def linear_rope_ok(m: int, n: int, k: int, head_dim: int, rotary_dim: int, page_size: int, x_dtype: torch.dtype,
+                   cache_dtype: torch.dtype, prenormed: bool = False) -> bool:
+    """Whether ``linear_rope_kv`` takes a projection of m rows onto n columns: a few rows (decoding), or a long
+    step with enough result tiles (256 x 128) to give every CU work without splitting K, heads of 128."""
+    if not (_backend is None and allow_mfma and x_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16):
+        return False
+    if 0 < m <= 16:
+        return k % 32 == 0 and head_dim % 16 == 0
+    tiles = -(-m // 256) * -(-n // 128)
+    return (rope_in_long_products and m > 128 and tiles >= 128 and k % 64 == 0 and 255 * k * 2 + 128 < 2 ** 32 and head_dim == 128
+            and rotary_dim % 8 == 0 and page_size % 8 == 0 and not prenormed)
 
 
 def linear_rope_kv(x, w: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, inv_freq: Optional[torch.Tensor],
                    rotary_dim: int, factor: float, num_heads: int, num_kv_heads: int, head_dim: int,
                    k_cache: torch.Tensor, v_cache: torch.Tensor, cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The q/k/v projection of at most 16 bfloat16 rows (or ``Prenormed`` rows) with the rotation and the
-    cache write in its epilogue: the same result as ``linear`` to float32 followed by ``rope_kv_write``
-    (w's q and k heads in paired order), without the kernel and the rows in between.  Returns q as
-    bfloat16 [m, heads, head_dim]."""
+    """The q/k/v projection of bfloat16 rows (at most 16, also ``Prenormed``; or a long step, see
+    ``linear_rope_ok``) with the rotation and the cache write in its epilogue: the same result as ``linear``
+    to float32 followed by ``rope_kv_write`` (w's q and k heads in paired order), without the kernel and the
+    rows in between.  Returns q as bfloat16 [m, heads, head_dim]."""
     x, pre = _pre_args(x)
     _dev_ok(x, w, positions, slots, inv_freq, k_cache, v_cache)
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_rope_kv: shapes {tuple(x.shape)} x {tuple(w.shape)}")
     m, k = x.shape
     n = w.shape[0]
-    _need(linear_rope_ok(m, k, head_dim, x.dtype, k_cache.dtype) and w.dtype == torch.bfloat16,
-          "linear_rope_kv: at most 16 bfloat16 rows, k % 32 == 0, head_dim % 16 == 0, a bfloat16 cache")
+    _need(linear_rope_ok(m, n, k, head_dim, rotary_dim, k_cache.shape[2] if k_cache.dim() == 4 else 0, x.dtype, k_cache.dtype,
+                         pre[1] != 0) and w.dtype == torch.bfloat16,
+          "linear_rope_kv: sizes or dtypes that the fused projection does not take (see linear_rope_ok)")
+    _need(m <= 16 or cos_sin is not None, "linear_rope_kv: a long step needs the table of cosines and sines")
     _need(n == (num_heads + 2 * num_kv_heads) * head_dim, f"linear_rope_kv: {n} weight rows for {num_heads} + 2 x {num_kv_heads} heads of {head_dim}")
     _i32(positions, m, "positions")
     _i32(slots, m, "slots")

@@ -85,8 +85,9 @@ class PagedAttention(Mixer):
         q = None
         if rot is not None and cache.writes:
             rows = x.x if isinstance(x, ops.Prenormed) else x
-            if ops.linear_rope_ok(rows.shape[0], rows.shape[1], self.head_dim, rows.dtype, cache.k.dtype):
-                # a few rows (decoding): the projection rotates and stores its rows itself
+            if ops.linear_rope_ok(rows.shape[0], self.wqkv.shape[0], rows.shape[1], self.head_dim, rot[1], cache.k.shape[2],
+                                  rows.dtype, cache.k.dtype, isinstance(x, ops.Prenormed)):
+                # a few rows (decoding) or a long step: the projection rotates and stores its rows itself
                 table = self.position.table(ctx, always=True) if hasattr(self.position, "table") else None
                 q = ops.linear_rope_kv(x, self.wqkv, ctx.positions, ctx.slot_mapping[cache.group], rot[0], rot[1], rot[2],
                                        self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v, table)

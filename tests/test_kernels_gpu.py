@@ -111,7 +111,9 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
 
 
 @pytest.mark.parametrize("m,heads,kv,d,rot,k,page", [(1, 4, 2, 64, 64, 256, 16), (8, 32, 8, 128, 128, 4096, 16),
-                                                    (16, 3, 1, 48, 32, 96, 8), (5, 6, 3, 16, 16, 2048, 32)])
+                                                    (16, 3, 1, 48, 32, 96, 8), (5, 6, 3, 16, 16, 2048, 32),
+                                                    (2100, 32, 8, 128, 128, 128, 16), (3000, 24, 8, 128, 64, 192, 8),
+                                                    (4300, 4, 2, 128, 128, 64, 16)])
 def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
     """The projection of a few rows that rotates and stores its rows in its epilogue gives the bits of the
     plain product followed by the rotation and cache-write kernel; and both agree with float64."""
@@ -122,8 +124,16 @@ def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
     x = torch.randn(m, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=g) * 0.1).to(torch.bfloat16)
     pos = torch.randint(0, 100000, (m,), generator=g, dtype=torch.int32)
-    pages = 5
-    slots = torch.randperm(pages * page, generator=g)[:m].to(torch.int32)
+    pages = 5 + (m + page - 1) // page
+    if m <= 16:
+        slots = torch.randperm(pages * page, generator=g)[:m].to(torch.int32)
+    else:   # a portion that starts three tokens into a page and walks shuffled pages, then scattered places
+        order = torch.randperm(pages, generator=g).tolist()
+        first = m * 3 // 4
+        sl = [order[(3 + i) // page] * page + (3 + i) % page for i in range(first)]
+        used = set(sl)
+        sl += [s_ for s_ in torch.randperm(pages * page, generator=g).tolist() if s_ not in used][: m - first]
+        slots = torch.tensor(sl, dtype=torch.int32)
     inv = rotary_inv_freq(d, 500000.0, None, rot)
     kc = torch.zeros(pages, kv, page, d, dtype=torch.bfloat16)
     vc = torch.zeros(pages, kv, d, page, dtype=torch.bfloat16)
@@ -131,9 +141,11 @@ def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
     k1, v1 = kc.to(DEV), vc.to(DEV)
     q1 = ops.rope_kv_write(ops.linear(xd, wd, torch.float32), pd, sd, invd, rot, 1.0, heads, kv, d, k1, v1, torch.bfloat16)
     k2, v2 = kc.to(DEV), vc.to(DEV)
-    q2 = ops.linear_rope_kv(xd, wd, pd, sd, invd, rot, 1.0, heads, kv, d, k2, v2)
+    assert ops.linear_rope_ok(m, n, k, d, rot, page, torch.bfloat16, torch.bfloat16)
+    q2 = ops.linear_rope_kv(xd, wd, pd, sd, invd, rot, 1.0, heads, kv, d, k2, v2,
+                            ops.rope_table(pd, invd, rot, 1.0) if m > 16 else None)
     assert torch.equal(q2, q1) and torch.equal(k2, k1) and torch.equal(v2, v1)
-    if rot:   # with the step's table of cosines and sines: the same bits again
+    if rot and m <= 16:   # with the step's table of cosines and sines: the same bits again
         k3, v3 = kc.to(DEV), vc.to(DEV)
         q3 = ops.linear_rope_kv(xd, wd, pd, sd, invd, rot, 1.0, heads, kv, d, k3, v3, ops.rope_table(pd, invd, rot, 1.0))
         assert torch.equal(q3, q1) and torch.equal(k3, k1) and torch.equal(v3, v1)
