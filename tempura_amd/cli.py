@@ -77,7 +77,7 @@ def cmd_run(args) -> int:
     from .sampling import SamplingParams
     eng = _engine_from_args(args)
     prompts = _prompts_from_args(args, eng.model.spec.vocab_size)
-    params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
+    params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p, typical_p=args.typical_p,
                             repeat_penalty=args.repeat_penalty, penalty_last_n=args.penalty_last_n,
                             presence_penalty=args.presence_penalty, frequency_penalty=args.frequency_penalty,
                             seed=args.sampling_seed, max_new_tokens=args.max_new_tokens,
@@ -144,6 +144,7 @@ def main(argv=None) -> int:
     p.add_argument("--top-k", type=int, default=50)
     p.add_argument("--top-p", type=float, default=1.0)
     p.add_argument("--min-p", type=float, default=0.0)
+    p.add_argument("--typical-p", type=float, default=1.0)
     p.add_argument("--repeat-penalty", type=float, default=1.0)
     p.add_argument("--penalty-last-n", type=int, default=64)
     p.add_argument("--presence-penalty", type=float, default=0.0)

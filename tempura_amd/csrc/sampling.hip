@@ -114,7 +114,9 @@ extern "C" int tp_apply_penalties(float* logits, int vocab, const int* rows, con
 
 // ---- filtered sampling ----------------------------------------------------------------
 // One block of 1024 threads per row:
-//   x = logit / temperature; drop x < max + ln(min_p); keep the top_k largest; softmax;
+//   x = logit / temperature; drop x < max + ln(min_p); typical-p: keep the tokens whose information
+//   -ln p lies closest to the entropy, up to a mass above typical_p
+//   (/root/reference/kernels/src/sampler_chain.rs:87-141); keep the top_k largest; softmax;
 //   keep the shortest prefix (by descending probability) whose mass reaches top_p;
 //   renormalise; walk the survivors in INDEX order and return the first index whose
 //   cumulative mass exceeds r (/root/reference/kernels/src/sampling.rs:229-333).
@@ -160,15 +162,24 @@ __device__ inline unsigned long long block_excl_scan(unsigned long long v, unsig
   return base + inc - v;
 }
 
+// The key that elements are selected by, largest first: the value itself, or (TYP) how close the element's
+// information -ln p is to the entropy H, closest first.  With d = v - max and p = exp(d) / Z:
+// -ln p - H = ln Z - d - (ln Z - sum p d) = mean_d - d, the distance of d from its mean under p.
+template <bool TYP>
+__device__ inline unsigned int select_key(float v, float maxv, float mean_d) {
+  if (TYP) return ~float_key(fabsf(mean_d - (v - maxv)));
+  return float_key(v);
+}
+
 // Radix selection from the top: finds the key K such that weight(key > K) < target <=
 // weight(key >= K), where an element's weight is 1 (MASS = false) or its fixed-point mass.
-// Only elements with key >= floor_key take part.  Returns K; *gt = weight(key > K),
+// Only elements whose VALUE key is >= floor_key take part.  Returns K; *gt = weight(key > K),
 // *eq_count = number of elements with key == K.
-template <bool MASS>
+template <bool MASS, bool TYP = false>
 __device__ unsigned int radix_select(const float* __restrict__ x, int n, float maxv, unsigned int floor_key,
                                      unsigned long long target, unsigned long long* hist /*256*/,
                                      unsigned int* cnt /*256*/, unsigned long long* sh /*4*/,
-                                     unsigned long long* gt_out, unsigned int* eq_count) {
+                                     unsigned long long* gt_out, unsigned int* eq_count, float mean_d = 0.f) {
   unsigned int prefix = 0;
   unsigned long long gt = 0;
   for (int pass = 0; pass < 4; ++pass) {
@@ -181,8 +192,8 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
     __syncthreads();
     for (int j = threadIdx.x; j < n; j += blockDim.x) {
       const float v = x[j];
-      const unsigned int key = float_key(v);
-      if (key < floor_key) continue;
+      if (float_key(v) < floor_key) continue;
+      const unsigned int key = select_key<TYP>(v, maxv, mean_d);
       if (pass > 0 && (key >> (shift + 8)) != prefix) continue;
       const unsigned int bin = (key >> shift) & 255u;
       atomicAdd(&cnt[bin], 1u);
@@ -231,10 +242,39 @@ __device__ void drop_surplus_ties(float* __restrict__ x, int n, unsigned int K, 
   __syncthreads();
 }
 
+// The typical-p cut: survivors with a selection key above K stay, those below go; the ones at K stay in index
+// order for as long as the mass before them is short of `need`.  Survivors without mass go as well (the
+// reference only lists tokens of positive probability).
+__device__ void typical_cut(float* __restrict__ x, int n, float maxv, unsigned int floor_key, float mean_d,
+                            unsigned int K, unsigned long long need, unsigned long long* lds) {
+  const int per = (n + SMP_THREADS - 1) / SMP_THREADS;
+  const int lo = min(n, (int)threadIdx.x * per), hi = min(n, lo + per);
+  unsigned long long mine = 0;
+  for (int j = lo; j < hi; ++j) {
+    const float v = x[j];
+    if (float_key(v) >= floor_key && select_key<true>(v, maxv, mean_d) == K) mine += fix_mass(v, maxv);
+  }
+  unsigned long long total;
+  unsigned long long before = block_excl_scan(mine, lds, &total);
+  for (int j = lo; j < hi; ++j) {
+    const float v = x[j];
+    if (float_key(v) < floor_key) continue;
+    const unsigned int key = select_key<true>(v, maxv, mean_d);
+    const unsigned long long q = fix_mass(v, maxv);
+    bool keep = key > K;
+    if (key == K) {
+      keep = before < need;
+      before += q;
+    }
+    if (!keep || q == 0) x[j] = -INFINITY;
+  }
+  __syncthreads();
+}
+
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int vocab, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
-    const float* __restrict__ rnd, int* __restrict__ out) {
+    const float* __restrict__ typical_p, const float* __restrict__ rnd, int* __restrict__ out) {
   __shared__ unsigned long long hist[256];
   __shared__ unsigned int cnt[256];
   __shared__ unsigned long long sh[4];
@@ -291,6 +331,29 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float thr = maxv + logf(mp);
     const unsigned int k2 = float_key(thr);
     if (k2 > floor_key) floor_key = k2;
+  }
+
+  // 2b. typical_p: the survivors nearest the entropy, nearest first, until their mass exceeds typical_p
+  const float typ = typical_p[row];
+  if (typ < 1.0f) {
+    unsigned long long part = 0;
+    float s1 = 0.f;
+    for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
+      const float v = x[j];
+      if (float_key(v) >= floor_key) {
+        part += fix_mass(v, maxv);
+        s1 += expf(v - maxv) * (v - maxv);
+      }
+    }
+    unsigned long long Z0;
+    block_excl_scan(part, scan, &Z0);
+    const float mean_d = block_sum(s1, fscratch) / ((float)Z0 * (1.0f / SMP_FIX));
+    unsigned long long target = (unsigned long long)((double)fmaxf(typ, 0.f) * (double)Z0) + 1;   // mass > typical_p
+    if (target > Z0) target = Z0;
+    unsigned long long gt;
+    unsigned int eq;
+    const unsigned int K = radix_select<true, true>(x, vocab, maxv, floor_key, target, hist, cnt, sh, &gt, &eq, mean_d);
+    typical_cut(x, vocab, maxv, floor_key, mean_d, K, target - gt, scan);
   }
 
   // 3. top_k: the k-th largest value among the survivors
@@ -368,12 +431,12 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
 }
 
 extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
-                         const int* top_k, const float* top_p, const float* min_p, const float* rnd, int* out,
-                         hipStream_t s) {
+                         const int* top_k, const float* top_p, const float* min_p, const float* typical_p,
+                         const float* rnd, int* out, hipStream_t s) {
   TP_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes");
   if (rows == 0) return 0;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, work, vocab, temperature, top_k,
-                     top_p, min_p, rnd, out);
+                     top_p, min_p, typical_p, rnd, out);
   TP_CHECK_LAUNCH("sample");
   return 0;
 }

@@ -536,24 +536,27 @@ def apply_penalties(logits: torch.Tensor, rows, tokens, counts, in_window, prese
           _ptr(fl[0]), _ptr(fl[1]), _ptr(fl[2]), n, _stream())
 
 
-def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, min_p, rnd) -> torch.Tensor:
+def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, min_p, rnd, typical_p=None) -> torch.Tensor:
     """float32 [m, vocab] and per-row options (host arrays) -> int32 [m] chosen tokens.
-    ``work`` is float32 scratch of at least [m, vocab].  temperature 0 rows return the argmax."""
+    ``work`` is float32 scratch of at least [m, vocab].  temperature 0 rows return the argmax.
+    ``typical_p`` None leaves that filter off (1.0) in every row."""
+    if typical_p is None:
+        typical_p = [1.0] * len(temperature)
     if _backend is not None:
-        return _backend.sample(logits, work, temperature, top_k, top_p, min_p, rnd)
+        return _backend.sample(logits, work, temperature, top_k, top_p, min_p, rnd, typical_p)
     import numpy as np
     _dev_ok(logits, work)
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits must be float32 [m, vocab]")
     m, vocab = logits.shape
     _need(work.dtype == torch.float32 and work.numel() >= m * vocab, "sample: work buffer too small")
-    for a in (temperature, top_k, top_p, min_p, rnd):
+    for a in (temperature, top_k, top_p, min_p, rnd, typical_p):
         _need(len(a) == m, "sample: one option per row")
     dev = logits.device
-    fl = _dev_array([temperature, top_p, min_p, rnd], np.float32, dev)
+    fl = _dev_array([temperature, top_p, min_p, rnd, typical_p], np.float32, dev)
     tk = _dev_array(top_k, np.int32, dev)
     out = torch.empty((m,), dtype=torch.int32, device=dev)
     _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
-          _ptr(fl[3]), _ptr(out), _stream())
+          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _stream())
     return out
 
 

@@ -13,7 +13,7 @@ class SamplingParams:
     top_k: int = 50                 # keep the k largest; 0 switches the filter off (the reference panics on 0)
     top_p: float = 1.0              # nucleus over the kept ones
     min_p: float = 0.0              # drop logits below max + ln(min_p)
-    typical_p: float = 1.0          # not implemented: anything but 1.0 is refused
+    typical_p: float = 1.0          # keep the tokens nearest the entropy until their mass exceeds it; 1.0 = off
     repeat_penalty: float = 1.0     # over the last `penalty_last_n` tokens of prompt + output
     penalty_last_n: int = 64
     presence_penalty: float = 0.0   # over generated tokens
@@ -32,8 +32,8 @@ class SamplingParams:
             raise ValueError("top_p must be in (0, 1]")
         if not (0 <= self.min_p <= 1.0):
             raise ValueError("min_p must be in [0, 1]")
-        if self.typical_p != 1.0:
-            raise ValueError("typical_p filtering is not implemented; leave it at 1.0")
+        if not (0 <= self.typical_p <= 1.0):
+            raise ValueError("typical_p must be in [0, 1]")
         if self.repeat_penalty <= 0:
             raise ValueError("repeat_penalty must be positive")
         if self.max_new_tokens < 0:

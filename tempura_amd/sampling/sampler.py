@@ -1,7 +1,7 @@
 """Next-token choice on the GPU for a batch of rows with per-row options.
 
 The reference samples on the CPU (/root/reference/kernels/src/sampling.rs:229-333);
-here the logits never leave the device: penalties, temperature, min-p, top-k, softmax,
+here the logits never leave the device: penalties, temperature, min-p, typical-p, top-k, softmax,
 top-p and the draw are kernels, and only the chosen token ids come back.
 
 Random numbers: draw number n of a request with seed s is a 24-bit fraction of a
@@ -57,11 +57,12 @@ class Sampler:
         top_k = np.asarray([p.top_k if 0 < p.top_k < self.vocab_size else 0 for p in params], dtype=np.int32)
         top_p = np.asarray([p.top_p for p in params], dtype=np.float32)
         min_p = np.asarray([p.min_p for p in params], dtype=np.float32)
+        typical_p = np.asarray([p.typical_p for p in params], dtype=np.float32)
         rnd = np.asarray([uniform_draw(self.default_seed if p.seed is None else p.seed, n)
                           for p, n in zip(params, draw_index)], dtype=np.float32)
         if self._work is None or self._work.shape[0] < m:
             self._work = torch.empty((max(m, 8), self.vocab_size), dtype=torch.float32, device=self.device)
-        return ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd).tolist()
+        return ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd, typical_p).tolist()
 
     def _penalised(self, logits, params, prompt_tokens, output_tokens):
         rows, toks, counts, inwin = [], [], [], []

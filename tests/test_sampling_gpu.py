@@ -8,10 +8,31 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def plain_sample(logits, temperature, top_k, top_p, min_p, r):
-    """temperature scale, min-p, top-k, softmax over the kept, top-p prefix, renormalise, walk the
+def plain_typical(x, typical_p):
+    """Keep the tokens whose information -ln p is nearest the entropy, nearest first (ties by index), until
+    their mass exceeds typical_p; the others become -inf (/root/reference/kernels/src/sampler_chain.rs:87-141)."""
+    p = torch.softmax(x, 0)
+    pos = p > 0
+    ent = -(p[pos] * p[pos].log()).sum()
+    score = torch.full_like(p, math.inf)
+    score[pos] = (-p[pos].log() - ent).abs()
+    order = torch.argsort(score, stable=True)
+    out = torch.full_like(x, -math.inf)
+    cum = 0.0
+    for i in order.tolist():
+        if not pos[i]:
+            break
+        cum += float(p[i])
+        out[i] = x[i]
+        if cum > typical_p:
+            break
+    return out
+
+
+def plain_sample(logits, temperature, top_k, top_p, min_p, r, typical_p=1.0):
+    """temperature scale, min-p, typical-p, top-k, softmax over the kept, top-p prefix, renormalise, walk the
     probabilities in INDEX order and return the first index whose cumulative sum exceeds r
-    (/root/reference/kernels/src/sampling.rs:229-333, min-p /root/reference/kernels/src/sampler_chain.rs:54-80)."""
+    (/root/reference/kernels/src/sampling.rs:192-333, min-p /root/reference/kernels/src/sampler_chain.rs:54-80)."""
     x = logits.double().clone()
     if temperature == 0:
         mx = x.max()
@@ -20,6 +41,8 @@ def plain_sample(logits, temperature, top_k, top_p, min_p, r):
         x = x / temperature
     if min_p > 0:
         x[x < x.max() + math.log(min_p)] = -math.inf
+    if typical_p < 1.0:
+        x = plain_typical(x, typical_p)
     V = x.numel()
     order = torch.argsort(x, descending=True, stable=True)
     k = V if top_k <= 0 else min(top_k, V)
@@ -40,13 +63,13 @@ def plain_sample(logits, temperature, top_k, top_p, min_p, r):
     return int(hit[0]) if hit.numel() else V - 1
 
 
-def _sample(logits, temperature, top_k, top_p, min_p, r):
+def _sample(logits, temperature, top_k, top_p, min_p, r, typical_p=1.0):
     from tempura_amd.kernels import ops
     ops.set_backend(None)
     m, v = logits.shape
     work = torch.empty(m, v, device=DEV)
     full = lambda a: [a] * m if not isinstance(a, (list, tuple)) else list(a)
-    return ops.sample(logits.to(DEV), work, full(temperature), full(top_k), full(top_p), full(min_p), full(r)).tolist()
+    return ops.sample(logits.to(DEV), work, full(temperature), full(top_k), full(top_p), full(min_p), full(r), full(typical_p)).tolist()
 
 
 @pytest.mark.parametrize("vocab", [16, 301, 4099])
@@ -59,6 +82,38 @@ def test_sample_matches_plain_rules(vocab, temperature, top_k, top_p, min_p):
     got = _sample(logits, temperature, top_k, top_p, min_p, rs)
     want = [plain_sample(logits[i], temperature, top_k, top_p, min_p, rs[i]) for i in range(24)]
     assert got == want
+
+
+@pytest.mark.parametrize("vocab", [16, 301, 4099])
+@pytest.mark.parametrize("temperature,top_k,top_p,min_p,typical_p", [(1.0, 0, 1.0, 0.0, 0.9), (0.8, 0, 1.0, 0.0, 0.5), (1.2, 20, 0.9, 0.0, 0.7),
+                                                                      (1.0, 0, 1.0, 0.05, 0.3), (1.0, 0, 1.0, 0.0, 0.0)])
+def test_typical_p_matches_plain_rules(vocab, temperature, top_k, top_p, min_p, typical_p):
+    g = torch.Generator().manual_seed(7 * vocab + int(typical_p * 10))
+    logits = torch.randn(24, vocab, generator=g) * 2.5
+    rs = [(i + 0.61) / 24 for i in range(24)]
+    got = _sample(logits, temperature, top_k, top_p, min_p, rs, typical_p)
+    want = [plain_sample(logits[i], temperature, top_k, top_p, min_p, rs[i], typical_p) for i in range(24)]
+    assert got == want
+
+
+def test_typical_p_drops_a_likely_but_untypical_token():
+    # token 0 holds 30 % of the mass, 700 others share the rest: the entropy is near the information of a tail
+    # token, so token 0 is the LEAST typical and leaves first, although every other filter would keep it
+    V = 701
+    lg = torch.full((1, V), math.log(0.7 / 700))
+    lg[0, 0] = math.log(0.3)
+    rows = lg.repeat(64, 1)
+    rs = [(i + 0.5) / 64 for i in range(64)]
+    assert 0 in _sample(rows, 1.0, 0, 1.0, 0.0, rs)                      # without the filter a draw below 0.3 takes it
+    got = _sample(rows, 1.0, 0, 1.0, 0.0, rs, 0.5005)
+    assert 0 not in got
+    # equal scores are admitted in index order: a mass above 0.5005 needs 501 of the 700 tail tokens
+    assert got == [plain_sample(lg[0], 1.0, 0, 1.0, 0.0, r, 0.5005) for r in rs]
+    assert 490 <= max(got) <= 501 and min(got) >= 1
+    # all logits equal: every token is equally typical, the first ones in index order whose mass exceeds 0.255 stay
+    flat = torch.zeros(32, 100)
+    got = _sample(flat, 1.0, 0, 1.0, 0.0, [(i + 0.5) / 32 for i in range(32)], 0.255)
+    assert max(got) == 25 and min(got) == 0
 
 
 def test_greedy_ties_and_fallthrough():
