@@ -274,7 +274,8 @@ __device__ void typical_cut(float* __restrict__ x, int n, float maxv, unsigned i
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int vocab, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
-    const float* __restrict__ typical_p, const float* __restrict__ rnd, int* __restrict__ out) {
+    const float* __restrict__ typical_p, const float* __restrict__ rnd, int* __restrict__ out,
+    float* __restrict__ info) {
   __shared__ unsigned long long hist[256];
   __shared__ unsigned int cnt[256];
   __shared__ unsigned long long sh[4];
@@ -285,9 +286,11 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   const int row = blockIdx.x;
   const float* lg = logits + (size_t)row * vocab;
   float* x = work + (size_t)row * vocab;
-  const float T = temperature[row];
+  const bool greedy = !(temperature[row] > 0.f);
+  const float T = greedy ? 1.0f : temperature[row];   // a greedy row that reports probabilities filters unscaled logits
+  float* inf = info == nullptr ? nullptr : info + 4 * row;
 
-  if (!(T > 0.f)) {  // greedy: argmax, last maximum wins
+  if (greedy) {  // argmax, last maximum wins
     float bv = -INFINITY;
     int bi = -1;
     for (int j = threadIdx.x; j < vocab; j += blockDim.x) argmax_merge(bv, bi, lg[j], j);
@@ -304,9 +307,13 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     if (threadIdx.x == 0) {
       for (int i = 1; i < SMP_WAVES; ++i) argmax_merge(bv, bi, vbest[i], ibest[i]);
       out[row] = bi < 0 ? vocab - 1 : bi;
+      ibest[0] = bi < 0 ? vocab - 1 : bi;
     }
-    return;
+    if (inf == nullptr) return;
+    __syncthreads();
   }
+  const int greedy_pick = greedy ? ibest[0] : -1;
+  __syncthreads();
 
   // 1. scale by the temperature, find the maximum
   float mx = -INFINITY;
@@ -320,7 +327,15 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   const float maxv = block_max(mx, fscratch);
   __syncthreads();
   if (maxv == -INFINITY) {  // nothing to choose from: the reference falls through to the last index
-    if (threadIdx.x == 0) out[row] = vocab - 1;
+    if (threadIdx.x == 0) {
+      if (!greedy) out[row] = vocab - 1;
+      if (inf != nullptr) {
+        inf[0] = 0.f;
+        inf[1] = 0.f;
+        inf[2] = INFINITY;      // no survivor
+        inf[3] = -INFINITY;
+      }
+    }
     return;
   }
 
@@ -399,6 +414,22 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     Z = gt + (need < (unsigned long long)eq ? need : (unsigned long long)eq) * q;
   }
 
+  // what a caller needs for log-probabilities of the final distribution: ln p(v) = (v - max) - ln Z for v >= floor
+  const float lnZ = logf((float)((double)Z * (1.0 / (double)SMP_FIX)));
+  if (inf != nullptr && threadIdx.x == 0) {
+    const unsigned int u = (floor_key & 0x80000000u) ? (floor_key & 0x7fffffffu) : ~floor_key;
+    inf[0] = maxv;
+    inf[1] = lnZ;
+    inf[2] = __uint_as_float(u);
+    if (greedy) {
+      const float v = x[greedy_pick];
+      inf[3] = (Z > 0 && float_key(v) >= floor_key) ? (v - maxv) - lnZ : -INFINITY;
+    } else if (Z == 0) {
+      inf[3] = -INFINITY;
+    }
+  }
+  if (greedy) return;
+
   // 6. draw: first index (index order) whose cumulative mass exceeds r * Z
   const float r = rnd[row];
   unsigned long long t = (unsigned long long)((double)r * (double)Z);
@@ -427,16 +458,90 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
       }
     }
     out[row] = pick;
+    if (inf != nullptr) inf[3] = (x[pick] - maxv) - lnZ;
+  }
+}
+
+// The n most probable tokens of the distribution a row was drawn from (value descending, ties by index), with their
+// log-probabilities (/root/reference/engine/src/model.rs:497-526).  `work` and `info` are what sample_kernel left.
+// ids beyond the number of survivors are -1.
+__global__ __launch_bounds__(SMP_THREADS) void top_logprobs_kernel(const float* __restrict__ work, const float* __restrict__ info,
+                                                                   int vocab, int n, int* __restrict__ ids,
+                                                                   float* __restrict__ lps) {
+  __shared__ int ibest[SMP_WAVES];
+  __shared__ float vbest[SMP_WAVES];
+  const int row = blockIdx.x;
+  const float* x = work + (size_t)row * vocab;
+  const float maxv = info[4 * row], lnZ = info[4 * row + 1], floorv = info[4 * row + 2];
+  float last_v = INFINITY;
+  int last_i = -1;
+  for (int i = 0; i < n; ++i) {
+    float bv = -INFINITY;
+    int bi = -1;
+    auto better = [](float v, int j, float bv, int bi) { return j >= 0 && (bi < 0 || v > bv || (v == bv && j < bi)); };
+    for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
+      const float v = x[j];
+      if (!(v >= floorv) || v == -INFINITY) continue;
+      if (!(v < last_v || (v == last_v && j > last_i))) continue;   // taken in an earlier turn
+      if (better(v, j, bv, bi)) {
+        bv = v;
+        bi = j;
+      }
+    }
+    for (int o = TP_WAVE / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, TP_WAVE);
+      const int oi = __shfl_xor(bi, o, TP_WAVE);
+      if (better(ov, oi, bv, bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x % TP_WAVE == 0) {
+      vbest[threadIdx.x / TP_WAVE] = bv;
+      ibest[threadIdx.x / TP_WAVE] = bi;
+    }
+    __syncthreads();
+    bv = vbest[0];
+    bi = ibest[0];
+    for (int w = 1; w < SMP_WAVES; ++w)
+      if (better(vbest[w], ibest[w], bv, bi)) {
+        bv = vbest[w];
+        bi = ibest[w];
+      }
+    if (threadIdx.x == 0) {
+      ids[row * n + i] = bi;
+      lps[row * n + i] = bi < 0 ? -INFINITY : (bv - maxv) - lnZ;
+    }
+    if (bi < 0) {
+      for (int k = i + 1 + threadIdx.x; k < n; k += blockDim.x) {
+        ids[row * n + k] = -1;
+        lps[row * n + k] = -INFINITY;
+      }
+      break;
+    }
+    last_v = bv;
+    last_i = bi;
   }
 }
 
 extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p, const float* typical_p,
-                         const float* rnd, int* out, hipStream_t s) {
+                         const float* rnd, int* out, float* info, hipStream_t s) {
   TP_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes");
   if (rows == 0) return 0;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, work, vocab, temperature, top_k,
-                     top_p, min_p, typical_p, rnd, out);
+                     top_p, min_p, typical_p, rnd, out, info);
   TP_CHECK_LAUNCH("sample");
+  return 0;
+}
+
+// `info` [rows, 4] and `work` as tp_sample left them; ids and lps are [rows, n].
+extern "C" int tp_top_logprobs(const float* work, const float* info, int rows, int vocab, int n, int* ids, float* lps,
+                               hipStream_t s) {
+  TP_REQUIRE(rows >= 0 && vocab > 0 && n >= 0, "top_logprobs: bad sizes");
+  if (rows == 0 || n == 0) return 0;
+  hipLaunchKernelGGL(top_logprobs_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, work, info, vocab, n, ids, lps);
+  TP_CHECK_LAUNCH("top_logprobs");
   return 0;
 }

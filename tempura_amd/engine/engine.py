@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import itertools
 import time
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple, Union
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple, Union
 
 import torch
 
@@ -75,7 +75,9 @@ class Engine:
 
     # ---- requests ------------------------------------------------------------
     def add_request(self, prompt_ids: Sequence[int], params: Optional[SamplingParams] = None,
-                    rid: Optional[Hashable] = None) -> Hashable:
+                    rid: Optional[Hashable] = None, logprobs_top_n: Optional[int] = None) -> Hashable:
+        """Queue a request.  With ``logprobs_top_n`` (0..20) every generated token gets a ``TokenLogprob``
+        record in ``request(rid).logprobs``."""
         params = params or SamplingParams()
         if rid is None:
             rid = next(self._ids)
@@ -86,7 +88,8 @@ class Engine:
             if t < 0 or t >= vocab:
                 raise ValueError(f"token id {t} outside the vocabulary of {vocab}")
         eos = params.eos_token_id if params.eos_token_id is not None else self.model.spec.eos_token_ids
-        req = Request(rid, [int(t) for t in prompt_ids], params, tuple(int(e) for e in eos))
+        req = Request(rid, [int(t) for t in prompt_ids], params, tuple(int(e) for e in eos),
+                      logprobs_top_n=logprobs_top_n)
         self.scheduler.add_request(req)
         self._requests[rid] = req
         self.counters["prompt_tokens"] += len(req.prompt)
@@ -113,9 +116,16 @@ class Engine:
         sampling = [it.request for it in items if it.samples]
         out: List[Tuple[Hashable, int, bool]] = []
         if sampling:
+            wanted = [r.logprobs_top_n for r in sampling if r.logprobs_top_n is not None]
             tokens = self.sampler.sample(
                 logits, [r.params for r in sampling], [len(r.output) for r in sampling],
-                [r.prompt for r in sampling], [r.output for r in sampling])
+                [r.prompt for r in sampling], [r.output for r in sampling], top_n=max(wanted) if wanted else None)
+            if wanted:
+                tokens, records = tokens
+                for req, rec in zip(sampling, records):
+                    if req.logprobs_top_n is not None:
+                        rec.top_logprobs = rec.top_logprobs[: req.logprobs_top_n]
+                        req.logprobs.append(rec)
             for req, tok in zip(sampling, tokens):
                 done = self.scheduler.append_token(req, tok)
                 self.counters["generated_tokens"] += 1
@@ -135,6 +145,52 @@ class Engine:
         while self.has_unfinished():
             self.step()
         return [list(self._requests[r].output) for r in rids]
+
+    def generate_with_logprobs(self, prompts: Sequence[Sequence[int]],
+                               params: Union[SamplingParams, Sequence[SamplingParams], None] = None, top_n: int = 0):
+        """``generate`` that also returns, per prompt, one ``TokenLogprob`` per generated token: the token's
+        log-probability under the distribution it was drawn from and the ``top_n`` (at most 20) most probable
+        tokens of that distribution (/root/reference/engine/src/model.rs:9817-9887)."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt")
+        rids = [self.add_request(p, sp, logprobs_top_n=top_n) for p, sp in zip(prompts, params)]
+        while self.has_unfinished():
+            self.step()
+        return ([list(self._requests[r].output) for r in rids], [list(self._requests[r].logprobs) for r in rids])
+
+    def generate_with_callback(self, prompts: Sequence[Sequence[int]],
+                               params: Union[SamplingParams, Sequence[SamplingParams], None],
+                               on_token: Callable[[int, int], bool]) -> List[List[int]]:
+        """``generate`` that hands every new token to ``on_token(prompt index, token)`` as soon as it is drawn;
+        a false return ends that prompt's generation there, the token kept
+        (/root/reference/engine/src/model.rs:9889-9960)."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt")
+        rids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        index = {r: i for i, r in enumerate(rids)}
+        while self.has_unfinished():
+            for rid, tok, done in self.step():
+                if rid in index and not on_token(index[rid], tok) and not done:
+                    self.abort(rid, "callback")
+        return [list(self._requests[r].output) for r in rids]
+
+    def abort(self, rid: Hashable, reason: str = "aborted") -> None:
+        """End a request now, wherever it stands; its pages and state slot are free at once."""
+        self.scheduler.abort(self._requests[rid], reason)
+
+    def sample_from_logits(self, logits: torch.Tensor, params: Optional[SamplingParams] = None, draw_index: int = 0,
+                           prompt_tokens: Sequence[int] = (), output_tokens: Sequence[int] = ()) -> int:
+        """One token from one row of logits ([vocab], any float dtype, host or device) by the engine's sampler
+        (/root/reference/engine/src/model.rs:363-368).  ``draw_index`` numbers the draw within its stream."""
+        row = logits.detach().to(device=self.device, dtype=torch.float32).reshape(1, -1).contiguous()
+        if row.shape[1] != self.model.spec.vocab_size:
+            raise ValueError(f"logits of {row.shape[1]} entries for a vocabulary of {self.model.spec.vocab_size}")
+        return int(self.sampler.sample(row, [params or SamplingParams()], [draw_index], [list(prompt_tokens)],
+                                       [list(output_tokens)])[0])
 
     def forward(self, token_ids: Sequence[int]) -> torch.Tensor:
         """Logits [vocab] (float32, host) after a whole prompt of a fresh request

@@ -45,6 +45,8 @@ class Request:
     preemptions: int = 0
     finish_reason: Optional[str] = None
     arrival: int = 0
+    logprobs_top_n: Optional[int] = None     # not None: keep a log-probability record per generated token
+    logprobs: List[object] = field(default_factory=list)
 
     @property
     def tokens(self) -> List[int]:
@@ -207,6 +209,16 @@ class Scheduler:
         elif req.num_tokens >= self.config.max_model_len:
             req.finish_reason = "max_model_len"
         return req.finish_reason is not None
+
+    def abort(self, req: Request, reason: str = "aborted") -> None:
+        """End a request from outside, wherever it stands (the reference ends a sequence whose client is
+        gone, /root/reference/server/src/engine_task.rs:64-66); what it holds is given back."""
+        if req.state == RequestState.FINISHED:
+            return
+        if req in self.waiting:
+            self.waiting.remove(req)
+        req.finish_reason = reason
+        self.finish(req)
 
     def finish(self, req: Request) -> None:
         """Give back the request's pages and state slot at once."""

@@ -536,14 +536,18 @@ def apply_penalties(logits: torch.Tensor, rows, tokens, counts, in_window, prese
           _ptr(fl[0]), _ptr(fl[1]), _ptr(fl[2]), n, _stream())
 
 
-def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, min_p, rnd, typical_p=None) -> torch.Tensor:
+def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, min_p, rnd, typical_p=None,
+           info: Optional[torch.Tensor] = None) -> torch.Tensor:
     """float32 [m, vocab] and per-row options (host arrays) -> int32 [m] chosen tokens.
     ``work`` is float32 scratch of at least [m, vocab].  temperature 0 rows return the argmax.
-    ``typical_p`` None leaves that filter off (1.0) in every row."""
+    ``typical_p`` None leaves that filter off (1.0) in every row.
+    ``info``: float32 [m, 4] that receives, per row, what log-probabilities of the filtered distribution need
+    (maximum, ln of the normaliser, smallest surviving value) and the chosen token's log-probability in column 3;
+    ``work`` then holds the filtered, scaled logits for ``top_logprobs``."""
     if typical_p is None:
         typical_p = [1.0] * len(temperature)
     if _backend is not None:
-        return _backend.sample(logits, work, temperature, top_k, top_p, min_p, rnd, typical_p)
+        return _backend.sample(logits, work, temperature, top_k, top_p, min_p, rnd, typical_p, info)
     import numpy as np
     _dev_ok(logits, work)
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: logits must be float32 [m, vocab]")
@@ -555,9 +559,29 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
     fl = _dev_array([temperature, top_p, min_p, rnd, typical_p], np.float32, dev)
     tk = _dev_array(top_k, np.int32, dev)
     out = torch.empty((m,), dtype=torch.int32, device=dev)
+    if info is not None:
+        _dev_ok(info)
+        _need(info.dtype == torch.float32 and info.is_contiguous() and tuple(info.shape) == (m, 4), "sample: info must be float32 [m, 4]")
     _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
-          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _stream())
+          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _stream())
     return out
+
+
+def top_logprobs(work: torch.Tensor, info: torch.Tensor, vocab: int, n: int):
+    """After ``sample(..., info=info)``: the ``n`` most probable tokens of each row's filtered distribution,
+    most probable first (ties by index), as (int32 [m, n] ids, float32 [m, n] log-probabilities); id -1 where a
+    row has fewer survivors."""
+    if _backend is not None:
+        return _backend.top_logprobs(work, info, vocab, n)
+    _dev_ok(work, info)
+    m = info.shape[0]
+    _need(info.dtype == torch.float32 and info.is_contiguous() and tuple(info.shape) == (m, 4), "top_logprobs: info must be float32 [m, 4]")
+    _need(work.dtype == torch.float32 and work.is_contiguous() and work.numel() >= m * vocab, "top_logprobs: work buffer too small")
+    _need(0 <= n <= vocab, "top_logprobs: n out of range")
+    ids = torch.empty((m, n), dtype=torch.int32, device=info.device)
+    lps = torch.empty((m, n), dtype=torch.float32, device=info.device)
+    _call("tp_top_logprobs", _ptr(work), _ptr(info), m, vocab, n, _ptr(ids), _ptr(lps), _stream())
+    return ids, lps
 
 
 def fill_normal(out: torch.Tensor, seed: int, mean: float, std: float) -> torch.Tensor:

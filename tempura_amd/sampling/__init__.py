@@ -1,4 +1,4 @@
 from .params import SamplingParams
-from .sampler import Sampler, uniform_draw
+from .sampler import Sampler, TokenLogprob, uniform_draw
 
-__all__ = ["SamplingParams", "Sampler", "uniform_draw"]
+__all__ = ["SamplingParams", "Sampler", "TokenLogprob", "uniform_draw"]

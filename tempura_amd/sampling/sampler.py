@@ -14,7 +14,8 @@ from __future__ import annotations
 
 import ctypes
 from collections import Counter
-from typing import List, Sequence
+from dataclasses import dataclass
+from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -34,6 +35,15 @@ def uniform_draw(seed: int, n: int) -> float:
     return (z >> 40) / float(1 << 24)
 
 
+@dataclass
+class TokenLogprob:
+    """A generated token with its log-probability and the most probable alternatives, most probable first
+    (/root/reference/engine/src/model.rs:475-486)."""
+    token_id: int
+    logprob: float
+    top_logprobs: List[Tuple[int, float]]
+
+
 class Sampler:
     def __init__(self, vocab_size: int, device, default_seed: int = 0):
         self.vocab_size = vocab_size
@@ -42,14 +52,18 @@ class Sampler:
         self._work = None
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], draw_index: Sequence[int],
-               prompt_tokens: Sequence[Sequence[int]], output_tokens: Sequence[Sequence[int]]) -> List[int]:
+               prompt_tokens: Sequence[Sequence[int]], output_tokens: Sequence[Sequence[int]],
+               top_n: Optional[int] = None):
         """``logits`` float32 [m, vocab] on the device; one ``SamplingParams`` per row;
         ``draw_index[i]`` is how many tokens row i's request has drawn before; the token
-        lists feed the penalties.  Returns the chosen token of each row."""
+        lists feed the penalties.  Returns the chosen token of each row.
+        With ``top_n`` (0..20) it returns (tokens, records) instead, a record per row being
+        ``TokenLogprob(token_id, logprob, top_logprobs)``: log-probabilities of the distribution the token was
+        drawn from, after temperature and filters (/root/reference/engine/src/model.rs:497-526)."""
         m = logits.shape[0]
         if m == 0:
-            return []
-        if all(p.is_greedy for p in params):
+            return [] if top_n is None else ([], [])
+        if top_n is None and all(p.is_greedy for p in params):
             return ops.argmax(logits).tolist()
         if any(p.has_penalties for p in params):
             logits = self._penalised(logits, params, prompt_tokens, output_tokens)
@@ -62,7 +76,16 @@ class Sampler:
                           for p, n in zip(params, draw_index)], dtype=np.float32)
         if self._work is None or self._work.shape[0] < m:
             self._work = torch.empty((max(m, 8), self.vocab_size), dtype=torch.float32, device=self.device)
-        return ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd, typical_p).tolist()
+        if top_n is None:
+            return ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd, typical_p).tolist()
+        top_n = max(0, min(int(top_n), 20, self.vocab_size))
+        info = torch.empty((m, 4), dtype=torch.float32, device=logits.device)
+        tokens = ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd, typical_p, info).tolist()
+        ids, lps = ops.top_logprobs(self._work, info, self.vocab_size, top_n)
+        ids, lps, chosen = ids.tolist(), lps.tolist(), info[:, 3].tolist()
+        records = [TokenLogprob(tok, chosen[r], [(i, lp) for i, lp in zip(ids[r], lps[r]) if i >= 0])
+                   for r, tok in enumerate(tokens)]
+        return tokens, records
 
     def _penalised(self, logits, params, prompt_tokens, output_tokens):
         rows, toks, counts, inwin = [], [], [], []

@@ -82,6 +82,63 @@ def test_temperature_sampling_seeded(tiny_dirs):
     assert alone[0] == a[2]
 
 
+def test_generate_with_logprobs(tiny_dirs):
+    """Greedy: the tokens of ``generate``, and records that agree with a softmax of the plain implementation's
+    logits over the top_k kept tokens (the reference reports the filtered distribution,
+    /root/reference/engine/src/model.rs:497-526)."""
+    from tempura_amd.sampling import SamplingParams
+    cfg, W = tiny_dirs.plain_model("A")
+    prompts = [helpers.random_tokens(256, n, seed=700 + n) for n in (5, 17)]
+    p = SamplingParams(temperature=0.0, top_k=8, max_new_tokens=6)
+    tokens, records = _engine(tiny_dirs, "A").generate_with_logprobs(prompts, p, top_n=3)
+    assert tokens == _engine(tiny_dirs, "A").generate(prompts, p)
+    for prompt, toks, recs in zip(prompts, tokens, records):
+        assert [r.token_id for r in recs] == toks
+        seq = list(prompt)
+        for tok, rec in zip(toks, recs):
+            lg = plain.forward(cfg, W, seq)[-1].double()
+            kept = torch.topk(lg, 8)
+            lp = torch.log_softmax(kept.values, 0)
+            assert rec.top_logprobs[0][0] == tok == int(kept.indices[0])
+            assert [i for i, _ in rec.top_logprobs] == kept.indices[:3].tolist()
+            assert abs(rec.logprob - float(lp[0])) < 1e-4
+            for (_, got), want in zip(rec.top_logprobs, lp[:3].tolist()):
+                assert abs(got - want) < 1e-4
+            seq.append(tok)
+    # requests with and without records in one batch
+    eng = _engine(tiny_dirs, "A")
+    r0 = eng.add_request(prompts[0], p, logprobs_top_n=0)
+    r1 = eng.add_request(prompts[1], p)
+    while eng.has_unfinished():
+        eng.step()
+    assert eng.request(r0).output == tokens[0] and eng.request(r1).output == tokens[1]
+    assert len(eng.request(r0).logprobs) == 6 and eng.request(r1).logprobs == []
+    assert all(r.top_logprobs == [] for r in eng.request(r0).logprobs)
+
+
+def test_generate_with_callback_and_abort(tiny_dirs):
+    from tempura_amd.sampling import SamplingParams
+    prompts = [helpers.random_tokens(256, n, seed=710 + n) for n in (5, 17, 30)]
+    p = SamplingParams(temperature=0.0, max_new_tokens=12)
+    full = _engine(tiny_dirs, "A").generate(prompts, p)
+    seen = {0: [], 1: [], 2: []}
+
+    def on_token(i, tok):
+        seen[i].append(tok)
+        return not (i == 1 and len(seen[1]) == 4)        # the second prompt stops after four tokens
+
+    eng = _engine(tiny_dirs, "A")
+    out = eng.generate_with_callback(prompts, p, on_token)
+    assert out == [full[0], full[1][:4], full[2]] and [seen[i] for i in range(3)] == out
+    assert all(pool.num_free == pool.num_pages for pool in eng.runner.cache.pools)
+    # one token from given logits, by the same sampler
+    lg = torch.randn(256)
+    assert eng.sample_from_logits(lg, SamplingParams(temperature=0.0)) == int(lg.argmax())
+    t = eng.sample_from_logits(lg, SamplingParams(temperature=0.9, top_k=5, seed=1), draw_index=3)
+    assert t in torch.topk(lg, 5).indices.tolist()
+    assert t == eng.sample_from_logits(lg, SamplingParams(temperature=0.9, top_k=5, seed=1), draw_index=3)
+
+
 def test_eos_and_length_limits(tiny_dirs):
     from tempura_amd.sampling import SamplingParams
     cfg, W = tiny_dirs.plain_model("A")

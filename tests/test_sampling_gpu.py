@@ -116,6 +116,45 @@ def test_typical_p_drops_a_likely_but_untypical_token():
     assert max(got) == 25 and min(got) == 0
 
 
+def test_logprobs_of_the_filtered_distribution():
+    """Per row: the chosen token's log-probability and the most probable survivors, from the distribution after
+    temperature and filters (/root/reference/engine/src/model.rs:497-526)."""
+    from tempura_amd.sampling import Sampler, SamplingParams
+    g = torch.Generator().manual_seed(11)
+    V = 4099
+    lg = (torch.randn(5, V, generator=g) * 3).to(DEV)
+    ps = [SamplingParams(temperature=0.0), SamplingParams(temperature=0.7, top_k=40, top_p=0.9, seed=5),
+          SamplingParams(temperature=1.0, top_k=0, seed=6), SamplingParams(temperature=1.3, top_k=3, seed=7),
+          SamplingParams(temperature=1.0, top_k=0, min_p=0.2, typical_p=0.6, seed=8)]
+    s = Sampler(V, DEV, default_seed=0)
+    toks, recs = s.sample(lg, ps, [0, 1, 2, 3, 4], [[]] * 5, [[]] * 5, top_n=5)
+    assert toks == s.sample(lg, ps, [0, 1, 2, 3, 4], [[]] * 5, [[]] * 5)
+    for r, (p, tok, rec) in enumerate(zip(ps, toks, recs)):
+        x = lg[r].double().cpu()
+        if p.temperature not in (0.0, 1.0):
+            x = x / p.temperature
+        if p.min_p > 0:
+            x[x < x.max() + math.log(p.min_p)] = -math.inf
+        if p.typical_p < 1:
+            x = plain_typical(x, p.typical_p)
+        if p.top_k > 0:
+            x[x < torch.topk(x, p.top_k).values[-1]] = -math.inf
+        pr = torch.softmax(x, 0)
+        if p.top_p < 1:
+            o = torch.argsort(pr, descending=True, stable=True)
+            cut = int(torch.nonzero(torch.cumsum(pr[o], 0) >= p.top_p)[0]) + 1
+            keep = torch.zeros(V, dtype=torch.bool)
+            keep[o[:cut]] = True
+            pr[~keep] = 0
+            pr /= pr.sum()
+        assert rec.token_id == tok and abs(rec.logprob - math.log(float(pr[tok]))) < 1e-4
+        n = min(5, int((pr > 0).sum()))
+        want = torch.topk(pr, n)
+        assert [i for i, _ in rec.top_logprobs] == want.indices.tolist()
+        assert all(abs(got - math.log(float(w))) < 1e-4 for (_, got), w in zip(rec.top_logprobs, want.values))
+    assert len(recs[3].top_logprobs) == 3, "three survivors of top_k = 3, although five were asked for"
+
+
 def test_greedy_ties_and_fallthrough():
     lg = torch.zeros(3, 100)
     lg[0, 5] = lg[0, 70] = 3.0                       # tie: the later index wins (model.rs:459-473)

@@ -154,3 +154,27 @@ def test_no_request_lost_under_a_tiny_pool(seed):
     assert got == want
     assert cache.free_pages() == [12]
     assert sched.pages_high_water[0] <= 12
+
+
+def test_abort_frees_at_once_wherever_the_request_stands():
+    sched, cache = make(num_pages=16, max_num_seqs=2)
+    a, b, c = req("a", 20, max_new=50), req("b", 20, max_new=50), req("c", 20, max_new=3)
+    for r in (a, b, c):
+        sched.add_request(r)
+    seen = []
+
+    def on_step(items):
+        seen.append([it.request.rid for it in items])
+        if len(seen) == 3:
+            sched.abort(a, "client gone")        # running, holds pages
+            sched.abort(c)                       # still waiting (two may run at once)
+            sched.abort(c)                       # a second abort changes nothing
+            assert not cache.has("a") and a.state == RequestState.FINISHED and a.finish_reason == "client gone"
+            assert c.state == RequestState.FINISHED and c.finish_reason == "aborted" and c.num_computed == 0
+            cache.check()
+
+    run(sched, cache, on_step=on_step)
+    assert b.finish_reason == "length" and len(b.output) == 50
+    assert all("a" not in s and "c" not in s for s in seen[3:])
+    assert sorted(r.rid for r in sched.finished) == ["a", "b", "c"]
+    assert cache.pools[0].num_free == 16
