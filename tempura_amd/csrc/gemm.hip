@@ -146,7 +146,7 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
                    const void* post_w, void* post_xg, float* post_ss, int layout, int defer_reduce, int* splits_out,
                    hipStream_t s);
 
-int tp_linear_rope_mfma(const void* x, const void* w, int M, int N, int K, const float* pre_ss, int pre_count,
+int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N, int K, const float* pre_ss, int pre_count,
                         float pre_eps, const int* positions, const int* slots, const double* inv_freq, int rotary_dim,
                         float factor, int n_heads, int n_kv, int head_dim, void* q_out, void* k_cache, void* v_cache,
                         int page_size, const float* cos_sin, hipStream_t s);
@@ -157,13 +157,14 @@ int tp_linear_rope_mfma(const void* x, const void* w, int M, int N, int K, const
 // [M, n_heads, head_dim], k into the cache place slots[m] and v into the transposed value cache (both
 // bfloat16), as tp_rope_kv_write does for the rows of a plain product.  cos_sin: the step's table from
 // tp_rope_table [M, rotary_dim / 2, 2], or nullptr (the epilogue then computes cosines and sines itself).
-extern "C" int tp_linear_rope(const void* x, const void* w, int M, int N, int K, const float* pre_ss, int pre_count,
+// w_tiled: the weight is in the tiled layout (see tp_linear_fused).
+extern "C" int tp_linear_rope(const void* x, const void* w, int w_tiled, int M, int N, int K, const float* pre_ss, int pre_count,
                               float pre_eps, const int* positions, const int* slots, const double* inv_freq,
                               int rotary_dim, float factor, int n_heads, int n_kv, int head_dim, void* q_out,
                               void* k_cache, void* v_cache, int page_size, const float* cos_sin, hipStream_t s) {
   TP_REQUIRE(x && w && positions && slots && q_out && k_cache && v_cache, "linear_rope: missing operand");
   TP_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "linear_rope: no frequency table");
-  const int r = tp_linear_rope_mfma(x, w, M, N, K, pre_ss, pre_count, pre_eps, positions, slots, inv_freq, rotary_dim,
+  const int r = tp_linear_rope_mfma(x, w, w_tiled, M, N, K, pre_ss, pre_count, pre_eps, positions, slots, inv_freq, rotary_dim,
                                     factor, n_heads, n_kv, head_dim, q_out, k_cache, v_cache, page_size, cos_sin, s);
   TP_REQUIRE(r == 0, "linear_rope: sizes M %d N %d K %d head_dim %d are not this product's (at most 16 rows, "
              "K %% 32 == 0, head_dim %% 16 == 0)", M, N, K, head_dim);
@@ -181,6 +182,9 @@ extern "C" int tp_linear_rope(const void* x, const void* w, int M, int N, int K,
 //
 // `layout` (bfloat16, at most 16 rows): bit 0, x is k-blocked [K / 8, M, 8] instead of [M, K]; bit 1, the
 // gated output (accumulate == 2) is written k-blocked [N / 16, M, 8] for a product that reads it so.
+// Bit 2 (bfloat16, any number of rows, N % 16 == 0, K % 64 == 0): w is tiled, [N / 16][K / 32][64][8]: the 16 x 32
+// block of rows 16 i.. and columns 32 j.. as 1,024 contiguous bytes, element (r, c) of the block at
+// ((c / 8) * 16 + r) * 8 + c % 8 (the matrix cores' operand order), blocks of a row group side by side.
 //
 // `defer_reduce` (products of 17..128 rows whose K is split over blocks): the partial sums stay in `scratch`
 // as [*splits_out, M, N] float32 and `out` is not touched; the caller's next kernel adds them (ascending).
@@ -192,9 +196,11 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   if (splits_out) *splits_out = 1;
   TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(accumulate != 1 || out_dt == TP_F32, "linear: accumulating output must be float32");
-  const bool split_norm = pre_ss != nullptr || post_w != nullptr || layout != 0;
-  TP_REQUIRE((layout & ~3) == 0 && (!(layout & 2) || accumulate == 2) && (!(layout & 1) || pre_ss == nullptr),
+  const bool split_norm = pre_ss != nullptr || post_w != nullptr || (layout & 3) != 0;
+  TP_REQUIRE((layout & ~7) == 0 && (!(layout & 2) || accumulate == 2) && (!(layout & 1) || pre_ss == nullptr),
              "linear: bad layout flags %d", layout);
+  TP_REQUIRE(!(layout & 4) || (in_dt == TP_BF16 && allow_mfma && N % 16 == 0 && K % 64 == 0),
+             "linear: tiled weights are bfloat16 with N %% 16 == 0 and K %% 64 == 0 (N=%d K=%d)", N, K);
   if (split_norm) {
     TP_REQUIRE(in_dt == TP_BF16 && allow_mfma && M <= 16 && K % 32 == 0,
                "linear: the split norm and the k-blocked layout need bfloat16 operands, at most 16 rows and K %% 32 == 0 (M=%d K=%d)", M, K);
@@ -216,6 +222,7 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
                                  pre_eps, post_w, post_xg, post_ss, layout, defer_reduce, splits_out, s);
     if (r >= 0) return r;
   }
+  TP_REQUIRE(!(layout & 4), "linear: no kernel for tiled weights at M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(!split_norm, "linear: sizes M=%d N=%d K=%d do not fit the split norm or the k-blocked layout", M, N, K);
   if (in_dt == TP_F32 && out_dt == TP_F32) {
     if (accumulate)

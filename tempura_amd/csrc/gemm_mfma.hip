@@ -36,7 +36,12 @@ __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8
 // Layouts of bfloat16 activations of at most 16 rows.  Row-major [M, K], or k-blocked [K / 8, M, 8]:
 // eight consecutive k of all rows side by side, so that the operand fragments that the lanes of a
 // wave fetch straight from global memory (16 bytes per row and k group) lie next to each other.
-enum { X_KBLOCKED = 1, OUT_KBLOCKED = 2 };
+// Layout of a weight.  Row-major [N, K], or tiled (N % 16 == 0, K % 64 == 0): [N / 16][K / 32][64][8], the operand
+// fragment of the MFMA for 16 weight rows and 32 of k as one run of 1,024 bytes, lane l's eight elements (row l % 16,
+// k group l / 16) at l * 16.  A wave's load of a fragment then covers eight whole cache lines instead of 64-byte
+// pieces of sixteen rows, which is what the address path of a CU can keep up with when the weights stream from HBM
+// (the down projection of 8 rows: 26.0 -> 23.4 us), and a stage of the pipelined kernels is a plain copy.
+enum { X_KBLOCKED = 1, OUT_KBLOCKED = 2, W_TILED = 4 };
 
 __device__ inline void store_gated(void* out, int layout, int M, int width, int m, int col, float v) {
   const size_t idx = (layout & OUT_KBLOCKED) ? ((size_t)(col >> 3) * M + m) * 8 + (col & 7) : (size_t)m * width + col;
@@ -146,7 +151,7 @@ __device__ inline void row_scale_finish(const RowScale& pre, const RowScaleLoads
 // MT: 16-row tiles of activations; NT: 16-row tiles of weights per block; WAVES: waves that
 // split K.  A wave takes K in runs of four consecutive 32-wide steps (256 contiguous bytes of
 // each weight row), run r going to wave r % WAVES.
-template <int MT, int NT, int WAVES, int DEPTH>
+template <int MT, int NT, int WAVES, int DEPTH, bool WT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16_t* __restrict__ x,
                                                                       const bf16_t* __restrict__ w,
                                                                       void* __restrict__ out, int mode, int M,
@@ -161,8 +166,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     const int wrow = min(n0 + j * 16 + (lane & 15), N - 1);
-    wp[j] = (const u32x4_t*)(w + (size_t)wrow * K + kofs);
+    wp[j] = WT ? (const u32x4_t*)(w + (size_t)min(n0 + j * 16, N - 16) * K) + lane
+                               : (const u32x4_t*)(w + (size_t)wrow * K + kofs);
   }
+  constexpr int wstep = WT ? 64 : 4;   // u32x4 units per 32 of k (a compile-time stride: the four loads of a run share one address)
   // x is [M, K] row-major, or (xblocked, M <= 16) [K / 8, M, 8]: eight consecutive k of all rows side by
   // side, so that the 16 bytes the lanes of a wave fetch lie next to each other
   const u32x4_t* xp[MT];
@@ -193,7 +200,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
         // steps past the end repeat the last one; their products are dropped below
         const int sidx = min(s0 + d * WAVES * 4 + u, steps - 1);
 #pragma unroll
-        for (int j = 0; j < NT; ++j) a[d][j][u] = wp[j][(size_t)sidx * 4];
+        for (int j = 0; j < NT; ++j) a[d][j][u] = wp[j][(size_t)sidx * wstep];
 #pragma unroll
         for (int t = 0; t < MT; ++t) b[d][t][u] = xp[t][(size_t)sidx * xstep];
       }
@@ -285,7 +292,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
 // before anything is multiplied, and again as soon as their registers are free, always in the order in
 // which they are consumed (loads return in order): a block has 256 bytes per lane in flight from its
 // first cycle.  (Measured against one chunk of prefetch: 5-10 % faster at 8 and 16 rows.)
-template <int NT, int WAVES>
+template <int NT, int WAVES, bool WT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                void* __restrict__ out, int mode, int M, int N, int K,
                                                                int layout, RowScale pre, NormPrep post, RopeOut rp) {
@@ -304,8 +311,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     const int wrow = min(n0 + j * 16 + (lane & 15), N - 1);
-    wp[j] = (const u32x4_t*)(w + (size_t)wrow * K + kofs);
+    wp[j] = WT ? (const u32x4_t*)(w + (size_t)min(n0 + j * 16, N - 16) * K) + lane
+                               : (const u32x4_t*)(w + (size_t)wrow * K + kofs);
   }
+  constexpr int wstep = WT ? 64 : 4;
   const int xrow = tid / TPR, xcol = (tid % TPR) * 8;
   const bool xload = xrow < M;
   const bf16_t* xsrc = x + (size_t)min(xrow, M - 1) * K + xcol;
@@ -322,7 +331,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_
     for (int u = 0; u < 4; ++u) {
       const int sidx = min(s0 + u, steps - 1);
 #pragma unroll
-      for (int j = 0; j < NT; ++j) a[slot][j][u] = wp[j][(size_t)sidx * 4];
+      for (int j = 0; j < NT; ++j) a[slot][j][u] = wp[j][(size_t)sidx * wstep];
     }
   };
   auto load_x = [&](int ch, int slot) {
@@ -641,10 +650,10 @@ static int g_tune_splits = 0, g_tune_mid = 0;                    // mid = 1: 17.
 static int g_tune_order = 0;   // large products: 1 tiled kernel, plain block order; 2 tiled, XCD patches; 3 pipelined kernel
 
 // Defined in gemm_pipe.hip; 0 when it took the product, -1 when the sizes are not its own.
-int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
                    size_t scratch_floats, int tune_splits, const RopeOut* rope, hipStream_t s);
 
-int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
                      size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s);
 
 extern int g_pipe_big;
@@ -669,8 +678,12 @@ template <int MT, int NT, int WAVES, int DEPTH>
 static void launch_skinny4(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, int layout,
                            RowScale pre, NormPrep post, const RopeOut& rp, hipStream_t s) {
   const int blocks = (N + 16 * NT - 1) / (16 * NT);
-  hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, NT, WAVES, DEPTH>), dim3(blocks), dim3(WAVES * 64), 0, s, x, w, out,
-                     mode, M, N, K, layout, pre, post, rp);
+  if (layout & W_TILED)
+    hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, NT, WAVES, DEPTH, true>), dim3(blocks), dim3(WAVES * 64), 0, s, x, w, out,
+                       mode, M, N, K, layout, pre, post, rp);
+  else
+    hipLaunchKernelGGL((gemm_skinny_mfma_kernel<MT, NT, WAVES, DEPTH, false>), dim3(blocks), dim3(WAVES * 64), 0, s, x, w, out,
+                       mode, M, N, K, layout, pre, post, rp);
 }
 
 template <int MT>
@@ -696,10 +709,14 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
     if (lds) {
       if (nt > 2) nt = 2;
       const int blocks = (N + 16 * nt - 1) / (16 * nt);
-      if (nt == 2)
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<2, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post, rp);
-      else
-        hipLaunchKernelGGL((gemm_skinny_lds_kernel<1, 8>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post, rp);
+      const bool wt = (layout & W_TILED) != 0;
+#define LDS_CASE(NT_, WT_) \
+  hipLaunchKernelGGL((gemm_skinny_lds_kernel<NT_, 8, WT_>), dim3(blocks), dim3(512), 0, s, x, w, out, mode, M, N, K, layout, pre, post, rp)
+      if (nt == 2 && wt) LDS_CASE(2, true);
+      else if (nt == 2) LDS_CASE(2, false);
+      else if (wt) LDS_CASE(1, true);
+      else LDS_CASE(1, false);
+#undef LDS_CASE
       return;
     }
   }
@@ -733,13 +750,14 @@ static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int mode,
 
 // The q/k/v projection of at most 16 rows with rotation and cache write in its epilogue (see RopeOut).
 // N = (n_heads + 2 n_kv) * head_dim.  Returns -1 for sizes this path does not take.
-int tp_linear_rope_mfma(const void* x, const void* w, int M, int N, int K, const float* pre_ss, int pre_count,
+int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N, int K, const float* pre_ss, int pre_count,
                         float pre_eps, const int* positions, const int* slots, const double* inv_freq, int rotary_dim,
                         float factor, int n_heads, int n_kv, int head_dim, void* q_out, void* k_cache, void* v_cache,
                         int page_size, const float* cos_sin, hipStream_t s) {
   if (M < 1 || (M > 16 && M <= 128) || K % 32 != 0 || head_dim % 16 != 0 || rotary_dim % 2 != 0 || rotary_dim > head_dim) return -1;
   if (N != (n_heads + 2 * n_kv) * head_dim || page_size < 1) return -1;
   if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return -1;
+  if (w_tiled && (N % 16 != 0 || K % 64 != 0)) return -1;
   const RowScale pre = {pre_ss, pre_count, 1.0f / (float)K, pre_eps};
   const NormPrep post = {nullptr, nullptr, nullptr};
   const RopeOut rp = {positions, slots, inv_freq, (const float2*)cos_sin, factor, rotary_dim, n_heads, n_kv, head_dim, page_size,
@@ -748,9 +766,9 @@ int tp_linear_rope_mfma(const void* x, const void* w, int M, int N, int K, const
     // long steps: the pipelined kernels, whose wave tiles (64 or 128 columns) must lie inside one head, with the
     // step's table of cosines and sines
     if (head_dim != 128 || rotary_dim % 8 != 0 || cos_sin == nullptr || pre_ss != nullptr || page_size % 8 != 0) return -1;
-    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, s);
+    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, s);
   }
-  launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, 0, pre, post, rp, s);
+  launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, w_tiled ? W_TILED : 0, pre, post, rp, s);
   return 0;
 }
 
@@ -762,7 +780,9 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
                    hipStream_t s) {
   if (splits_out) *splits_out = 1;
   if (K % 32 != 0) return -1;
-  if (layout != 0 && M > 16) return -1;
+  const int w_tiled = (layout & W_TILED) != 0;
+  if (w_tiled && (N % 16 != 0 || K % 64 != 0)) return -1;
+  if ((layout & (X_KBLOCKED | OUT_KBLOCKED)) != 0 && M > 16) return -1;
   if ((layout & OUT_KBLOCKED) && accumulate != 2) return -1;
   if ((pre_ss != nullptr || post_w != nullptr) && M > 16) return -1;
   if (post_w != nullptr && accumulate != 1) return -1;
@@ -791,11 +811,13 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
     // (measured at 128 rows: N = 28,672 59 us against 77 us, the narrow products a few us slower)
     const bool pipe = g_tune_order ? g_tune_order == 3 : (M > 128 || (M > 64 && N >= 16384));
     const bool pipe64 = !pipe && M <= 128 && scratch != nullptr && g_tune_mid != 2;
-    if (pipe && tp_linear_pipe(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, nullptr, s) == 0) {
+    if (pipe && tp_linear_pipe(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, nullptr, s) == 0) {
       // taken by the pipelined kernel
-    } else if (pipe64 && tp_linear_pipe64(xb, wb, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, defer_reduce,
-                                          splits_out, s) == 0) {
+    } else if (pipe64 && tp_linear_pipe64(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits,
+                                          defer_reduce, splits_out, s) == 0) {
       // taken by the 64-row pipelined kernel
+    } else if (w_tiled) {
+      return -1;   // the kernels below read row-major weights only
     } else if (M > 128 || scratch == nullptr) {
       dim3 grid((N + 127) / 128, (M + 127) / 128);
       if (grid.y > 65535) return -1;

@@ -19,6 +19,9 @@
 //  * blocks go to the eight XCDs round robin; the blocks that one XCD runs at a time form a patch of
 //    (row blocks x column blocks) that share their operand tiles through that XCD's L2.
 //  * the result leaves through LDS, so that every store covers whole cache lines (emit_tile).
+//  * the weights may come tiled (wt: [N / 16][K / 32][64][8], a 16 x 32 block in the matrix cores' operand order as
+//    1,024 contiguous bytes): a load then copies one block to LDS as it is, the fragment read is the lane's own
+//    16 bytes of it, and nothing of the above swizzle applies to that operand.
 // One barrier per 64 of K.  Sizes: K % 64 == 0; any M and N (loads clamp to the last row, stores are
 // masked).  The sum over K runs in ascending order for every output element.
 // Further down: the same pipeline on 256 x 256 block tiles (gemm_pipe_big_kernel; the host mixes both tile
@@ -479,7 +482,7 @@ __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0
 // and a second kernel adds the splits in ascending order and applies the epilogue.
 __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                         void* __restrict__ out, float* __restrict__ partial, int mode,
-                                                        int M, int N, int K, int pm, int ldo, RopeOut rp) {
+                                                        int M, int N, int K, int pm, int ldo, RopeOut rp, int wt) {
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE_BYTES];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -525,18 +528,25 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     const int grow = i < 8 ? min(row, M - 1 - m0) : min(row, N - 1 - n0);
     voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
+    if (wt && i >= 8) {   // block u of the stage's weights: row group u / 2 of the block tile, first or second 32 of k
+      const int u = wave * 4 + i - 8;
+      const int grp = min(u / 2, (N - n0) / 16 - 1);
+      voff[i] = ((unsigned)grp * (unsigned)(K / 32) + (u & 1)) * 1024u + lane * 16;
+    }
   }
+  const int wkstep = wt ? 2048 : BK * 2;     // bytes from one stage's weights to the next
+  const unsigned boff0 = wt ? lane * 16 : off0, boff1 = wt ? 1024 + lane * 16 : off1;
   const unsigned char* xk = (const unsigned char*)x + ((size_t)m0 * K + (size_t)kt_first * BK) * 2;
-  const unsigned char* wk = (const unsigned char*)w + ((size_t)n0 * K + (size_t)kt_first * BK) * 2;
+  const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2 + (size_t)kt_first * wkstep;
 #pragma unroll
   for (int p = 0; p < NS; ++p)
-    if (p < KT) issue_stage(stages + p * STAGE_BYTES, xk + p * BK * 2, wk + p * BK * 2, voff, wave);
+    if (p < KT) issue_stage(stages + p * STAGE_BYTES, xk + p * BK * 2, wk + p * wkstep, voff, wave);
   xk += NS * BK * 2;  // the next stage to load is that of tile NS
-  wk += NS * BK * 2;
+  wk += NS * wkstep;
   Frags fa, fb;
   if (KT > 2) WAIT_VM(2 * LPW); else WAIT_VM(0);
   __builtin_amdgcn_s_barrier();
-  READ_ALL(fa, lds0 + arow + off0, lds0 + brow + off0);
+  READ_ALL(fa, lds0 + arow + off0, lds0 + brow + boff0);
   wait_frags(fa);
   // Tile kt: the first half step multiplies fa and reads the second half's fragments; then tile kt + 1
   // must have landed for every wave (barrier), which also means that every wave is done reading tile
@@ -546,30 +556,30 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
   for (; kt + NS < KT; ++kt) {
     const int sn = st + 1 == NS ? 0 : st + 1;
     const unsigned cur = lds0 + st * STAGE_BYTES, nxt = lds0 + sn * STAGE_BYTES;
-    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fb);
     WAIT_VM(LPW);  // tile kt + 2 may stay in flight
     __builtin_amdgcn_s_barrier();
-    half_step<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, stages + st * STAGE_BYTES, xk, wk, voff, wave);
+    half_step<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE_BYTES, xk, wk, voff, wave);
     wait_frags(fa);
     xk += BK * 2;
-    wk += BK * 2;
+    wk += wkstep;
     st = sn;
   }
   for (; kt + 1 < KT; ++kt) {  // nothing left to load
     const int sn = st + 1 == NS ? 0 : st + 1;
     const unsigned cur = lds0 + st * STAGE_BYTES, nxt = lds0 + sn * STAGE_BYTES;
-    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fb);
     WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
-    half_step<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, nullptr, nullptr, nullptr, voff, wave);
+    half_step<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fa);
     st = sn;
   }
   {
     const unsigned cur = lds0 + st * STAGE_BYTES;
-    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fb);
     half_step<false, false>(acc, fb, fa, 0, 0, nullptr, nullptr, nullptr, voff, wave);
   }
@@ -708,7 +718,7 @@ __device__ inline void read_all_big(FragsBig& f, unsigned aaddr, unsigned baddr)
 // No split of K here.  N: the columns of this launch (a multiple of 256); ldo as above.
 __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                             void* __restrict__ out, int mode, int M, int N, int K,
-                                                            int pm, int ldo, RopeOut rp) {
+                                                            int pm, int ldo, RopeOut rp, int wt) {
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NSB * STAGE_BIG];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -742,18 +752,24 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     const int grow = i < 8 ? min(row, M - 1 - m0) : row;   // (every w row of the launch exists)
     voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
+    if (wt && i >= 8) {   // block u of the stage's weights: row group u / 2 of the block tile, first or second 32 of k
+      const int u = wave * 8 + (i & 7);
+      voff[i] = ((unsigned)(u / 2) * (unsigned)(K / 32) + (u & 1)) * 1024u + lane * 16;
+    }
   }
+  const int wkstep = wt ? 2048 : BK * 2;
+  const unsigned boff0 = wt ? lane * 16 : off0, boff1 = wt ? 1024 + lane * 16 : off1;
   const unsigned char* xk = (const unsigned char*)x + (size_t)m0 * K * 2;
   const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2;
 #pragma unroll
   for (int p = 0; p < NSB; ++p)
-    if (p < KT) issue_stage_big(stages + p * STAGE_BIG, xk + p * BK * 2, wk + p * BK * 2, voff, wave);
+    if (p < KT) issue_stage_big(stages + p * STAGE_BIG, xk + p * BK * 2, wk + p * wkstep, voff, wave);
   xk += NSB * BK * 2;
-  wk += NSB * BK * 2;
+  wk += NSB * wkstep;
   FragsBig f;
   if (KT > 1) WAIT_VM(LPWB); else WAIT_VM(0);
   __builtin_amdgcn_s_barrier();
-  read_all_big(f, lds0 + arow + off0, lds0 + brow + off0);
+  read_all_big(f, lds0 + arow + off0, lds0 + brow + boff0);
   // Tile kt: the first half step multiplies the fragments of its first 32 of K and reads those of the second;
   // then tile kt + 1 must have landed for every wave (barrier), which also means that every wave is done
   // reading tile kt's stage: the second half step refills it with tile kt + 2 while it multiplies and reads
@@ -761,25 +777,25 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
   int st = 0, kt = 0;
   for (; kt + NSB < KT; ++kt) {
     const unsigned cur = lds0 + st * STAGE_BIG, nxt = lds0 + (st ^ 1) * STAGE_BIG;
-    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
-    half_step_big<1, true, true>(acc, f, nxt + arow + off0, nxt + brow + off0, stages + st * STAGE_BIG, xk, wk, voff, wave);
+    half_step_big<1, true, true>(acc, f, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE_BIG, xk, wk, voff, wave);
     xk += BK * 2;
-    wk += BK * 2;
+    wk += wkstep;
     st ^= 1;
   }
   for (; kt + 1 < KT; ++kt) {  // nothing left to load
     const unsigned cur = lds0 + st * STAGE_BIG, nxt = lds0 + (st ^ 1) * STAGE_BIG;
-    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
-    half_step_big<1, true, false>(acc, f, nxt + arow + off0, nxt + brow + off0, nullptr, nullptr, nullptr, voff, wave);
+    half_step_big<1, true, false>(acc, f, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
     st ^= 1;
   }
   {
     const unsigned cur = lds0 + st * STAGE_BIG;
-    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     half_step_big<1, false, false>(acc, f, 0, 0, nullptr, nullptr, nullptr, voff, wave);
   }
   // The MFMAs are assembly, so the compiler does not know that their results take time: wait out the last ones
@@ -878,7 +894,7 @@ __device__ inline void half_step64(f32x4_t (&acc)[2][4], const Frags64& cur, Fra
 
 __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              void* __restrict__ out, float* __restrict__ partial,
-                                                             int mode, int M, int N, int K) {
+                                                             int mode, int M, int N, int K, int wt) {
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE64];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -909,9 +925,16 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     const int grow = i < 2 ? min(row, M - 1 - m0) : min(row, N - 1 - n0);
     voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
+    if (wt && i >= 2) {   // block u of the stage's weights: row group u / 2 of the block tile, first or second 32 of k
+      const int u = wave * 4 + i - 2;
+      const int grp = min(u / 2, (N - n0) / 16 - 1);
+      voff[i] = ((unsigned)grp * (unsigned)(K / 32) + (u & 1)) * 1024u + lane * 16;
+    }
   }
+  const int wkstep = wt ? 2048 : BK * 2;
+  const unsigned boff0 = wt ? lane * 16 : off0, boff1 = wt ? 1024 + lane * 16 : off1;
   const unsigned char* xk = (const unsigned char*)x + ((size_t)m0 * K + (size_t)kt_first * BK) * 2;
-  const unsigned char* wk = (const unsigned char*)w + ((size_t)n0 * K + (size_t)kt_first * BK) * 2;
+  const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2 + (size_t)kt_first * wkstep;
   auto issue_stage64 = [&](unsigned char* buf, const unsigned char* xs, const unsigned char* ws) {
     issue_one64<0>(buf, xs, ws, voff, wave);
     issue_one64<1>(buf, xs, ws, voff, wave);
@@ -922,45 +945,45 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
   };
 #pragma unroll
   for (int p = 0; p < NS; ++p)
-    if (p < KT) issue_stage64(stages + p * STAGE64, xk + p * BK * 2, wk + p * BK * 2);
+    if (p < KT) issue_stage64(stages + p * STAGE64, xk + p * BK * 2, wk + p * wkstep);
   xk += NS * BK * 2;
-  wk += NS * BK * 2;
+  wk += NS * wkstep;
   Frags64 fa, fb;
   if (KT > 2) WAIT_VM(2 * LPW64); else WAIT_VM(0);
   __builtin_amdgcn_s_barrier();
 #define READ_ALL64(f, aaddr, baddr) \
   read_one<0>(f, aaddr, baddr); read_one<1>(f, aaddr, baddr); read_one<2>(f, aaddr, baddr); \
   read_one<3>(f, aaddr, baddr); read_one<4>(f, aaddr, baddr); read_one<5>(f, aaddr, baddr)
-  READ_ALL64(fa, lds0 + arow + off0, lds0 + brow + off0);
+  READ_ALL64(fa, lds0 + arow + off0, lds0 + brow + boff0);
   wait_frags(fa);
   int st = 0, kt = 0;
   for (; kt + NS < KT; ++kt) {
     const int sn = st + 1 == NS ? 0 : st + 1;
     const unsigned cur = lds0 + st * STAGE64, nxt = lds0 + sn * STAGE64;
-    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fb);
     WAIT_VM(LPW64);
     __builtin_amdgcn_s_barrier();
-    half_step64<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, stages + st * STAGE64, xk, wk, voff, wave);
+    half_step64<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE64, xk, wk, voff, wave);
     wait_frags(fa);
     xk += BK * 2;
-    wk += BK * 2;
+    wk += wkstep;
     st = sn;
   }
   for (; kt + 1 < KT; ++kt) {
     const int sn = st + 1 == NS ? 0 : st + 1;
     const unsigned cur = lds0 + st * STAGE64, nxt = lds0 + sn * STAGE64;
-    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fb);
     WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
-    half_step64<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + off0, nullptr, nullptr, nullptr, voff, wave);
+    half_step64<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fa);
     st = sn;
   }
   {
     const unsigned cur = lds0 + st * STAGE64;
-    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + off1, nullptr, nullptr, nullptr, voff, wave);
+    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     wait_frags(fb);
     half_step64<false, false>(acc, fb, fa, 0, 0, nullptr, nullptr, nullptr, voff, wave);
   }
@@ -984,9 +1007,10 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
 // Returns 0 when launched, -1 when the sizes are not this kernel's.  `scratch` (optional) is room for
 // float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
 int g_pipe_big = 0;   // tuning: 1 = 256 x 256 tiles for every whole block of 256 columns, 2 = never
-int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
                    size_t scratch_floats, int tune_splits, const RopeOut* rope, hipStream_t s) {
   if ((mode == OUT_ROPE) != (rope != nullptr)) return -1;
+  if (w_tiled && N % 16 != 0) return -1;
   if (K % BK != 0 || K < BK) return -1;
   if ((size_t)(BM - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;  // a lane's source offset is 32 bits
   if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
@@ -1034,7 +1058,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
     const long Q2 = (nb_big + 7) / 8, QS2 = (Q2 + pq - 1) / pq;
     const long blocks2 = 8 * QS2 * MS * 32;
     hipLaunchKernelGGL(gemm_pipe_big_kernel, dim3((unsigned)blocks2), dim3(256), 0, s, x, w, out, mode, M, nb_big * BNB, K,
-                       pm, ldo, rp);
+                       pm, ldo, rp, w_tiled);
     const int n_done = nb_big * BNB;
     if (n_done == N) return 0;
     // the rest of the columns
@@ -1046,11 +1070,11 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
     void* out2 = out == nullptr ? nullptr : (char*)out + (size_t)(mode == OUT_SWIGLU ? n_done / 2 : n_done) * esz;
     rp.col0 = n_done;
     hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocksr, 1), dim3(256), 0, s, x, w + (size_t)n_done * K, out2, scratch,
-                       mode, M, N2, K, pm, ldo, rp);
+                       mode, M, N2, K, pm, ldo, rp, w_tiled);
     return 0;
   }
   hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks, splits), dim3(256), 0, s, x, w, out, scratch, mode, M, N, K,
-                     pm, ldo, rp);
+                     pm, ldo, rp, w_tiled);
   if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
@@ -1061,9 +1085,10 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, void* out, int mode, int M,
 
 // The 64-row pipeline (17..128 rows).  `defer`: when K is split, leave the partial sums in `scratch` for the
 // caller's next kernel and report their number through *splits_out.
-int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, void* out, int mode, int M, int N, int K, float* scratch,
+int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
                      size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s) {
   if (K % BK != 0 || K < BK || M > 128) return -1;
+  if (w_tiled && N % 16 != 0) return -1;
   if ((size_t)(BM64 - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;
   if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
   const int MB = (M + BM64 - 1) / BM64, NB = (N + BN - 1) / BN;
@@ -1082,7 +1107,7 @@ int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, void* out, int mode, int 
   }
   const bool leave = defer && splits > 1 && splits_out != nullptr && mode != OUT_SWIGLU;
   hipLaunchKernelGGL(gemm_pipe64_kernel, dim3((unsigned)tiles, splits), dim3(256), 0, s, x, w, out,
-                     splits > 1 ? scratch : nullptr, mode, M, N, K);
+                     splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled);
   if (leave) {
     *splits_out = splits;
   } else if (splits > 1) {

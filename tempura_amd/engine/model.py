@@ -14,6 +14,7 @@ from typing import Callable, Dict, List, Optional, Tuple
 import torch
 
 from ..config.spec import ModelSpec
+from ..kernels import ops
 from ..parts.base import CacheSpec, StateSpec, WeightInfo, build_part, part_class
 from ..parts.inventory import expected_weights
 
@@ -88,6 +89,8 @@ class CausalLM:
 
         def add(t):
             nonlocal total
+            if isinstance(t, ops.TiledWeight):
+                t = t.data
             if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
                 seen.add(t.data_ptr())
                 total += t.numel() * t.element_size()

@@ -12,6 +12,7 @@ product does.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -184,6 +185,69 @@ class KBlocked:
         return self.data.permute(1, 0, 2).reshape(self.rows, self.width).contiguous()
 
 
+class TiledWeight:
+    """A bfloat16 weight [n, k] (n % 16 == 0, k % 64 == 0) stored tiled, ``data`` [n / 16, k / 32, 64, 8]: the block
+    of rows 16 i.. and columns 32 j.. as 1,024 contiguous bytes in the matrix cores' operand order, lane l = (column
+    group l / 16, row l % 16) holding eight consecutive columns.  The products read it with whole-cache-line loads
+    where the row-major form makes a wave fetch 64-byte pieces of sixteen rows.  Made by ``tile_weight``; taken by
+    ``linear``, ``linear_swiglu`` and ``linear_rope_kv``."""
+    __slots__ = ("data", "n", "k")
+
+    def __init__(self, data, n, k):
+        self.data, self.n, self.k = data, n, k
+
+    @property
+    def shape(self):
+        return (self.n, self.k)
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def dim(self) -> int:
+        return 2
+
+    def rows(self, lo: int, hi: int) -> "TiledWeight":
+        """Rows lo..hi (multiples of 16) as a weight of their own; no copy."""
+        _need(lo % 16 == 0 and hi % 16 == 0 and 0 <= lo < hi <= self.n, f"tiled weight: rows {lo}..{hi} of {self.n}")
+        return TiledWeight(self.data[lo // 16: hi // 16], hi - lo, self.k)
+
+    def row_major(self) -> torch.Tensor:
+        """The plain [n, k] tensor (a copy)."""
+        return self.data.view(self.n // 16, self.k // 32, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(self.n, self.k).contiguous()
+
+
+#: weights that fit are stored tiled (False, or TEMPURA_TILE_WEIGHTS=0 in the environment: every weight stays row-major)
+tile_weights = os.environ.get("TEMPURA_TILE_WEIGHTS", "1") != "0"
+
+
+def tile_weight(w: torch.Tensor):
+    """A weight [n, k] for the products: ``TiledWeight`` when it is bfloat16 on the GPU with n % 16 == 0 and
+    k % 64 == 0 and the matrix-core kernels are in use, else ``w`` itself.  No value changes."""
+    if not (tile_weights and _backend is None and allow_mfma and isinstance(w, torch.Tensor) and w.is_cuda
+            and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[0] % 16 == 0 and w.shape[1] % 64 == 0):
+        return w
+    n, k = w.shape
+    data = w.view(n // 16, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(n // 16, k // 32, 64, 8)
+    return TiledWeight(data, n, k)
+
+
+def weight_rows(w, lo: int, hi: int):
+    """Rows lo..hi of a weight, tiled or not, without a copy."""
+    return w.rows(lo, hi) if isinstance(w, TiledWeight) else w[lo:hi]
+
+
+def _w_args(w):
+    """(tensor whose memory the kernel reads, layout bit) of a weight."""
+    if isinstance(w, TiledWeight):
+        return w.data, 4
+    return w, 0
+
+
 class Partials:
     """The float32 partial sums [splits, m, n] of a product whose K was split over blocks, not yet added:
     the kernel that consumes the rows adds them (in ascending order), which saves the reduction kernel.
@@ -223,7 +287,8 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     if _backend is not None:
         return _backend.linear_swiglu(x, w, blocked_out) if blocked_out else _backend.linear_swiglu(x, w)
     x, pre = _pre_args(x)
-    _dev_ok(x, w)
+    wd, wl = _w_args(w)
+    _dev_ok(x, wd)
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_swiglu: shapes {tuple(x.shape)} x {tuple(w.shape)}")
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "linear_swiglu: operands must be bfloat16")
     m, k = x.shape
@@ -235,8 +300,8 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     else:
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     scratch, nscratch = _splitk_scratch(x, m, n)
-    _call("tp_linear_fused", _ptr(x), _ptr(w), _BF16, _ptr(out.data if blocked_out else out), _BF16, 2, m, n, k, 1,
-          _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), 2 if blocked_out else 0,
+    _call("tp_linear_fused", _ptr(x), _ptr(wd), _BF16, _ptr(out.data if blocked_out else out), _BF16, 2, m, n, k, 1,
+          _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), (2 if blocked_out else 0) | wl,
           0, _ptr(None), _stream())
     return out
 
@@ -271,17 +336,18 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
             return _backend.linear(x, w, out_dtype, residual, next_norm)
         return _backend.linear(x, w, out_dtype, residual)
     layout = 0
+    wd, wl = _w_args(w)
     if isinstance(x, KBlocked):
         _need(allow_mfma and x.data.dtype == torch.bfloat16 and tuple(x.data.shape) == (x.width // 8, x.rows, 8)
               and x.width % 32 == 0, "linear: malformed k-blocked rows")
         kb, layout = x, 1
         x, pre = x.data, (_ptr(None), 0, ctypes.c_float(0.0))
         m, k = kb.rows, kb.width
-        _dev_ok(x, w, residual)
+        _dev_ok(x, wd, residual)
         _need(w.dim() == 2 and w.shape[1] == k and w.dtype == torch.bfloat16, f"linear: shapes {(m, k)} x {tuple(w.shape)}")
     else:
         x, pre = _pre_args(x)
-        _dev_ok(x, w, residual)
+        _dev_ok(x, wd, residual)
         _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
         _need(x.dtype == w.dtype, f"linear: operand dtypes differ ({x.dtype}, {w.dtype})")
         m, k = x.shape
@@ -302,11 +368,12 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
         post = (_ptr(weight), _ptr(handed.x), _ptr(handed.ss))
     scratch, nscratch = _splitk_scratch(x, m, n) if allow_mfma else (None, 0)
     # 17..128 rows: the partial sums of a split K may stay unadded for the kernel that consumes the rows
-    defer = scratch is not None and 16 < m <= 128 and layout == 0 and \
+    layout |= wl
+    defer = scratch is not None and 16 < m <= 128 and (layout & 3) == 0 and \
         ((next_norm is not None and residual is not None and split_norm_ok(m, n, x.dtype) and n % 4 == 0 and n <= 16384) or
          (partial_ok and residual is None and out_dtype == torch.float32))
     splits = ctypes.c_int(1)
-    _call("tp_linear_fused", _ptr(x), _ptr(w), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
+    _call("tp_linear_fused", _ptr(x), _ptr(wd), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
           ctypes.c_size_t(nscratch), *pre, *post, layout, int(defer), ctypes.byref(splits), _stream())
     if defer and splits.value > 1:
         if next_norm is None:
@@ -346,7 +413,8 @@ def linear_rope_kv(x, w: torch.Tensor, positions: torch.Tensor, slots: torch.Ten
     to float32 followed by ``rope_kv_write`` (w's q and k heads in paired order), without the kernel and the
     rows in between.  Returns q as bfloat16 [m, heads, head_dim]."""
     x, pre = _pre_args(x)
-    _dev_ok(x, w, positions, slots, inv_freq, k_cache, v_cache)
+    wd, wl = _w_args(w)
+    _dev_ok(x, wd, positions, slots, inv_freq, k_cache, v_cache)
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_rope_kv: shapes {tuple(x.shape)} x {tuple(w.shape)}")
     m, k = x.shape
     n = w.shape[0]
@@ -369,7 +437,7 @@ def linear_rope_kv(x, w: torch.Tensor, positions: torch.Tensor, slots: torch.Ten
         _need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and tuple(cos_sin.shape) == (m, rotary_dim // 2, 2),
               "linear_rope_kv: table must be float32 [m, rotary_dim / 2, 2]")
     q = torch.empty((m, num_heads, head_dim), dtype=torch.bfloat16, device=x.device)
-    _call("tp_linear_rope", _ptr(x), _ptr(w), m, n, k, *pre, _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
+    _call("tp_linear_rope", _ptr(x), _ptr(wd), int(wl != 0), m, n, k, *pre, _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
           ctypes.c_float(factor), num_heads, num_kv_heads, head_dim, _ptr(q), _ptr(k_cache), _ptr(v_cache),
           k_cache.shape[2], _ptr(cos_sin), _stream())
     return q

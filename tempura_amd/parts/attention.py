@@ -72,8 +72,9 @@ class PagedAttention(Mixer):
         w = self.spec.weights
         # One [q_dim + 2 kv_dim, hidden] matrix: one product instead of three.
         parts = [self._paired(get(w["q"])), self._paired(get(w["k"])), get(w["v"])]
-        self.wqkv = torch.cat([self._to_device(t) for t in parts], dim=0).contiguous()
-        self.wo = self._to_device(get(w["o"]))
+        # (stored tiled where the sizes allow: the products then read whole cache lines)
+        self.wqkv = ops.tile_weight(torch.cat([self._to_device(t) for t in parts], dim=0).contiguous())
+        self.wo = ops.tile_weight(self._to_device(get(w["o"])))
         self.position.load_weights(get)
 
     def cache_spec(self):
@@ -109,7 +110,7 @@ class PagedAttention(Mixer):
             qkv = ops.linear(x, self.wqkv, torch.float32, partial_ok=rot is not None)
         else:
             # A call that reads another call's cache needs queries only.
-            qkv = ops.linear(x, self.wqkv[: self.q_dim], torch.float32, partial_ok=rot is not None)
+            qkv = ops.linear(x, ops.weight_rows(self.wqkv, 0, self.q_dim), torch.float32, partial_ok=rot is not None)
         if rot is None:
             q = qkv[:, : self.q_dim]
             k = qkv[:, self.q_dim: self.q_dim + self.kv_dim] if cache.writes else None

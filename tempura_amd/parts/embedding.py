@@ -57,7 +57,7 @@ class OutputHead(Part):
             self.weight = embedding.weight      # same device buffer, no copy
             self.tied = True
         else:
-            self.weight = self._to_device(t)
+            self.weight = ops.tile_weight(self._to_device(t))     # (a tied matrix stays as the embedding reads it)
 
     def forward(self, x):
         """normed rows [m, hidden] -> float32 logits [m, vocab]."""

@@ -36,10 +36,10 @@ class SwiGLU(FeedForward):
         # eight of up, so that the product's epilogue applies silu(g) * u to its float32 sums.
         self.fused = self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
         if self.fused:
-            self.w13 = ops.interleave_gate_up(gate, up)
+            self.w13 = ops.tile_weight(ops.interleave_gate_up(gate, up))
         else:
-            self.w13 = torch.cat([gate, up], dim=0).contiguous()
-        self.w2 = self._to_device(get(w["down"]))
+            self.w13 = ops.tile_weight(torch.cat([gate, up], dim=0).contiguous())
+        self.w2 = ops.tile_weight(self._to_device(get(w["down"])))
 
     def forward(self, x, ctx, residual, next_norm=None):
         if self.fused:

@@ -149,6 +149,11 @@ def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
         k3, v3 = kc.to(DEV), vc.to(DEV)
         q3 = ops.linear_rope_kv(xd, wd, pd, sd, invd, rot, 1.0, heads, kv, d, k3, v3, ops.rope_table(pd, invd, rot, 1.0))
         assert torch.equal(q3, q1) and torch.equal(k3, k1) and torch.equal(v3, v1)
+    if n % 16 == 0 and k % 64 == 0:   # the weight stored tiled: the same bits
+        k4, v4 = kc.to(DEV), vc.to(DEV)
+        q4 = ops.linear_rope_kv(xd, ops.tile_weight(wd), pd, sd, invd, rot, 1.0, heads, kv, d, k4, v4,
+                                ops.rope_table(pd, invd, rot, 1.0) if m > 16 else None)
+        assert torch.equal(q4, q1) and torch.equal(k4, k1) and torch.equal(v4, v1)
     kr, vr = kc.clone(), vc.clone()
     qr = emu.rope_kv_write(x.double() @ w.double().T, pos, slots, inv, rot, 1.0, heads, kv, d, kr, vr, torch.float64)
     _close(q2, qr, 1e-2, "q")
@@ -333,6 +338,62 @@ def test_linear_mfma(m, n, k):
         _close(one[0], got[0].double().cpu(), 2e-6, "row alone vs in a batch")
         again = ops.linear(xd, wd, torch.float32)
         assert torch.equal(again, got), "the same call must give the same bits"
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 16, 64), (1, 4096, 4096), (8, 208, 192), (8, 6144, 4096), (16, 1024, 14336), (16, 48, 128),
+                                   (17, 48, 64), (33, 1008, 320), (64, 4096, 1024), (100, 16400, 128), (128, 512, 2048),
+                                   (129, 256, 2048), (200, 304, 192), (300, 4096, 4096), (700, 1040, 448), (1000, 816, 192),
+                                   (2048, 8448, 128), (2100, 6144, 128), (2300, 1024, 256)])
+def test_tiled_weights_give_the_same_bits(m, n, k):
+    """A weight stored tiled (16 x 32 blocks in the matrix cores' operand order) is the same weight: every product
+    that takes it returns the bits it returns for the row-major tensor: plain, bfloat16 out, into a residual, gated,
+    with the split norm and k-blocked rows (at most 16 rows), with the partial sums left to the consumer (17..128
+    rows) and under both tile sizes of the long products."""
+    ops = _ops()
+    lib = ops.library()
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.randn(n, k, generator=g).to(torch.bfloat16).to(DEV)
+    res = torch.randn(m, n, generator=g).to(DEV)
+    t = ops.tile_weight(w)
+    assert isinstance(t, ops.TiledWeight) and t.shape == (n, k) and torch.equal(t.row_major(), w)
+    assert torch.equal(t.rows(16, n).row_major(), w[16:]) if n > 16 else True
+    nw = (torch.rand(n, generator=g) + 0.5).to(DEV)
+    for mode in (0, 5, 6) if m > 128 else (0,):
+        lib.tp_linear_tune_tile(mode)
+        try:
+            assert torch.equal(ops.linear(x, t, torch.float32), ops.linear(x, w, torch.float32)), f"f32 out, tile mode {mode}"
+            assert torch.equal(ops.linear(x, t, torch.bfloat16), ops.linear(x, w, torch.bfloat16)), f"bf16 out, tile mode {mode}"
+            assert torch.equal(ops.linear(x, t, torch.float32, residual=res.clone()),
+                               ops.linear(x, w, torch.float32, residual=res.clone())), f"residual, tile mode {mode}"
+            a, b = ops.linear_swiglu(x, t, blocked_out=True), ops.linear_swiglu(x, w, blocked_out=True)
+            if m <= 16:
+                assert isinstance(a, ops.KBlocked) and torch.equal(a.data, b.data), "gated, k-blocked"
+            else:
+                assert torch.equal(a, b), f"gated, tile mode {mode}"
+        finally:
+            lib.tp_linear_tune_tile(0)
+    if n > 16:      # a slice of whole row groups is a weight of its own
+        assert torch.equal(ops.linear(x, ops.weight_rows(t, 16, n), torch.float32), ops.linear(x, w[16:].contiguous(), torch.float32))
+    if m <= 128:    # the next norm prepared (at most 16 rows) or the partial sums left to the norm kernel (17..128)
+        ra, rb = res.clone(), res.clone()
+        ha = ops.linear(x, t, torch.float32, residual=ra, next_norm=(nw, 1e-5))
+        hb = ops.linear(x, w, torch.float32, residual=rb, next_norm=(nw, 1e-5))
+        assert torch.equal(ra, rb)
+        if isinstance(hb[1], ops.Prenormed):
+            assert torch.equal(ha[1].x, hb[1].x) and torch.equal(ha[1].ss, hb[1].ss)
+            # ... and such rows as the input of the next product
+            w2 = torch.randn(64, n, generator=g).to(torch.bfloat16).to(DEV)
+            if n % 64 == 0:
+                assert torch.equal(ops.linear(ha[1], ops.tile_weight(w2), torch.float32), ops.linear(hb[1], w2, torch.float32))
+        elif hb[1] is not None:
+            assert torch.equal(ha[1], hb[1])
+        pa, pb = ops.linear(x, t, torch.float32, partial_ok=True), ops.linear(x, w, torch.float32, partial_ok=True)
+        assert type(pa) is type(pb)
+        assert torch.equal(pa.data, pb.data) if isinstance(pa, ops.Partials) else torch.equal(pa, pb)
+    if m <= 16 and k % 32 == 0:     # k-blocked rows in
+        kb = ops.KBlocked(x.view(m, k // 8, 8).permute(1, 0, 2).contiguous(), m, k)
+        assert torch.equal(ops.linear(kb, t, torch.float32), ops.linear(kb, w, torch.float32))
 
 
 @pytest.mark.parametrize("m,n,k", [(300, 512, 128), (1000, 816, 192), (257, 256, 64), (2048, 8448, 128), (2100, 6144, 128)])
