@@ -283,7 +283,7 @@ def _pre_args(x):
 def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     """bfloat16 x [m, k] (or ``Prenormed``), interleaved gate/up weight [2i, k] -> bfloat16 [m, i] =
     silu(x g^T) * (x u^T), the gate applied to the float32 accumulators (no rounding in between).
-    With ``blocked_out`` the result comes as ``KBlocked`` when there are at most 16 rows (else as a tensor)."""
+    With ``blocked_out`` the result comes as ``KBlocked`` when there are at most 16 rows and i % 32 == 0 (else as a tensor)."""
     if _backend is not None:
         return _backend.linear_swiglu(x, w, blocked_out) if blocked_out else _backend.linear_swiglu(x, w)
     x, pre = _pre_args(x)
@@ -294,7 +294,8 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     m, k = x.shape
     n = w.shape[0]
     _need(n % 16 == 0 and k % 32 == 0, "linear_swiglu: needs 2i % 16 == 0 and k % 32 == 0")
-    blocked_out = blocked_out and allow_mfma and 0 < m <= 16   # (the product that takes such rows is an MFMA kernel)
+    # (the product that takes such rows is an MFMA kernel over K in steps of 32)
+    blocked_out = blocked_out and allow_mfma and 0 < m <= 16 and (n // 2) % 32 == 0
     if blocked_out:
         out = KBlocked(torch.empty((n // 16, m, 8), dtype=torch.bfloat16, device=x.device), m, n // 2)
     else:

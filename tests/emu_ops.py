@@ -64,7 +64,7 @@ class EmuOps:
         g, u = y[:, :, 0].reshape(x.shape[0], -1), y[:, :, 1].reshape(x.shape[0], -1)
         out = (g / (1.0 + torch.exp(-g)) * u).to(torch.bfloat16)
         m, i = out.shape
-        if blocked_out and 0 < m <= 16:
+        if blocked_out and 0 < m <= 16 and i % 32 == 0:
             return KBlocked(out.reshape(m, i // 8, 8).permute(1, 0, 2).contiguous(), m, i)
         return out
 

@@ -38,9 +38,17 @@ CONFIGS: Dict[str, LlamaConfig] = {
                      num_key_value_heads=2, head_dim=64, vocab_size=512, max_position_embeddings=2048,
                      rms_norm_eps=1e-5, rope_theta=500000.0,
                      rope_scaling=RopeScaling("llama3", 8.0, 1.0, 4.0, 128), tie_word_embeddings=False),
+    # E: head size 80 (a multiple of 16, no power of two), groups of 3, an odd vocabulary, pages of 64, and a
+    #    feed-forward width (136) that the gated product takes but the k-blocked hand-over between the two
+    #    feed-forward products does not (it steps by 32)
+    "E": LlamaConfig(hidden_size=160, intermediate_size=136, num_hidden_layers=2, num_attention_heads=6,
+                     num_key_value_heads=2, head_dim=80, vocab_size=1001, max_position_embeddings=4096,
+                     rms_norm_eps=1e-4, rope_theta=1000000.0, rope_scaling=None, tie_word_embeddings=True),
 }
 #: weights are N(0, STD): large enough that attention is peaked and faults show
 STD = 0.15
+STD_OF = {"E": 0.1}
+SEED_OF = {"A": 11, "B": 23, "C": 37, "D": 41, "E": 53}
 
 
 class TinyModels:
@@ -53,7 +61,7 @@ class TinyModels:
         if key not in self._made:
             d = os.path.join(self.root, f"{name}_{dtype}")
             cfg = LlamaConfig.from_dict(CONFIGS[name].to_dict())
-            write_random_model(cfg, d, seed={"A": 11, "B": 23, "C": 37, "D": 41}[name], std=STD, norm_jitter=0.2, dtype=dtype)
+            write_random_model(cfg, d, seed=SEED_OF[name], std=STD_OF.get(name, STD), norm_jitter=0.2, dtype=dtype)
             self._made[key] = d
         return self._made[key]
 
@@ -151,8 +159,9 @@ def schedule_mixed(lengths: Dict[str, int], max_tokens: int, seed: int, max_live
 LENGTHS = {"A": {"a0": 5, "a1": 17, "a2": 33, "a3": 150, "a4": 97, "a5": 64},
            "B": {"b0": 1, "b1": 9, "b2": 40, "b3": 63, "b4": 120, "b5": 201},
            "C": {"c0": 3, "c1": 49, "c2": 130, "c3": 75, "c4": 25, "c5": 88},
-           "D": {"d0": 7, "d1": 300, "d2": 41, "d3": 170, "d4": 96, "d5": 33}}
-PAGE_SIZE = {"A": 16, "B": 8, "C": 32, "D": 16}
+           "D": {"d0": 7, "d1": 300, "d2": 41, "d3": 170, "d4": 96, "d5": 33},
+           "E": {"e0": 2, "e1": 129, "e2": 64, "e3": 260, "e4": 31, "e5": 65}}
+PAGE_SIZE = {"A": 16, "B": 8, "C": 32, "D": 16, "E": 64}
 
 
 def requests_for(name: str) -> Dict[str, List[int]]:

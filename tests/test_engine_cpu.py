@@ -25,7 +25,7 @@ def _runner(tiny_dirs, name, max_tokens):
     return ModelRunner(model, ps, (max_tokens + ps - 1) // ps, max_requests=4)
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_every_cutting_matches_plain(tiny_dirs, name, mode):
     cfg, W = tiny_dirs.plain_model(name)

@@ -46,7 +46,7 @@ def _compare(got, ref, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_tail", "portions", "mixed"])
 def test_replay_modes(tiny_dirs, name, dtype, mode):
     requests = helpers.requests_for(name)
@@ -95,7 +95,7 @@ def test_long_decoding(tiny_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_first_tokens(tiny_dirs, name, dtype):
     """The first tokens of a sequence, one by one from position 0 (one key, then two, ...)."""
     cfg, W = tiny_dirs.plain_model(name, dtype)
