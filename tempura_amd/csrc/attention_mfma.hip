@@ -695,7 +695,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 }
 
 // ---- dispatch ------------------------------------------------------------------------------
-static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave
+static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave; 2 / 3: 32 / 16 query rows per wave
 extern "C" void tp_attention_tune(int v) { g_attn_tune = v; }
 
 template <int D>
@@ -712,16 +712,29 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
     }
   }
   if (has_multi) {
-    constexpr int NQ = (D <= 128) ? 2 : 1;
-    const dim3 grid((max_q_len + 16 * NQ - 1) / (16 * NQ), a.n_kv * ((group + 3) / 4), n_req);
+    // A wave owns 32 query rows (two tiles: half the key and value reads per product) when that still gives
+    // every CU its two blocks; otherwise 16 rows and twice the blocks (a portion of 512 tokens behind a long
+    // prefix: a fifth faster).  Both give the same bits: a query column never sees another's values.
+    const int kv_groups = a.n_kv * ((group + 3) / 4);
+    const long blocks2 = (long)((max_q_len + 31) / 32) * kv_groups * n_req;
+    const bool two = g_attn_tune == 2 || (g_attn_tune != 3 && blocks2 >= 512);
+    const int rows = two ? 32 : 16;
+    const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
+    const int skip = num_single > 0 ? 1 : 0;
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
       if (g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
-        hipLaunchKernelGGL((attn_prefill_lds_kernel<D, NQ>), grid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0);
+        if (two)
+          hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), grid, dim3(256), 0, s, a, skip);
+        else
+          hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 1>), grid, dim3(256), 0, s, a, skip);
         return 0;
       }
     }
-    hipLaunchKernelGGL((attn_prefill_kernel<D, NQ>), grid, dim3(256), 0, s, a, num_single > 0 ? 1 : 0);
+    if (two)
+      hipLaunchKernelGGL((attn_prefill_kernel<D, 2>), grid, dim3(256), 0, s, a, skip);
+    else
+      hipLaunchKernelGGL((attn_prefill_kernel<D, 1>), grid, dim3(256), 0, s, a, skip);
   }
   return 0;
 }

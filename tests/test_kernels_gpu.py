@@ -221,7 +221,7 @@ def test_rope_kv_write_long_step(dtype, heads, kv, d, page, n):
     assert torch.equal(k1, kd) and torch.equal(v1, vd)
 
 
-def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, allow_fast=True):
+def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, allow_fast=True, tune=0):
     ops = _ops()
     g = torch.Generator().manual_seed(seed)
     R = len(q_lens)
@@ -244,12 +244,15 @@ def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, a
     scale = 1.0 / math.sqrt(d)
     ref = emu.paged_attention(q, kc, vc, bt, cu, cl, tr, scale, window, max(q_lens), max(ctx_lens)).double()
     ops.allow_fast_attention = allow_fast
+    ops.library().tp_attention_tune(tune)
     try:
         got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), cu.to(DEV), cl.to(DEV), tr.to(DEV),
                                   scale, window, max(q_lens), max(ctx_lens))
     finally:
         ops.allow_fast_attention = True
+        ops.library().tp_attention_tune(0)
     _close(got, ref, 2e-5 if dtype == torch.float32 else 1.2e-2, f"attention h{heads} kv{kv} d{d} page{page}")
+    return got
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -528,6 +531,10 @@ def test_attention_mfma(heads, kv, d, page):
     _attention_case(bf, heads, kv, d, page, [70, 33], [70, 97], 0, seed=13)                            # portions only
     _attention_case(bf, heads, kv, d, page, [20, 1, 6, 1], [50, 77, 6, 300], 13, seed=14)              # window
     _attention_case(bf, heads, kv, d, page, [40, 1], [200, 200], 64, seed=15)                          # window longer than a step
+    # a wave takes 32 query rows when there are many blocks and 16 when there are few: the same bits
+    for q_lens, ctx_lens, window in (([70, 33, 1], [70, 97, 40], 0), ([45, 100], [300, 100], 50)):
+        a, b = (_attention_case(bf, heads, kv, d, page, q_lens, ctx_lens, window, seed=17, tune=t) for t in (2, 3))
+        assert torch.equal(a, b)
 
 
 def test_attention_mfma_long_decode():
