@@ -81,7 +81,13 @@ struct AttnArgs {
   int n_heads, n_kv, page_size, window, num_splits;
   int page_shift;   // log2(page_size), or -1
   float scale_log2;
+  // portions whose keys are split over blocks (few query blocks, a long context): the number of parts and
+  // their partial results, [token, head, part] of PART_STRIDE(D) floats: O (unnormalised), maximum, sum
+  int portion_splits;
+  float* portion_scratch;
+  const int* token_req;
 };
+#define PART_STRIDE(D) ((D) + 4)
 
 // The keys and values of one step of 32 keys, as MFMA operand fragments.
 template <int D>
@@ -338,7 +344,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   // query blocks; the longest query blocks come first.
   const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
   const int by = lin % gridDim.y, bx = (lin / gridDim.y) % gridDim.x;
-  const int r = lin / (gridDim.x * gridDim.y);
+  const int rz = lin / (gridDim.x * gridDim.y);
+  const int r = rz / a.portion_splits, part = rz % a.portion_splits;   // (gridDim.z = requests * parts)
   const int q_start = a.cu_seqlens[r];
   const int q_len = a.cu_seqlens[r + 1] - q_start;
   if (q_len <= 0 || (skip_single && q_len == 1)) return;
@@ -374,7 +381,31 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   const int last_pos = pos0 + min(q0 + 16 * NQ, q_len) - 1;
   int first = 0;
   if (a.window > 0) first = max(0, pos0 + q0 - a.window + 1) & ~31;
-  const int nsteps = (last_pos - first) / 32 + 1;
+  int nsteps = (last_pos - first) / 32 + 1;
+  if (a.portion_splits > 1) {
+    // this block's share of the steps; a block without any writes partial results that weigh nothing
+    const int per_part = (nsteps + a.portion_splits - 1) / a.portion_splits;
+    const int s_begin = part * per_part;
+    nsteps = min(nsteps, s_begin + per_part) - s_begin;
+    first += s_begin * 32;
+    if (nsteps <= 0) {
+      if (active) {
+#pragma unroll
+        for (int nq = 0; nq < NQ; ++nq) {
+          const int qi = q0 + nq * 16 + c;
+          if (qi >= q_len) continue;
+          float* pr = a.portion_scratch + (((size_t)(q_start + qi) * a.n_heads + head) * a.portion_splits + part) * PART_STRIDE(D);
+#pragma unroll
+          for (int dt = 0; dt < D / 16; ++dt) *(f32x4_t*)(pr + dt * 16 + 4 * g) = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+          if (g == 0) {
+            pr[D] = -INFINITY;
+            pr[D + 1] = 0.f;
+          }
+        }
+      }
+      return;
+    }
+  }
   const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this block
 
   // what this lane fetches in each of its loads of a step: load t = wave + 4 i; t < KI is a piece of
@@ -562,7 +593,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     lt += __shfl_xor(lt, 32, 64);
     const float inv = 1.0f / lt;
     const int qi = q0 + nq * 16 + c;
-    if (qi < q_len) {
+    if (qi < q_len && a.portion_splits > 1) {
+      float* pr = a.portion_scratch + (((size_t)(q_start + qi) * a.n_heads + head) * a.portion_splits + part) * PART_STRIDE(D);
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) *(f32x4_t*)(pr + dt * 16 + 4 * g) = o[nq][dt];
+      if (g == 0) {
+        pr[D] = m[nq];
+        pr[D + 1] = lt;
+      }
+    } else if (qi < q_len) {
       bf16_t* orow = a.out + ((size_t)(q_start + qi) * a.n_heads + head) * D;
 #pragma unroll
       for (int dt = 0; dt < D / 16; ++dt) {
@@ -694,12 +733,40 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   }
 }
 
+// The same for the rows of portions whose keys were split over blocks: out[token, head, :] from the parts
+// [token, head, part] of PART_STRIDE(D) floats, in ascending order.  grid: (tokens, heads); block: one wave.
+__global__ __launch_bounds__(64) void attn_combine_rows_kernel(const float* __restrict__ scratch,
+                                                               const int* __restrict__ cu_seqlens,
+                                                               const int* __restrict__ token_req,
+                                                               bf16_t* __restrict__ out, int n_heads, int D,
+                                                               int parts, int skip_single) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int r = token_req[t];
+  if (skip_single && cu_seqlens[r + 1] - cu_seqlens[r] == 1) return;   // (the decode kernels wrote this row)
+  const int stride = PART_STRIDE(D);
+  const float* base = scratch + ((size_t)t * n_heads + h) * parts * stride;
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < parts) {
+    ms = base[(size_t)lane * stride + D];
+    ls = base[(size_t)lane * stride + D + 1];
+  }
+  const float mg = wave_max(ms);
+  const float mu = (mg == -INFINITY) ? 0.f : mg;
+  const float ws = __builtin_amdgcn_exp2f(ms - mu);  // 0 for lanes without a part
+  const float inv = 1.0f / wave_sum(ws * ls);
+  for (int d = lane; d < D; d += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < parts; ++s) acc = fmaf(__shfl(ws, s, 64), base[(size_t)s * stride + d], acc);
+    out[((size_t)t * n_heads + h) * D + d] = float_to_bf16(acc * inv);
+  }
+}
+
 // ---- dispatch ------------------------------------------------------------------------------
 static int g_attn_tune = 0;   // 1: portions take the kernel that loads keys and values per wave; 2 / 3: 32 / 16 query rows per wave
 extern "C" void tp_attention_tune(int v) { g_attn_tune = v; }
 
 template <int D>
-static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_single, hipStream_t s) {
+static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int num_single, hipStream_t s) {
   const int group = a.n_heads / a.n_kv;
   const bool has_multi = num_single < n_req;
   if (num_single > 0) {
@@ -719,8 +786,19 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
     const long blocks2 = (long)((max_q_len + 31) / 32) * kv_groups * n_req;
     const bool two = g_attn_tune == 2 || (g_attn_tune != 3 && blocks2 >= 512);
     const int rows = two ? 32 : 16;
-    const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
     const int skip = num_single > 0 ? 1 : 0;
+    if constexpr (D == 32 || D == 64 || D == 128) {
+      if (a.portion_splits > 1 && g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
+        // few query blocks under a long context: the keys of each are split over blocks (of 32 query rows)
+        const dim3 sgrid((max_q_len + 31) / 32, kv_groups, n_req * a.portion_splits);
+        hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), sgrid, dim3(256), 0, s, a, skip);
+        hipLaunchKernelGGL(attn_combine_rows_kernel, dim3(n_tokens, a.n_heads), dim3(64), 0, s, a.portion_scratch,
+                           a.cu_seqlens, a.token_req, a.out, a.n_heads, D, a.portion_splits, skip);
+        return 0;
+      }
+    }
+    a.portion_splits = 1;   // (the kernels below do not split)
+    const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
       if (g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
@@ -742,8 +820,11 @@ static int launch_all(const AttnArgs& a, int n_req, int max_q_len, int num_singl
 int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                             int table_width, const int* cu_seqlens, const int* context_lens, void* out, int n_tokens,
                             int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
-                            int max_q_len, int num_single, int num_splits, float* scratch, hipStream_t s) {
+                            int max_q_len, int num_single, int num_splits, float* scratch, const int* token_req,
+                            int portion_splits, float* portion_scratch, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
+  if (portion_splits < 1 || portion_splits > 64 || (portion_splits > 1 && (portion_scratch == nullptr || token_req == nullptr))) return -1;
+  if ((long)n_req * portion_splits > 65535) return -1;
   if (n_req > 65535 || n_req <= 0) return -1;
   if (num_single > 0 && (num_splits < 1 || num_splits > 64)) return -1;
   if (num_single > 0 && num_splits > 1 && scratch == nullptr) return -1;
@@ -765,12 +846,15 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
     if ((1 << b) == page_size) a.page_shift = b;
   a.window = window;
   a.num_splits = num_splits;
+  a.portion_splits = portion_splits;
+  a.portion_scratch = portion_scratch;
+  a.token_req = token_req;
   a.scale_log2 = scale * 1.4426950408889634f;
   switch (head_dim) {
-    case 32: launch_all<32>(a, n_req, max_q_len, num_single, s); break;
-    case 64: launch_all<64>(a, n_req, max_q_len, num_single, s); break;
-    case 96: launch_all<96>(a, n_req, max_q_len, num_single, s); break;
-    case 128: launch_all<128>(a, n_req, max_q_len, num_single, s); break;
+    case 32: launch_all<32>(a, n_tokens, n_req, max_q_len, num_single, s); break;
+    case 64: launch_all<64>(a, n_tokens, n_req, max_q_len, num_single, s); break;
+    case 96: launch_all<96>(a, n_tokens, n_req, max_q_len, num_single, s); break;
+    case 128: launch_all<128>(a, n_tokens, n_req, max_q_len, num_single, s); break;
     default: return -1;
   }
   TP_CHECK_LAUNCH("paged_attention (mfma)");

@@ -537,6 +537,27 @@ def test_attention_mfma(heads, kv, d, page):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("heads,kv,d,page", [(8, 2, 128, 16), (6, 3, 64, 32), (5, 1, 32, 64)])
+def test_attention_portions_with_split_keys(heads, kv, d, page):
+    """Few query blocks under a long context: the keys of a portion are split over blocks and the parts combined.
+    Parts of 64 keys here, so that there are many (more than some blocks have steps: empty parts), beside single
+    decoded tokens, with and without a window; the unsplit kernel's result is within rounding."""
+    ops = _ops()
+    bf = torch.bfloat16
+    cases = (([40, 1, 5, 1], [700, 300, 41, 64], 0), ([33, 2], [1000, 515], 0), ([70, 1], [400, 130], 100))
+    keep = ops.portion_min_keys, ops.portion_target_blocks
+    try:
+        for q_lens, ctx_lens, window in cases:
+            ops.portion_min_keys, ops.portion_target_blocks = 64, 4096
+            a = _attention_case(bf, heads, kv, d, page, q_lens, ctx_lens, window, seed=18)
+            ops.portion_target_blocks = 1
+            b = _attention_case(bf, heads, kv, d, page, q_lens, ctx_lens, window, seed=18)
+            assert not torch.equal(a, b), "the split path did not run"
+            _close(a, b.double().cpu(), 8e-3, "split against unsplit")
+    finally:
+        ops.portion_min_keys, ops.portion_target_blocks = keep
+
+
 def test_attention_mfma_long_decode():
     _attention_case(torch.bfloat16, 8, 2, 128, 16, [1, 1], [3000, 2049], 0, seed=16)
 
