@@ -521,9 +521,11 @@ portion_scratch_limit = 256 << 20
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     cu_seqlens: torch.Tensor, context_lens: torch.Tensor, token_req: torch.Tensor,
                     scale: float, window: int, max_q_len: int, max_context_len: int,
-                    num_single: Optional[int] = None) -> torch.Tensor:
+                    num_single: Optional[int] = None, portion_avg_keys: Optional[int] = None) -> torch.Tensor:
     """q [n, heads, head_dim] over k [pages, kv_heads, page_size, head_dim] and transposed
-    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim]."""
+    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim].
+    ``portion_avg_keys``: the keys a query row of the longer requests attends to, on average (None: estimated
+    from the longest request); it decides whether splitting their keys over blocks pays."""
     if _backend is not None:
         return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
                                         token_req, scale, window, max_q_len, max_context_len)
@@ -561,7 +563,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         # every portion are split over blocks until the chip is full (T = 512 behind 7,680 keys: 236 -> 138 us).
         q_blocks = -(-(n - num_single) // 32) + (r - num_single)
         blocks = q_blocks * kvh * ((heads // kvh + 3) // 4)
-        parts = max(1, min(16, portion_target_blocks // blocks, max_context_len // portion_min_keys, 65535 // r))
+        if portion_avg_keys is None:
+            portion_avg_keys = max_context_len - max_q_len // 2
+        if window > 0:
+            portion_avg_keys = min(portion_avg_keys, window)
+        # (a part costs its partial results, about what 260 keys cost: parts of few keys are a loss)
+        parts = max(1, min(16, portion_target_blocks // blocks, portion_avg_keys // portion_min_keys, 65535 // r))
         if parts > 1 and n * heads * parts * (d + 4) * 4 > portion_scratch_limit:
             parts = 1
         if parts > 1:

@@ -544,7 +544,7 @@ def test_attention_portions_with_split_keys(heads, kv, d, page):
     decoded tokens, with and without a window; the unsplit kernel's result is within rounding."""
     ops = _ops()
     bf = torch.bfloat16
-    cases = (([40, 1, 5, 1], [700, 300, 41, 64], 0), ([33, 2], [1000, 515], 0), ([70, 1], [400, 130], 100))
+    cases = (([40, 1, 5, 1], [700, 300, 41, 64], 0), ([33, 2], [1000, 515], 0), ([70, 1], [900, 130], 300))
     keep = ops.portion_min_keys, ops.portion_target_blocks
     try:
         for q_lens, ctx_lens, window in cases:
