@@ -88,15 +88,15 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int table_width, const int* cu_seqlens, const int* context_lens, void* out, int n_tokens,
                             int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
                             int max_q_len, int num_single, int num_splits, float* scratch, const int* token_req,
-                            int portion_splits, float* portion_scratch, hipStream_t s);
+                            int portion_splits, int portion_min_steps, float* portion_scratch, hipStream_t s);
 
 extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, const void* v_cache,
                                   const int* block_tables, int table_width, const int* cu_seqlens,
                                   const int* context_lens, const int* token_req, void* out, int n_tokens,
                                   int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale,
                                   int window, int max_q_len, int max_ctx, int allow_fast, int num_single,
-                                  int num_splits, float* scratch, int portion_splits, float* portion_scratch,
-                                  hipStream_t s) {
+                                  int num_splits, float* scratch, int portion_splits, int portion_min_steps,
+                                  float* portion_scratch, hipStream_t s) {
   // num_single: how many requests bring exactly one token (they go to the split decode kernel,
   // which, with more than one split, needs `scratch` of n_req * n_heads * num_splits * (head_dim + 2)
   // floats).  portion_splits > 1: the keys of every longer request are split over that many blocks,
@@ -113,7 +113,7 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
     const int rc = tp_paged_attention_fast(q, k_cache, v_cache, block_tables, table_width, cu_seqlens,
                                            context_lens, out, n_tokens, n_req, n_heads, n_kv, head_dim,
                                            page_size, scale, window, max_q_len, num_single, num_splits, scratch, token_req,
-                                           portion_splits, portion_scratch, s);
+                                           portion_splits, portion_min_steps, portion_scratch, s);
     if (rc >= 0) return rc;
   }
   const dim3 grid(n_tokens, n_heads);

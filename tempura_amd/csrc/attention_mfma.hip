@@ -81,9 +81,11 @@ struct AttnArgs {
   int n_heads, n_kv, page_size, window, num_splits;
   int page_shift;   // log2(page_size), or -1
   float scale_log2;
-  // portions whose keys are split over blocks (few query blocks, a long context): the number of parts and
-  // their partial results, [token, head, part] of PART_STRIDE(D) floats: O (unnormalised), maximum, sum
+  // portions whose keys are split over blocks (few query blocks, long contexts): the largest number of parts
+  // (a query block with few steps gets fewer, or stays whole and writes its rows itself) and their partial
+  // results, [token, head, part] of PART_STRIDE(D) floats: O (unnormalised), maximum, sum
   int portion_splits;
+  int portion_min_steps;   // a query block is split into at most (its steps / this) parts
   float* portion_scratch;
   const int* token_req;
 };
@@ -327,6 +329,11 @@ __device__ inline u32x4_t attn_lds_read(unsigned addr) {
   return v;
 }
 
+// Into how many parts the keys of a query block with `steps` steps of 32 keys are split.
+__device__ __host__ inline int portion_parts(int steps, int max_parts, int min_steps) {
+  return max_parts <= 1 ? 1 : min(max_parts, max(1, steps / min_steps));
+}
+
 template <int D, int NQ>
 __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, int skip_single) {
   constexpr int C = D / 8;             // 16-byte chunks per key row
@@ -382,29 +389,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   int first = 0;
   if (a.window > 0) first = max(0, pos0 + q0 - a.window + 1) & ~31;
   int nsteps = (last_pos - first) / 32 + 1;
-  if (a.portion_splits > 1) {
-    // this block's share of the steps; a block without any writes partial results that weigh nothing
-    const int per_part = (nsteps + a.portion_splits - 1) / a.portion_splits;
-    const int s_begin = part * per_part;
-    nsteps = min(nsteps, s_begin + per_part) - s_begin;
+  const int my_parts = portion_parts(nsteps, a.portion_splits, a.portion_min_steps);
+  if (part >= my_parts) return;
+  if (my_parts > 1) {   // this block's share of the steps (never empty: my_parts <= nsteps)
+    const int s_begin = (int)((long)part * nsteps / my_parts), s_end = (int)((long)(part + 1) * nsteps / my_parts);
     first += s_begin * 32;
-    if (nsteps <= 0) {
-      if (active) {
-#pragma unroll
-        for (int nq = 0; nq < NQ; ++nq) {
-          const int qi = q0 + nq * 16 + c;
-          if (qi >= q_len) continue;
-          float* pr = a.portion_scratch + (((size_t)(q_start + qi) * a.n_heads + head) * a.portion_splits + part) * PART_STRIDE(D);
-#pragma unroll
-          for (int dt = 0; dt < D / 16; ++dt) *(f32x4_t*)(pr + dt * 16 + 4 * g) = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-          if (g == 0) {
-            pr[D] = -INFINITY;
-            pr[D + 1] = 0.f;
-          }
-        }
-      }
-      return;
-    }
+    nsteps = s_end - s_begin;
   }
   const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this block
 
@@ -593,7 +583,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     lt += __shfl_xor(lt, 32, 64);
     const float inv = 1.0f / lt;
     const int qi = q0 + nq * 16 + c;
-    if (qi < q_len && a.portion_splits > 1) {
+    if (qi < q_len && my_parts > 1) {
       float* pr = a.portion_scratch + (((size_t)(q_start + qi) * a.n_heads + head) * a.portion_splits + part) * PART_STRIDE(D);
 #pragma unroll
       for (int dt = 0; dt < D / 16; ++dt) *(f32x4_t*)(pr + dt * 16 + 4 * g) = o[nq][dt];
@@ -734,17 +724,27 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
 }
 
 // The same for the rows of portions whose keys were split over blocks: out[token, head, :] from the parts
-// [token, head, part] of PART_STRIDE(D) floats, in ascending order.  grid: (tokens, heads); block: one wave.
+// [token, head, part] of PART_STRIDE(D) floats, in ascending order.  A row's query block (of 32 rows) may have
+// been split into fewer parts than the most, or not at all (then the attention kernel wrote the row itself):
+// the count is worked out here as it is there.  grid: (tokens, heads); block: one wave.
 __global__ __launch_bounds__(64) void attn_combine_rows_kernel(const float* __restrict__ scratch,
                                                                const int* __restrict__ cu_seqlens,
+                                                               const int* __restrict__ context_lens,
                                                                const int* __restrict__ token_req,
                                                                bf16_t* __restrict__ out, int n_heads, int D,
-                                                               int parts, int skip_single) {
+                                                               int max_parts, int min_steps, int window, int skip_single) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = token_req[t];
-  if (skip_single && cu_seqlens[r + 1] - cu_seqlens[r] == 1) return;   // (the decode kernels wrote this row)
+  const int q_start = cu_seqlens[r], q_len = cu_seqlens[r + 1] - q_start;
+  if (skip_single && q_len == 1) return;   // (the decode kernels wrote this row)
+  const int pos0 = context_lens[r] - q_len;
+  const int q0 = ((t - q_start) / 32) * 32;
+  const int last_pos = pos0 + min(q0 + 32, q_len) - 1;
+  const int first = window > 0 ? (max(0, pos0 + q0 - window + 1) & ~31) : 0;
+  const int parts = portion_parts((last_pos - first) / 32 + 1, max_parts, min_steps);
+  if (parts == 1) return;
   const int stride = PART_STRIDE(D);
-  const float* base = scratch + ((size_t)t * n_heads + h) * parts * stride;
+  const float* base = scratch + ((size_t)t * n_heads + h) * max_parts * stride;
   float ms = -INFINITY, ls = 0.f;
   if (lane < parts) {
     ms = base[(size_t)lane * stride + D];
@@ -793,7 +793,8 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
         const dim3 sgrid((max_q_len + 31) / 32, kv_groups, n_req * a.portion_splits);
         hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), sgrid, dim3(256), 0, s, a, skip);
         hipLaunchKernelGGL(attn_combine_rows_kernel, dim3(n_tokens, a.n_heads), dim3(64), 0, s, a.portion_scratch,
-                           a.cu_seqlens, a.token_req, a.out, a.n_heads, D, a.portion_splits, skip);
+                           a.cu_seqlens, a.context_lens, a.token_req, a.out, a.n_heads, D, a.portion_splits,
+                           a.portion_min_steps, a.window, skip);
         return 0;
       }
     }
@@ -821,8 +822,9 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int table_width, const int* cu_seqlens, const int* context_lens, void* out, int n_tokens,
                             int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
                             int max_q_len, int num_single, int num_splits, float* scratch, const int* token_req,
-                            int portion_splits, float* portion_scratch, hipStream_t s) {
+                            int portion_splits, int portion_min_steps, float* portion_scratch, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
+  if (portion_min_steps < 1) return -1;
   if (portion_splits < 1 || portion_splits > 64 || (portion_splits > 1 && (portion_scratch == nullptr || token_req == nullptr))) return -1;
   if ((long)n_req * portion_splits > 65535) return -1;
   if (n_req > 65535 || n_req <= 0) return -1;
@@ -847,6 +849,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
   a.window = window;
   a.num_splits = num_splits;
   a.portion_splits = portion_splits;
+  a.portion_min_steps = portion_min_steps;
   a.portion_scratch = portion_scratch;
   a.token_req = token_req;
   a.scale_log2 = scale * 1.4426950408889634f;

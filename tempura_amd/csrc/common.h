@@ -45,6 +45,14 @@ __device__ inline float to_float(float v) { return v; }
 __device__ inline float to_float(bf16_t v) { return bf16_to_float(v); }
 __device__ inline void from_float(float* p, float v) { *p = v; }
 __device__ inline void from_float(bf16_t* p, float v) { *p = float_to_bf16(v); }
+// four neighbouring results as one store (p aligned to four elements)
+__device__ inline void from_float4(float* p, float a, float b, float c, float d) { *(float4*)p = make_float4(a, b, c, d); }
+__device__ inline void from_float4(bf16_t* p, float a, float b, float c, float d) {
+  uint2 u;
+  u.x = (uint32_t)float_to_bf16(a).bits | ((uint32_t)float_to_bf16(b).bits << 16);
+  u.y = (uint32_t)float_to_bf16(c).bits | ((uint32_t)float_to_bf16(d).bits << 16);
+  *(uint2*)p = u;
+}
 
 // cosine and sine (times factor) of pos * inv_freq: the product in float64, reduced to [0, 2 pi) there,
 // sine and cosine of the small rest in float32 (every kernel that rotates uses this one routine)

@@ -74,10 +74,7 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
       const int j = (threadIdx.x + i * blockDim.x) * 4;
       if (j < hidden) {
         const float4 wv = *(const float4*)(w + j);
-        from_float(o + j, v[i].x * scale * wv.x);
-        from_float(o + j + 1, v[i].y * scale * wv.y);
-        from_float(o + j + 2, v[i].z * scale * wv.z);
-        from_float(o + j + 3, v[i].w * scale * wv.w);
+        from_float4(o + j, v[i].x * scale * wv.x, v[i].y * scale * wv.y, v[i].z * scale * wv.z, v[i].w * scale * wv.w);
       }
     }
     return;

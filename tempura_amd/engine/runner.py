@@ -60,7 +60,6 @@ class StepContext:
         self.max_q_len = 0
         self.max_context_len = 0
         self.num_single = 0          # requests that bring exactly one token
-        self.portion_avg_keys = 0    # keys that a query row of the longer requests attends to, on average
         self.page_size = 0
         self.q_starts: List[int] = []
         self.q_lens: List[int] = []
@@ -234,8 +233,6 @@ class ModelRunner:
         ctx.max_q_len = max(q_lens)
         ctx.num_single = sum(1 for n in q_lens if n == 1)
         ctx.max_context_len = int(ctx_lens.max())
-        multi = [(n, int(c)) for n, c in zip(q_lens, ctx_lens) if n > 1]
-        ctx.portion_avg_keys = sum(n * (c - (n - 1) // 2) for n, c in multi) // max(1, sum(n for n, _ in multi))
         ctx.page_size = self.page_size
         ctx.q_starts = [int(c) for c in cu[:-1]]
         ctx.q_lens = q_lens

@@ -513,7 +513,7 @@ decode_target_blocks = 256
 #: portions of prompts with fewer query blocks than this have their keys split over blocks (1: never)
 portion_target_blocks = 1024
 #: in parts of at least this many keys
-portion_min_keys = 512
+portion_min_keys = 1024
 #: and only while the partial results stay below this many bytes
 portion_scratch_limit = 256 << 20
 
@@ -521,11 +521,9 @@ portion_scratch_limit = 256 << 20
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     cu_seqlens: torch.Tensor, context_lens: torch.Tensor, token_req: torch.Tensor,
                     scale: float, window: int, max_q_len: int, max_context_len: int,
-                    num_single: Optional[int] = None, portion_avg_keys: Optional[int] = None) -> torch.Tensor:
+                    num_single: Optional[int] = None) -> torch.Tensor:
     """q [n, heads, head_dim] over k [pages, kv_heads, page_size, head_dim] and transposed
-    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim].
-    ``portion_avg_keys``: the keys a query row of the longer requests attends to, on average (None: estimated
-    from the longest request); it decides whether splitting their keys over blocks pays."""
+    v [pages, kv_heads, head_dim, page_size] -> [n, heads * head_dim]."""
     if _backend is not None:
         return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
                                         token_req, scale, window, max_q_len, max_context_len)
@@ -563,15 +561,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     parts, part_scratch = 1, None
     if fast and num_single < r and d in (32, 64, 128) and page_size & (page_size - 1) == 0 and page_size >= max(8, 512 // d):
         # Few query blocks under a long context (a portion of a prompt behind a long cached prefix): the keys of
-        # every portion are split over blocks until the chip is full (T = 512 behind 7,680 keys: 236 -> 138 us).
+        # every portion are split over blocks until the chip is full (T = 512 behind 7,680 keys: 219 -> 137 us).
         q_blocks = -(-(n - num_single) // 32) + (r - num_single)
         blocks = q_blocks * kvh * ((heads // kvh + 3) // 4)
-        if portion_avg_keys is None:
-            portion_avg_keys = max_context_len - max_q_len // 2
-        if window > 0:
-            portion_avg_keys = min(portion_avg_keys, window)
-        # (a part costs its partial results, about what 260 keys cost: parts of few keys are a loss)
-        parts = max(1, min(16, portion_target_blocks // blocks, portion_avg_keys // portion_min_keys, 65535 // r))
+        # (a query block is split into at most as many parts as it has portion_min_keys keys: the short blocks
+        # of a prompt from an empty cache stay whole)
+        parts = max(1, min(16, portion_target_blocks // blocks, max_context_len // portion_min_keys, 65535 // r))
         if parts > 1 and n * heads * parts * (d + 4) * 4 > portion_scratch_limit:
             parts = 1
         if parts > 1:
@@ -579,7 +574,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _call("tp_paged_attention", _ptr(q), _dt(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), width,
           _ptr(cu_seqlens), _ptr(context_lens), _ptr(token_req), _ptr(out), n, r, heads, kvh, d, page_size,
           ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(fast),
-          int(num_single), int(splits), _ptr(scratch), int(parts), _ptr(part_scratch), _stream())
+          int(num_single), int(splits), _ptr(scratch), int(parts), max(1, portion_min_keys // 32), _ptr(part_scratch), _stream())
     return out
 
 

@@ -97,7 +97,7 @@ class PagedAttention(Mixer):
         a = ops.paged_attention(
             q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
             ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
-            ctx.num_single, getattr(ctx, "portion_avg_keys", None) or None)
+            ctx.num_single)
         if next_norm is None:
             ops.linear(a, self.wo, torch.float32, residual=residual)
             return None

@@ -540,8 +540,9 @@ def test_attention_mfma(heads, kv, d, page):
 @pytest.mark.parametrize("heads,kv,d,page", [(8, 2, 128, 16), (6, 3, 64, 32), (5, 1, 32, 64)])
 def test_attention_portions_with_split_keys(heads, kv, d, page):
     """Few query blocks under a long context: the keys of a portion are split over blocks and the parts combined.
-    Parts of 64 keys here, so that there are many (more than some blocks have steps: empty parts), beside single
-    decoded tokens, with and without a window; the unsplit kernel's result is within rounding."""
+    Parts of at least 64 keys here, so that there are many (query blocks with few steps get fewer parts, or stay
+    whole and write their rows themselves), beside single decoded tokens, with and without a window; the unsplit
+    kernel's result is within rounding."""
     ops = _ops()
     bf = torch.bfloat16
     cases = (([40, 1, 5, 1], [700, 300, 41, 64], 0), ([33, 2], [1000, 515], 0), ([70, 1], [900, 130], 300))
