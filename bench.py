@@ -15,6 +15,7 @@ from __future__ import annotations
 import argparse
 import copy
 import json
+import os
 import random
 import sys
 import time
@@ -36,6 +37,7 @@ def parse_args():
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-chain", action="store_true", help="wait for each step's tokens on the host before queueing the next step")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--point-steps", type=int, default=1000, help="timed steps of the batch-1 and batch-64 points")
@@ -121,12 +123,27 @@ def main() -> int:
         for rid in rids:
             runner.add_request(rid)
             runner.step([StepEntry(rid, prompt(args.prompt_len), [])])
-        last = [rng.randrange(V) for _ in rids]
+        # The first step takes its tokens from the host; from then on a step takes the tokens the argmax kernel
+        # chose (still on the device) and is queued behind it at once, while the tokens of the step before
+        # travel to the host, where serving needs them one step later (the engine's loop does the same).
+        lg = runner.step([StepEntry(rid, [rng.randrange(V)], [0]) for rid in rids])
+        chosen = ops.argmax(lg)
+        coming = ops.HostCopy(chosen)
+        seen = []
 
         def one():
-            nonlocal last
-            lg = runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, last)])
-            last = ops.argmax(lg).tolist()          # the next tokens come back to the host, as in serving
+            nonlocal chosen, coming
+            if args.no_chain:                       # (for comparison: wait for the tokens, then queue the step)
+                lg = runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, coming.result())])
+                chosen = ops.argmax(lg)
+                coming = ops.HostCopy(chosen)
+                return
+            lg = runner.step_chained(rids, chosen)
+            nxt = ops.argmax(lg)
+            nxt_coming = ops.HostCopy(nxt)
+            runner.prepare_decode(rids)             # stage the step after this one while the GPU works
+            seen.append(coming.result()[0])         # the tokens of the step before, on the host
+            chosen, coming = nxt, nxt_coming
 
         for _ in range(n_warm):
             one()

@@ -19,7 +19,8 @@ from ..sampling import Sampler, SamplingParams
 from .loading import load_model, parse_dtype, random_model
 from .model import CausalLM
 from .runner import ModelRunner, StepEntry
-from .scheduler import Request, RequestState, Scheduler, SchedulerConfig
+from ..cache import PagesExhausted
+from .scheduler import Request, RequestState, ScheduledItem, Scheduler, SchedulerConfig
 
 
 class Engine:
@@ -27,11 +28,16 @@ class Engine:
                  seed: int = 0, page_size: int = 16, kv_pages: Optional[int] = None,
                  gpu_memory_utilization: float = 0.9, max_batch_size: int = 64,
                  max_seq_len: Optional[int] = None, max_num_batched_tokens: int = 2048,
-                 prefill_chunk_size: int = 512, device: str = "cuda:0", use_graph: bool = True):
+                 prefill_chunk_size: int = 512, device: str = "cuda:0", use_graph: bool = True,
+                 chain_steps: bool = True):
         """``model``: a folder with config.json and safetensors, or (with ``random_weights``) a typed
         configuration such as ``LlamaConfig``/``PRESETS[name]``.
         ``kv_pages``: cache pages per group; by default as many as ``gpu_memory_utilization`` of the
-        free memory holds, but no more than ``max_batch_size`` requests of ``max_seq_len`` need."""
+        free memory holds, but no more than ``max_batch_size`` requests of ``max_seq_len`` need.
+        ``chain_steps``: while every running request is decoding and nobody waits, the next step is queued
+        behind the sampling kernel (its tokens stay on the device) before the host has read this step's
+        tokens, so the GPU does not wait for the host between steps; a request that ends on the token just
+        read has then one row computed for nothing.  What the caller sees does not change."""
         self.device = torch.device(device)
         if isinstance(model, str):
             if random_weights:
@@ -58,7 +64,9 @@ class Engine:
         self.sampler = Sampler(spec.vocab_size, self.device, default_seed=seed)
         self._ids = itertools.count()
         self._requests: Dict[Hashable, Request] = {}
-        self.counters = {"steps": 0, "prompt_tokens": 0, "generated_tokens": 0, "batched_tokens": 0}
+        self.counters = {"steps": 0, "prompt_tokens": 0, "generated_tokens": 0, "batched_tokens": 0, "chained_steps": 0}
+        self.chain_steps = bool(chain_steps) and use_graph and self.device.type == "cuda"
+        self._ahead = None      # (requests, logits) of a step that is already queued
 
     def _pages_from_memory(self, utilization: float, max_batch_size: int) -> int:
         m = self.model
@@ -101,16 +109,28 @@ class Engine:
     def step(self) -> List[Tuple[Hashable, int, bool]]:
         """One scheduler decision, one model step, one sampling pass.
         Returns (request id, new token, finished) for every request that got a token."""
-        items = self.scheduler.schedule()
-        if not items:
-            return []
-        entries = []
-        for it in items:
-            toks = it.request.tokens[it.start: it.start + it.count]
-            entries.append(StepEntry(it.request.rid, toks, [it.count - 1] if it.samples else []))
-        logits = self.runner.step(entries)
-        self.counters["steps"] += 1
-        self.counters["batched_tokens"] += sum(it.count for it in items)
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None:
+            # This step was queued while the last one's tokens were read.  Rows of requests that ended on those
+            # tokens (or were aborted since) are dropped; their pages are back already.
+            reqs, logits = ahead
+            live = [i for i, r in enumerate(reqs) if r.state != RequestState.FINISHED]
+            if not live:
+                return self.step() if self.has_unfinished() else []
+            items = [ScheduledItem(reqs[i], reqs[i].num_tokens - 1, 1, True) for i in live]
+            if len(live) < len(reqs):
+                logits = logits[torch.tensor(live, dtype=torch.long, device=self.device)]
+        else:
+            items = self.scheduler.schedule()
+            if not items:
+                return []
+            entries = []
+            for it in items:
+                toks = it.request.tokens[it.start: it.start + it.count]
+                entries.append(StepEntry(it.request.rid, toks, [it.count - 1] if it.samples else []))
+            logits = self.runner.step(entries)
+            self.counters["steps"] += 1
+            self.counters["batched_tokens"] += sum(it.count for it in items)
         for it in items:
             self.scheduler.advance(it)
         sampling = [it.request for it in items if it.samples]
@@ -119,7 +139,8 @@ class Engine:
             wanted = [r.logprobs_top_n for r in sampling if r.logprobs_top_n is not None]
             tokens = self.sampler.sample(
                 logits, [r.params for r in sampling], [len(r.output) for r in sampling],
-                [r.prompt for r in sampling], [r.output for r in sampling], top_n=max(wanted) if wanted else None)
+                [r.prompt for r in sampling], [r.output for r in sampling], top_n=max(wanted) if wanted else None,
+                meanwhile=self._queue_next(items) if not wanted else None)
             if wanted:
                 tokens, records = tokens
                 for req, rec in zip(sampling, records):
@@ -133,6 +154,34 @@ class Engine:
                     self.scheduler.finish(req)
                 out.append((req.rid, int(tok), done))
         return out
+
+    def _queue_next(self, items) -> Optional[Callable]:
+        """What to do between the launch of the sampling kernels and the wait for their tokens: when this was a
+        step of single tokens and nobody waits, the next step will bring one token for the same requests, less
+        those that reach their length now, so it is queued at once with the tokens still on the device (a
+        request that ends on its token leaves a row computed for nothing).  None when that does not apply."""
+        if not self.chain_steps or self.scheduler.waiting or not all(it.count == 1 and it.samples for it in items):
+            return None
+        limit = self.scheduler.config.max_model_len
+        keep = [i for i, it in enumerate(items)
+                if len(it.request.output) + 1 < it.request.params.max_new_tokens and it.request.num_tokens + 1 < limit]
+        if not keep:
+            return None
+        reqs = [items[i].request for i in keep]
+
+        def queue(chosen: torch.Tensor) -> None:
+            rids = [r.rid for r in reqs]
+            toks = chosen if len(keep) == len(items) else chosen[torch.tensor(keep, dtype=torch.long, device=self.device)]
+            try:
+                logits = self.runner.step_chained(rids, toks.to(torch.int32))
+            except PagesExhausted:
+                return              # the scheduler decides who gives way, in the next call
+            self.counters["steps"] += 1
+            self.counters["chained_steps"] += 1
+            self.counters["batched_tokens"] += len(rids)
+            self._ahead = (reqs, logits)
+            self.runner.prepare_decode(rids)
+        return queue
 
     def generate(self, prompts: Sequence[Sequence[int]], params: Union[SamplingParams, Sequence[SamplingParams], None] = None
                  ) -> List[List[int]]:

@@ -86,11 +86,17 @@ class _DecodeGraph:
         self.sizes = [rows, rows, rows, rows] + [rows * self.width] * n_groups + [rows] * n_groups
         self.offs = np.cumsum([0] + self.sizes)
         total = int(self.offs[-1])
-        self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
-        self.host_np = self.host.numpy()
+        # two pinned buffers taken in turn (the next step may be staged while the last copy is still queued),
+        # and a small one for the tokens alone
+        self.hosts = [torch.empty(total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.host_nps = [h.numpy() for h in self.hosts]
+        self.copied = [torch.cuda.Event() for _ in range(2)]
+        self.turn = 0
+        self.tok_host = torch.empty(rows, dtype=torch.int32, pin_memory=True)
+        self.tok_np = self.tok_host.numpy()
+        self.tok_copied = torch.cuda.Event()
         self.packed = torch.zeros(total, dtype=torch.int32, device=runner.device)
         self.fixed = torch.arange(rows + 1, dtype=torch.int32, device=runner.device)
-        self.copied = torch.cuda.Event()
         self.graph = None
         self.logits = None
 
@@ -144,6 +150,8 @@ class ModelRunner:
         self.use_graph = bool(use_graph) and self.device.type == "cuda" and not model.state_specs and \
             all(getattr(p, "graph_safe", False) for layer in model.layers for p in layer.parts())
         self.graph_steps = 0
+        self._prepared = None          # (request ids, graph) of a decode step staged ahead by prepare_decode
+        self.staged_steps = 0          # decode steps that found their inputs staged
         self._graphs: Dict[tuple, _DecodeGraph] = {}
         self._graph_pool = None
 
@@ -152,9 +160,11 @@ class ModelRunner:
         return self.cache.has(rid)
 
     def add_request(self, rid) -> None:
+        self._prepared = None
         self.cache.add(rid)
 
     def end_request(self, rid) -> None:
+        self._prepared = None
         self.cache.release(rid)
 
     def num_cached(self, rid) -> int:
@@ -256,17 +266,58 @@ class ModelRunner:
             self._graphs[key] = g
         return g
 
-    def _fill_graph_inputs(self, g: _DecodeGraph, entries: Sequence[StepEntry]) -> None:
-        g.copied.synchronize()                     # the last copy out of the pinned buffer has finished
-        self.cache.fill_decode([e.rid for e in entries], [e.tokens[0] for e in entries], g.rows, g.width,
-                               [self.pools.scratch_page(gi) for gi in range(len(self.cache.groups))], g.host_np)
-        g.packed.copy_(g.host, non_blocking=True)
-        g.copied.record()
+    def _fill_graph_inputs(self, g: _DecodeGraph, rids: Sequence, tokens: Sequence[int]) -> None:
+        i = g.turn
+        g.turn ^= 1
+        g.copied[i].synchronize()                  # the last copy out of this pinned buffer has finished
+        self.cache.fill_decode(rids, tokens, g.rows, g.width,
+                               [self.pools.scratch_page(gi) for gi in range(len(self.cache.groups))], g.host_nps[i])
+        g.packed.copy_(g.hosts[i], non_blocking=True)
+        g.copied[i].record()
 
-    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        ctx_len = self.cache.max_num_tokens([e.rid for e in entries]) + 1
-        g = self._graph_for(len(entries), ctx_len)
-        self._fill_graph_inputs(g, entries)
+    def prepare_decode(self, rids: Sequence) -> bool:
+        """A hint that changes no result: the next step will most likely bring one token for each of these
+        requests, in this order.  Pages are reserved and everything of that step but its tokens (positions,
+        lengths, tables, cache rows) is staged and sent now, while the GPU is still busy with the step before;
+        when the step comes and is what was announced, only its tokens follow.  Anything else in between
+        (another step, a request added or ended) drops the staging.  False when nothing was staged."""
+        self._prepared = None
+        rids = list(rids)
+        if not self.use_graph or not rids or len(set(rids)) != len(rids) or not all(self.cache.has(r) for r in rids):
+            return False
+        ctx_len = self.cache.max_num_tokens(rids) + 1
+        if ctx_len > self.model.spec.max_positions:
+            return False
+        try:
+            self.cache.reserve_many(rids, [1] * len(rids))
+        except PagesExhausted:
+            return False
+        g = self._graph_for(len(rids), ctx_len)
+        if g.graph is None:
+            return False
+        self._fill_graph_inputs(g, rids, [0] * len(rids))
+        self._prepared = (tuple(rids), g)
+        return True
+
+    def _graph_step(self, rids: Sequence, tokens, want_rows: Optional[Sequence[int]] = None) -> torch.Tensor:
+        """``tokens``: a list of ints, or an int32 device tensor [len(rids)] (tokens the host has not seen yet)."""
+        on_device = torch.is_tensor(tokens)
+        n = len(rids)
+        prepared, self._prepared = self._prepared, None
+        if prepared is not None and prepared[0] == tuple(rids):
+            g = prepared[1]                         # staged already: only the tokens are new
+            self.staged_steps += 1
+            if not on_device:
+                g.tok_copied.synchronize()
+                g.tok_np[:n] = tokens
+                g.packed[:n].copy_(g.tok_host[:n], non_blocking=True)
+                g.tok_copied.record()
+        else:
+            ctx_len = self.cache.max_num_tokens(rids) + 1
+            g = self._graph_for(n, ctx_len)
+            self._fill_graph_inputs(g, rids, [0] * n if on_device else tokens)
+        if on_device:
+            g.packed[:n].copy_(tokens)
         if g.graph is None:
             ctx = g.context(self)
             tok = g.view(0)
@@ -281,10 +332,35 @@ class ModelRunner:
             g.graph = graph
         g.graph.replay()
         self.graph_steps += 1
-        rows = [r for r, e in enumerate(entries) if len(e.want) > 0]
-        if len(rows) == len(entries):
-            return g.logits[: len(entries)]
-        return g.logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows else g.logits[:0]
+        if want_rows is None or len(want_rows) == n:
+            return g.logits[:n]
+        return g.logits[torch.tensor(want_rows, dtype=torch.long, device=self.device)] if want_rows else g.logits[:0]
+
+    def step_chained(self, rids: Sequence, tokens: torch.Tensor) -> torch.Tensor:
+        """A step of one token per request whose tokens are still on the device: ``tokens`` int32 [len(rids)],
+        for instance what the sampling kernel chose after the step before, which the host has not read yet.
+        The step is queued behind that kernel at once, so the GPU goes from one step to the next without
+        waiting for the host.  The tokens must be valid ids (they are not checked here); every request must be
+        live; needs the graph path.  Returns the logits of every row (a view of the graph's output buffer)."""
+        rids = list(rids)
+        if not self.use_graph:
+            raise ValueError("step_chained needs use_graph")
+        if not rids or len(set(rids)) != len(rids):
+            raise ValueError("step_chained: one entry per request, at least one")
+        if not (torch.is_tensor(tokens) and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.numel() == len(rids)
+                and tokens.device.type == torch.device(self.device).type):
+            raise ValueError("step_chained: tokens must be an int32 device tensor with one id per request")
+        for rid in rids:
+            if not self.cache.has(rid):
+                raise ValueError(f"request {rid!r} is not live; add_request first")
+            if self.cache.num_tokens(rid) + 1 > self.model.spec.max_positions:
+                raise ValueError(f"request {rid!r}: one more token exceeds max positions {self.model.spec.max_positions}")
+        self.cache.reserve_many(rids, [1] * len(rids))
+        logits = self._graph_step(rids, tokens)
+        self.cache.commit_many(rids, [1] * len(rids))
+        self.steps_run += 1
+        self.tokens_run += len(rids)
+        return logits
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the batch; returns float32 logits [sum of wanted places, vocab] on the device,
@@ -294,11 +370,13 @@ class ModelRunner:
         self._check_entries(entries)
         self.reserve(entries)
         if self.use_graph and all(len(e.tokens) == 1 for e in entries):
-            logits = self._graph_step(entries)
+            logits = self._graph_step([e.rid for e in entries], [e.tokens[0] for e in entries],
+                                      [r for r, e in enumerate(entries) if len(e.want) > 0])
             self.cache.commit_many([e.rid for e in entries], [1] * len(entries))
             self.steps_run += 1
             self.tokens_run += len(entries)
             return logits
+        self._prepared = None
         tok_dev, ctx, starts = self.build_context(entries)
         # A request that starts at position 0 gets a cleared state (also after a recompute).
         if self.pools.state:

@@ -602,6 +602,33 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
+class HostCopy:
+    """A small device tensor on its way to the host: the copy into pinned memory is queued when the object is
+    made, ``result()`` waits for that copy alone (not for work queued behind it) and returns a list.  The pinned
+    buffers are taken in turn from a ring, so at most ``RING`` copies may be outstanding."""
+    RING = 8
+    _ring: list = []
+    _next = 0
+
+    def __init__(self, t: torch.Tensor):
+        cls = HostCopy
+        n = t.numel()
+        if not cls._ring:
+            cls._ring = [None] * cls.RING
+        slot = cls._ring[cls._next]
+        if slot is None or slot[0].numel() < n or slot[0].dtype != t.dtype:
+            slot = (torch.empty(max(n, 256), dtype=t.dtype, pin_memory=True), torch.cuda.Event())
+            cls._ring[cls._next] = slot
+        cls._next = (cls._next + 1) % cls.RING
+        self._buf, self._event, self._n = slot[0], slot[1], n
+        self._buf[:n].copy_(t.reshape(-1), non_blocking=True)
+        self._event.record()
+
+    def result(self) -> list:
+        self._event.synchronize()
+        return self._buf[: self._n].tolist()
+
+
 def _dev_array(values, dtype, device) -> torch.Tensor:
     import numpy as np
     return torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=dtype))).to(device)

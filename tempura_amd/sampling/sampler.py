@@ -53,18 +53,26 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], draw_index: Sequence[int],
                prompt_tokens: Sequence[Sequence[int]], output_tokens: Sequence[Sequence[int]],
-               top_n: Optional[int] = None):
+               top_n: Optional[int] = None, meanwhile=None):
         """``logits`` float32 [m, vocab] on the device; one ``SamplingParams`` per row;
         ``draw_index[i]`` is how many tokens row i's request has drawn before; the token
         lists feed the penalties.  Returns the chosen token of each row.
         With ``top_n`` (0..20) it returns (tokens, records) instead, a record per row being
         ``TokenLogprob(token_id, logprob, top_logprobs)``: log-probabilities of the distribution the token was
-        drawn from, after temperature and filters (/root/reference/engine/src/model.rs:497-526)."""
+        drawn from, after temperature and filters (/root/reference/engine/src/model.rs:497-526).
+        ``meanwhile``: called with the chosen tokens (int32 on the device) once the kernels are launched and
+        before the tokens are waited for: host work that can run while the GPU does, such as queueing the
+        next step behind them."""
         m = logits.shape[0]
         if m == 0:
             return [] if top_n is None else ([], [])
         if top_n is None and all(p.is_greedy for p in params):
-            return ops.argmax(logits).tolist()
+            chosen = ops.argmax(logits)
+            if meanwhile is None:
+                return chosen.tolist()
+            coming = ops.HostCopy(chosen)          # (queued before whatever `meanwhile` queues)
+            meanwhile(chosen)
+            return coming.result()
         if any(p.has_penalties for p in params):
             logits = self._penalised(logits, params, prompt_tokens, output_tokens)
         temp = np.asarray([p.temperature for p in params], dtype=np.float32)
@@ -77,7 +85,12 @@ class Sampler:
         if self._work is None or self._work.shape[0] < m:
             self._work = torch.empty((max(m, 8), self.vocab_size), dtype=torch.float32, device=self.device)
         if top_n is None:
-            return ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd, typical_p).tolist()
+            chosen = ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd, typical_p)
+            if meanwhile is None:
+                return chosen.tolist()
+            coming = ops.HostCopy(chosen)
+            meanwhile(chosen)
+            return coming.result()
         top_n = max(0, min(int(top_n), 20, self.vocab_size))
         info = torch.empty((m, 4), dtype=torch.float32, device=logits.device)
         tokens = ops.sample(logits, self._work, temp, top_k, top_p, min_p, rnd, typical_p, info).tolist()

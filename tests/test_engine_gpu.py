@@ -152,6 +152,50 @@ def test_eos_and_length_limits(tiny_dirs):
     assert out == ref
 
 
+def test_steps_queued_ahead_change_nothing(tiny_dirs):
+    """While all requests decode, the engine queues the next step before it has read this step's tokens.  The
+    tokens and the final state are those of an engine that does not: with requests
+    of different lengths, one that ends on an EOS token (its row in the step already queued is dropped), seeded
+    temperature sampling with penalties, a request added and one aborted on the way."""
+    from tempura_amd.sampling import SamplingParams
+    cfg, W = tiny_dirs.plain_model("A")
+    prompts = [helpers.random_tokens(256, n, seed=700 + n) for n in (9, 30, 4, 17)]
+    ref = [plain.greedy_generate(cfg, W, p, 24) for p in prompts]
+    eos = ref[1][9]                                           # request 1 stops early
+    params = [SamplingParams(temperature=0.0, max_new_tokens=24),
+              SamplingParams(temperature=0.0, max_new_tokens=24, eos_token_id=[eos]),
+              SamplingParams(temperature=0.0, max_new_tokens=7),
+              SamplingParams(temperature=0.9, top_k=20, seed=5, repeat_penalty=1.2, presence_penalty=0.3, max_new_tokens=24)]
+
+    def run(chain):
+        eng = _engine(tiny_dirs, "A", chain_steps=chain)
+        rids = [eng.add_request(p, sp) for p, sp in zip(prompts, params)]
+        events, calls = [], 0
+        while eng.has_unfinished():
+            events.append(eng.step())
+            calls += 1
+            if calls == 12:
+                rids.append(eng.add_request(prompts[0][:5], SamplingParams(temperature=0.0, max_new_tokens=6)))
+            if calls == 20:
+                eng.abort(rids[0])
+        outs = [list(eng.request(r).output) for r in rids]
+        assert eng.runner.cache.free_pages() == [64]
+        return outs, events, eng.stats()
+
+    outs0, events0, st0 = run(False)
+    outs1, events1, st1 = run(True)
+    assert st0["chained_steps"] == 0 and st1["chained_steps"] > 10
+    assert outs1 == outs0
+    for outs, events in ((outs0, events0), (outs1, events1)):      # every token was reported once, in order
+        seen = {}
+        for call in events:
+            for rid, tok, _done in call:
+                seen.setdefault(rid, []).append(tok)
+        assert [seen.get(i, []) for i in range(len(outs))] == outs
+    assert outs1[1] == ref[1][: ref[1].index(eos) + 1] and outs1[2] == ref[2][:7]
+    assert st1["generated_tokens"] == st0["generated_tokens"]
+
+
 def test_command_line(tiny_dirs, tmp_path):
     cfg, W = tiny_dirs.plain_model("A")
     model = tiny_dirs.path("A", "float32")

@@ -83,6 +83,39 @@ def test_graph_replays_match_eager(tiny_dirs, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_staged_ahead_change_nothing(tiny_dirs, dtype):
+    """``prepare_decode`` is a hint: steps that find their inputs staged give the bits of steps that do not, and a
+    hint that does not come true (other requests, another order, a request ended in between) is dropped."""
+    from tempura_amd.engine.runner import StepEntry
+    name = "D"
+    reqs = {rid: toks for rid, toks in list(helpers.requests_for(name).items())[1:4]}
+
+    def run(hints):
+        runner = _runner(tiny_dirs, name, dtype, 1024, helpers.PAGE_SIZE[name], use_graph=True)
+        for rid, toks in reqs.items():
+            runner.add_request(rid)
+            runner.step([StepEntry(rid, toks[:5], [])])
+        live, out = list(reqs), []
+        for i in range(5, 30):
+            if i == 20:                                    # a request ends between a hint and its step
+                runner.end_request(live.pop(1))
+            out.append(runner.step([StepEntry(rid, [reqs[rid][i]], [0]) for rid in live]).clone())
+            hint = hints(i, live)
+            if hint is not None:
+                runner.prepare_decode(hint)
+        return out, runner
+
+    plain_out, r0 = run(lambda i, live: None)
+    staged_out, r1 = run(lambda i, live: list(live))
+    wrong_out, r2 = run(lambda i, live: list(reversed(live)) if i % 2 else live[:1])
+    assert r0.staged_steps == 0 and r1.staged_steps >= 22 and r2.staged_steps == 0
+    for a, b, c in zip(plain_out, staged_out, wrong_out):
+        assert torch.equal(a, b) and torch.equal(a, c)
+    for r in (r0, r1, r2):
+        r.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(tiny_dirs, dtype):
     """700 tokens decoded one by one after a short prompt (config A, 44 pages of 16)."""
     cfg, W = tiny_dirs.plain_model("A", dtype)
