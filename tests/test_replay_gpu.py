@@ -85,12 +85,13 @@ def test_graph_replays_match_eager(tiny_dirs, name, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_steps_staged_ahead_change_nothing(tiny_dirs, dtype):
     """``prepare_decode`` is a hint: steps that find their inputs staged give the bits of steps that do not, and a
-    hint that does not come true (other requests, another order, a request ended in between) is dropped."""
+    hint that does not come true (other requests, another order, a request ended in between) is dropped.
+    ``step_chained`` (tokens from device memory) gives the same bits again, staged or not."""
     from tempura_amd.engine.runner import StepEntry
     name = "D"
     reqs = {rid: toks for rid, toks in list(helpers.requests_for(name).items())[1:4]}
 
-    def run(hints):
+    def run(hints, on_device=False):
         runner = _runner(tiny_dirs, name, dtype, 1024, helpers.PAGE_SIZE[name], use_graph=True)
         for rid, toks in reqs.items():
             runner.add_request(rid)
@@ -99,7 +100,11 @@ def test_decode_steps_staged_ahead_change_nothing(tiny_dirs, dtype):
         for i in range(5, 30):
             if i == 20:                                    # a request ends between a hint and its step
                 runner.end_request(live.pop(1))
-            out.append(runner.step([StepEntry(rid, [reqs[rid][i]], [0]) for rid in live]).clone())
+            if on_device:                                  # the tokens come from device memory
+                toks = torch.tensor([reqs[rid][i] for rid in live], dtype=torch.int32, device="cuda:0")
+                out.append(runner.step_chained(live, toks).clone())
+            else:
+                out.append(runner.step([StepEntry(rid, [reqs[rid][i]], [0]) for rid in live]).clone())
             hint = hints(i, live)
             if hint is not None:
                 runner.prepare_decode(hint)
@@ -108,10 +113,12 @@ def test_decode_steps_staged_ahead_change_nothing(tiny_dirs, dtype):
     plain_out, r0 = run(lambda i, live: None)
     staged_out, r1 = run(lambda i, live: list(live))
     wrong_out, r2 = run(lambda i, live: list(reversed(live)) if i % 2 else live[:1])
-    assert r0.staged_steps == 0 and r1.staged_steps >= 22 and r2.staged_steps == 0
-    for a, b, c in zip(plain_out, staged_out, wrong_out):
-        assert torch.equal(a, b) and torch.equal(a, c)
-    for r in (r0, r1, r2):
+    chained_out, r3 = run(lambda i, live: list(live), on_device=True)
+    chained_cold, r4 = run(lambda i, live: None, on_device=True)
+    assert r0.staged_steps == 0 and r1.staged_steps >= 22 and r2.staged_steps == 0 and r3.staged_steps >= 22
+    for a, b, c, d, e in zip(plain_out, staged_out, wrong_out, chained_out, chained_cold):
+        assert torch.equal(a, b) and torch.equal(a, c) and torch.equal(a, d) and torch.equal(a, e)
+    for r in (r0, r1, r2, r3, r4):
         r.cache.check()
 
 
