@@ -31,6 +31,8 @@ def _add_engine_args(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048, help="token budget of one step")
     ap.add_argument("--prefill-chunk-size", type=int, default=512, help="largest prompt portion in one step")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps as a HIP graph")
+    ap.add_argument("--no-chain-steps", action="store_true",
+                    help="wait for a step's tokens on the host before queueing the next decode step")
 
 
 def _engine_from_args(args):
@@ -53,7 +55,8 @@ def _engine_from_args(args):
                   page_size=args.block_size, kv_pages=args.kv_blocks,
                   gpu_memory_utilization=args.gpu_memory_utilization, max_batch_size=args.max_batch_size,
                   max_seq_len=args.max_seq_len, max_num_batched_tokens=args.max_num_batched_tokens,
-                  prefill_chunk_size=args.prefill_chunk_size, use_graph=not args.no_graph)
+                  prefill_chunk_size=args.prefill_chunk_size, use_graph=not args.no_graph,
+                  chain_steps=not args.no_chain_steps)
 
 
 def _prompts_from_args(args, vocab: int):
