@@ -170,12 +170,30 @@ def main(argv=None) -> int:
 
     p = sub.add_parser("replay", help="trace replay (same as bin/trace_run)", add_help=False)
     p.set_defaults(fn=None)
+    p = sub.add_parser("bench", help="decode and prefill throughput of a named size (bench.py of the checkout)", add_help=False)
+    p.set_defaults(fn=None)
 
     if argv is None:
         argv = sys.argv[1:]
     if argv and argv[0] == "replay":
         from .replay import main as replay_main
         return replay_main(argv[1:])
+    if argv and argv[0] == "bench":
+        # bench.py lies beside the package in a checkout (the measuring harness calls it by that path)
+        import os
+        import runpy
+        script = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")
+        if not os.path.isfile(script):
+            raise SystemExit(f"tempura bench: {script} not found (it ships with the source checkout)")
+        rest = list(argv[1:])
+        if rest and not rest[0].startswith("-"):
+            rest = ["--model-config", rest[0]] + rest[1:]       # `tempura bench llama-3.2-3b`
+        sys.argv = [script] + rest
+        try:
+            runpy.run_path(script, run_name="__main__")
+        except SystemExit as e:
+            return int(e.code or 0)
+        return 0
     args = ap.parse_args(argv)
     return args.fn(args)
 
