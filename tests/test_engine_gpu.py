@@ -214,6 +214,40 @@ def test_command_line(tiny_dirs, tmp_path):
     assert '"stats"' in p.stderr
 
 
+def test_model_width_layer_against_plain(tmp_path):
+    """One layer with the widths of Llama-3.1-8B (hidden 4096, 32 heads of 128 in 8 groups, intermediate 14336;
+    a vocabulary of 8,192 keeps the folder at half a gigabyte) against the plain float64 implementation, which
+    shares nothing with the kernels: a prompt of 600 tokens whole, in uneven portions, and with its last 32
+    tokens one by one through the graph, in float32 and in bfloat16 (weights N(0, 0.02), stored as bfloat16)."""
+    from tempura_amd.config import LlamaConfig, RopeScaling
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner, StepEntry
+    from tempura_amd.kernels import ops
+    from tempura_amd.weights import write_random_model
+    ops.set_backend(None)
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=1, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, vocab_size=8192, max_position_embeddings=131072,
+                      rms_norm_eps=1e-5, rope_theta=500000.0, rope_scaling=RopeScaling("llama3", 8.0, 1.0, 4.0, 8192),
+                      tie_word_embeddings=False)
+    folder = str(tmp_path / "wide")
+    write_random_model(cfg, folder, seed=3, std=0.02, dtype="bfloat16")
+    pc, W = plain.read_model_dir(folder)
+    toks = helpers.random_tokens(8192, 600, seed=1)
+    ref = plain.forward(pc, W, toks)
+    cuts = {"whole": [(0, 600)], "portions": [(0, 300), (300, 17), (317, 2), (319, 160), (479, 121)],
+            "tail": [(0, 568)] + [(i, 1) for i in range(568, 600)]}
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 2e-2)):
+        model = load_model(folder, dtype, "cuda:0")
+        for mode, steps in cuts.items():
+            runner = ModelRunner(model, 16, 48, max_requests=2, use_graph=(mode == "tail"))
+            runner.add_request("x")
+            got = torch.cat([runner.step([StepEntry("x", toks[s: s + n], list(range(n)))]).cpu().clone() for s, n in steps])
+            err = helpers.rel_err(got, ref)
+            assert err <= tol, f"{dtype}/{mode}: {err:.3e} from the plain implementation, first at {helpers.first_difference(got, ref, tol)}"
+        del model
+        torch.cuda.empty_cache()
+
+
 def test_model_sized_layers_bfloat16_against_float32():
     """Two layers with the sizes of Llama-3.1-8B (hidden 4096, 32 heads of 128 in 8 groups, intermediate 14336,
     vocabulary 128256) and the same weights in both precisions: the bfloat16 engine (pipelined products of
