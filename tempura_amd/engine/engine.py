@@ -65,7 +65,7 @@ class Engine:
         self._ids = itertools.count()
         self._requests: Dict[Hashable, Request] = {}
         self.counters = {"steps": 0, "prompt_tokens": 0, "generated_tokens": 0, "batched_tokens": 0, "chained_steps": 0}
-        self.chain_steps = bool(chain_steps) and use_graph and self.device.type == "cuda"
+        self.chain_steps = bool(chain_steps) and self.runner.use_graph     # (a model with parts that cannot be captured runs eagerly)
         self._ahead = None      # (requests, logits) of a step that is already queued
 
     def _pages_from_memory(self, utilization: float, max_batch_size: int) -> int:

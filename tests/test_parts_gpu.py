@@ -191,6 +191,18 @@ def test_toy_mixer_with_state_on_the_gpu(tmp_path, dtype):
     for r, t in reqs.items():
         ref = toy_parts.plain_toy_forward(cfg, W, t)
         assert helpers.rel_err(got[r], ref) < helpers.TOL[dtype], r
+    if dtype == "float32":
+        # and through the entry point (which then neither replays graphs nor queues steps ahead)
+        from tempura_amd.engine import Engine
+        from tempura_amd.sampling import SamplingParams
+        eng = Engine(model, dtype=dtype, page_size=8, kv_pages=24, max_batch_size=3)
+        assert not eng.chain_steps
+        outs = eng.generate([reqs["q"], reqs["p"][:5]], SamplingParams(temperature=0.0, max_new_tokens=6))
+        for prompt, out in zip([reqs["q"], reqs["p"][:5]], outs):
+            seq = list(prompt)
+            for tok in out:         # greedy by the plain implementation, token by token
+                assert tok == int(torch.argmax(toy_parts.plain_toy_forward(cfg, W, seq)[-1]))
+                seq.append(tok)
 
 
 def test_toy_routed_ffn_and_learned_position_on_the_gpu(tmp_path):
