@@ -244,6 +244,8 @@ class Engine:
     def forward(self, token_ids: Sequence[int]) -> torch.Tensor:
         """Logits [vocab] (float32, host) after a whole prompt of a fresh request
         (the reference's ``forward``, /root/reference/engine/src/model.rs:308)."""
+        if self._ahead is not None:      # a queued step's logits live in a graph's output buffer: keep a copy
+            self._ahead = (self._ahead[0], self._ahead[1].clone())
         rid = ("forward", next(self._ids))
         self.runner.add_request(rid)
         try:
