@@ -79,6 +79,8 @@ def main() -> int:
     print(f"[bench] model built in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     pages = max_batch * ((args.context + args.page_size - 1) // args.page_size) + 8
     runner = ModelRunner(model, args.page_size, pages, max_requests=max_batch, use_graph=not args.no_graph)
+    if not runner.use_graph:
+        args.no_chain = True          # (a step can only be queued ahead of its tokens where steps replay a graph)
     rng = random.Random(0)
     V = cfg.vocab_size
     elem = 2 if args.dtype == "bfloat16" else 4
@@ -191,7 +193,7 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "global_batch": args.batch, "seq_len": args.context, "prompt_len": args.prompt_len,
             "page_size": args.page_size, "weights": "random N(0,0.02)", "parallelism": "single GPU",
-            "graph": not args.no_graph,
+            "graph": not args.no_graph, "steps_queued_ahead": not args.no_chain,
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
