@@ -84,7 +84,15 @@ def _ptr(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
+
+
 def _stream():
+    """The current stream's handle (of the current device).  Asked for at every launch: the direct call is
+    some 8 us cheaper than ``torch.cuda.current_stream()``, a quarter of an eager launch's host time."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(_raw_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
