@@ -25,7 +25,17 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int vocab, int c
   const int lo = chunk * per, hi = min(vocab, lo + per);
   float bv = -INFINITY;
   int bi = -1;
-  for (int j = lo + threadIdx.x; j < hi; j += blockDim.x) argmax_merge(bv, bi, row[j], j);
+  // four loads in flight per thread (the merge is a pure function of value and index, so the order is free)
+  int j = lo + threadIdx.x;
+  const int bd = blockDim.x;
+  for (; j + 3 * bd < hi; j += 4 * bd) {
+    const float v0 = row[j], v1 = row[j + bd], v2 = row[j + 2 * bd], v3 = row[j + 3 * bd];
+    argmax_merge(bv, bi, v0, j);
+    argmax_merge(bv, bi, v1, j + bd);
+    argmax_merge(bv, bi, v2, j + 2 * bd);
+    argmax_merge(bv, bi, v3, j + 3 * bd);
+  }
+  for (; j < hi; j += bd) argmax_merge(bv, bi, row[j], j);
   for (int o = TP_WAVE / 2; o > 0; o >>= 1) {
     const float ov = __shfl_xor(bv, o, TP_WAVE);
     const int oi = __shfl_xor(bi, o, TP_WAVE);
