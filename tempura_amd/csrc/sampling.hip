@@ -200,17 +200,28 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
       cnt[i] = 0;
     }
     __syncthreads();
-    for (int j = threadIdx.x; j < n; j += blockDim.x) {
-      const float v = x[j];
-      if (float_key(v) < floor_key) continue;
+    auto take = [&](float v) {
+      if (float_key(v) < floor_key) return;
       const unsigned int key = select_key<TYP>(v, maxv, mean_d);
-      if (pass > 0 && (key >> (shift + 8)) != prefix) continue;
+      if (pass > 0 && (key >> (shift + 8)) != prefix) return;
       const unsigned int bin = (key >> shift) & 255u;
       atomicAdd(&cnt[bin], 1u);
       if (MASS)
         atomicAdd(&hist[bin], fix_mass(v, maxv));
       else
         atomicAdd(&hist[bin], 1ull);
+    };
+    {   // four loads in flight per thread (counts and fixed-point masses do not depend on the order)
+      const int bd = blockDim.x;
+      int j = threadIdx.x;
+      for (; j + 3 * bd < n; j += 4 * bd) {
+        const float v0 = x[j], v1 = x[j + bd], v2 = x[j + 2 * bd], v3 = x[j + 3 * bd];
+        take(v0);
+        take(v1);
+        take(v2);
+        take(v3);
+      }
+      for (; j < n; j += bd) take(x[j]);
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -327,12 +338,27 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
 
   // 1. scale by the temperature, find the maximum
   float mx = -INFINITY;
-  for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
-    float v = lg[j];
-    if (T != 1.0f) v = v / T;
-    if (!(v == v)) v = -INFINITY;  // NaN never survives
-    x[j] = v;
-    mx = fmaxf(mx, v);
+  {
+    auto scale = [&](float v) {
+      if (T != 1.0f) v = v / T;
+      if (!(v == v)) v = -INFINITY;  // NaN never survives
+      return v;
+    };
+    const int bd = blockDim.x;
+    int j = threadIdx.x;
+    for (; j + 3 * bd < vocab; j += 4 * bd) {   // four loads in flight per thread
+      const float v0 = scale(lg[j]), v1 = scale(lg[j + bd]), v2 = scale(lg[j + 2 * bd]), v3 = scale(lg[j + 3 * bd]);
+      x[j] = v0;
+      x[j + bd] = v1;
+      x[j + 2 * bd] = v2;
+      x[j + 3 * bd] = v3;
+      mx = fmaxf(fmaxf(mx, v0), fmaxf(v1, fmaxf(v2, v3)));
+    }
+    for (; j < vocab; j += bd) {
+      const float v = scale(lg[j]);
+      x[j] = v;
+      mx = fmaxf(mx, v);
+    }
   }
   const float maxv = block_max(mx, fscratch);
   __syncthreads();
@@ -392,17 +418,25 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     if (K > floor_key) floor_key = K;
   }
 
-  // 4. total mass of the survivors
+  // 4. total mass of the survivors (left to the draw, which sums the same masses wave by wave, when nothing
+  // needs it earlier: no top_p and no report)
+  const float tp = top_p[row];
+  const bool need_mass_now = (tp < 1.0f && tp > 0.f) || inf != nullptr || greedy;
   unsigned long long part = 0;
-  for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
-    const float v = x[j];
-    if (float_key(v) >= floor_key) part += fix_mass(v, maxv);
+  if (need_mass_now) {
+    auto mass = [&](float v) { return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull; };
+    const int bd = blockDim.x;
+    int j = threadIdx.x;
+    for (; j + 3 * bd < vocab; j += 4 * bd) {   // four loads in flight per thread; integer sums, any order
+      const float v0 = x[j], v1 = x[j + bd], v2 = x[j + 2 * bd], v3 = x[j + 3 * bd];
+      part += mass(v0) + mass(v1) + mass(v2) + mass(v3);
+    }
+    for (; j < vocab; j += bd) part += mass(x[j]);
   }
-  unsigned long long Z;
-  block_excl_scan(part, scan, &Z);
+  unsigned long long Z = 0;
+  if (need_mass_now) block_excl_scan(part, scan, &Z);
 
   // 5. top_p: the shortest prefix by descending probability whose mass reaches top_p
-  const float tp = top_p[row];
   if (tp < 1.0f && tp > 0.f) {
     unsigned long long target = (unsigned long long)((double)tp * (double)Z);
     if (target < 1) target = 1;
@@ -441,34 +475,64 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   if (greedy) return;
 
   // 6. draw: first index (index order) whose cumulative mass exceeds r * Z
+  // Every wave owns a contiguous range of the row and sums its mass with coalesced loads; the wave whose range
+  // holds the target then walks it 64 elements at a time with a prefix sum over its lanes.
+  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  const int per_wave = ((vocab + SMP_WAVES - 1) / SMP_WAVES + TP_WAVE - 1) / TP_WAVE * TP_WAVE;
+  const int wlo = min(vocab, wave * per_wave), whi = min(vocab, wlo + per_wave);
+  auto mass = [&](int j) {
+    if (j >= whi) return 0ull;
+    const float v = x[j];
+    return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull;
+  };
+  unsigned long long mine = 0;
+  for (int j = wlo + lane; j < whi; j += 4 * TP_WAVE)
+    mine += mass(j) + mass(j + TP_WAVE) + mass(j + 2 * TP_WAVE) + mass(j + 3 * TP_WAVE);
+#pragma unroll
+  for (int o = TP_WAVE / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, TP_WAVE);
+  __syncthreads();
+  if (lane == 0) scan[wave] = mine;
+  __syncthreads();
+  unsigned long long total = 0;
+  for (int i = 0; i < SMP_WAVES; ++i) total += scan[i];
+  if (!need_mass_now) Z = total;
+  if (total == 0 || Z == 0) {       // nothing left to draw from: the last index
+    if (threadIdx.x == 0) out[row] = vocab - 1;
+    return;
+  }
   const float r = rnd[row];
   unsigned long long t = (unsigned long long)((double)r * (double)Z);
   if (t >= Z) t = Z - 1;
-  const int per = (vocab + SMP_THREADS - 1) / SMP_THREADS;
-  const int lo = min(vocab, (int)threadIdx.x * per), hi = min(vocab, lo + per);
-  unsigned long long mine = 0;
-  for (int j = lo; j < hi; ++j) {
-    const float v = x[j];
-    if (float_key(v) >= floor_key) mine += fix_mass(v, maxv);
-  }
-  unsigned long long total;
-  unsigned long long base = block_excl_scan(mine, scan, &total);
-  if (threadIdx.x == 0 && total == 0) out[row] = vocab - 1;
-  if (mine > 0 && base <= t && t < base + mine) {
-    unsigned long long c = base;
-    int pick = hi - 1;
-    for (int j = lo; j < hi; ++j) {
-      const float v = x[j];
-      if (float_key(v) >= floor_key) {
-        c += fix_mass(v, maxv);
-        if (c > t) {
-          pick = j;
-          break;
-        }
-      }
+  unsigned long long base = 0, before = 0;
+  int chosen_wave = -1;
+  for (int i = 0; i < SMP_WAVES; ++i) {
+    const unsigned long long w = scan[i];
+    if (chosen_wave < 0 && t < before + w) {
+      chosen_wave = i;
+      base = before;
     }
-    out[row] = pick;
-    if (inf != nullptr) inf[3] = (x[pick] - maxv) - lnZ;
+    before += w;
+  }
+  if (wave == chosen_wave) {
+    unsigned long long c = base;
+    for (int j0 = wlo; j0 < whi; j0 += TP_WAVE) {
+      const unsigned long long q = mass(j0 + lane);
+      unsigned long long inc = q;
+#pragma unroll
+      for (int o = 1; o < TP_WAVE; o <<= 1) {
+        const unsigned long long up = __shfl_up(inc, o, TP_WAVE);
+        if (lane >= o) inc += up;
+      }
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(q > 0 && c + inc > t);
+      if (hit != 0) {   // (the first lane whose running mass passes the target: index order)
+        if (lane == (int)__builtin_ctzll(hit)) {
+          out[row] = j0 + lane;
+          if (inf != nullptr) inf[3] = (x[j0 + lane] - maxv) - lnZ;
+        }
+        break;
+      }
+      c += __shfl(inc, TP_WAVE - 1, TP_WAVE);
+    }
   }
 }
 
