@@ -637,9 +637,42 @@ class HostCopy:
         return self._buf[: self._n].tolist()
 
 
-def _dev_array(values, dtype, device) -> torch.Tensor:
-    import numpy as np
-    return torch.from_numpy(np.ascontiguousarray(np.asarray(values, dtype=dtype))).to(device)
+class _Staging:
+    """Small per-call option arrays on their way to the device through pinned memory: the copy is queued behind
+    the work in flight instead of making the host wait for it (a pageable copy would).  Buffers are taken in
+    turn from a ring and reused once their copy has run."""
+    RING = 8
+    _ring: list = []
+    _next = 0
+
+    @classmethod
+    def send(cls, arrays, device) -> list:
+        """``arrays``: numpy arrays of 4-byte elements, each [rows..]; returns device tensors of the same shapes
+        and dtypes (views of one packed transfer)."""
+        import numpy as np
+        total = sum(a.size for a in arrays)
+        if not cls._ring:
+            cls._ring = [None] * cls.RING
+        slot = cls._ring[cls._next]
+        if slot is None or slot[0].numel() < total:
+            slot = (torch.empty(max(total, 1024), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+            cls._ring[cls._next] = slot
+        cls._next = (cls._next + 1) % cls.RING
+        host, event = slot
+        event.synchronize()                       # the copy that last used this buffer has run
+        flat = host.numpy()
+        views, off = [], 0
+        for a in arrays:
+            flat[off: off + a.size] = np.ascontiguousarray(a).reshape(-1).view(np.int32)
+            off += a.size
+        dev = host[:total].to(device, non_blocking=True)
+        event.record()
+        off = 0
+        for a in arrays:
+            t = dev[off: off + a.size]
+            views.append((t.view(torch.float32) if a.dtype == np.float32 else t).view(a.shape))
+            off += a.size
+        return views
 
 
 def apply_penalties(logits: torch.Tensor, rows, tokens, counts, in_window, presence, frequency, repeat) -> None:
@@ -656,8 +689,8 @@ def apply_penalties(logits: torch.Tensor, rows, tokens, counts, in_window, prese
     _need(len(presence) == m and len(frequency) == m and len(repeat) == m, "apply_penalties: one penalty per row")
     _need(all(0 <= r < m for r in rows), "apply_penalties: row out of range")
     dev = logits.device
-    ints = _dev_array([rows, tokens, counts, in_window], np.int32, dev)
-    fl = _dev_array([presence, frequency, repeat], np.float32, dev)
+    ints, fl = _Staging.send([np.asarray([rows, tokens, counts, in_window], dtype=np.int32),
+                              np.asarray([presence, frequency, repeat], dtype=np.float32)], dev)
     _call("tp_apply_penalties", _ptr(logits), vocab, _ptr(ints[0]), _ptr(ints[1]), _ptr(ints[2]), _ptr(ints[3]),
           _ptr(fl[0]), _ptr(fl[1]), _ptr(fl[2]), n, _stream())
 
@@ -682,8 +715,8 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
     for a in (temperature, top_k, top_p, min_p, rnd, typical_p):
         _need(len(a) == m, "sample: one option per row")
     dev = logits.device
-    fl = _dev_array([temperature, top_p, min_p, rnd, typical_p], np.float32, dev)
-    tk = _dev_array(top_k, np.int32, dev)
+    fl, tk = _Staging.send([np.asarray([temperature, top_p, min_p, rnd, typical_p], dtype=np.float32),
+                            np.asarray(top_k, dtype=np.int32)], dev)
     out = torch.empty((m,), dtype=torch.int32, device=dev)
     if info is not None:
         _dev_ok(info)
