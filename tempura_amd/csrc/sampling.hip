@@ -185,13 +185,18 @@ __device__ inline unsigned int select_key(float v, float maxv, float mean_d) {
 // weight(key >= K), where an element's weight is 1 (MASS = false) or its fixed-point mass.
 // Only elements whose VALUE key is >= floor_key take part.  Returns K; *gt = weight(key > K),
 // *eq_count = number of elements with key == K.
+// After the first pass the elements of the chosen bin are copied to `cand` (LDS, SMP_CAND entries) when they fit,
+// and the other three passes run over those few instead of the whole row: the k-th largest of 128,256 logits
+// shares its first byte (sign and seven exponent bits) with a few thousand others at most.
+#define SMP_CAND 4096
 template <bool MASS, bool TYP = false>
 __device__ unsigned int radix_select(const float* __restrict__ x, int n, float maxv, unsigned int floor_key,
                                      unsigned long long target, unsigned long long* hist /*256*/,
-                                     unsigned int* cnt /*256*/, unsigned long long* sh /*4*/,
+                                     unsigned int* cnt /*256*/, unsigned long long* sh /*4*/, float* cand /*SMP_CAND*/,
                                      unsigned long long* gt_out, unsigned int* eq_count, float mean_d = 0.f) {
   unsigned int prefix = 0;
   unsigned long long gt = 0;
+  int n_cand = -1;          // >= 0: the passes run over cand[0 .. n_cand)
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 24 - 8 * pass;
     __syncthreads();
@@ -206,12 +211,11 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
       if (pass > 0 && (key >> (shift + 8)) != prefix) return;
       const unsigned int bin = (key >> shift) & 255u;
       atomicAdd(&cnt[bin], 1u);
-      if (MASS)
-        atomicAdd(&hist[bin], fix_mass(v, maxv));
-      else
-        atomicAdd(&hist[bin], 1ull);
+      if (MASS) atomicAdd(&hist[bin], fix_mass(v, maxv));   // (counting: the weight of a bin is its count)
     };
-    {   // four loads in flight per thread (counts and fixed-point masses do not depend on the order)
+    if (n_cand >= 0) {
+      for (int j = threadIdx.x; j < n_cand; j += blockDim.x) take(cand[j]);
+    } else {   // four loads in flight per thread (counts and fixed-point masses do not depend on the order)
       const int bd = blockDim.x;
       int j = threadIdx.x;
       for (; j + 3 * bd < n; j += 4 * bd) {
@@ -228,16 +232,40 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
       unsigned long long run = gt;
       int b = 255;
       for (; b > 0; --b) {
-        if (run + hist[b] >= target) break;
-        run += hist[b];
+        const unsigned long long w = MASS ? hist[b] : (unsigned long long)cnt[b];
+        if (run + w >= target) break;
+        run += w;
       }
       sh[0] = run;
       sh[1] = (unsigned long long)b;
       sh[2] = (unsigned long long)cnt[b];
+      sh[3] = 0;            // (the candidates' counter)
     }
     __syncthreads();
     gt = sh[0];
     prefix = (prefix << 8) | (unsigned int)sh[1];
+    if (pass == 0 && sh[2] <= (unsigned long long)SMP_CAND) {
+      // gather the chosen bin's elements (their order does not matter: counts and integer masses)
+      const unsigned int want = prefix;
+      auto gather = [&](float v) {
+        if (float_key(v) < floor_key) return;
+        if ((select_key<TYP>(v, maxv, mean_d) >> 24) != want) return;
+        const unsigned long long at = atomicAdd(&sh[3], 1ull);
+        if (at < (unsigned long long)SMP_CAND) cand[at] = v;
+      };
+      const int bd = blockDim.x;
+      int j = threadIdx.x;
+      for (; j + 3 * bd < n; j += 4 * bd) {
+        const float v0 = x[j], v1 = x[j + bd], v2 = x[j + 2 * bd], v3 = x[j + 3 * bd];
+        gather(v0);
+        gather(v1);
+        gather(v2);
+        gather(v3);
+      }
+      for (; j < n; j += bd) gather(x[j]);
+      __syncthreads();
+      n_cand = (int)sh[3];   // (== sh[2], the bin's count)
+    }
   }
   *gt_out = gt;
   *eq_count = (unsigned int)sh[2];
@@ -300,6 +328,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   __shared__ unsigned long long hist[256];
   __shared__ unsigned int cnt[256];
   __shared__ unsigned long long sh[4];
+  __shared__ float cand[SMP_CAND];
   __shared__ unsigned long long scan[SMP_WAVES];
   __shared__ float fscratch[32];
   __shared__ int ibest[SMP_WAVES];
@@ -403,7 +432,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     if (target > Z0) target = Z0;
     unsigned long long gt;
     unsigned int eq;
-    const unsigned int K = radix_select<true, true>(x, vocab, maxv, floor_key, target, hist, cnt, sh, &gt, &eq, mean_d);
+    const unsigned int K = radix_select<true, true>(x, vocab, maxv, floor_key, target, hist, cnt, sh, cand, &gt, &eq, mean_d);
     typical_cut(x, vocab, maxv, floor_key, mean_d, K, target - gt, scan);
   }
 
@@ -412,7 +441,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   if (k > 0 && k < vocab) {
     unsigned long long gt;
     unsigned int eq;
-    const unsigned int K = radix_select<false>(x, vocab, maxv, floor_key, (unsigned long long)k, hist, cnt, sh, &gt, &eq);
+    const unsigned int K = radix_select<false>(x, vocab, maxv, floor_key, (unsigned long long)k, hist, cnt, sh, cand, &gt, &eq);
     // fewer than k survivors: K lands on the smallest surviving bin and nothing is cut
     if (gt + eq > (unsigned long long)k) drop_surplus_ties(x, vocab, K, (unsigned long long)k - gt, scan);
     if (K > floor_key) floor_key = K;
@@ -442,7 +471,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     if (target < 1) target = 1;
     unsigned long long gt;
     unsigned int eq;
-    const unsigned int K = radix_select<true>(x, vocab, maxv, floor_key, target, hist, cnt, sh, &gt, &eq);
+    const unsigned int K = radix_select<true>(x, vocab, maxv, floor_key, target, hist, cnt, sh, cand, &gt, &eq);
     // each tie at K has the same mass q; take as many as the target still needs
     float kv;
     {
