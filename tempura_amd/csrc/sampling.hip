@@ -146,7 +146,9 @@ __device__ inline unsigned int float_key(float f) {
 }
 
 __device__ inline unsigned long long fix_mass(float x, float maxv) {
-  return (unsigned long long)(expf(x - maxv) * SMP_FIX);
+  const float d = x - maxv;
+  if (d < -27.8f) return 0ull;   // exp(d) * 2^40 < 1 truncates to 0 anyway: the far tail costs no exponential
+  return (unsigned long long)(expf(d) * SMP_FIX);
 }
 
 // Exclusive prefix sum over the block in thread order; *total gets the block's sum.
