@@ -322,11 +322,84 @@ __device__ void typical_cut(float* __restrict__ x, int n, float maxv, unsigned i
   __syncthreads();
 }
 
+// Step 1 of sample_kernel for a whole row on many CUs: x = logit / temperature (NaN -> -inf), written to `work`,
+// and the maximum of each of SMP_CHUNKS pieces of the row to part_max[row, piece].  grid: (rows, SMP_CHUNKS).
+#define SMP_CHUNKS 32
+__global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restrict__ logits, float* __restrict__ work,
+                                                           int vocab, const float* __restrict__ temperature,
+                                                           float* __restrict__ part_max) {
+  __shared__ float fscratch[32];
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const float* lg = logits + (size_t)row * vocab;
+  float* x = work + (size_t)row * vocab;
+  const float T = temperature[row] > 0.f ? temperature[row] : 1.0f;
+  const int per = (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS;
+  const int lo = min(vocab, chunk * per), hi = min(vocab, lo + per);
+  auto scale = [&](float v) {
+    if (T != 1.0f) v = v / T;
+    if (!(v == v)) v = -INFINITY;  // NaN never survives
+    return v;
+  };
+  float mx = -INFINITY;
+  const int bd = blockDim.x;
+  int j = lo + threadIdx.x;
+  for (; j + 3 * bd < hi; j += 4 * bd) {
+    const float v0 = scale(lg[j]), v1 = scale(lg[j + bd]), v2 = scale(lg[j + 2 * bd]), v3 = scale(lg[j + 3 * bd]);
+    x[j] = v0;
+    x[j + bd] = v1;
+    x[j + 2 * bd] = v2;
+    x[j + 3 * bd] = v3;
+    mx = fmaxf(fmaxf(mx, v0), fmaxf(v1, fmaxf(v2, v3)));
+  }
+  for (; j < hi; j += bd) {
+    const float v = scale(lg[j]);
+    x[j] = v;
+    mx = fmaxf(mx, v);
+  }
+  mx = block_max(mx, fscratch);
+  if (threadIdx.x == 0) part_max[row * SMP_CHUNKS + chunk] = mx;
+}
+
+// For rows that are only scaled (and perhaps cut by min_p) before the draw: the fixed-point mass of each of the
+// SMP_CHUNKS pieces, part_mass[row, piece], against the row's maximum from sample_scale_kernel.  The draw then
+// looks at one piece only.  grid: (rows, SMP_CHUNKS).
+__global__ __launch_bounds__(256) void sample_mass_kernel(const float* __restrict__ work, int vocab,
+                                                          const float* __restrict__ min_p,
+                                                          const float* __restrict__ part_max,
+                                                          unsigned long long* __restrict__ part_mass) {
+  __shared__ unsigned long long wsum[4];
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const float* x = work + (size_t)row * vocab;
+  float maxv = part_max[row * SMP_CHUNKS];
+  for (int i = 1; i < SMP_CHUNKS; ++i) maxv = fmaxf(maxv, part_max[row * SMP_CHUNKS + i]);
+  unsigned int floor_key = float_key(-INFINITY) + 1u;
+  const float mp = min_p[row];
+  if (mp > 0.f && maxv != -INFINITY) {
+    const unsigned int k2 = float_key(maxv + logf(mp));
+    if (k2 > floor_key) floor_key = k2;
+  }
+  const int per = (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS;
+  const int lo = min(vocab, chunk * per), hi = min(vocab, lo + per);
+  auto mass = [&](int j) {
+    if (j >= hi) return 0ull;
+    const float v = x[j];
+    return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull;
+  };
+  unsigned long long mine = 0;
+  const int bd = blockDim.x;
+  for (int j = lo + threadIdx.x; j < hi; j += 4 * bd) mine += mass(j) + mass(j + bd) + mass(j + 2 * bd) + mass(j + 3 * bd);
+#pragma unroll
+  for (int o = TP_WAVE / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, TP_WAVE);
+  if (threadIdx.x % TP_WAVE == 0) wsum[threadIdx.x / TP_WAVE] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) part_mass[row * SMP_CHUNKS + chunk] = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+}
+
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int vocab, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
     const float* __restrict__ typical_p, const float* __restrict__ rnd, int* __restrict__ out,
-    float* __restrict__ info) {
+    float* __restrict__ info, const float* __restrict__ part_max, const unsigned long long* __restrict__ part_mass) {
   __shared__ unsigned long long hist[256];
   __shared__ unsigned int cnt[256];
   __shared__ unsigned long long sh[4];
@@ -369,7 +442,9 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
 
   // 1. scale by the temperature, find the maximum
   float mx = -INFINITY;
-  {
+  if (part_max != nullptr) {   // sample_scale_kernel did this step on many CUs
+    if (threadIdx.x < SMP_CHUNKS) mx = part_max[row * SMP_CHUNKS + threadIdx.x];
+  } else {
     auto scale = [&](float v) {
       if (T != 1.0f) v = v / T;
       if (!(v == v)) v = -INFINITY;  // NaN never survives
@@ -413,6 +488,56 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float thr = maxv + logf(mp);
     const unsigned int k2 = float_key(thr);
     if (k2 > floor_key) floor_key = k2;
+  }
+
+  // The short way for a row that is only scaled (and cut by min_p): the masses of its pieces are there already
+  // (sample_mass_kernel, same maximum and floor), so the draw finds its piece and walks that one alone.
+  {
+    const int k0 = top_k[row];
+    const float tp0 = top_p[row];
+    if (part_mass != nullptr && !greedy && inf == nullptr && !(typical_p[row] < 1.0f) && !(k0 > 0 && k0 < vocab) &&
+        !(tp0 < 1.0f && tp0 > 0.f)) {
+      const unsigned long long* pm = part_mass + (size_t)row * SMP_CHUNKS;
+      unsigned long long Z = 0;
+      for (int i = 0; i < SMP_CHUNKS; ++i) Z += pm[i];
+      if (Z == 0) {
+        if (threadIdx.x == 0) out[row] = vocab - 1;
+        return;
+      }
+      unsigned long long t = (unsigned long long)((double)rnd[row] * (double)Z);
+      if (t >= Z) t = Z - 1;
+      unsigned long long c = 0;
+      int piece = 0;
+      for (; piece < SMP_CHUNKS - 1; ++piece) {
+        if (t < c + pm[piece]) break;
+        c += pm[piece];
+      }
+      if (threadIdx.x >= TP_WAVE) return;      // one wave walks the piece, 64 elements at a time
+      const int lane = threadIdx.x;
+      const int per = (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS;
+      const int lo = min(vocab, piece * per), hi = min(vocab, lo + per);
+      for (int j0 = lo; j0 < hi; j0 += TP_WAVE) {
+        const int j = j0 + lane;
+        unsigned long long q = 0;
+        if (j < hi) {
+          const float v = x[j];
+          if (float_key(v) >= floor_key) q = fix_mass(v, maxv);
+        }
+        unsigned long long inc = q;
+#pragma unroll
+        for (int o = 1; o < TP_WAVE; o <<= 1) {
+          const unsigned long long up = __shfl_up(inc, o, TP_WAVE);
+          if (lane >= o) inc += up;
+        }
+        const unsigned long long hit = __builtin_amdgcn_ballot_w64(q > 0 && c + inc > t);
+        if (hit != 0) {
+          if (lane == (int)__builtin_ctzll(hit)) out[row] = j;
+          return;
+        }
+        c += __shfl(inc, TP_WAVE - 1, TP_WAVE);
+      }
+      return;
+    }
   }
 
   // 2b. typical_p: the survivors nearest the entropy, nearest first, until their mass exceeds typical_p
@@ -632,11 +757,23 @@ __global__ __launch_bounds__(SMP_THREADS) void top_logprobs_kernel(const float* 
 
 extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p, const float* typical_p,
-                         const float* rnd, int* out, float* info, hipStream_t s) {
+                         const float* rnd, int* out, float* info, float* part_max, unsigned long long* part_mass,
+                         hipStream_t s) {
+  // part_max: scratch of rows * 32 floats, or null (the row's first step then runs inside the one block per row);
+  // part_mass: scratch of rows * 32 64-bit integers, given when some row is only scaled before the draw
   TP_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes");
   if (rows == 0) return 0;
+  if (part_max != nullptr && vocab >= 4096 && rows <= 65535)
+    hipLaunchKernelGGL(sample_scale_kernel, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, logits, work, vocab, temperature,
+                       part_max);
+  else
+    part_max = nullptr;
+  if (part_max != nullptr && part_mass != nullptr && info == nullptr)
+    hipLaunchKernelGGL(sample_mass_kernel, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, work, vocab, min_p, part_max, part_mass);
+  else
+    part_mass = nullptr;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, work, vocab, temperature, top_k,
-                     top_p, min_p, typical_p, rnd, out, info);
+                     top_p, min_p, typical_p, rnd, out, info, part_max, part_mass);
   TP_CHECK_LAUNCH("sample");
   return 0;
 }

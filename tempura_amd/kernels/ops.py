@@ -718,11 +718,17 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
     fl, tk = _Staging.send([np.asarray([temperature, top_p, min_p, rnd, typical_p], dtype=np.float32),
                             np.asarray(top_k, dtype=np.int32)], dev)
     out = torch.empty((m,), dtype=torch.int32, device=dev)
+    part_max = torch.empty((m * 32,), dtype=torch.float32, device=dev)    # (maxima of 32 pieces of each row)
+    # rows that are only scaled (and cut by min_p) before the draw get the masses of their pieces from a kernel
+    # of many blocks; worth it when there is such a row
+    plain_rows = any(t > 0 and not (0 < k < vocab) and not (0.0 < p < 1.0) and not (ty < 1.0)
+                     for t, k, p, ty in zip(temperature, top_k, top_p, typical_p))
+    part_mass = torch.empty((m * 32,), dtype=torch.int64, device=dev) if plain_rows and info is None else None
     if info is not None:
         _dev_ok(info)
         _need(info.dtype == torch.float32 and info.is_contiguous() and tuple(info.shape) == (m, 4), "sample: info must be float32 [m, 4]")
     _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
-          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _stream())
+          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _ptr(part_max), _ptr(part_mass), _stream())
     return out
 
 
