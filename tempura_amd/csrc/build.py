@@ -151,7 +151,8 @@ def ensure_built(verbose: bool = True) -> str:
 
 
 # ---- the host library: plain C++ (no GPU code), needed on machines without a GPU too ------------
-HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+# (no contraction into fused multiply-adds: counter_normal.h must round as the device kernel does)
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-pthread", "-ffp-contract=off"]
 
 
 def host_sources() -> List[str]:
@@ -160,7 +161,7 @@ def host_sources() -> List[str]:
 
 def _host_lib_name() -> str:
     h = hashlib.sha256()
-    for p in host_sources():
+    for p in host_sources() + [os.path.join(HERE, "counter_normal.h")]:
         h.update(os.path.basename(p).encode())
         with open(p, "rb") as f:
             h.update(f.read())

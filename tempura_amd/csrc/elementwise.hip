@@ -3,6 +3,7 @@
 #include <stdarg.h>
 
 #include "common.h"
+#include "counter_normal.h"
 
 static thread_local char g_error[512] = "";
 
@@ -459,28 +460,17 @@ extern "C" int tp_swiglu(const void* gu, int in_dt, void* out, int out_dt, int m
 }
 
 // ---- seeded normal fill ------------------------------------------------------------------
-// out[i] = mean + std * N(0, 1) where the normal deviate of element i depends only on
-// (seed, i): a SplitMix64 hash gives two uniforms, Box-Muller turns them into a deviate.
-// Used to make random weights of large models directly in device memory.
-__device__ inline unsigned long long splitmix64(unsigned long long z) {
-  z += 0x9E3779B97F4A7C15ull;
-  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-  return z ^ (z >> 31);
-}
-
+// out[i] = mean + std * N(0, 1) where the deviate of element i depends only on (seed, i) and has the same
+// bits as the host library's (counter_normal.h): random weights of large models are made directly in device
+// memory and can still be regenerated on the host.
 template <typename T>
-__global__ void fill_normal_kernel(T* __restrict__ out, size_t n, unsigned long long seed, float mean, float std) {
+__global__ void fill_normal_kernel(T* __restrict__ out, size_t n, unsigned long long seed, double mean, double std) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const unsigned long long h = splitmix64(seed ^ splitmix64((unsigned long long)i));
-  const float u1 = ((float)(unsigned int)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
-  const float u2 = (float)(unsigned int)((h >> 8) & 0xffffffu) * (1.0f / 16777216.0f);
-  const float z = sqrtf(-2.0f * logf(u1)) * cosf(6.283185307179586f * u2);
-  from_float(out + i, mean + std * z);
+  from_float(out + i, cn_element(seed, i, mean, std));
 }
 
-extern "C" int tp_fill_normal(void* out, int dt, size_t n, unsigned long long seed, float mean, float std,
+extern "C" int tp_fill_normal(void* out, int dt, size_t n, unsigned long long seed, double mean, double std,
                               hipStream_t s) {
   if (n == 0) return 0;
   const dim3 grid((unsigned)((n + 255) / 256));

@@ -35,8 +35,8 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
                  norm_jitter: float = 0.0, on_device: bool = None, values_as=None) -> CausalLM:
     """A model with seeded random weights made tensor by tensor, never written to disk
     (for sizes whose folder would be tens of gigabytes).  With ``on_device`` (the default on a
-    GPU) each tensor is filled by a kernel in device memory; its values then differ from the
-    host generator's that ``write_random_model`` uses.  ``values_as`` (a dtype name) rounds the matrix
+    GPU) each tensor is filled by a kernel in device memory, with the same values as the host
+    generator's that ``write_random_model`` uses.  ``values_as`` (a dtype name) rounds the matrix
     values to that type first, so that a float32 model can hold exactly a bfloat16 model's weights."""
     from ..kernels import ops
     from ..weights.random_init import _tensor_seed

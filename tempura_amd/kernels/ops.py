@@ -750,10 +750,11 @@ def top_logprobs(work: torch.Tensor, info: torch.Tensor, vocab: int, n: int):
 
 
 def fill_normal(out: torch.Tensor, seed: int, mean: float, std: float) -> torch.Tensor:
-    """Fill a device tensor with mean + std * N(0, 1); element i depends only on (seed, i)."""
+    """Fill a device tensor with mean + std * N(0, 1); element i depends only on (seed, i) and has the bits
+    that ``weights.random_init.fill_normal_host`` gives it on the host."""
     if _backend is not None:
         return _backend.fill_normal(out, seed, mean, std)
     _dev_ok(out)
     _call("tp_fill_normal", _ptr(out), _dt(out), ctypes.c_size_t(out.numel()), ctypes.c_ulonglong(seed & (2 ** 64 - 1)),
-          ctypes.c_float(mean), ctypes.c_float(std), _stream())
+          ctypes.c_double(mean), ctypes.c_double(std), _stream())
     return out

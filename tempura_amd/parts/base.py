@@ -23,6 +23,7 @@ class WeightInfo:
     shape: Tuple[int, ...]
     init: str = "normal"          # "normal" (N(0, std)) or "ones"
     optional: bool = False        # True: absence is legal (tied output head)
+    kind: str = "float"           # "float": a weight (stored F32, BF16 or F16); "int": an integer table (kept as int32)
 
 
 @dataclass(frozen=True)

@@ -43,9 +43,11 @@ class SamplingParams:
 
     @property
     def is_greedy(self) -> bool:
-        """Pure greedy: plain argmax of the untouched logits
-        (/root/reference/kernel-api/src/lib.rs:286-290)."""
-        return self.temperature == 0.0 and self.presence_penalty == 0.0 and self.frequency_penalty == 0.0
+        """Pure greedy: plain argmax of the untouched logits.  The reference's rule leaves the repetition
+        penalty out (/root/reference/kernel-api/src/lib.rs:286-290) because its serving path hands that
+        penalty no earlier tokens; here the penalty does see the request's history, so a temperature-0 row
+        with any penalty takes the argmax of the penalised logits, whatever else is in the batch."""
+        return self.temperature == 0.0 and not self.has_penalties
 
     @property
     def has_penalties(self) -> bool:

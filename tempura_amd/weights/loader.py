@@ -4,14 +4,24 @@ Every ``*.safetensors`` file in the folder is read in path order; a later file's
 tensor replaces an earlier one of the same name; an empty folder is an error
 (/root/reference/engine/src/loader.rs:119-145).  bfloat16 stays bfloat16, float16
 is widened exactly to float32, a tensor stored in 32-bit stays 32-bit, integer
-tables become int32.  All faults of a checkpoint
-(missing and unexpected tensors, wrong shapes) are reported in ONE error; the
-reference stops at the first (/root/reference/engine/src/weights.rs:28-42,150-195)
-and checks element counts only (weights.rs:230-238).
+tables become int32.  A weight must be stored as F32, BF16 or F16 and an integer table
+as an integer type; anything else is refused by name (the reference reads the bytes of
+any other type as if they were float32, /root/reference/engine/src/loader.rs:191-208).
+All faults of a checkpoint (missing and unexpected tensors, wrong shapes, wrong element
+types) are reported in ONE error; the reference stops at the first
+(/root/reference/engine/src/weights.rs:28-42,150-195) and checks element counts only
+(weights.rs:230-238).
+
+A folder may hold ``integrity.json``, ``{"tensor_hashes": {name: sha256 of the stored
+bytes}}``; every tensor it names is then verified while it is loaded
+(/root/reference/engine/src/loader.rs:147-182 hashes the widened float32 values; here
+the bytes as stored, so that a bfloat16 checkpoint is never widened just to be hashed).
 """
 from __future__ import annotations
 
 import glob
+import hashlib
+import json
 import os
 from typing import Callable, Dict, List, Optional
 
@@ -25,11 +35,17 @@ class WeightsError(ValueError):
     """A checkpoint that does not fit the model.  ``missing``, ``unexpected`` and
     ``wrong_shape`` (name -> (expected, found)) carry the details."""
 
-    def __init__(self, message, missing=(), unexpected=(), wrong_shape=None):
+    def __init__(self, message, missing=(), unexpected=(), wrong_shape=None, wrong_dtype=None):
         super().__init__(message)
         self.missing = list(missing)
         self.unexpected = list(unexpected)
         self.wrong_shape = dict(wrong_shape or {})
+        self.wrong_dtype = dict(wrong_dtype or {})      # name -> (accepted tags, found tag)
+
+
+#: element types a checkpoint may store a tensor of each kind in
+ACCEPTED_TAGS = {"float": ("F32", "BF16", "F16"), "int": ("I64", "I32", "I16", "I8", "U8")}
+MANIFEST_NAME = "integrity.json"
 
 
 class Checkpoint:
@@ -56,15 +72,23 @@ class Checkpoint:
         return self._where[name].dtype_tag(name)
 
     def tensor(self, name: str) -> torch.Tensor:
-        """The tensor on the host in its kept dtype."""
+        """The tensor on the host in its kept dtype: bfloat16, float32 and int32 as stored, float16 widened
+        (exactly) to float32, other integers to int32.  Any other stored type is refused."""
+        tag = self.dtype_tag(name)
+        if tag not in ACCEPTED_TAGS["float"] and tag not in ACCEPTED_TAGS["int"]:
+            raise WeightsError(f"tensor {name} is stored as {tag}: weights must be F32, BF16 or F16, integer tables an integer type",
+                               wrong_dtype={name: (ACCEPTED_TAGS["float"] + ACCEPTED_TAGS["int"], tag)})
         t = self._where[name].tensor(name)
         if t.dtype == torch.float16:
             return t.to(torch.float32)      # exact widening
-        if t.dtype == torch.float64:
-            return t.to(torch.float32)
-        if t.dtype in (torch.int64, torch.int16, torch.int8, torch.uint8, torch.bool):
+        if t.dtype in (torch.int64, torch.int16, torch.int8, torch.uint8):
             return t.to(torch.int32)
-        return t                            # bfloat16, float32, int32 as stored
+        return t
+
+    def sha256(self, name: str) -> str:
+        """Hex digest of the tensor's bytes as stored."""
+        t = self._where[name].tensor(name).contiguous()
+        return hashlib.sha256(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"").hexdigest()
 
     def close(self) -> None:
         for f in self.files:
@@ -76,11 +100,16 @@ def check_checkpoint(ckpt: Checkpoint, expected: Dict[str, WeightInfo]) -> None:
     have = set(ckpt.names())
     missing = sorted(n for n, info in expected.items() if n not in have and not info.optional)
     unexpected = sorted(n for n in have if n not in expected)
-    wrong = {}
+    wrong, wrong_dt = {}, {}
     for n, info in expected.items():
-        if n in have and tuple(ckpt.shape(n)) != tuple(info.shape):
+        if n not in have:
+            continue
+        if tuple(ckpt.shape(n)) != tuple(info.shape):
             wrong[n] = (tuple(info.shape), tuple(ckpt.shape(n)))
-    if missing or unexpected or wrong:
+        accepted = ACCEPTED_TAGS[getattr(info, "kind", "float")]
+        if ckpt.dtype_tag(n) not in accepted:
+            wrong_dt[n] = (accepted, ckpt.dtype_tag(n))
+    if missing or unexpected or wrong or wrong_dt:
         lines = [f"checkpoint in {ckpt.model_dir} does not fit the model:"]
         if missing:
             lines.append(f"  missing tensors ({len(missing)}): " + ", ".join(missing))
@@ -89,11 +118,41 @@ def check_checkpoint(ckpt: Checkpoint, expected: Dict[str, WeightInfo]) -> None:
         if wrong:
             lines.append(f"  wrong shapes ({len(wrong)}): " + ", ".join(
                 f"{n} expected {list(e)} found {list(f)}" for n, (e, f) in sorted(wrong.items())))
-        raise WeightsError("\n".join(lines), missing, unexpected, wrong)
+        if wrong_dt:
+            lines.append(f"  wrong element types ({len(wrong_dt)}): " + ", ".join(
+                f"{n} stored as {f}, accepted {'/'.join(a)}" for n, (a, f) in sorted(wrong_dt.items())))
+        raise WeightsError("\n".join(lines), missing, unexpected, wrong, wrong_dt)
 
 
-def load_into(model, model_dir: str) -> None:
-    """Check the folder's tensors against ``model`` and load them, tensor by tensor."""
+def write_manifest(model_dir: str) -> str:
+    """Write ``integrity.json`` for the folder's tensors as they are now; returns its path."""
+    ckpt = Checkpoint(model_dir)
+    hashes = {n: ckpt.sha256(n) for n in sorted(ckpt.names())}
+    ckpt.close()
+    path = os.path.join(model_dir, MANIFEST_NAME)
+    with open(path, "w") as f:
+        json.dump({"tensor_hashes": hashes}, f, indent=1, sort_keys=True)
+    return path
+
+
+def read_manifest(model_dir: str) -> Optional[Dict[str, str]]:
+    path = os.path.join(model_dir, MANIFEST_NAME)
+    if not os.path.exists(path):
+        return None
+    try:
+        with open(path) as f:
+            hashes = json.load(f)["tensor_hashes"]
+        if not isinstance(hashes, dict) or not all(isinstance(v, str) for v in hashes.values()):
+            raise ValueError("tensor_hashes must map names to hex digests")
+    except (OSError, ValueError, KeyError, TypeError) as e:
+        raise WeightsError(f"{path}: not an integrity manifest: {e}") from e
+    return hashes
+
+
+def load_into(model, model_dir: str, verify: Optional[bool] = None) -> None:
+    """Check the folder's tensors against ``model`` and load them, tensor by tensor.
+    ``verify``: None checks the tensors against ``integrity.json`` when the folder has one, True demands
+    one, False skips it."""
     try:
         ckpt = Checkpoint(model_dir)
     except SafetensorsError as e:
@@ -101,12 +160,23 @@ def load_into(model, model_dir: str) -> None:
     expected = model.expected_weights()
     check_checkpoint(ckpt, expected)
     have = set(ckpt.names())
+    manifest = read_manifest(model_dir) if verify is not False else None
+    if verify is True and manifest is None:
+        raise WeightsError(f"{model_dir} has no {MANIFEST_NAME} to verify against")
+    if manifest:
+        absent = sorted(n for n in manifest if n not in have)
+        if absent:
+            raise WeightsError(f"{MANIFEST_NAME} names tensors the checkpoint does not hold: " + ", ".join(absent), absent)
 
     def get(name: str, optional: bool = False) -> Optional[torch.Tensor]:
         if name not in have:
             if optional:
                 return None
             raise WeightsError(f"missing tensor {name}", [name])
+        if manifest and name in manifest:
+            got = ckpt.sha256(name)
+            if got != manifest[name].lower():
+                raise WeightsError(f"tensor {name} fails its integrity check: expected sha256 {manifest[name]}, got {got}")
         return ckpt.tensor(name)
 
     model.load_weights(get)

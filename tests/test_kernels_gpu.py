@@ -623,3 +623,41 @@ def test_linear_swiglu(m, inter, k):
         r1 = res.clone().to(DEV)
         ops.linear(blk, w2.to(DEV), torch.float32, residual=r1)
         _close(r1, want, 2e-5, "product of k-blocked rows")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seed,n,mean,std", [(0, 1, 0.0, 0.02), (7, 4_000_037, 0.0, 0.02), (2 ** 63 + 11, 1_000_000, 1.0, 0.2)])
+def test_fill_normal_has_the_host_generator_s_bits(dtype, seed, n, mean, std):
+    """The device kernel, the host library and the numpy twin (tests/plain_random.py) agree on every element."""
+    import numpy as np
+    import plain_random
+    from tempura_amd.weights.random_init import fill_normal_host
+    ops = _ops()
+    dev = ops.fill_normal(torch.empty(n, dtype=dtype, device=DEV), seed, mean, std).cpu()
+    host = fill_normal_host(torch.empty(n, dtype=dtype), seed, mean, std)
+    assert torch.equal(dev.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       host.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    twin = torch.from_numpy(plain_random.fill_normal((min(n, 300_000),), seed, mean, std)).to(dtype)
+    assert torch.equal(dev[: twin.numel()], twin)
+
+
+def test_device_made_model_equals_the_written_folder(tmp_path):
+    """A model made in device memory holds the weights of the folder written from the same configuration and seed."""
+    import helpers
+    from tempura_amd.config import LlamaConfig
+    from tempura_amd.engine.loading import load_model, random_model
+    _ops()
+    cfg = LlamaConfig.from_dict(helpers.CONFIGS["D"].to_dict())
+    from tempura_amd.weights import write_random_model
+    for dtype in ("float32", "bfloat16"):
+        d = write_random_model(cfg, str(tmp_path / dtype), seed=5, std=0.1, norm_jitter=0.1, dtype=dtype)
+        a = load_model(d, dtype, DEV)
+        b = random_model(cfg, seed=5, dtype=dtype, device=DEV, std=0.1, norm_jitter=0.1)
+        for la, lb in zip(a.layers, b.layers):
+            for pa, pb in zip(la.parts(), lb.parts()):
+                for key, va in vars(pa).items():
+                    vb = getattr(pb, key)
+                    va, vb = getattr(va, "data", va), getattr(vb, "data", vb)
+                    if isinstance(va, torch.Tensor):
+                        assert torch.equal(va, vb), f"{type(pa).__name__}.{key} differs ({dtype})"
+        assert torch.equal(a.embedding.weight, b.embedding.weight) and torch.equal(a.final_norm.weight, b.final_norm.weight)
