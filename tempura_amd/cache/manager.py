@@ -68,6 +68,9 @@ class CacheManager:
             raise ValueError(native.last_error())
         self.pools = [_PoolView(self, g, int(n)) for g, n in enumerate(num_pages)]
         self._slot_of: Dict[Hashable, int] = {}
+        #: bumped by everything that changes what a request holds or where its next token goes (add, release,
+        #: commit, truncate): whoever keeps values derived from the tables compares it before using them
+        self.generation = 0
         self._g_buf = (ctypes.c_int * max(1, len(self.groups)))()
 
     def __del__(self):
@@ -96,6 +99,7 @@ class CacheManager:
         if s < 0:
             raise RuntimeError(native.last_error())
         self._slot_of[rid] = s
+        self.generation += 1
         return s
 
     def release(self, rid) -> None:
@@ -103,6 +107,7 @@ class CacheManager:
         s = self._slot_of.pop(rid, None)
         if s is None:
             raise ValueError(f"request {rid!r} is not live (released twice?)")
+        self.generation += 1
         if self._lib.cc_release(self._h, s) != 0:
             raise RuntimeError(native.last_error())
 
@@ -150,11 +155,13 @@ class CacheManager:
         self.commit_many([rid], [n_new])
 
     def commit_many(self, rids: Sequence, n_new: Sequence[int]) -> None:
+        self.generation += 1
         if self._lib.cc_commit(self._h, len(rids), _ints([self._slot(r) for r in rids]), _ints([int(n) for n in n_new])) != 0:
             raise RuntimeError(native.last_error())
 
     def truncate(self, rid, num_tokens: int) -> None:
         """Forget tokens past ``num_tokens`` and return whole pages beyond them."""
+        self.generation += 1
         if self._lib.cc_truncate(self._h, self._slot(rid), int(num_tokens)) != 0:
             raise ValueError(native.last_error())
 

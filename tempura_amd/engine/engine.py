@@ -162,6 +162,8 @@ class Engine:
         request that ends on its token leaves a row computed for nothing).  None when that does not apply."""
         if not self.chain_steps or self.scheduler.waiting or not all(it.count == 1 and it.samples for it in items):
             return None
+        if len(items) != len(self.scheduler.running):
+            return None         # a running request was left out of this step: the scheduler must see it again
         limit = self.scheduler.config.max_model_len
         keep = [i for i, it in enumerate(items)
                 if len(it.request.output) + 1 < it.request.params.max_new_tokens and it.request.num_tokens + 1 < limit]

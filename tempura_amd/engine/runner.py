@@ -150,7 +150,7 @@ class ModelRunner:
         self.use_graph = bool(use_graph) and self.device.type == "cuda" and not model.state_specs and \
             all(getattr(p, "graph_safe", False) for layer in model.layers for p in layer.parts())
         self.graph_steps = 0
-        self._prepared = None          # (request ids, graph) of a decode step staged ahead by prepare_decode
+        self._prepared = None          # (request ids, graph, cache generation) of a decode step staged ahead by prepare_decode
         self.staged_steps = 0          # decode steps that found their inputs staged
         self._graphs: Dict[tuple, _DecodeGraph] = {}
         self._graph_pool = None
@@ -296,7 +296,7 @@ class ModelRunner:
         if g.graph is None:
             return False
         self._fill_graph_inputs(g, rids, [0] * len(rids))
-        self._prepared = (tuple(rids), g)
+        self._prepared = (tuple(rids), g, self.cache.generation)
         return True
 
     def _graph_step(self, rids: Sequence, tokens, want_rows: Optional[Sequence[int]] = None) -> torch.Tensor:
@@ -304,7 +304,10 @@ class ModelRunner:
         on_device = torch.is_tensor(tokens)
         n = len(rids)
         prepared, self._prepared = self._prepared, None
-        if prepared is not None and prepared[0] == tuple(rids):
+        # (staged values are good only while nothing was added, ended, committed or truncated since: the scheduler
+        # changes the cache manager directly, and a request that was preempted and readmitted, or a request
+        # name used again, would otherwise find another request's positions and pages)
+        if prepared is not None and prepared[0] == tuple(rids) and prepared[2] == self.cache.generation:
             g = prepared[1]                         # staged already: only the tokens are new
             self.staged_steps += 1
             if not on_device:

@@ -95,6 +95,14 @@ class Scheduler:
     def add_request(self, req: Request) -> None:
         if not req.prompt:
             raise ValueError(f"request {req.rid!r}: empty prompt")
+        if req.params.max_new_tokens == 0:
+            # nothing to generate: finished as it arrives, without a step and without a sampled token
+            req.arrival = self._arrivals
+            self._arrivals += 1
+            req.finish_reason = "length"
+            req.state = RequestState.FINISHED
+            self.finished.append(req)
+            return
         total = len(req.prompt) + req.params.max_new_tokens
         limit = self.config.max_model_len
         if len(req.prompt) >= limit and req.params.max_new_tokens > 0:

@@ -144,6 +144,32 @@ def test_generate_and_preemption_on_host(tiny_dirs):
     assert tight.stats()["preemptions"] > 0 and tight.runner.cache.free_pages() == [6]
 
 
+def test_zero_new_tokens_and_a_request_left_out_of_a_step(tiny_dirs):
+    from tempura_amd.engine import Engine
+    from tempura_amd.sampling import SamplingParams
+    cfg, W = tiny_dirs.plain_model("A")
+    prompts = [helpers.random_tokens(256, n, seed=900 + n) for n in (4, 6, 9)]
+    kw = dict(dtype="float32", device="cpu", page_size=16, max_batch_size=4, kv_pages=32)
+    eng = Engine(tiny_dirs.path("A"), **kw)
+    outs = eng.generate(prompts, [SamplingParams(temperature=0.0, max_new_tokens=n) for n in (0, 3, 0)])
+    assert outs == [[], plain.greedy_generate(cfg, W, prompts[1], 3), []]
+    assert eng.stats()["generated_tokens"] == 3
+    # A token budget below the number of decoding requests leaves one out of the step.  Such a step must not be
+    # followed by a step queued ahead for the same requests (the one left out would wait until the others end).
+    eng = Engine(tiny_dirs.path("A"), max_num_batched_tokens=32, **kw)
+    eng.chain_steps = True                       # (what a GPU engine has; the decision is host logic)
+    for p in prompts:
+        eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=6))
+    eng.step()
+    assert all(r.is_decoding for r in eng.scheduler.running) and len(eng.scheduler.running) == 3
+    items = eng.scheduler.schedule()
+    assert len(items) == 3 and eng._queue_next(items) is not None, "every running request decodes: the next step may be queued"
+    eng.scheduler.config.max_num_batched_tokens = 2
+    items = eng.scheduler.schedule()
+    assert len(items) == 2 and all(it.count == 1 and it.samples for it in items)
+    assert eng._queue_next(items) is None
+
+
 def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
     """A mixer defined in the tests, with per-request state and no paged cache, in an architecture of its own."""
     import toy_parts

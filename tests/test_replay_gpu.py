@@ -122,6 +122,36 @@ def test_decode_steps_staged_ahead_change_nothing(tiny_dirs, dtype):
         r.cache.check()
 
 
+def test_staged_inputs_are_dropped_when_the_cache_changed_behind_the_runner(tiny_dirs):
+    """The scheduler ends and readmits requests on the cache manager itself.  A decode step that was staged for
+    the same request names before such a change must not replay the old positions and pages."""
+    from tempura_amd.engine.runner import StepEntry
+    name, dtype = "D", "float32"
+    reqs = {rid: toks for rid, toks in list(helpers.requests_for(name).items())[1:3]}
+    rids = list(reqs)
+    ref = _reference(tiny_dirs, name, dtype)
+    runner = _runner(tiny_dirs, name, dtype, 1024, helpers.PAGE_SIZE[name], use_graph=True)
+    for rid in rids:
+        runner.add_request(rid)
+        runner.step([StepEntry(rid, reqs[rid][:9], [])])
+    runner.step([StepEntry(rid, [reqs[rid][9]], [0]) for rid in rids])            # captures the graph
+    assert runner.prepare_decode(rids)
+    # preempted and readmitted behind the runner's back, as the scheduler does it: another length, other pages
+    runner.cache.release(rids[0])
+    runner.cache.add(rids[0])
+    runner.step([StepEntry(rids[0], reqs[rids[0]][:4], [])])
+    assert runner.prepare_decode(rids)
+    runner.cache.release(rids[0])
+    runner.cache.add(rids[0])
+    runner.step([StepEntry(rids[0], reqs[rids[0]][:6], [])])
+    before = runner.staged_steps
+    got = runner.step([StepEntry(rids[0], [reqs[rids[0]][6]], [0]), StepEntry(rids[1], [reqs[rids[1]][10]], [0])]).cpu()
+    assert runner.staged_steps == before, "the stale staging was used"
+    assert helpers.rel_err(got[0], ref[rids[0]][6]) <= helpers.TOL[dtype]
+    assert helpers.rel_err(got[1], ref[rids[1]][10]) <= helpers.TOL[dtype]
+    runner.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(tiny_dirs, dtype):
     """700 tokens decoded one by one after a short prompt (config A, 44 pages of 16)."""

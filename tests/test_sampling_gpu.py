@@ -225,3 +225,24 @@ def test_sampler_class_rows_with_different_options():
     assert out[1] in lg[1].topk(10).indices.tolist()
     assert out[2] != int(lg[2].argmax()), "a huge presence penalty bans the generated token"
     assert s.sample(lg, ps, [0, 3, 1], [[], [], []], [[], [], [int(lg[2].argmax())]]) == out
+
+
+def test_temperature_zero_with_repetition_penalty_does_not_depend_on_the_batch():
+    """A temperature-0 row with a repetition penalty takes the argmax of the penalised logits whether it is alone,
+    beside a sampled row, or asked for log-probabilities."""
+    from tempura_amd.sampling import Sampler, SamplingParams
+    V = 300
+    lg = torch.zeros(2, V)
+    lg[0, 17], lg[0, 40] = 5.0, 4.0             # the penalty (5.0 / 1.3 < 4.0) moves the maximum from 17 to 40
+    lg[1] = torch.randn(V, generator=torch.Generator().manual_seed(4))
+    lg = lg.to(DEV)
+    s = Sampler(V, torch.device(DEV), default_seed=1)
+    greedy = SamplingParams(temperature=0.0, repeat_penalty=1.3)
+    assert not greedy.is_greedy and SamplingParams(temperature=0.0).is_greedy
+    hist = [3, 17, 9]
+    alone = s.sample(lg[:1], [greedy], [0], [hist], [[]])
+    beside = s.sample(lg, [greedy, SamplingParams(temperature=0.9, seed=3)], [0, 0], [hist, []], [[], []])
+    with_lp, recs = s.sample(lg[:1], [greedy], [0], [hist], [[]], top_n=2)
+    assert alone == [40] and beside[0] == 40 and with_lp == [40] and recs[0].token_id == 40
+    assert s.sample(lg[:1], [SamplingParams(temperature=0.0)], [0], [hist], [[]]) == [17]
+    assert float(lg[0, 17]) == 5.0, "the caller's logits are left as they were"

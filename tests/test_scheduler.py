@@ -178,3 +178,14 @@ def test_abort_frees_at_once_wherever_the_request_stands():
     assert all("a" not in s and "c" not in s for s in seen[3:])
     assert sorted(r.rid for r in sched.finished) == ["a", "b", "c"]
     assert cache.pools[0].num_free == 16
+
+
+def test_nothing_to_generate_finishes_on_arrival():
+    sched, cache = make()
+    r = req("z", 5, max_new=0)
+    sched.add_request(r)
+    assert r.state == RequestState.FINISHED and r.finish_reason == "length" and r.output == []
+    assert not sched.has_unfinished() and cache.live_requests() == []
+    sched.add_request(req("a", 5, max_new=2))
+    steps = run(sched, cache)
+    assert [s[0][0] for s in steps] == ["a", "a"]

@@ -125,3 +125,53 @@ def test_compute_dtype_conversion(tmp_path):
     load_into(mbf, d2)
     assert mbf.layers[0].mixer.wo.dtype == torch.bfloat16
     assert mbf.final_norm.weight.dtype == torch.float32
+
+
+def test_other_element_types_are_refused_by_name(tmp_path):
+    """A weight stored as F64, an integer or BOOL is not converted silently: the one error names it
+    (the reference would read such bytes as float32, /root/reference/engine/src/loader.rs:191-208)."""
+    cfg, model = _model("A")
+    w = random_weights(cfg, 0, dtype="float32")
+    w["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(64, 64, dtype=torch.int32)
+    w["model.layers.1.mlp.down_proj.weight"] = w["model.layers.1.mlp.down_proj.weight"].double()
+    w["model.norm.weight"] = torch.ones(64, dtype=torch.bool)
+    del w["model.layers.1.mlp.up_proj.weight"]
+    os.makedirs(tmp_path / "m")
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), w.items())
+    with pytest.raises(WeightsError) as ei:
+        load_into(model, str(tmp_path / "m"))
+    e = ei.value
+    assert set(e.wrong_dtype) == {"model.layers.0.self_attn.q_proj.weight", "model.layers.1.mlp.down_proj.weight", "model.norm.weight"}
+    assert e.wrong_dtype["model.layers.1.mlp.down_proj.weight"][1] == "F64"
+    assert e.missing == ["model.layers.1.mlp.up_proj.weight"], "still one error for every fault"
+    assert "q_proj.weight stored as I32" in str(e)
+    ck = Checkpoint(str(tmp_path / "m"))
+    with pytest.raises(WeightsError, match="F64"):
+        ck.tensor("model.layers.1.mlp.down_proj.weight")
+
+
+def test_integrity_manifest(tmp_path):
+    from tempura_amd.weights.loader import MANIFEST_NAME, write_manifest
+    cfg, model = _model("A")
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=3, dtype="bfloat16")
+    with pytest.raises(WeightsError, match="no integrity.json"):
+        load_into(model, d, verify=True)
+    path = write_manifest(d)
+    assert os.path.basename(path) == MANIFEST_NAME
+    load_into(model, d)                    # verified because the manifest is there
+    load_into(model, d, verify=True)
+    # one changed value in one tensor
+    w = {n: Checkpoint(d).tensor(n).clone() for n in Checkpoint(d).names()}
+    w["model.layers.1.mlp.gate_proj.weight"][3, 5] += 1.0
+    write_safetensors(os.path.join(d, "model.safetensors"), w.items())
+    with pytest.raises(WeightsError, match="gate_proj.weight fails its integrity check"):
+        load_into(model, d)
+    load_into(model, d, verify=False)
+    # a manifest that names a tensor the folder lacks
+    with open(path) as f:
+        m = json.load(f)
+    m["tensor_hashes"]["model.layers.9.ghost"] = "00"
+    with open(path, "w") as f:
+        json.dump(m, f)
+    with pytest.raises(WeightsError, match="ghost"):
+        load_into(model, d)
