@@ -98,8 +98,19 @@ struct KvFrags {
   bf16x8_t v[D / 16];
 };
 
+// A lane's value fragment holds eight consecutive key places of one element.  Places past the last key that
+// exists hold whatever the page's previous owner (or a padded row) left there; their probabilities are 0, but
+// 0 * NaN and 0 * Inf are NaN, so one request's non-finite values would reach the next owner of the page.
+// The mask keeps the first `n` places (n <= 0: none, n >= 8: all) and clears the others to +0.
+__device__ inline u32x4_t attn_existing_keys(int n) {
+  u32x4_t keep;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) keep[w] = (2 * w < n ? 0x0000ffffu : 0u) | (2 * w + 1 < n ? 0xffff0000u : 0u);
+  return keep;
+}
+
 // Fetch the fragments of the step starting at key j0 (kvh: kv head; ctx: keys that exist; keys
-// past the end are clamped to the last one and masked later).
+// past the end are clamped to the last one and masked later, values past the end are cleared).
 template <int D>
 __device__ inline void attn_load(const AttnArgs& a, const int* __restrict__ table, int kvh, int ctx, int j0,
                                  KvFrags<D>& f) {
@@ -118,6 +129,12 @@ __device__ inline void attn_load(const AttnArgs& a, const int* __restrict__ tabl
   const int kb = min(j0 + 8 * g, (ctx - 1) & ~7);
   const int vpage = table[kb / ps];
   const bf16_t* vr = a.v_cache + ((size_t)(vpage * a.n_kv + kvh) * D + c) * ps + kb % ps;
+  if (j0 + 32 > ctx) {   // the step that holds the last key
+    const u32x4_t keep = attn_existing_keys(ctx - (j0 + 8 * g));
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt) f.v[dt] = frag_of(*(const u32x4_t*)(vr + (size_t)dt * 16 * ps) & keep);
+    return;
+  }
 #pragma unroll
   for (int dt = 0; dt < D / 16; ++dt) f.v[dt] = frag_of(*(const u32x4_t*)(vr + (size_t)dt * 16 * ps));
 }
@@ -566,6 +583,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     for (int dt = 0; dt < D / 16; ++dt) {
       asm volatile("" : "+v"(vv[dt]));
       vf[dt] = frag_of(vv[dt]);
+    }
+    if (j0 + 32 > ctx) {   // the step that holds the last key: places past it are cleared (see attn_existing_keys)
+      const u32x4_t keep = attn_existing_keys(ctx - (j0 + 8 * g));
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) vf[dt] = frag_of(vv[dt] & keep);
     }
     attn_pv<D, NQ>(vf, pf, alpha, moved, o);
     stage = nstage;

@@ -221,7 +221,7 @@ def test_rope_kv_write_long_step(dtype, heads, kv, d, page, n):
     assert torch.equal(k1, kd) and torch.equal(v1, vd)
 
 
-def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, allow_fast=True, tune=0):
+def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, allow_fast=True, tune=0, poison=False):
     ops = _ops()
     g = torch.Generator().manual_seed(seed)
     R = len(q_lens)
@@ -243,6 +243,16 @@ def _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed, a
     tr = torch.repeat_interleave(torch.arange(R, dtype=torch.int32), torch.tensor(q_lens))
     scale = 1.0 / math.sqrt(d)
     ref = emu.paged_attention(q, kc, vc, bt, cu, cl, tr, scale, window, max(q_lens), max(ctx_lens)).double()
+    if poison:
+        # every cache place that holds no key of its request is NaN: the rest of each last page, the spare pages
+        used = torch.zeros(pages, page, dtype=torch.bool)
+        for r, c in enumerate(ctx_lens):
+            for i in range(c):
+                used[bt[r, i // page], i % page] = True
+        kc = kc.clone()
+        vc = vc.clone()
+        kc[~used[:, None, :].expand(pages, kv, page)] = float("nan")
+        vc.transpose(2, 3)[~used[:, None, :].expand(pages, kv, page)] = float("nan")
     ops.allow_fast_attention = allow_fast
     ops.library().tp_attention_tune(tune)
     try:
@@ -557,6 +567,19 @@ def test_attention_portions_with_split_keys(heads, kv, d, page):
             _close(a, b.double().cpu(), 8e-3, "split against unsplit")
     finally:
         ops.portion_min_keys, ops.portion_target_blocks = keep
+
+
+@pytest.mark.parametrize("dtype,fast,heads,kv,d,page", [(torch.bfloat16, True, 8, 2, 128, 16), (torch.bfloat16, True, 6, 3, 96, 32),
+                                                        (torch.bfloat16, True, 4, 2, 64, 8), (torch.bfloat16, True, 5, 1, 32, 64),
+                                                        (torch.bfloat16, False, 4, 2, 48, 16), (torch.float32, False, 4, 2, 80, 16)])
+def test_attention_ignores_what_lies_past_the_last_key(dtype, fast, heads, kv, d, page):
+    """A page keeps what its previous owner wrote; if that was not finite, nothing of it may reach the new
+    owner: NaN in every cache place that holds no key (the matrix-core kernels fetch eight key places of a value
+    at once, and 0 * NaN is NaN)."""
+    for q_lens, ctx_lens, window in (([37, 9, 1, 1, 1], [37, 61, 33, 130, 1], 0), ([1, 1, 1], [700, 31, 257], 0),
+                                     ([70, 33], [70, 97], 0), ([20, 1, 6, 1], [50, 77, 6, 300], 13)):
+        got = _attention_case(dtype, heads, kv, d, page, q_lens, ctx_lens, window, seed=21, allow_fast=fast, poison=True)
+        assert bool(torch.isfinite(got.float()).all())
 
 
 def test_attention_mfma_long_decode():
