@@ -58,7 +58,8 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
         if info.init == "ones":
             t = torch.ones(info.shape, dtype=torch.float32, device=dev)
             if norm_jitter:
-                ops.fill_normal(t, _tensor_seed(seed, name), 1.0, norm_jitter)
+                # (rounded to the stored type as a written folder's norm weights are)
+                t = ops.fill_normal(t, _tensor_seed(seed, name), 1.0, norm_jitter).to(store).to(torch.float32)
             return t
         t = torch.empty(info.shape, dtype=parse_dtype(values_as) if values_as else store, device=dev)
         return ops.fill_normal(t, _tensor_seed(seed, name), 0.0, std).to(store)

@@ -96,12 +96,19 @@ def rope(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, attn_
     return torch.cat([x0 * c - x1 * s, x0 * s + x1 * c], dim=-1)
 
 
+def as_bfloat16(x: torch.Tensor) -> torch.Tensor:
+    """x rounded to bfloat16 (nearest, ties to even) and widened again: what storing it in 16 bits does."""
+    return x.to(torch.float32).to(torch.bfloat16).to(x.dtype)
+
+
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, window: Optional[int] = None,
-              kv_offset: int = 0) -> torch.Tensor:
+              kv_offset: int = 0, stored=None) -> torch.Tensor:
     """q [T, nH, D], k, v [S, nKV, D] with S = kv_offset + T; kv head of head h is
     h // (nH / nKV); query row s sees keys j <= (S - T) + s and, with a window w, j >= limit - w + 1;
     score = dot * scale; softmax over the visible keys; out = sum p_j v_j.
-    /root/reference/kernels/src/attention.rs:28-87"""
+    /root/reference/kernels/src/attention.rs:28-87
+    ``stored``: see ``forward``; here it rounds the unnormalised probabilities that are multiplied with the
+    values (their sum is taken before the rounding)."""
     T, nH, D = q.shape
     S, nKV, _ = k.shape
     group = nH // nKV
@@ -115,8 +122,11 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, w
                 start = limit - window + 1
             scores = (k[start: limit + 1, kv_h] @ q[s, h]) * scale
             p = torch.exp(scores - scores.max())
-            p = p / p.sum()
-            out[s, h] = p @ v[start: limit + 1, kv_h]
+            if stored is None:
+                p = p / p.sum()
+                out[s, h] = p @ v[start: limit + 1, kv_h]
+            else:
+                out[s, h] = (stored(p) @ v[start: limit + 1, kv_h]) / p.sum()
     return out.reshape(T, nH * D)
 
 
@@ -125,10 +135,13 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu_ffn(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor) -> torch.Tensor:
+def swiglu_ffn(x: torch.Tensor, wg: torch.Tensor, wu: torch.Tensor, wd: torch.Tensor, stored=None) -> torch.Tensor:
     """down(silu(gate(x)) * up(x)), weights [out, in], y = x W^T.
     /root/reference/engine/src/model.rs:1203-1231,1301-1313"""
-    return (silu(x @ wg.T) * (x @ wu.T)) @ wd.T
+    a = silu(x @ wg.T) * (x @ wu.T)
+    if stored is not None:
+        a = stored(a)
+    return a @ wd.T
 
 
 # ---- whole model --------------------------------------------------------------------------
@@ -143,14 +156,20 @@ def layer_window(cfg: dict, layer: int) -> Optional[int]:
 
 
 def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=torch.float64,
-            position_offset: int = 0) -> torch.Tensor:
+            position_offset: int = 0, stored=None) -> torch.Tensor:
     """Logits [T, vocab] at every position of one whole sequence, no cache.
     ``position_offset`` shifts every position (positions are session.position + t,
     /root/reference/engine/src/model.rs:686-688); only distances count, so logits must not change.
     Order inside a layer: norm, q/k/v, rope on q and k, attention, o, add, norm, feed-forward, add
     (/root/reference/engine/src/model.rs:952-1314); then final norm and output projection
     (model.rs:1355-1398), the output matrix being the embedding when the file has none
-    (/root/reference/engine/src/weights.rs:156-166)."""
+    (/root/reference/engine/src/weights.rs:156-166).
+    ``stored`` (for instance ``as_bfloat16``) is applied to every value that 16-bit serving keeps in 16 bits
+    between two operations: the normed rows fed to a product, q, k and v, the unnormalised probabilities, the
+    attention output and the gated activations; everything else (sums, norms, softmax statistics, the residual
+    stream) stays exact.  The distance of such a run from the exact one is the rounding noise that the storage
+    type alone explains, the yardstick the 16-bit engine is measured with."""
+    keep = stored if stored is not None else (lambda t: t)
     W = {k: v.to(dtype) for k, v in weights.items()}
     H = cfg["hidden_size"]
     nH = cfg["num_attention_heads"]
@@ -168,17 +187,17 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
     scale = 1.0 / math.sqrt(D)                                          # model.rs:1078
     for l in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{l}."
-        x = rmsnorm(h, W[p + "input_layernorm.weight"], eps)
+        x = keep(rmsnorm(h, W[p + "input_layernorm.weight"], eps))
         q = (x @ W[p + "self_attn.q_proj.weight"].T).reshape(T, nH, D)
         k = (x @ W[p + "self_attn.k_proj.weight"].T).reshape(T, nKV, D)
-        v = (x @ W[p + "self_attn.v_proj.weight"].T).reshape(T, nKV, D)
-        q = rope(q, pos, inv_freq)
-        k = rope(k, pos, inv_freq)
-        a = attention(q, k, v, scale, layer_window(cfg, l))
+        v = keep((x @ W[p + "self_attn.v_proj.weight"].T).reshape(T, nKV, D))
+        q = keep(rope(q, pos, inv_freq))
+        k = keep(rope(k, pos, inv_freq))
+        a = keep(attention(q, k, v, scale, layer_window(cfg, l), stored=stored))
         h = h + a @ W[p + "self_attn.o_proj.weight"].T
-        x = rmsnorm(h, W[p + "post_attention_layernorm.weight"], eps)
-        h = h + swiglu_ffn(x, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
-    x = rmsnorm(h, W["model.norm.weight"], eps)
+        x = keep(rmsnorm(h, W[p + "post_attention_layernorm.weight"], eps))
+        h = h + swiglu_ffn(x, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"], stored)
+    x = keep(rmsnorm(h, W["model.norm.weight"], eps))
     lm = W["lm_head.weight"] if ("lm_head.weight" in W and not cfg.get("tie_word_embeddings", False)) \
         else W["model.embed_tokens.weight"]
     return x @ lm.T
