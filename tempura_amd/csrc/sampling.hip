@@ -2,6 +2,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "no_alloc.h"
 
 // ---- argmax -----------------------------------------------------------------------
 // One block per row.  On exact ties the LAST maximum wins, as the reference's greedy
@@ -86,6 +87,39 @@ extern "C" int tp_argmax(const float* logits, int* out, int rows, int vocab, voi
   if (chunks > 1) hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(TP_WAVE), 0, s, pv, pi, chunks, vocab, out);
   TP_CHECK_LAUNCH("argmax");
   return 0;
+}
+
+// ---- argmax without a workspace argument (see no_alloc.h) ---------------------------------
+// The partial results live in a device array of the library itself.  In host code the array's name is only a
+// stand-in for the symbol: its device address is looked up per device, and that pointer is what kernels get.
+static __device__ __align__(256) unsigned char argmax_static_scratch[TP_ARGMAX_STATIC_MAX_ROWS * 64 * 8];
+#define TP_MAX_DEVICES 64
+static void* g_argmax_static_ptr[TP_MAX_DEVICES] = {};
+
+extern "C" int tp_argmax_static_init(void) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  TP_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  TP_REQUIRE(dev >= 0 && dev < TP_MAX_DEVICES, "argmax_static: device %d outside the table of %d", dev, TP_MAX_DEVICES);
+  if (__atomic_load_n(&g_argmax_static_ptr[dev], __ATOMIC_ACQUIRE) != nullptr) return 0;
+  void* ptr = nullptr;
+  e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(argmax_static_scratch));
+  TP_REQUIRE(e == hipSuccess && ptr != nullptr, "argmax_static: hipGetSymbolAddress failed on device %d: %s", dev,
+             hipGetErrorString(e));
+  __atomic_store_n(&g_argmax_static_ptr[dev], ptr, __ATOMIC_RELEASE);   // (two threads racing here store the same address)
+  return 0;
+}
+
+extern "C" int tp_argmax_static(const float* logits, int* out, int rows, int vocab, hipStream_t s) {
+  TP_REQUIRE(rows >= 0 && vocab > 0, "argmax_static: bad sizes");
+  TP_REQUIRE(rows <= TP_ARGMAX_STATIC_MAX_ROWS, "argmax_static: %d rows, the library's scratch array holds %d", rows,
+             TP_ARGMAX_STATIC_MAX_ROWS);
+  if (rows == 0) return 0;
+  if (tp_argmax_static_init() != 0) return 1;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  TP_REQUIRE(e == hipSuccess && dev >= 0 && dev < TP_MAX_DEVICES, "argmax_static: hipGetDevice failed");
+  return tp_argmax(logits, out, rows, vocab, g_argmax_static_ptr[dev], s);
 }
 
 // ---- penalties ----------------------------------------------------------------------
