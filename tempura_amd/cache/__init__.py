@@ -1,5 +1,5 @@
-from .pages import PagePool, PagesExhausted
-from .manager import CacheManager
+from .manager import CacheManager, PagesExhausted
 from .pools import CachePools, LayerCache
+from .rules import VisibilityRule, register_rule
 
-__all__ = ["PagePool", "PagesExhausted", "CacheManager", "CachePools", "LayerCache"]
+__all__ = ["PagesExhausted", "CacheManager", "CachePools", "LayerCache", "VisibilityRule", "register_rule"]

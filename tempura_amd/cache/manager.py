@@ -4,8 +4,9 @@ groups, and slots for fixed-size per-request state.
 Layers whose mixers have the same ``CacheSpec`` form a group; each group has a
 page pool of its own and every request has one block table per group (logical
 page -> physical page), shared by all cache slots of the group.  A ``full``
-group keeps every page until the request ends; a ``window`` group gives a page
-back as soon as no later query can see any key in it.  Pages return to the free
+group keeps every page until the request ends; a group with another visibility
+rule (``window``, ``chunk``; cache/rules.py) gives a page back as soon as no later
+query can see any key in it.  Pages return to the free
 list at once and are handed out again (most recently freed first).
 
 This is host bookkeeping only: it never touches device memory.  The bookkeeping
@@ -24,7 +25,18 @@ import numpy as np
 
 from ..parts.base import CacheSpec
 from . import native
-from .pages import PagesExhausted
+from .rules import rule_args
+
+
+class PagesExhausted(RuntimeError):
+    """Not enough free pages (the reference's ``PoolExhausted{need_pages, free_pages}``,
+    /root/reference/engine/src/cutile_kv_cache.rs:31-44)."""
+
+    def __init__(self, need: int, free: int, group: int = 0):
+        super().__init__(f"cache group {group}: need {need} pages, {free} free")
+        self.need = need
+        self.free = free
+        self.group = group
 
 
 class _PoolView:
@@ -60,9 +72,10 @@ class CacheManager:
             raise ValueError("num_pages must be >= 0")
         self.max_requests = int(max_requests)
         self._lib = native.lib()
-        kinds = [1 if (s.kind == "window" and s.window is not None) else 0 for s in self.groups]
-        windows = [int(s.window) if s.window is not None else 0 for s in self.groups]
-        self._h = ctypes.c_void_p(self._lib.cc_create(len(self.groups), _ints(kinds), _ints(windows), self.page_size,
+        # what each group's queries can still see: a rule of the core and its integers (cache/rules.py)
+        args = [rule_args(s) for s in self.groups]
+        self._h = ctypes.c_void_p(self._lib.cc_create(len(self.groups), _ints([a[0] for a in args]),
+                                                      _ints([p for a in args for p in a[1]]), self.page_size,
                                                       _ints([int(n) for n in num_pages]), self.max_requests))
         if not self._h:
             raise ValueError(native.last_error())
@@ -197,6 +210,28 @@ class CacheManager:
                                       out.ctypes.data_as(ctypes.c_void_p))
         if rc != 0:
             raise RuntimeError(native.last_error())
+
+    def fill_step(self, slots: Sequence[int], n_new: np.ndarray, tokens: np.ndarray, n_want: np.ndarray, want: np.ndarray,
+                  vocab: int, max_positions: int, scratch_pages: Sequence[int], out: np.ndarray):
+        """Pack the device inputs of a step into ``out`` (int32): see ``cc_fill_step`` in the host library for the
+        layout.  The step is checked (``ValueError``) and its pages are reserved (``PagesExhausted``) in the same call;
+        a step that is refused changes nothing.  ``slots``: the state slots of the step's requests (``state_slot``).  Returns the meta list
+        [N, M, total, largest count, largest context, single-token requests, widths per group], or None when
+        ``out`` is too small (then ``self.last_fill_need`` says how many ints are needed)."""
+        meta = (ctypes.c_int * (6 + max(1, len(self.groups))))()
+        rc = self._lib.cc_fill_step(self._h, len(slots), _ints(slots), n_new.ctypes.data_as(ctypes.c_void_p),
+                                    tokens.ctypes.data_as(ctypes.c_void_p), n_want.ctypes.data_as(ctypes.c_void_p),
+                                    want.ctypes.data_as(ctypes.c_void_p), int(vocab), int(max_positions),
+                                    _ints([int(p) for p in scratch_pages]), out.ctypes.data_as(ctypes.c_void_p),
+                                    ctypes.c_long(out.size), meta)
+        if rc == 1:
+            raise PagesExhausted(meta[0], meta[1], meta[2])
+        if rc == 2:
+            self.last_fill_need = int(meta[2])
+            return None
+        if rc != 0:
+            raise ValueError(native.last_error())
+        return list(meta)
 
     # ---- statistics and invariants -------------------------------------
     def free_pages(self) -> List[int]:

@@ -21,12 +21,10 @@ def lib():
             raise RuntimeError(f"cannot load the host library {path}: {e}") from e
         l.cc_last_error.restype = ctypes.c_char_p
         l.cc_create.restype = ctypes.c_void_p
-        l.pp_create.restype = ctypes.c_void_p
         l.cc_waste_ratio.restype = ctypes.c_double
         for name in ("cc_destroy", "cc_add", "cc_release", "cc_num_tokens", "cc_pages_needed", "cc_reserve", "cc_commit",
                      "cc_truncate", "cc_table_len", "cc_table", "cc_slots", "cc_free_pages", "cc_num_live",
-                     "cc_waste_ratio", "cc_check", "cc_fill_decode", "pp_destroy", "pp_num_free", "pp_alloc", "pp_free",
-                     "pp_is_held", "pp_check"):
+                     "cc_waste_ratio", "cc_check", "cc_fill_decode", "cc_fill_step", "hr_fill_normal"):
             getattr(l, name).argtypes = None
         _lib = l
     return _lib

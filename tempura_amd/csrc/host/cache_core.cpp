@@ -1,6 +1,7 @@
 // Host bookkeeping of the paged cache, in C++ behind a C interface: page pools (LIFO free lists with
-// conservation checks), per-request block tables per cache group, window groups that give pages back,
-// state slots, and the packing of a decode step's device inputs.  It never touches device memory.
+// conservation checks), per-request block tables per cache group, groups whose queries stop seeing old keys
+// and give those pages back, state slots, and the packing of a step's device inputs (a decode step's, and
+// any mixed step's).  It never touches device memory.
 //
 // The reference keeps the same bookkeeping natively: a LIFO page allocator whose invariant is
 // available + in_use == total (/root/reference/engine/src/kv_cache.rs:762-795,
@@ -81,21 +82,29 @@ struct Request {
   std::vector<int> first_live;             // per group: first logical page still held
 };
 
-enum { KIND_FULL = 0, KIND_WINDOW = 1 };
+// ---- what a group's queries can still see ------------------------------------------------------
+// A group's rule is data: a code into RULES and up to RULE_PARAMS integers.  A rule gives the first key that
+// a query at position `pos` can see; it must never decrease as pos grows, because the pages below it go back
+// to the pool for good.  Another rule is one more function and one more line of the table; the host side
+// names the codes in one place (tempura_amd/cache/rules.py).
+enum { RULE_PARAMS = 4 };
+typedef int (*FirstVisible)(int pos, const int* params);
+int rule_all(int, const int*) { return 0; }                                        // every key, always
+int rule_last_n(int pos, const int* p) { return p[0] > 0 ? std::max(0, pos - p[0] + 1) : 0; }   // a window of p[0] keys
+int rule_chunk(int pos, const int* p) { return p[0] > 0 ? pos / p[0] * p[0] : 0; }  // the query's own chunk of p[0] positions
+const FirstVisible RULES[] = {rule_all, rule_last_n, rule_chunk};
+const int NUM_RULES = (int)(sizeof(RULES) / sizeof(RULES[0]));
 
 struct Core {
   int page_size = 0, max_requests = 0;
-  std::vector<int> kind, window;
+  std::vector<int> rule, params;   // per group: code, RULE_PARAMS integers
   std::vector<Pool> pools;
   std::vector<Request> reqs;
   std::vector<int> free_state;
 
   int n_groups() const { return (int)pools.size(); }
   // first logical page a query at position `start` can still see
-  int first_needed(int g, int start) const {
-    if (kind[g] == KIND_WINDOW && window[g] > 0) return std::max(0, start - window[g] + 1) / page_size;
-    return 0;
-  }
+  int first_needed(int g, int start) const { return RULES[rule[g]](start, &params[(size_t)g * RULE_PARAMS]) / page_size; }
   // pages group g must allocate so that the request can take n_new more tokens
   int pages_needed(const Request& r, int g, int n_new) const {
     const int end = r.num_tokens + n_new;
@@ -147,35 +156,19 @@ extern "C" {
 
 const char* cc_last_error() { return g_error.c_str(); }
 
-// ---- a page pool on its own ---------------------------------------------------------------
-void* pp_create(int num_pages) {
-  if (num_pages < 0) {
-    fail("num_pages must be >= 0");
-    return nullptr;
-  }
-  return new Pool(num_pages);
-}
-void pp_destroy(void* h) { delete (Pool*)h; }
-int pp_num_free(void* h) { return ((Pool*)h)->num_free(); }
-int pp_alloc(void* h) {  // the page, or -1 when none is free
-  Pool* p = (Pool*)h;
-  if (p->free_list.empty()) return fail("need 1 pages, 0 free");
-  return p->alloc();
-}
-int pp_free(void* h, int page) { return ((Pool*)h)->release(page); }
-int pp_is_held(void* h, int page) {
-  Pool* p = (Pool*)h;
-  return page >= 0 && page < p->num_pages && p->held[page];
-}
-int pp_check(void* h) { return ((Pool*)h)->check(); }
-
 // ---- the cache manager -----------------------------------------------------------------------
-void* cc_create(int n_groups, const int* kind, const int* window, int page_size, const int* num_pages,
+// rule[g]: a code into RULES; params: RULE_PARAMS integers per group.
+void* cc_create(int n_groups, const int* rule, const int* params, int page_size, const int* num_pages,
                 int max_requests) {
   if (page_size <= 0 || n_groups < 0 || max_requests < 0) {
     fail("page_size must be positive");
     return nullptr;
   }
+  for (int g = 0; g < n_groups; ++g)
+    if (rule[g] < 0 || rule[g] >= NUM_RULES) {
+      fail("group %d: unknown visibility rule %d (the core has %d)", g, rule[g], NUM_RULES);
+      return nullptr;
+    }
   Core* c = new Core;
   c->page_size = page_size;
   c->max_requests = max_requests;
@@ -185,8 +178,8 @@ void* cc_create(int n_groups, const int* kind, const int* window, int page_size,
       fail("num_pages must be >= 0");
       return nullptr;
     }
-    c->kind.push_back(kind[g]);
-    c->window.push_back(window[g]);
+    c->rule.push_back(rule[g]);
+    for (int i = 0; i < RULE_PARAMS; ++i) c->params.push_back(params[(size_t)g * RULE_PARAMS + i]);
     c->pools.emplace_back(num_pages[g]);
   }
   c->reqs.resize(max_requests);
@@ -429,6 +422,125 @@ int cc_fill_decode(void* h, int n, const int* reqs, const int* tokens, int rows,
       if (lp >= (int)table.size() || table[lp] < 0) return fail("position %d has no page reserved", p);
       maps[(size_t)g * rows + i] = table[lp] * c->page_size + p % c->page_size;
     }
+  }
+  return 0;
+}
+
+// A whole step in one call: check it, reserve its pages, and pack its device inputs into one int32 buffer.
+// Request reqs[i] brings n_new[i] tokens (tokens: all of them, flattened) and wants the logits at n_want[i] of
+// its places (want: indices into its own tokens, flattened).  With N tokens, R requests and M wanted places:
+//   tokens[N] positions[N] token_req[N] cu_seqlens[R + 1] context_lens[R] state_slots[R] logit_rows[M]
+//   then per group block_tables[R, width_g], then per group slot_mapping[N]
+// width_g is the longest table of the step in group g (at least 1); entries without a page point at the
+// scratch page.  meta receives {N, M, total, largest n_new, largest context, requests with one token, widths...}.
+// Returns 0; 1 when a pool cannot give the step's pages (meta = {need, free, group}); 2 when `capacity` ints
+// do not hold the buffer (meta[2] says how many are needed); -1 for a step that is refused (a token outside
+// the vocabulary, a wanted place outside its tokens, a request twice, a length above max_positions).  With
+// 1, 2 or a refused step nothing has changed: no page is reserved and nothing is written.
+int cc_fill_step(void* h, int n, const int* reqs, const int* n_new, const int* tokens, const int* n_want, const int* want,
+                 int vocab, int max_positions, const int* scratch_page, int* out, long capacity, int* meta) {
+  Core* c = (Core*)h;
+  const int G = c->n_groups(), ps = c->page_size;
+  if (n <= 0) return fail("a step needs at least one entry");
+  long N = 0, M = 0;
+  int max_q = 0, max_ctx = 0, singles = 0;
+  std::vector<int> width(G, 1);
+  std::vector<long> need(G, 0);
+  std::vector<uint8_t> in_step(c->max_requests, 0);
+  for (int i = 0; i < n; ++i) {
+    Request* r = c->live(reqs[i]);
+    if (!r) return -1;
+    if (in_step[reqs[i]]) return fail("entry %d: its request appears twice in one step", i);
+    in_step[reqs[i]] = 1;
+    if (n_new[i] <= 0) return fail("entry %d: a step entry needs at least one token", i);
+    if (n_want[i] < 0) return fail("entry %d: negative count of wanted places", i);
+    const long end = (long)r->num_tokens + n_new[i];
+    if (end > max_positions) return fail("entry %d: %ld tokens exceed max positions %d", i, end, max_positions);
+    for (int j = 0; j < n_new[i]; ++j) {
+      const int t = tokens[N + j];
+      if (t < 0 || t >= vocab) return fail("entry %d: token id %d outside the vocabulary of %d", i, t, vocab);
+    }
+    for (int j = 0; j < n_want[i]; ++j) {
+      const int w = want[M + j];
+      if (w < 0 || w >= n_new[i]) return fail("entry %d: wanted place %d outside its %d tokens", i, w, n_new[i]);
+    }
+    N += n_new[i];
+    M += n_want[i];
+    max_q = std::max(max_q, n_new[i]);
+    max_ctx = std::max(max_ctx, (int)end);
+    singles += n_new[i] == 1;
+    for (int g = 0; g < G; ++g) {
+      width[g] = std::max(width[g], std::max((int)r->tables[g].size(), (int)((end + ps - 1) / ps)));
+      need[g] += c->pages_needed(*r, g, n_new[i]);
+    }
+  }
+  for (int g = 0; g < G; ++g)
+    if (need[g] > c->pools[g].num_free()) {
+      meta[0] = (int)need[g];
+      meta[1] = c->pools[g].num_free();
+      meta[2] = g;
+      return 1;
+    }
+  long total = 3 * N + (n + 1) + 2L * n + M + (long)G * N;
+  for (int g = 0; g < G; ++g) total += (long)n * width[g];
+  if (total > 0x7fffffffL) return fail("the step's inputs exceed 2^31 integers");
+  meta[0] = (int)N;
+  meta[1] = (int)M;
+  meta[2] = (int)total;
+  meta[3] = max_q;
+  meta[4] = max_ctx;
+  meta[5] = singles;
+  for (int g = 0; g < G; ++g) meta[6 + g] = width[g];
+  if (total > capacity) return 2;
+  for (int i = 0; i < n; ++i) c->grow(c->reqs[reqs[i]], n_new[i]);
+
+  int* tok = out;
+  int* pos = tok + N;
+  int* treq = pos + N;
+  int* cu = treq + N;
+  int* ctxl = cu + (n + 1);
+  int* slot = ctxl + n;
+  int* rows = slot + n;
+  int* tables = rows + M;
+  int* maps = tables;
+  for (int g = 0; g < G; ++g) maps += (long)n * width[g];
+  long t0 = 0, w0 = 0;
+  cu[0] = 0;
+  for (int i = 0; i < n; ++i) {
+    const Request& r = c->reqs[reqs[i]];
+    const int cnt = n_new[i];
+    for (int j = 0; j < cnt; ++j) {
+      tok[t0 + j] = tokens[t0 + j];
+      pos[t0 + j] = r.num_tokens + j;
+      treq[t0 + j] = i;
+    }
+    for (int j = 0; j < n_want[i]; ++j) rows[w0 + j] = (int)t0 + want[w0 + j];
+    cu[i + 1] = (int)(t0 + cnt);
+    ctxl[i] = r.num_tokens + cnt;
+    slot[i] = reqs[i];
+    t0 += cnt;
+    w0 += n_want[i];
+  }
+  int* bt = tables;
+  int* mp = maps;
+  for (int g = 0; g < G; ++g) {
+    const int wd = width[g];
+    t0 = 0;
+    for (int i = 0; i < n; ++i) {
+      const Request& r = c->reqs[reqs[i]];
+      const std::vector<int>& table = r.tables[g];
+      int* row = bt + (long)i * wd;
+      // pages a rule has given back, and what lies past the table, point at the scratch page; no query reads them
+      for (int lp = 0; lp < wd; ++lp) row[lp] = (lp < (int)table.size() && table[lp] >= 0) ? table[lp] : scratch_page[g];
+      for (int j = 0; j < n_new[i]; ++j) {
+        const int p = r.num_tokens + j, lp = p / ps;
+        if (lp >= (int)table.size() || table[lp] < 0) return fail("entry %d: position %d has no page in group %d", i, p, g);
+        mp[t0 + j] = table[lp] * ps + p % ps;
+      }
+      t0 += n_new[i];
+    }
+    bt += (long)n * wd;
+    mp += N;
   }
   return 0;
 }

@@ -67,6 +67,9 @@ class Engine:
         self.counters = {"steps": 0, "prompt_tokens": 0, "generated_tokens": 0, "batched_tokens": 0, "chained_steps": 0}
         self.chain_steps = bool(chain_steps) and self.runner.use_graph     # (a model with parts that cannot be captured runs eagerly)
         self._ahead = None      # (requests, logits) of a step that is already queued
+        #: what the last call of ``step`` ran: single decoded tokens, prompt tokens in portions, requests, and
+        #: whether the step had been queued ahead
+        self.last_step = {"decode_tokens": 0, "prompt_tokens": 0, "requests": 0, "queued_ahead": False}
 
     def _pages_from_memory(self, utilization: float, max_batch_size: int) -> int:
         m = self.model
@@ -120,17 +123,21 @@ class Engine:
             items = [ScheduledItem(reqs[i], reqs[i].num_tokens - 1, 1, True) for i in live]
             if len(live) < len(reqs):
                 logits = logits[torch.tensor(live, dtype=torch.long, device=self.device)]
+            self.last_step = {"decode_tokens": len(items), "prompt_tokens": 0, "requests": len(items), "queued_ahead": True}
         else:
             items = self.scheduler.schedule()
             if not items:
                 return []
             entries = []
             for it in items:
-                toks = it.request.tokens[it.start: it.start + it.count]
+                toks = it.request.step_tokens(it.start, it.count)
                 entries.append(StepEntry(it.request.rid, toks, [it.count - 1] if it.samples else []))
             logits = self.runner.step(entries)
             self.counters["steps"] += 1
             self.counters["batched_tokens"] += sum(it.count for it in items)
+            decoding = sum(1 for it in items if it.count == 1 and it.samples and it.request.output)
+            self.last_step = {"decode_tokens": decoding, "prompt_tokens": sum(it.count for it in items) - decoding,
+                              "requests": len(items), "queued_ahead": False}
         for it in items:
             self.scheduler.advance(it)
         sampling = [it.request for it in items if it.samples]
@@ -267,4 +274,6 @@ class Engine:
         s["cache_bytes"] = self.runner.pools.bytes()
         s["weight_bytes"] = self.model.weight_bytes()
         s["graph_steps"] = self.runner.graph_steps
+        s["eager_steps"] = self.runner.host_steps["pack"]
+        s["eager_step_pack_ms"] = 1e3 * self.runner.host_seconds["pack"] / max(1, self.runner.host_steps["pack"])
         return s

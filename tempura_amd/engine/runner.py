@@ -9,6 +9,9 @@ sequence of n tokens, or m sequences of exactly one token,
 """
 from __future__ import annotations
 
+import itertools
+import re
+import time
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
@@ -122,6 +125,43 @@ class _DecodeGraph:
         return ctx
 
 
+class _PackedStaging:
+    """Host buffers for the packed inputs of eager steps on their way to the device.  On a GPU they are pinned
+    and taken in turn from a small ring, so that the copy is queued behind the work in flight instead of making
+    the host wait for it (a copy from pageable memory would); a buffer is used again once its copy has run."""
+    RING = 4
+
+    def __init__(self, device):
+        self.device = device
+        self.cuda = torch.device(device).type == "cuda"
+        self.slots = [None] * self.RING          # (tensor, numpy view, event)
+        self.turn = 0
+
+    def take(self, need: int) -> np.ndarray:
+        """A host buffer of at least ``need`` int32 (the next of the ring), free to be written.  The ring moves
+        on when the buffer is sent; a buffer that is taken and not sent is simply taken again."""
+        slot = self.slots[self.turn]
+        if slot is None or slot[0].numel() < need:
+            size = max(4096, 1 << int(need - 1).bit_length())
+            t = torch.empty(size, dtype=torch.int32, pin_memory=self.cuda)
+            slot = (t, t.numpy(), torch.cuda.Event() if self.cuda else None)
+            self.slots[self.turn] = slot
+        elif slot[2] is not None:
+            slot[2].synchronize()                # the copy that last used this buffer has run
+        return slot[1]
+
+    def send(self, total: int) -> torch.Tensor:
+        """The first ``total`` ints of the buffer taken last, as a device tensor."""
+        t, arr, event = self.slots[self.turn]
+        self.turn = (self.turn + 1) % self.RING
+        if not self.cuda:
+            return t[:total].clone()
+        dev = torch.empty(total, dtype=torch.int32, device=self.device)
+        dev.copy_(t[:total], non_blocking=True)
+        event.record()
+        return dev
+
+
 class ModelRunner:
     def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
                  cache_dtype: Optional[torch.dtype] = None, use_graph: bool = False):
@@ -146,6 +186,10 @@ class ModelRunner:
                                                 self.pools.state.get(call.cache)))
         self.steps_run = 0
         self.tokens_run = 0
+        self._staging = _PackedStaging(self.device)
+        #: host time spent packing the inputs of eager steps, and how many such steps there were
+        self.host_seconds = {"pack": 0.0}
+        self.host_steps = {"pack": 0}
         # Decode-only steps replay a captured graph when every part of the model allows it.
         self.use_graph = bool(use_graph) and self.device.type == "cuda" and not model.state_specs and \
             all(getattr(p, "graph_safe", False) for layer in model.layers for p in layer.parts())
@@ -198,57 +242,78 @@ class ModelRunner:
         """Pages for every entry, or ``PagesExhausted`` with nothing changed."""
         self.cache.reserve_many([e.rid for e in entries], [len(e.tokens) for e in entries])
 
-    def build_context(self, entries: Sequence[StepEntry]):
-        """Host side of a step: flatten the batch and describe it (pages must be reserved)."""
-        n_groups = len(self.cache.groups)
+    def _pack_step(self, entries: Sequence[StepEntry]):
+        """Host side of a step, one call into the host library: the step is checked, its pages are reserved (all or
+        nothing, ``PagesExhausted``) and its device inputs are packed into one pinned buffer that goes to the
+        device in one copy.  Returns (tokens on the device, context).  A refused step changes nothing."""
+        t_start = time.perf_counter()
         R = len(entries)
-        q_lens = [len(e.tokens) for e in entries]
-        starts = [self.cache.num_tokens(e.rid) for e in entries]
-        N = sum(q_lens)
-        cu = np.zeros(R + 1, dtype=np.int32)
-        cu[1:] = np.cumsum(q_lens)
-        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
-        positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, q_lens)])
-        token_req = np.repeat(np.arange(R, dtype=np.int32), q_lens)
-        ctx_lens = np.asarray([s + n for s, n in zip(starts, q_lens)], dtype=np.int32)
-        state_slots = np.asarray([self.cache.state_slot(e.rid) for e in entries], dtype=np.int32)
-        rows: List[int] = []
-        for r, e in enumerate(entries):
-            rows.extend(int(cu[r]) + int(w) for w in e.want)
-        logit_rows = np.asarray(rows, dtype=np.int32)
-        tables, slots = [], []
-        for g in range(n_groups):
-            width = max(1, max(len(self.cache.table(e.rid, g)) for e in entries))
-            bt = np.full((R, width), self.pools.scratch_page(g), dtype=np.int32)
-            for r, e in enumerate(entries):
-                t = np.asarray(self.cache.table(e.rid, g), dtype=np.int32)
-                # Pages a window has given back stay pointed at the scratch page; no query reads them.
-                bt[r, : len(t)] = np.where(t >= 0, t, self.pools.scratch_page(g))
-            tables.append(bt)
-            slots.append(np.concatenate([self.cache.slots(e.rid, g, s, n)
-                                         for e, s, n in zip(entries, starts, q_lens)]).astype(np.int32))
-
-        # One packed host buffer, one copy to the device, then views.
-        pieces = [tokens, positions, token_req, cu, ctx_lens, state_slots, logit_rows] + \
-                 [t.reshape(-1) for t in tables] + slots
-        offs = np.cumsum([0] + [p.size for p in pieces])
-        packed = torch.from_numpy(np.concatenate(pieces)).to(self.device)
-        view = [packed[offs[i]: offs[i + 1]] for i in range(len(pieces))]
-
+        cache = self.cache
+        try:
+            slots = [cache._slot_of[e.rid] for e in entries]
+        except KeyError:
+            bad = next(e.rid for e in entries if not cache.has(e.rid))
+            raise ValueError(f"request {bad!r} is not live; add_request first") from None
+        try:
+            n_new = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=R)
+            pieces = [np.asarray(e.tokens, dtype=np.int32) for e in entries]
+            tokens = pieces[0].reshape(-1) if R == 1 else np.concatenate(pieces, axis=None)
+            n_want = np.fromiter((len(e.want) for e in entries), dtype=np.int32, count=R)
+            want = np.fromiter(itertools.chain.from_iterable(e.want for e in entries), dtype=np.int32, count=int(n_want.sum()))
+        except OverflowError:
+            raise ValueError(f"a token id or wanted place outside the vocabulary of {self.model.spec.vocab_size}") from None
+        tokens = np.ascontiguousarray(tokens)
+        scratch = [self.pools.scratch_page(g) for g in range(len(cache.groups))]
+        spec = self.model.spec
+        guess = 4 * int(tokens.size) + 4 * R + int(want.size) + len(cache.groups) * (int(tokens.size) + R * 64) + 64
+        while True:
+            host = self._staging.take(guess)
+            try:
+                meta = cache.fill_step(slots, n_new, tokens, n_want, want, spec.vocab_size, spec.max_positions, scratch, host)
+            except ValueError as e:
+                msg = str(e)
+                m = re.match(r"entry (\d+): (.*)", msg)
+                if m:
+                    msg = f"request {entries[int(m.group(1))].rid!r}: {m.group(2)}"
+                raise ValueError(msg) from None
+            if meta is not None:
+                break
+            guess = cache.last_fill_need
+        N, M, total, max_q, max_ctx, singles = meta[:6]
+        widths = meta[6: 6 + len(cache.groups)]
+        n_groups = len(cache.groups)
+        # what parts that loop over requests on the host may read (the pinned buffer is used again later)
+        o = 3 * N
+        cu = host[o: o + R + 1].copy()
+        ctx_lens = host[o + R + 1: o + 2 * R + 1].copy()
+        packed = self._staging.send(total)
         ctx = StepContext()
         ctx.num_tokens, ctx.num_requests = N, R
-        tok_dev, ctx.positions, ctx.token_req, ctx.cu_seqlens, ctx.context_lens, ctx.state_slots, ctx.logit_rows = view[:7]
-        ctx.block_tables = [view[7 + g].view(R, tables[g].shape[1]) for g in range(n_groups)]
-        ctx.slot_mapping = view[7 + n_groups: 7 + 2 * n_groups]
-        ctx.max_q_len = max(q_lens)
-        ctx.num_single = sum(1 for n in q_lens if n == 1)
-        ctx.max_context_len = int(ctx_lens.max())
+        tok_dev = packed[:N]
+        ctx.positions = packed[N: 2 * N]
+        ctx.token_req = packed[2 * N: 3 * N]
+        ctx.cu_seqlens = packed[o: o + R + 1]
+        ctx.context_lens = packed[o + R + 1: o + 2 * R + 1]
+        ctx.state_slots = packed[o + 2 * R + 1: o + 3 * R + 1]
+        o += 3 * R + 1
+        ctx.logit_rows = packed[o: o + M]
+        o += M
+        ctx.block_tables = []
+        for g in range(n_groups):
+            ctx.block_tables.append(packed[o: o + R * widths[g]].view(R, widths[g]))
+            o += R * widths[g]
+        ctx.slot_mapping = [packed[o + g * N: o + (g + 1) * N] for g in range(n_groups)]
+        ctx.max_q_len = max_q
+        ctx.num_single = singles
+        ctx.max_context_len = max_ctx
         ctx.page_size = self.page_size
-        ctx.q_starts = [int(c) for c in cu[:-1]]
-        ctx.q_lens = q_lens
-        ctx.ctx_lens = [int(c) for c in ctx_lens]
-        ctx.state_slot_list = [int(s) for s in state_slots]
-        return tok_dev, ctx, starts
+        ctx.q_starts = cu[:-1].tolist()
+        ctx.q_lens = n_new.tolist()
+        ctx.ctx_lens = ctx_lens.tolist()
+        ctx.state_slot_list = slots
+        self.host_seconds["pack"] += time.perf_counter() - t_start
+        self.host_steps["pack"] += 1
+        return tok_dev, ctx
 
     # ---- decode steps as a graph -----------------------------------------
     def _graph_for(self, rows: int, ctx_len: int) -> Optional[_DecodeGraph]:
@@ -370,9 +435,11 @@ class ModelRunner:
         ordered by entry and then by ``want``.  After a decode-only step the result is a view of
         the graph's output buffer: use it before the next step."""
         entries = list(entries)
-        self._check_entries(entries)
-        self.reserve(entries)
+        if not entries:
+            raise ValueError("a step needs at least one entry")
         if self.use_graph and all(len(e.tokens) == 1 for e in entries):
+            self._check_entries(entries)
+            self.reserve(entries)
             logits = self._graph_step([e.rid for e in entries], [e.tokens[0] for e in entries],
                                       [r for r, e in enumerate(entries) if len(e.want) > 0])
             self.cache.commit_many([e.rid for e in entries], [1] * len(entries))
@@ -380,17 +447,16 @@ class ModelRunner:
             self.tokens_run += len(entries)
             return logits
         self._prepared = None
-        tok_dev, ctx, starts = self.build_context(entries)
+        tok_dev, ctx = self._pack_step(entries)
         # A request that starts at position 0 gets a cleared state (also after a recompute).
         if self.pools.state:
-            fresh = [ctx.state_slot_list[r] for r, s in enumerate(starts) if s == 0]
+            fresh = [s for s, n, c in zip(ctx.state_slot_list, ctx.q_lens, ctx.ctx_lens) if c == n]
             if fresh:
                 idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
                 for t in self.pools.state.values():
                     t.index_fill_(0, idx, 0)
         logits = self.model.forward(tok_dev, ctx, self.layer_caches)
-        for e in entries:
-            self.cache.commit(e.rid, len(e.tokens))
+        self.cache.commit_many([e.rid for e in entries], ctx.q_lens)
         self.steps_run += 1
         self.tokens_run += ctx.num_tokens
         return logits

@@ -23,7 +23,10 @@ from dataclasses import dataclass, field
 from enum import Enum
 from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 from ..cache import CacheManager
+from ..cache.rules import rule_of
 from ..sampling.params import SamplingParams
 
 
@@ -47,6 +50,7 @@ class Request:
     arrival: int = 0
     logprobs_top_n: Optional[int] = None     # not None: keep a log-probability record per generated token
     logprobs: List[object] = field(default_factory=list)
+    _array: Optional[object] = field(default=None, repr=False, compare=False)
 
     @property
     def tokens(self) -> List[int]:
@@ -55,6 +59,17 @@ class Request:
     @property
     def num_tokens(self) -> int:
         return len(self.prompt) + len(self.output)
+
+    def step_tokens(self, start: int, count: int):
+        """Tokens start .. start + count - 1 of prompt + output, as a step entry takes them: the newest token alone
+        as a list, a portion as a slice of an int32 array that is made once per prefill (not once per step)."""
+        n = self.num_tokens
+        if count == 1 and start == n - 1 and self.output:
+            return self.output[-1:]
+        arr = self._array
+        if arr is None or arr.size != n:
+            arr = self._array = np.asarray(self.prompt + self.output, dtype=np.int32)
+        return arr[start: start + count]
 
     @property
     def is_decoding(self) -> bool:
@@ -110,12 +125,13 @@ class Scheduler:
         # It must fit the pool when it is the only request, or it could never finish.
         need_tokens = min(total, limit)
         ps = self.cache.page_size
+        step = min(self.config.prefill_chunk_size, self.config.max_num_batched_tokens)
         for g, pool in enumerate(self.cache.pools):
             spec = self.cache.groups[g]
-            tokens_held = need_tokens
-            if spec.kind == "window" and spec.window is not None:
-                tokens_held = min(need_tokens, spec.window + min(self.config.prefill_chunk_size,
-                                                                 self.config.max_num_batched_tokens) + ps)
+            # (a group that gives pages back holds what its rule still shows plus the step in flight and a page of slack)
+            tokens_held = rule_of(spec.kind).held_tokens(spec, need_tokens, step)
+            if tokens_held < need_tokens:
+                tokens_held = min(need_tokens, tokens_held + ps)
             if (tokens_held + ps - 1) // ps > pool.num_pages:
                 raise ValueError(
                     f"request {req.rid!r}: needs {(tokens_held + ps - 1) // ps} pages of cache group {g}, the pool has {pool.num_pages}")

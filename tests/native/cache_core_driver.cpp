@@ -9,7 +9,7 @@
 #include <vector>
 
 extern "C" {
-void* cc_create(int n_groups, const int* kind, const int* window, int page_size, const int* num_pages, int max_requests);
+void* cc_create(int n_groups, const int* rule, const int* params, int page_size, const int* num_pages, int max_requests);
 void cc_destroy(void*);
 int cc_add(void*);
 int cc_release(void*, int);
@@ -39,7 +39,7 @@ int main(int argc, char** argv) {
   const unsigned seed = argc > 1 ? (unsigned)atoi(argv[1]) : 1;
   std::mt19937 rng(seed);
   auto pick = [&](int n) { return (int)(rng() % (unsigned)n); };
-  const int kinds[2] = {0, 1}, windows[2] = {0, 24}, pages[2] = {40, 14};
+  const int kinds[2] = {0, 1}, windows[8] = {0, 0, 0, 0, 24, 0, 0, 0}, pages[2] = {40, 14};
   const int page_size = 4 << pick(3), max_req = 5;
   void* c = cc_create(2, kinds, windows, page_size, pages, max_req);
   REQUIRE(c != nullptr);

@@ -4,28 +4,32 @@ import random
 
 import pytest
 
-from tempura_amd.cache import CacheManager, PagePool, PagesExhausted
+from tempura_amd.cache import CacheManager, PagesExhausted
 from tempura_amd.parts import CacheSpec
 
 FULL = CacheSpec("full", 2, 16)
 WIN = CacheSpec("window", 2, 16, window=24)
 
 
-def test_page_pool_conservation_and_double_free():
+def test_pages_are_conserved_and_used_again_most_recent_first():
     # invariant available + in_use == total (/root/reference/kernel-api/src/lib.rs:604-618)
-    p = PagePool(4)
-    a, b = p.alloc(), p.alloc()
-    assert p.num_free == 2 and p.num_held == 2 and a != b
-    p.free(a)
-    with pytest.raises(ValueError, match="freed twice"):
-        p.free(a)
-    with pytest.raises(ValueError, match="out of range"):
-        p.free(9)
-    assert p.alloc() == a                       # most recently freed page is used again first
-    p.alloc(), p.alloc()
+    m = CacheManager([FULL], page_size=4, num_pages=4, max_requests=3)
+    for rid in "ab":
+        m.add(rid)
+        m.reserve(rid, 4)
+        m.commit(rid, 4)
+    (pa,), (pb,) = m.table("a", 0), m.table("b", 0)
+    assert pa != pb and m.free_pages() == [2]
+    m.release("a")
+    with pytest.raises(ValueError, match="not live"):
+        m.release("a")                          # nothing is freed twice
+    m.add("c")
+    m.reserve("c", 12)
+    assert m.table("c", 0)[0] == pa             # the most recently freed page is used again first
+    m.add("a")
     with pytest.raises(PagesExhausted):
-        p.alloc()
-    p.check()
+        m.reserve("a", 1)
+    m.check()
 
 
 def test_reserve_commit_release():
@@ -190,3 +194,33 @@ def test_fill_decode_packs_what_the_tables_say():
         m.fill_decode(["a"], [1], rows, 3, scratch, out)          # a table of six pages does not fit three columns
     with pytest.raises(RuntimeError):
         m.fill_decode(["c", "a", "b", "c", "a"], [1] * 5, rows, width, scratch, out)   # more requests than rows
+
+
+def test_visibility_rules_are_data():
+    """A group's rule is a code of the host library and a few integers, named in cache/rules.py: ``chunk`` (a
+    query sees the keys of its own aligned chunk) needs no line of the manager, and another kind that maps to one
+    of the library's functions is registered from outside."""
+    from tempura_amd.cache import VisibilityRule, register_rule
+    chunk = CacheSpec("chunk", 2, 16, window=16)
+    m = CacheManager([FULL, chunk], page_size=8, num_pages=[16, 4], max_requests=2)
+    m.add("a")
+    for n in (5, 20, 7, 1, 30):
+        m.reserve("a", n)
+        m.commit("a", n)
+        m.check()
+    # 63 tokens: the next query (position 63) lies in chunk 48..63, so pages below key 48 are back
+    assert m.num_tokens("a") == 63 and [p >= 0 for p in m.table("a", 1)] == [False] * 6 + [True] * 2
+    assert all(p >= 0 for p in m.table("a", 0)) and m.free_pages() == [8, 2]
+    m.reserve("a", 1)
+    m.commit("a", 1)                                 # position 64 opens a new chunk: nothing before it is seen again
+    assert [p >= 0 for p in m.table("a", 1)] == [False] * 8
+    m.release("a")
+    # a kind of one's own over the library's "last n keys" rule, with twice the spec's number
+    register_rule("window2x", VisibilityRule(1, lambda s: (2 * s.window,), lambda s, total, step: min(total, 2 * s.window + step)))
+    m = CacheManager([CacheSpec("window2x", 1, 8, window=8)], page_size=8, num_pages=8, max_requests=1)
+    m.add("b")
+    m.reserve("b", 40)
+    m.commit("b", 40)                                # the next query at 40 sees keys 25..40: pages 0..2 are back
+    assert [p >= 0 for p in m.table("b", 0)] == [False] * 3 + [True] * 2
+    with pytest.raises(ValueError, match="no visibility rule"):
+        CacheManager([CacheSpec("sinks", 1, 8)], page_size=8, num_pages=8, max_requests=1)
