@@ -242,9 +242,3 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   TP_CHECK_LAUNCH("linear");
   return 0;
 }
-
-extern "C" int tp_linear(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,
-                         int N, int K, int allow_mfma, float* scratch, size_t scratch_floats, hipStream_t s) {
-  return tp_linear_fused(x, w, in_dt, out, out_dt, accumulate, M, N, K, allow_mfma, scratch, scratch_floats, nullptr, 0,
-                         0.f, nullptr, nullptr, nullptr, 0, 0, nullptr, s);
-}

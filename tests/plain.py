@@ -155,13 +155,40 @@ def layer_window(cfg: dict, layer: int) -> Optional[int]:
     return None
 
 
-def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtype=torch.float64,
+def decoder_layer(cfg: dict, get, l: int, h: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, stored=None) -> torch.Tensor:
+    """One layer on the residual stream h [T, hidden] of one whole sequence: norm, q/k/v, rope on q and k,
+    attention, o, add, norm, feed-forward, add (/root/reference/engine/src/model.rs:952-1314).
+    ``get(name)`` returns the layer's tensors by checkpoint name."""
+    keep = stored if stored is not None else (lambda t: t)
+    H = cfg["hidden_size"]
+    nH = cfg["num_attention_heads"]
+    nKV = cfg.get("num_key_value_heads", nH)
+    D = cfg.get("head_dim") or H // nH
+    eps = cfg.get("rms_norm_eps", 1e-5)
+    T = h.shape[0]
+    scale = 1.0 / math.sqrt(D)                                          # model.rs:1078
+    p = f"model.layers.{l}."
+    x = keep(rmsnorm(h, get(p + "input_layernorm.weight"), eps))
+    q = (x @ get(p + "self_attn.q_proj.weight").T).reshape(T, nH, D)
+    k = (x @ get(p + "self_attn.k_proj.weight").T).reshape(T, nKV, D)
+    v = keep((x @ get(p + "self_attn.v_proj.weight").T).reshape(T, nKV, D))
+    q = keep(rope(q, pos, inv_freq))
+    k = keep(rope(k, pos, inv_freq))
+    a = keep(attention(q, k, v, scale, layer_window(cfg, l), stored=stored))
+    h = h + a @ get(p + "self_attn.o_proj.weight").T
+    x = keep(rmsnorm(h, get(p + "post_attention_layernorm.weight"), eps))
+    return h + swiglu_ffn(x, get(p + "mlp.gate_proj.weight"), get(p + "mlp.up_proj.weight"), get(p + "mlp.down_proj.weight"), stored)
+
+
+def forward(cfg: dict, weights, tokens: List[int], dtype=torch.float64,
             position_offset: int = 0, stored=None) -> torch.Tensor:
     """Logits [T, vocab] at every position of one whole sequence, no cache.
+    ``weights``: tensors by checkpoint name, or a function name -> tensor (or None for a tensor the checkpoint
+    does not hold) that is asked for each tensor when it is needed, so that a large model can be streamed layer
+    by layer.
     ``position_offset`` shifts every position (positions are session.position + t,
     /root/reference/engine/src/model.rs:686-688); only distances count, so logits must not change.
-    Order inside a layer: norm, q/k/v, rope on q and k, attention, o, add, norm, feed-forward, add
-    (/root/reference/engine/src/model.rs:952-1314); then final norm and output projection
+    Layers in order (``decoder_layer``), then final norm and output projection
     (model.rs:1355-1398), the output matrix being the embedding when the file has none
     (/root/reference/engine/src/weights.rs:156-166).
     ``stored`` (for instance ``as_bfloat16``) is applied to every value that 16-bit serving keeps in 16 bits
@@ -169,11 +196,23 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
     attention output and the gated activations; everything else (sums, norms, softmax statistics, the residual
     stream) stays exact.  The distance of such a run from the exact one is the rounding noise that the storage
     type alone explains, the yardstick the 16-bit engine is measured with."""
-    keep = stored if stored is not None else (lambda t: t)
-    W = {k: v.to(dtype) for k, v in weights.items()}
+    return forward_many(cfg, weights, [tokens], [stored], dtype, position_offset)[0][0]
+
+
+def forward_many(cfg: dict, weights, sequences, stored_variants=(None,), dtype=torch.float64, position_offset: int = 0):
+    """``forward`` for several sequences and several ``stored`` variants at once: result[i][j] is the logits of
+    sequence i under variant j.  Every tensor is fetched once per layer and used for all of them, so a model
+    whose weights are streamed (``weights`` a function) is read once."""
+    if callable(weights):
+        fetch = weights
+    else:
+        fetch = weights.get
+
+    def get(name):
+        t = fetch(name)
+        return None if t is None else t.to(dtype)
     H = cfg["hidden_size"]
     nH = cfg["num_attention_heads"]
-    nKV = cfg.get("num_key_value_heads", nH)
     D = cfg.get("head_dim") or H // nH
     eps = cfg.get("rms_norm_eps", 1e-5)
     theta = cfg.get("rope_theta", 10000.0)
@@ -181,26 +220,31 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
     if rs is not None and rs.get("rope_type", rs.get("type")) in (None, "default"):
         rs = None
     inv_freq = rope_inv_freq(D, theta, rs)
-    T = len(tokens)
-    pos = torch.arange(T) + position_offset
-    h = W["model.embed_tokens.weight"][torch.tensor(tokens)]           # model.rs:672-684, no scaling
-    scale = 1.0 / math.sqrt(D)                                          # model.rs:1078
+    embed = get("model.embed_tokens.weight")
+    hs = [[embed[torch.tensor(tokens)] for _ in stored_variants] for tokens in sequences]    # model.rs:672-684, no scaling
+    pos = [torch.arange(len(tokens)) + position_offset for tokens in sequences]
     for l in range(cfg["num_hidden_layers"]):
-        p = f"model.layers.{l}."
-        x = keep(rmsnorm(h, W[p + "input_layernorm.weight"], eps))
-        q = (x @ W[p + "self_attn.q_proj.weight"].T).reshape(T, nH, D)
-        k = (x @ W[p + "self_attn.k_proj.weight"].T).reshape(T, nKV, D)
-        v = keep((x @ W[p + "self_attn.v_proj.weight"].T).reshape(T, nKV, D))
-        q = keep(rope(q, pos, inv_freq))
-        k = keep(rope(k, pos, inv_freq))
-        a = keep(attention(q, k, v, scale, layer_window(cfg, l), stored=stored))
-        h = h + a @ W[p + "self_attn.o_proj.weight"].T
-        x = keep(rmsnorm(h, W[p + "post_attention_layernorm.weight"], eps))
-        h = h + swiglu_ffn(x, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"], stored)
-    x = keep(rmsnorm(h, W["model.norm.weight"], eps))
-    lm = W["lm_head.weight"] if ("lm_head.weight" in W and not cfg.get("tie_word_embeddings", False)) \
-        else W["model.embed_tokens.weight"]
-    return x @ lm.T
+        held = {}
+
+        def layer_get(name):
+            if name not in held:
+                held[name] = get(name)
+            return held[name]
+        for i in range(len(sequences)):
+            for j, stored in enumerate(stored_variants):
+                hs[i][j] = decoder_layer(cfg, layer_get, l, hs[i][j], pos[i], inv_freq, stored)
+    norm_w = get("model.norm.weight")
+    lm = None if cfg.get("tie_word_embeddings", False) else get("lm_head.weight")
+    if lm is None:
+        lm = embed
+    out = []
+    for i in range(len(sequences)):
+        row = []
+        for j, stored in enumerate(stored_variants):
+            x = rmsnorm(hs[i][j], norm_w, eps)
+            row.append((stored(x) if stored is not None else x) @ lm.T)
+        out.append(row)
+    return out
 
 
 def greedy_generate(cfg: dict, weights: Dict[str, torch.Tensor], prompt: List[int], n_new: int) -> List[int]:

@@ -248,6 +248,105 @@ def test_model_width_layer_against_plain(tmp_path):
         torch.cuda.empty_cache()
 
 
+def _wide_config(layers, vocab):
+    from tempura_amd.config import LlamaConfig, RopeScaling
+    return LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=layers, num_attention_heads=32,
+                       num_key_value_heads=8, head_dim=128, vocab_size=vocab, max_position_embeddings=131072,
+                       rms_norm_eps=1e-5, rope_theta=500000.0, rope_scaling=RopeScaling("llama3", 8.0, 1.0, 4.0, 8192),
+                       tie_word_embeddings=False)
+
+
+def test_model_width_mixed_schedule_against_plain(tmp_path):
+    """Two layers with the widths of Llama-3.1-8B under the mixed schedule: up to four live requests, portions of
+    some beside single decoded tokens of others, the last 32 tokens of each one by one (decode-only steps replay
+    the graph), and so few pages that finished requests' pages are used again; float32 and bfloat16 against the
+    plain float64 implementation.  The q and k projections are scaled up (scores 16 times those of N(0, 0.02)
+    weights), so that attention is peaked and a wrong key or page moves the logits far beyond the bound."""
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.kernels import ops
+    from tempura_amd.weights import random_weights, write_safetensors
+    ops.set_backend(None)
+    cfg = _wide_config(2, 8192)
+    W = random_weights(cfg, seed=4, std=0.02, dtype="bfloat16")
+    for name in W:
+        if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
+            W[name] = (W[name].float() * 4.0).to(torch.bfloat16)
+    folder = tmp_path / "wide2"
+    folder.mkdir()
+    (folder / "config.json").write_text(cfg.to_json())
+    write_safetensors(str(folder / "model.safetensors"), W.items())
+    del W
+    pc, PW = plain.read_model_dir(str(folder))
+    lengths = {"w0": 150, "w1": 97, "w2": 210, "w3": 64, "w4": 131, "w5": 40}
+    requests = {rid: helpers.random_tokens(8192, n, seed=300 + i) for i, (rid, n) in enumerate(lengths.items())}
+    max_tokens = 256 + 192 + 64                 # room for about three requests: pages must come back and be used again
+    steps = helpers.schedule_mixed(lengths, max_tokens, seed=9)
+    assert max(len(e) for e, _ in steps) >= 3 and any(len(e) > 1 and all(c == 1 for _, _, c in e) for e, _ in steps)
+    for dtype in ("float32", "bfloat16"):
+        refs = {rid: helpers.plain_reference(pc, PW, toks, dtype) for rid, toks in requests.items()}
+        model = load_model(str(folder), dtype, "cuda:0")
+        runner = ModelRunner(model, 16, max_tokens // 16, max_requests=4, use_graph=True)
+        got = helpers.run_schedule(runner, requests, steps)
+        assert runner.graph_steps > 0 and not runner.cache.live_requests()
+        for rid, (exact, bound) in refs.items():
+            err = helpers.rel_err(got[rid], exact)
+            assert err <= bound, f"{dtype}: request {rid} differs from the plain implementation by {err:.3e} (bound {bound:.3e}), " \
+                                 f"first at {helpers.first_difference(got[rid], exact, bound)}"
+        del model, runner
+        torch.cuda.empty_cache()
+
+
+def test_full_depth_model_against_plain_streamed():
+    """All 32 layers of the Llama-3.1-8B preset (vocabulary 128,256), weights made in device memory, under a mixed
+    schedule of three requests (portions, single tokens, pages used again): the float32 engine and the bfloat16
+    engine against the plain float64 implementation, which gets every tensor from the same generator, one at a
+    time (``fill_normal`` has the bits of its numpy twin, tests/plain_random.py), so that no layer's weights are
+    ever held twice."""
+    from tempura_amd.config import PRESETS, LlamaConfig
+    from tempura_amd.engine.loading import random_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.kernels import ops
+    import plain_random
+    ops.set_backend(None)
+    cfg = LlamaConfig.from_dict(PRESETS["llama-3.1-8b"].to_dict())
+    cfg.validate()
+    seed, std = 6, 0.02
+    pc = json.loads(cfg.to_json())
+    expected = None
+
+    def get(name):
+        """The tensor as the device generator makes it (bfloat16 values), widened on the host."""
+        info = expected[name]
+        if info.init == "ones":
+            return torch.ones(info.shape, dtype=torch.float64)
+        t = ops.fill_normal(torch.empty(info.shape, dtype=torch.bfloat16, device="cuda:0"), plain_random.tensor_key(seed, name), 0.0, std)
+        return t.cpu().double()
+
+    lengths = {"f0": 96, "f1": 40, "f2": 70}
+    requests = {rid: helpers.random_tokens(cfg.vocab_size, n, seed=400 + i) for i, (rid, n) in enumerate(lengths.items())}
+    max_tokens = 128 + 64
+    steps = helpers.schedule_mixed(lengths, max_tokens, seed=3)
+    refs = None
+    for dtype in ("float32", "bfloat16"):
+        model = random_model(cfg, seed=seed, dtype=dtype, device="cuda:0", std=std, values_as="bfloat16")
+        if refs is None:
+            expected = model.expected_weights()
+            both = plain.forward_many(pc, get, list(requests.values()), [None, plain.as_bfloat16])      # one pass over the weights
+            exact = {rid: both[i][0] for i, rid in enumerate(requests)}
+            noisy = {rid: both[i][1] for i, rid in enumerate(requests)}
+            refs = {"float32": {rid: (exact[rid], helpers.TOL["float32"]) for rid in requests},
+                    "bfloat16": {rid: (exact[rid], helpers.BF16_FACTOR * helpers.rel_err(noisy[rid], exact[rid])) for rid in requests}}
+        runner = ModelRunner(model, 16, max_tokens // 16, max_requests=4, use_graph=True)
+        got = helpers.run_schedule(runner, requests, steps)
+        for rid, (ex, bound) in refs[dtype].items():
+            err = helpers.rel_err(got[rid], ex)
+            assert err <= bound, f"{dtype}: request {rid} differs from the plain implementation by {err:.3e} (bound {bound:.3e}), " \
+                                 f"first at {helpers.first_difference(got[rid], ex, bound)}"
+        del model, runner
+        torch.cuda.empty_cache()
+
+
 def test_model_sized_layers_bfloat16_against_float32():
     """Two layers with the sizes of Llama-3.1-8B (hidden 4096, 32 heads of 128 in 8 groups, intermediate 14336,
     vocabulary 128256) and the same weights in both precisions: the bfloat16 engine (pipelined products of

@@ -59,6 +59,48 @@ def test_replay_modes(tiny_dirs, name, dtype, mode):
     _compare(got, _reference(tiny_dirs, name, dtype), dtype, f"{name}/{dtype}/{mode}")
 
 
+def test_cutting_modes_against_each_other(tiny_dirs, capsys):
+    """The four ways of cutting compared with each other, not only with the plain implementation (float32,
+    config A).  Every kernel computes a row in an order that does not involve other rows; the one thing that
+    changes with a step's size is which product kernel runs: steps of at most eight rows take the kernel that
+    splits K over a block's threads, longer steps the tiled one, and the two add in different orders.  So a
+    position's logits are bit-equal between two modes whenever both ran it in a step of the same class, and
+    differ by float32 rounding otherwise; the measured differences are printed."""
+    name, dtype = "A", "float32"
+    requests = helpers.requests_for(name)
+    results, classes = {}, {}
+    for mode in ("whole", "bulk_tail", "portions", "mixed"):
+        steps, max_tokens = helpers.schedule_for(name, mode)
+        runner = _runner(tiny_dirs, name, dtype, max_tokens, helpers.PAGE_SIZE[name])
+        results[mode] = helpers.run_schedule(runner, requests, steps)
+        cls = {rid: [None] * len(t) for rid, t in requests.items()}
+        for entries, _ in steps:
+            rows = sum(c for _, _, c in entries)
+            for rid, start, count in entries:
+                for i in range(start, start + count):
+                    cls[rid][i] = rows <= 8
+        classes[mode] = cls
+    report = []
+    for mode in ("bulk_tail", "portions", "mixed"):
+        same = other = 0
+        worst = 0.0
+        for rid in requests:
+            a, b = results["whole"][rid], results[mode][rid]
+            scale = float(a.abs().max())
+            for i in range(a.shape[0]):
+                if classes["whole"][rid][i] == classes[mode][rid][i]:
+                    assert torch.equal(a[i], b[i]), f"{mode}: request {rid} position {i} ran the same kernels and differs"
+                    same += 1
+                else:
+                    worst = max(worst, float((a[i] - b[i]).abs().max()) / scale)
+                    other += 1
+        assert worst <= 2e-6, f"{mode}: {worst:.3e} between two orders of float32 addition"
+        report.append(f"{mode} vs whole: {same} positions bit-equal, {other} under the other product kernel, largest difference {worst:.2e}")
+    assert any("0 under" not in r for r in report), "no position was run by the other kernel: the comparison is empty"
+    with capsys.disabled():
+        print("\n  " + "\n  ".join(report))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C", "D"])
 def test_graph_replays_match_eager(tiny_dirs, name, dtype):
