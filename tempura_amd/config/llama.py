@@ -311,15 +311,12 @@ class LlamaConfig:
                     "down": f"{p}.mlp.down_proj.weight",
                 },
             )
-            layers.append(LayerSpec(
-                block="prenorm",
-                mixer=mixer,
-                ffn=ffn,
-                mixer_norm=PartSpec("rmsnorm", {"eps": self.rms_norm_eps},
-                                    {"weight": f"{p}.input_layernorm.weight"}),
-                ffn_norm=PartSpec("rmsnorm", {"eps": self.rms_norm_eps},
-                                  {"weight": f"{p}.post_attention_layernorm.weight"}),
-            ))
+            layers.append(LayerSpec("prenorm", {
+                "mixer_norm": PartSpec("rmsnorm", {"eps": self.rms_norm_eps}, {"weight": f"{p}.input_layernorm.weight"}),
+                "mixer": mixer,
+                "ffn_norm": PartSpec("rmsnorm", {"eps": self.rms_norm_eps}, {"weight": f"{p}.post_attention_layernorm.weight"}),
+                "ffn": ffn,
+            }))
         embed_name = "model.embed_tokens.weight"
         return ModelSpec(
             architecture=self.architecture,

@@ -36,17 +36,26 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """A block: how a mixer, a feed-forward and their norms are arranged.
+    """A block: a registered arrangement and the parts it arranges, by the names the arrangement gives them.
 
-    ``block`` names a registered arrangement (``"prenorm"``: x + mixer(norm(x)),
-    then x + ffn(norm(x))).
+    ``block`` names the arrangement (``"prenorm"``: x + mixer(norm(x)), then x + ffn(norm(x)), whose parts are
+    ``mixer_norm``, ``mixer``, ``ffn_norm`` and ``ffn``).  Which names an arrangement reads, and which category of
+    part (mixer, ffn, norm) each is, is the arrangement's business: one with other norms, or without a
+    feed-forward, has other names and needs no change here.  ``spec.mixer`` reads ``spec.parts["mixer"]``.
     """
 
     block: str
-    mixer: PartSpec
-    ffn: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    parts: Dict[str, PartSpec] = field(default_factory=dict)
+
+    def __getattr__(self, name: str) -> PartSpec:
+        parts = object.__getattribute__(self, "parts")
+        try:
+            return parts[name]
+        except KeyError:
+            raise AttributeError(f"block {self.block!r} has no part named {name!r} (it has {sorted(parts)})") from None
+
+    def __hash__(self):
+        return hash((self.block, tuple(sorted((k, hash(v)) for k, v in self.parts.items()))))
 
 
 @dataclass(frozen=True)

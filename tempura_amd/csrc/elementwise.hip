@@ -459,6 +459,39 @@ extern "C" int tp_swiglu(const void* gu, int in_dt, void* out, int out_dt, int m
   return 0;
 }
 
+// ---- rows of 4-byte elements: gather and clear ------------------------------------------------
+// out[i, :] = src[rows[i], :] (rows null: out[i, :] = src[i, :]); the element type only has to be four bytes wide
+// (float32 logits, int32 token ids).  grid: (rows out, column blocks of 1024); block: 256 threads, four elements each.
+__global__ void copy_rows4_kernel(const uint32_t* __restrict__ src, const int* __restrict__ rows, uint32_t* __restrict__ out,
+                                  int width) {
+  const int i = blockIdx.x;
+  const size_t from = (size_t)(rows ? rows[i] : i) * width, to = (size_t)i * width;
+  for (int j = blockIdx.y * 1024 + threadIdx.x; j < min(width, (int)(blockIdx.y + 1) * 1024); j += 256) out[to + j] = src[from + j];
+}
+
+extern "C" int tp_copy_rows4(const void* src, const int* rows, void* out, int n, int width, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && width > 0, "copy_rows: bad sizes");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(copy_rows4_kernel, dim3(n, (width + 1023) / 1024), dim3(256), 0, s, (const uint32_t*)src, rows,
+                     (uint32_t*)out, width);
+  TP_CHECK_LAUNCH("copy_rows");
+  return 0;
+}
+
+// t[rows[i], :] = 0 for rows of `width` 4-byte elements.
+__global__ void zero_rows4_kernel(uint32_t* __restrict__ t, const int* __restrict__ rows, int width) {
+  const size_t at = (size_t)rows[blockIdx.x] * width;
+  for (int j = blockIdx.y * 1024 + threadIdx.x; j < min(width, (int)(blockIdx.y + 1) * 1024); j += 256) t[at + j] = 0u;
+}
+
+extern "C" int tp_zero_rows4(void* t, const int* rows, int n, int width, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && width > 0, "zero_rows: bad sizes");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(zero_rows4_kernel, dim3(n, (width + 1023) / 1024), dim3(256), 0, s, (uint32_t*)t, rows, width);
+  TP_CHECK_LAUNCH("zero_rows");
+  return 0;
+}
+
 // ---- seeded normal fill ------------------------------------------------------------------
 // out[i] = mean + std * N(0, 1) where the deviate of element i depends only on (seed, i) and has the same
 // bits as the host library's (counter_normal.h): random weights of large models are made directly in device

@@ -15,6 +15,7 @@ from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple, Un
 import torch
 
 from ..config import load_config
+from ..kernels import ops
 from ..sampling import Sampler, SamplingParams
 from .loading import load_model, parse_dtype, random_model
 from .model import CausalLM
@@ -122,7 +123,7 @@ class Engine:
                 return self.step() if self.has_unfinished() else []
             items = [ScheduledItem(reqs[i], reqs[i].num_tokens - 1, 1, True) for i in live]
             if len(live) < len(reqs):
-                logits = logits[torch.tensor(live, dtype=torch.long, device=self.device)]
+                logits = ops.take_rows(logits, live)
             self.last_step = {"decode_tokens": len(items), "prompt_tokens": 0, "requests": len(items), "queued_ahead": True}
         else:
             items = self.scheduler.schedule()
@@ -180,9 +181,9 @@ class Engine:
 
         def queue(chosen: torch.Tensor) -> None:
             rids = [r.rid for r in reqs]
-            toks = chosen if len(keep) == len(items) else chosen[torch.tensor(keep, dtype=torch.long, device=self.device)]
+            toks = chosen if len(keep) == len(items) else ops.take_rows(chosen, keep)
             try:
-                logits = self.runner.step_chained(rids, toks.to(torch.int32))
+                logits = self.runner.step_chained(rids, toks)
             except PagesExhausted:
                 return              # the scheduler decides who gives way, in the next call
             self.counters["steps"] += 1
@@ -254,7 +255,7 @@ class Engine:
         """Logits [vocab] (float32, host) after a whole prompt of a fresh request
         (the reference's ``forward``, /root/reference/engine/src/model.rs:308)."""
         if self._ahead is not None:      # a queued step's logits live in a graph's output buffer: keep a copy
-            self._ahead = (self._ahead[0], self._ahead[1].clone())
+            self._ahead = (self._ahead[0], ops.take_rows(self._ahead[1]))
         rid = ("forward", next(self._ids))
         self.runner.add_request(rid)
         try:

@@ -35,6 +35,11 @@ class CausalLM:
         self._plan_caches()
 
     # ---- caches --------------------------------------------------------
+    def _cache_owner(self, layer: int):
+        """The part of a layer whose cache and state needs its calls have (a block says which; by default its mixer)."""
+        block = self.layers[layer]
+        return block.cache_owner() if hasattr(block, "cache_owner") else block.mixer
+
     def _plan_caches(self) -> None:
         """Group cache slots by what their mixers need."""
         n_slots = 1 + max((c.cache for c in self.order), default=-1)
@@ -51,7 +56,7 @@ class CausalLM:
         self.state_specs: Dict[int, StateSpec] = {}
         counts: List[int] = []
         for slot in range(n_slots):
-            mixer = self.layers[self.order[owner[slot]].layer].mixer
+            mixer = self._cache_owner(self.order[owner[slot]].layer)
             cs = mixer.cache_spec()
             if cs is None:
                 self.slot_group.append((-1, 0))
@@ -68,8 +73,8 @@ class CausalLM:
         self.slots_per_group = counts
         for i, call in enumerate(self.order):
             if not self.call_writes[i]:
-                mine = self.layers[call.layer].mixer.cache_spec()
-                theirs = self.layers[self.order[owner[call.cache]].layer].mixer.cache_spec()
+                mine = self._cache_owner(call.layer).cache_spec()
+                theirs = self._cache_owner(self.order[owner[call.cache]].layer).cache_spec()
                 if mine != theirs:
                     raise ValueError(f"run order entry {i} reads cache slot {call.cache} whose layout differs from its own")
 

@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager, CachePools, LayerCache, PagesExhausted
+from ..kernels import ops
 from .model import CausalLM
 
 
@@ -402,7 +403,7 @@ class ModelRunner:
         self.graph_steps += 1
         if want_rows is None or len(want_rows) == n:
             return g.logits[:n]
-        return g.logits[torch.tensor(want_rows, dtype=torch.long, device=self.device)] if want_rows else g.logits[:0]
+        return ops.take_rows(g.logits, want_rows) if want_rows else g.logits[:0]
 
     def step_chained(self, rids: Sequence, tokens: torch.Tensor) -> torch.Tensor:
         """A step of one token per request whose tokens are still on the device: ``tokens`` int32 [len(rids)],
@@ -452,9 +453,8 @@ class ModelRunner:
         if self.pools.state:
             fresh = [s for s, n, c in zip(ctx.state_slot_list, ctx.q_lens, ctx.ctx_lens) if c == n]
             if fresh:
-                idx = torch.tensor(fresh, dtype=torch.long, device=self.device)
                 for t in self.pools.state.values():
-                    t.index_fill_(0, idx, 0)
+                    ops.zero_rows(t, fresh)
         logits = self.model.forward(tok_dev, ctx, self.layer_caches)
         self.cache.commit_many([e.rid for e in entries], ctx.q_lens)
         self.steps_run += 1

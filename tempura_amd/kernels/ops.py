@@ -749,6 +749,43 @@ def top_logprobs(work: torch.Tensor, info: torch.Tensor, vocab: int, n: int):
     return ids, lps
 
 
+def take_rows(t: torch.Tensor, rows=None) -> torch.Tensor:
+    """A new tensor holding rows ``rows`` (a list of indices; None: all of them, a plain copy) of a float32 or
+    int32 tensor [n] or [n, width], by the library's own copy kernel."""
+    if _backend is not None:
+        return _backend.take_rows(t, rows)
+    import numpy as np
+    _dev_ok(t)
+    _need(t.dtype in (torch.float32, torch.int32) and t.dim() in (1, 2), "take_rows: needs float32 or int32 [n] or [n, width]")
+    n_in = t.shape[0]
+    width = 1 if t.dim() == 1 else t.shape[1]
+    if rows is None:
+        n, idx = n_in, None
+    else:
+        n = len(rows)
+        _need(all(0 <= int(r) < n_in for r in rows), "take_rows: row out of range")
+        idx = _Staging.send([np.asarray(rows, dtype=np.int32)], t.device)[0] if n else None
+    out = torch.empty((n,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+    if n and width:
+        _call("tp_copy_rows4", _ptr(t), _ptr(idx), _ptr(out), n, width, _stream())
+    return out
+
+
+def zero_rows(t: torch.Tensor, rows) -> None:
+    """t[rows] = 0 in place for a float32 or int32 tensor [n, ...] (rows: a list of indices)."""
+    if _backend is not None:
+        return _backend.zero_rows(t, rows)
+    import numpy as np
+    _dev_ok(t)
+    _need(t.dtype in (torch.float32, torch.int32) and t.dim() >= 1, "zero_rows: needs a float32 or int32 tensor")
+    n_in = t.shape[0]
+    width = t[0].numel() if n_in else 0
+    _need(all(0 <= int(r) < n_in for r in rows), "zero_rows: row out of range")
+    if len(rows) and width:
+        idx = _Staging.send([np.asarray(rows, dtype=np.int32)], t.device)[0]
+        _call("tp_zero_rows4", _ptr(t), _ptr(idx), len(rows), width, _stream())
+
+
 def fill_normal(out: torch.Tensor, seed: int, mean: float, std: float) -> torch.Tensor:
     """Fill a device tensor with mean + std * N(0, 1); element i depends only on (seed, i) and has the bits
     that ``weights.random_init.fill_normal_host`` gives it on the host."""

@@ -15,30 +15,47 @@ from __future__ import annotations
 from .base import build_part, part_class, register_part
 
 
-class PreNormBlock:
+class ArrangedBlock:
+    """Base of the arrangements: builds the parts a ``LayerSpec`` names, by the categories the arrangement
+    declares in ``ROLES`` (name -> ``"mixer"``, ``"ffn"`` or ``"norm"``), in that order, each as an attribute of
+    its name.  A subclass writes ``forward(h, ctx, cache)`` and registers itself under ``"block"``; the model
+    asks ``cache_owner()`` which part's cache and state needs a call of the layer has."""
+
     category = "block"
+    ROLES: dict = {}
 
     def __init__(self, layer_spec, hidden_size, dtype, device):
         self.layer_spec = layer_spec
-        self.mixer_norm = build_part("norm", layer_spec.mixer_norm, hidden_size, dtype, device)
-        self.mixer = build_part("mixer", layer_spec.mixer, hidden_size, dtype, device)
-        self.ffn_norm = build_part("norm", layer_spec.ffn_norm, hidden_size, dtype, device)
-        self.ffn = build_part("ffn", layer_spec.ffn, hidden_size, dtype, device)
+        missing = [name for name in self.ROLES if name not in layer_spec.parts]
+        extra = [name for name in layer_spec.parts if name not in self.ROLES]
+        if missing or extra:
+            raise ValueError(f"block {layer_spec.block!r} arranges the parts {sorted(self.ROLES)}: "
+                             f"missing {missing}, not its own {extra}")
+        for name, cat in self.ROLES.items():
+            setattr(self, name, build_part(cat, layer_spec.parts[name], hidden_size, dtype, device))
 
     def parts(self):
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+        return [getattr(self, name) for name in self.ROLES]
+
+    def cache_owner(self):
+        """The part whose ``cache_spec()`` / ``state_spec()`` this layer's cache slot serves."""
+        return self.mixer
 
     @classmethod
     def expected_weights(cls, layer_spec, hidden_size):
         out = {}
-        for cat, ps in (("norm", layer_spec.mixer_norm), ("mixer", layer_spec.mixer),
-                        ("norm", layer_spec.ffn_norm), ("ffn", layer_spec.ffn)):
+        for name, cat in cls.ROLES.items():
+            ps = layer_spec.parts[name]
             out.update(part_class(cat, ps.kind).expected_weights(ps, hidden_size))
         return out
 
     def load_weights(self, get):
         for p in self.parts():
             p.load_weights(get)
+
+
+class PreNormBlock(ArrangedBlock):
+    ROLES = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "ffn"}
 
     def entry_norm(self, m):
         """What the part before this block needs to prepare this block's first norm for ``m`` rows, or None."""

@@ -117,7 +117,7 @@ class Sampler:
                 inwin.append(1 if tok in window else 0)
         if not rows:
             return logits
-        out = logits.clone()
+        out = ops.take_rows(logits)          # (the caller's logits stay as they are)
         ops.apply_penalties(out, rows, toks, counts, inwin,
                             [p.presence_penalty for p in params], [p.frequency_penalty for p in params],
                             [p.repeat_penalty for p in params])

@@ -125,3 +125,10 @@ class EmuOps:
         v = logits.shape[1]
         flipped = torch.flip(logits, dims=[1])
         return (v - 1 - torch.argmax(flipped, dim=1)).to(torch.int32)
+
+    def take_rows(self, t, rows=None):
+        return t.clone() if rows is None else t[torch.tensor(list(rows), dtype=torch.long)].clone()
+
+    def zero_rows(self, t, rows):
+        if len(rows):
+            t[torch.tensor(list(rows), dtype=torch.long)] = 0

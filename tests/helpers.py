@@ -89,12 +89,24 @@ TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 BF16_FACTOR = 2.0
 
 
+def float32_bound(cfg: dict) -> float:
+    """The float32 engine's bound for a model of these widths.  A float32 sum of K terms carries a rounding error
+    that grows like sqrt(K); ``TOL["float32"]`` was set on models whose longest sum has a few hundred terms, and a
+    model whose products run over thousands gets the constant times sqrt(K / 512) (the Llama-3.1-8B widths, K up to
+    14,336: 1.06e-4; every tiny configuration: the constant itself).  A wrong key, page or position costs 1e-2 and
+    more at any width."""
+    H = cfg["hidden_size"]
+    nH = cfg["num_attention_heads"]
+    K = max(H, cfg["intermediate_size"], nH * (cfg.get("head_dim") or H // nH))
+    return TOL["float32"] * max(1.0, (K / 512.0) ** 0.5)
+
+
 def plain_reference(cfg, W, tokens, dtype: str):
     """(exact logits [T, vocab] of the plain implementation, bound on rel_err for an engine of ``dtype``): the
-    constant in float32; in bfloat16 ``BF16_FACTOR`` times the rounding noise of bfloat16 storage on this request."""
+    constant in float32 (``float32_bound``: scaled up for wide models); in bfloat16 ``BF16_FACTOR`` times the rounding noise of bfloat16 storage on this request."""
     exact = plain.forward(cfg, W, tokens)
     if dtype == "float32":
-        return exact, TOL["float32"]
+        return exact, float32_bound(cfg)
     rounded = plain.forward(cfg, W, tokens, stored=plain.as_bfloat16)
     return exact, BF16_FACTOR * rel_err(rounded, exact)
 

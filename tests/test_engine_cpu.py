@@ -222,3 +222,38 @@ def test_toy_routed_ffn_and_learned_position_register_build_and_step(tmp_path):
     for r in reqs:
         assert helpers.first_difference(got[r], ref[r], 1e-6) is None, r
     assert runner.cache.free_pages() == [12, 8]
+
+
+def test_toy_block_arrangements_with_other_parts_register_build_and_step(tmp_path):
+    """Two block arrangements defined in the tests: one with norms before and after the mixer and the feed-forward
+    (six named parts), one with a mixer and no feed-forward.  ``LayerSpec`` carries the parts by the names the
+    arrangement gives them, so neither needs a change to the framework's files."""
+    import toy_parts
+    from tempura_amd.config import load_config
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.weights import write_random_model
+    cfg = toy_parts.ToySandwichConfig()
+    spec = cfg.build_spec()
+    assert sorted(spec.layers[0].parts) == ["ffn", "mixer", "post_ffn_norm", "post_mixer_norm", "pre_ffn_norm", "pre_mixer_norm"]
+    assert sorted(spec.layers[1].parts) == ["mixer", "norm"] and spec.layers[1].mixer.kind == "attention"
+    with pytest.raises(AttributeError, match="no part named"):
+        spec.layers[1].ffn
+    d = write_random_model(cfg, str(tmp_path / "sandwich"), seed=8, std=0.2, norm_jitter=0.1, dtype="float32")
+    assert type(load_config(d)) is toy_parts.ToySandwichConfig
+    model = load_model(d, "float32", "cpu")
+    assert model.slots_per_group == [3] and len(model.expected_weights()) == 3 + 4 * 3 + (4 + 3) * 2 + 1
+    _, W = plain.read_model_dir(d)
+    runner = ModelRunner(model, 8, 12, max_requests=3)
+    reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=20 + i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30}.items())}
+    ref = {r: toy_parts.plain_sandwich_forward(cfg, W, t) for r, t in reqs.items()}
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
+             ([("p", 10, 11), ("r", 17, 13)], ["p", "r"])]
+    got = helpers.run_schedule(runner, reqs, steps)
+    for r in reqs:
+        assert helpers.first_difference(got[r], ref[r], 1e-6) is None, r
+    # a spec that names parts the arrangement does not have is refused when the block is built
+    from tempura_amd.config import LayerSpec
+    from tempura_amd.parts import part_class
+    with pytest.raises(ValueError, match="missing"):
+        part_class("block", "prenorm")(LayerSpec("prenorm", {"mixer": spec.layers[1].mixer}), cfg.hidden_size, torch.float32, "cpu")

@@ -260,8 +260,9 @@ def test_model_width_mixed_schedule_against_plain(tmp_path):
     """Two layers with the widths of Llama-3.1-8B under the mixed schedule: up to four live requests, portions of
     some beside single decoded tokens of others, the last 32 tokens of each one by one (decode-only steps replay
     the graph), and so few pages that finished requests' pages are used again; float32 and bfloat16 against the
-    plain float64 implementation.  The q and k projections are scaled up (scores 16 times those of N(0, 0.02)
-    weights), so that attention is peaked and a wrong key or page moves the logits far beyond the bound."""
+    plain float64 implementation.  The q and k projections are doubled (scores four times those of N(0, 0.02)
+    weights: a standard deviation of about 6.5 over a few hundred keys), so that attention is sharply peaked and
+    a wrong key or page moves the logits far beyond the bound."""
     from tempura_amd.engine.loading import load_model
     from tempura_amd.engine.runner import ModelRunner
     from tempura_amd.kernels import ops
@@ -271,7 +272,7 @@ def test_model_width_mixed_schedule_against_plain(tmp_path):
     W = random_weights(cfg, seed=4, std=0.02, dtype="bfloat16")
     for name in W:
         if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
-            W[name] = (W[name].float() * 4.0).to(torch.bfloat16)
+            W[name] = (W[name].float() * 2.0).to(torch.bfloat16)
     folder = tmp_path / "wide2"
     folder.mkdir()
     (folder / "config.json").write_text(cfg.to_json())
@@ -335,7 +336,7 @@ def test_full_depth_model_against_plain_streamed():
             both = plain.forward_many(pc, get, list(requests.values()), [None, plain.as_bfloat16])      # one pass over the weights
             exact = {rid: both[i][0] for i, rid in enumerate(requests)}
             noisy = {rid: both[i][1] for i, rid in enumerate(requests)}
-            refs = {"float32": {rid: (exact[rid], helpers.TOL["float32"]) for rid in requests},
+            refs = {"float32": {rid: (exact[rid], helpers.float32_bound(pc)) for rid in requests},
                     "bfloat16": {rid: (exact[rid], helpers.BF16_FACTOR * helpers.rel_err(noisy[rid], exact[rid])) for rid in requests}}
         runner = ModelRunner(model, 16, max_tokens // 16, max_requests=4, use_graph=True)
         got = helpers.run_schedule(runner, requests, steps)

@@ -684,3 +684,23 @@ def test_device_made_model_equals_the_written_folder(tmp_path):
                     if isinstance(va, torch.Tensor):
                         assert torch.equal(va, vb), f"{type(pa).__name__}.{key} differs ({dtype})"
         assert torch.equal(a.embedding.weight, b.embedding.weight) and torch.equal(a.final_norm.weight, b.final_norm.weight)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.int32])
+@pytest.mark.parametrize("n,width", [(1, 1), (7, 301), (64, 128256), (5, 1024), (3, 1025)])
+def test_take_rows_and_zero_rows(dtype, n, width):
+    ops = _ops()
+    g = torch.Generator().manual_seed(n + width)
+    src = (torch.randn(n, width, generator=g) * 100).to(dtype)
+    d = src.to(DEV)
+    rows = [int(r) for r in torch.randint(0, n, (max(1, n // 2 + 1),), generator=g)]
+    assert torch.equal(ops.take_rows(d, rows).cpu(), src[rows])
+    assert torch.equal(ops.take_rows(d).cpu(), src) and ops.take_rows(d).data_ptr() != d.data_ptr()
+    assert torch.equal(ops.take_rows(d[:, 0].contiguous(), rows).cpu(), src[rows, 0])
+    assert ops.take_rows(d, []).shape == (0, width)
+    ops.zero_rows(d, sorted(set(rows)))
+    want = src.clone()
+    want[sorted(set(rows))] = 0
+    assert torch.equal(d.cpu(), want)
+    with pytest.raises(Exception, match="out of range"):
+        ops.take_rows(d, [n])

@@ -63,9 +63,10 @@ def test_cutting_modes_against_each_other(tiny_dirs, capsys):
     """The four ways of cutting compared with each other, not only with the plain implementation (float32,
     config A).  Every kernel computes a row in an order that does not involve other rows; the one thing that
     changes with a step's size is which product kernel runs: steps of at most eight rows take the kernel that
-    splits K over a block's threads, longer steps the tiled one, and the two add in different orders.  So a
-    position's logits are bit-equal between two modes whenever both ran it in a step of the same class, and
-    differ by float32 rounding otherwise; the measured differences are printed."""
+    splits K over a block's threads, longer steps the tiled one, and the two add in different orders.  A position
+    reads the keys and values of the positions before it, so its logits are bit-equal between two modes whenever
+    both ran it AND everything before it in steps of the same class, and differ by float32 rounding otherwise;
+    the measured differences are printed."""
     name, dtype = "A", "float32"
     requests = helpers.requests_for(name)
     results, classes = {}, {}
@@ -87,8 +88,10 @@ def test_cutting_modes_against_each_other(tiny_dirs, capsys):
         for rid in requests:
             a, b = results["whole"][rid], results[mode][rid]
             scale = float(a.abs().max())
+            alike = True
             for i in range(a.shape[0]):
-                if classes["whole"][rid][i] == classes[mode][rid][i]:
+                alike = alike and classes["whole"][rid][i] == classes[mode][rid][i]
+                if alike:
                     assert torch.equal(a[i], b[i]), f"{mode}: request {rid} position {i} ran the same kernels and differs"
                     same += 1
                 else:

@@ -4,7 +4,9 @@ nothing under tempura_amd/ knows about them.
   beside attention in others (``ToyForCausalLM``);
 * a feed-forward with routing (each token goes to the expert its router scores highest) and a position
   encoding that is not rotary (a learned vector per position, added to queries and keys), in layers beside
-  the library's own parts (``ToyRoutedForCausalLM``)."""
+  the library's own parts (``ToyRoutedForCausalLM``);
+* a block arrangement with other parts than the library's: norms before AND after the mixer and the feed-forward
+  (six named parts), and a second kind of layer that has a mixer and no feed-forward at all (``ToySandwichForCausalLM``)."""
 from __future__ import annotations
 
 import json
@@ -14,7 +16,7 @@ from typing import Dict, List
 import torch
 
 from tempura_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, register_architecture
-from tempura_amd.parts import FeedForward, Mixer, PositionEncoding, StateSpec, WeightInfo, register_part
+from tempura_amd.parts import ArrangedBlock, FeedForward, Mixer, PositionEncoding, StateSpec, WeightInfo, register_part
 
 
 class DecaySumMixer(Mixer):
@@ -146,12 +148,12 @@ class ToyConfig:
                                                "head_dim": self.head_dim, "scale": self.head_dim ** -0.5, "window": None,
                                                "position": PartSpec("rope", {"head_dim": self.head_dim, "theta": 1e4, "scaling": None})},
                                  {"q": f"{p}.q", "k": f"{p}.k", "v": f"{p}.v", "o": f"{p}.o"})
-            layers.append(LayerSpec(
-                "prenorm", mixer,
-                PartSpec("swiglu", {"intermediate_size": self.intermediate_size},
-                         {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"}),
-                PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": f"{p}.n1"}),
-                PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": f"{p}.n2"})))
+            layers.append(LayerSpec("prenorm", {
+                "mixer": mixer,
+                "ffn": PartSpec("swiglu", {"intermediate_size": self.intermediate_size},
+                                {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"}),
+                "mixer_norm": PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": f"{p}.n1"}),
+                "ffn_norm": PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": f"{p}.n2"})}))
         return ModelSpec(self.architecture, self.hidden_size, self.vocab_size, self.max_position_embeddings, layers,
                          [LayerCall(l) for l in range(self.num_hidden_layers)],
                          PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": "toy.norm"}),
@@ -202,10 +204,11 @@ class ToyRoutedConfig:
         swiglu = lambda p: PartSpec("swiglu", {"intermediate_size": self.intermediate_size},
                                     {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"})
         norm = lambda n: PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": n})
+        block = lambda mixer, ffn, n1, n2: LayerSpec("prenorm", {"mixer": mixer, "ffn": ffn, "mixer_norm": n1, "ffn_norm": n2})
         layers = [
-            LayerSpec("prenorm", self._attention("r.0", learned("r.0"), None), routed("r.0"), norm("r.0.n1"), norm("r.0.n2")),
-            LayerSpec("prenorm", self._attention("r.1", rope, 12), swiglu("r.1"), norm("r.1.n1"), norm("r.1.n2")),
-            LayerSpec("prenorm", self._attention("r.2", learned("r.2"), None), routed("r.2"), norm("r.2.n1"), norm("r.2.n2")),
+            block(self._attention("r.0", learned("r.0"), None), routed("r.0"), norm("r.0.n1"), norm("r.0.n2")),
+            block(self._attention("r.1", rope, 12), swiglu("r.1"), norm("r.1.n1"), norm("r.1.n2")),
+            block(self._attention("r.2", learned("r.2"), None), routed("r.2"), norm("r.2.n1"), norm("r.2.n2")),
         ]
         return ModelSpec(self.architecture, self.hidden_size, self.vocab_size, self.max_position_embeddings, layers,
                          [LayerCall(0), LayerCall(1), LayerCall(2)],
@@ -279,3 +282,99 @@ def plain_toy_forward(cfg: ToyConfig, W: Dict[str, torch.Tensor], tokens: List[i
         x = plain.rmsnorm(h, W[f"{p}.n2"], 1e-5)
         h = h + plain.swiglu_ffn(x, W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
     return plain.rmsnorm(h, W["toy.norm"], 1e-5) @ W["toy.embed"].T
+
+
+class SandwichBlock(ArrangedBlock):
+    """h += post_mixer_norm(mixer(pre_mixer_norm(h))); h += post_ffn_norm(ffn(pre_ffn_norm(h))): six parts, two of
+    them norms that the library's own arrangement does not have.  A part adds its result into the stream it is
+    handed, so the block hands it a zero stream and norms what comes back."""
+    ROLES = {"pre_mixer_norm": "norm", "mixer": "mixer", "post_mixer_norm": "norm",
+             "pre_ffn_norm": "norm", "ffn": "ffn", "post_ffn_norm": "norm"}
+
+    def forward(self, h, ctx, cache):
+        y = torch.zeros_like(h)
+        self.mixer.forward(self.pre_mixer_norm.forward(h), ctx, cache, y)
+        h += self.post_mixer_norm.forward(y).float()
+        y = torch.zeros_like(h)
+        self.ffn.forward(self.pre_ffn_norm.forward(h), ctx, y)
+        h += self.post_ffn_norm.forward(y).float()
+
+
+class MixerOnlyBlock(ArrangedBlock):
+    """h += mixer(norm(h)) and nothing else: a layer without a feed-forward."""
+    ROLES = {"norm": "norm", "mixer": "mixer"}
+
+    def forward(self, h, ctx, cache):
+        self.mixer.forward(self.norm.forward(h), ctx, cache, h)
+
+
+register_part("block", "toy_sandwich", SandwichBlock)
+register_part("block", "toy_mixer_only", MixerOnlyBlock)
+
+
+@dataclass
+class ToySandwichConfig:
+    """Layer 0: the sandwich arrangement around attention and SwiGLU; layer 1: attention alone; layer 2: sandwich."""
+    hidden_size: int = 64
+    vocab_size: int = 120
+    num_attention_heads: int = 4
+    num_key_value_heads: int = 2
+    head_dim: int = 16
+    intermediate_size: int = 96
+    max_position_embeddings: int = 128
+    architecture: str = "ToySandwichForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        keys = cls.__dataclass_fields__
+        return cls(**{k: v for k, v in d.items() if k in keys})
+
+    def to_json(self):
+        d = {k: getattr(self, k) for k in self.__dataclass_fields__}
+        d["architectures"] = [self.architecture]
+        return json.dumps(d)
+
+    def build_spec(self) -> ModelSpec:
+        rope = PartSpec("rope", {"head_dim": self.head_dim, "theta": 1e4, "scaling": None})
+        norm = lambda n: PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": n})
+        attn = lambda p: PartSpec("attention", {"num_heads": self.num_attention_heads, "num_kv_heads": self.num_key_value_heads,
+                                                "head_dim": self.head_dim, "scale": self.head_dim ** -0.5, "window": None,
+                                                "position": rope}, {"q": f"{p}.q", "k": f"{p}.k", "v": f"{p}.v", "o": f"{p}.o"})
+        swiglu = lambda p: PartSpec("swiglu", {"intermediate_size": self.intermediate_size},
+                                    {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"})
+        sandwich = lambda p: LayerSpec("toy_sandwich", {
+            "pre_mixer_norm": norm(f"{p}.n1"), "mixer": attn(p), "post_mixer_norm": norm(f"{p}.n2"),
+            "pre_ffn_norm": norm(f"{p}.n3"), "ffn": swiglu(p), "post_ffn_norm": norm(f"{p}.n4")})
+        layers = [sandwich("s.0"), LayerSpec("toy_mixer_only", {"norm": norm("s.1.n1"), "mixer": attn("s.1")}), sandwich("s.2")]
+        return ModelSpec(self.architecture, self.hidden_size, self.vocab_size, self.max_position_embeddings, layers,
+                         [LayerCall(0), LayerCall(1), LayerCall(2)], norm("s.norm"),
+                         PartSpec("embedding", {}, {"weight": "s.embed"}), PartSpec("lm_head", {"tied": False}, {"weight": "s.head"}))
+
+
+register_architecture("ToySandwichForCausalLM", ToySandwichConfig)
+
+
+def plain_sandwich_forward(cfg: ToySandwichConfig, W: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
+    """Whole sequence, no cache, float64: the sandwich toy model written out plainly."""
+    import plain
+    W = {k: v.double() for k, v in W.items()}
+    T = len(tokens)
+    H, KV, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    h = W["s.embed"][torch.tensor(tokens)]
+    inv = plain.rope_inv_freq(D, 1e4, None)
+    pos = torch.arange(T)
+
+    def attend(p, x):
+        q = plain.rope((x @ W[f"{p}.q"].T).reshape(T, H, D), pos, inv)
+        k = plain.rope((x @ W[f"{p}.k"].T).reshape(T, KV, D), pos, inv)
+        v = (x @ W[f"{p}.v"].T).reshape(T, KV, D)
+        return plain.attention(q, k, v, D ** -0.5) @ W[f"{p}.o"].T
+    for l in range(3):
+        p = f"s.{l}"
+        if l == 1:
+            h = h + attend(p, plain.rmsnorm(h, W[f"{p}.n1"], 1e-5))
+            continue
+        h = h + plain.rmsnorm(attend(p, plain.rmsnorm(h, W[f"{p}.n1"], 1e-5)), W[f"{p}.n2"], 1e-5)
+        y = plain.swiglu_ffn(plain.rmsnorm(h, W[f"{p}.n3"], 1e-5), W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
+        h = h + plain.rmsnorm(y, W[f"{p}.n4"], 1e-5)
+    return plain.rmsnorm(h, W["s.norm"], 1e-5) @ W["s.head"].T
