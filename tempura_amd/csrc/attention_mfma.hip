@@ -109,6 +109,9 @@ __device__ inline u32x4_t attn_existing_keys(int n) {
   return keep;
 }
 
+// (per-wave loads of keys and values: a decode step reads a request's cache once, so the loads are nontemporal)
+#define ATTN_KV_LOAD(p) __builtin_nontemporal_load(p)
+
 // Fetch the fragments of the step starting at key j0 (kvh: kv head; ctx: keys that exist; keys
 // past the end are clamped to the last one and masked later, values past the end are cleared).
 template <int D>
@@ -123,7 +126,7 @@ __device__ inline void attn_load(const AttnArgs& a, const int* __restrict__ tabl
     const int page = table[key / ps];
     const bf16_t* kr = a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + key % ps) * D + g * 8;
 #pragma unroll
-    for (int dk = 0; dk < D / 32; ++dk) f.k[t][dk] = frag_of(*(const u32x4_t*)(kr + dk * 32));
+    for (int dk = 0; dk < D / 32; ++dk) f.k[t][dk] = frag_of(ATTN_KV_LOAD((const u32x4_t*)(kr + dk * 32)));
   }
   // values: eight consecutive keys of element d per lane
   const int kb = min(j0 + 8 * g, (ctx - 1) & ~7);
@@ -132,11 +135,11 @@ __device__ inline void attn_load(const AttnArgs& a, const int* __restrict__ tabl
   if (j0 + 32 > ctx) {   // the step that holds the last key
     const u32x4_t keep = attn_existing_keys(ctx - (j0 + 8 * g));
 #pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt) f.v[dt] = frag_of(*(const u32x4_t*)(vr + (size_t)dt * 16 * ps) & keep);
+    for (int dt = 0; dt < D / 16; ++dt) f.v[dt] = frag_of(ATTN_KV_LOAD((const u32x4_t*)(vr + (size_t)dt * 16 * ps)) & keep);
     return;
   }
 #pragma unroll
-  for (int dt = 0; dt < D / 16; ++dt) f.v[dt] = frag_of(*(const u32x4_t*)(vr + (size_t)dt * 16 * ps));
+  for (int dt = 0; dt < D / 16; ++dt) f.v[dt] = frag_of(ATTN_KV_LOAD((const u32x4_t*)(vr + (size_t)dt * 16 * ps)));
 }
 
 // One step of 32 keys starting at j0 for NQ query tiles, on fetched fragments.  qpos[nq] is the

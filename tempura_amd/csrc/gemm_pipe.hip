@@ -866,7 +866,8 @@ __device__ inline void issue_one64(unsigned char* buf, const unsigned char* xk, 
                                    const unsigned (&voff)[LPW64], int wave) {
   const int t = I < 2 ? wave * 2 + I : 8 + wave * 4 + (I - 2);
   const unsigned char* src = (I < 2 ? xk : wk) + voff[I];
-  __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+  // (the weights are read once per step: nontemporal, aux bit 1; the few activation rows stay cached)
+  __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, I < 2 ? 0 : 2);
 }
 template <bool READ, bool LOAD>
 __device__ inline void half_step64(f32x4_t (&acc)[2][4], const Frags64& cur, Frags64& nxt, unsigned aaddr, unsigned baddr,
