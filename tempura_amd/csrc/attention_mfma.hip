@@ -733,7 +733,11 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   const float mu = (mg == -INFINITY) ? 0.f : mg;
   const float ws = __builtin_amdgcn_exp2f(ms - mu);  // 0 for lanes without a split
   const float inv = 1.0f / wave_sum(ws * ls);
-  for (int d = lane; d < D; d += 64) {
+  // (every lane runs every turn of these loops, also where the head size is no multiple of 64: a lane that sat
+  // out a turn could not hand its split's weight to the others, and with more than 32 splits of a head size of
+  // 32 or 96 the lanes that hold the later splits' weights would sit out)
+  for (int d0 = 0; d0 < D; d0 += 64) {
+    const int d = min(d0 + lane, D - 1);
     float acc = 0.f;
     int s = 0;
     for (; s + 8 <= num_splits; s += 8) {   // eight independent loads in flight
@@ -744,7 +748,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
       for (int u = 0; u < 8; ++u) acc = fmaf(__shfl(ws, s + u, 64), v[u], acc);
     }
     for (; s < num_splits; ++s) acc = fmaf(__shfl(ws, s, 64), base[(size_t)s * (D + 2) + d], acc);
-    out[((size_t)q_start * n_heads + h) * D + d] = float_to_bf16(acc * inv);
+    if (d0 + lane < D) out[((size_t)q_start * n_heads + h) * D + d] = float_to_bf16(acc * inv);
   }
 }
 
@@ -779,10 +783,11 @@ __global__ __launch_bounds__(64) void attn_combine_rows_kernel(const float* __re
   const float mu = (mg == -INFINITY) ? 0.f : mg;
   const float ws = __builtin_amdgcn_exp2f(ms - mu);  // 0 for lanes without a part
   const float inv = 1.0f / wave_sum(ws * ls);
-  for (int d = lane; d < D; d += 64) {
+  for (int d0 = 0; d0 < D; d0 += 64) {      // (every lane runs every turn: see attn_combine_kernel)
+    const int d = min(d0 + lane, D - 1);
     float acc = 0.f;
     for (int s = 0; s < parts; ++s) acc = fmaf(__shfl(ws, s, 64), base[(size_t)s * stride + d], acc);
-    out[((size_t)t * n_heads + h) * D + d] = float_to_bf16(acc * inv);
+    if (d0 + lane < D) out[((size_t)t * n_heads + h) * D + d] = float_to_bf16(acc * inv);
   }
 }
 

@@ -518,6 +518,8 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int,
 allow_fast_attention = True
 #: the split decode kernel aims at this many blocks (of four waves) in flight
 decode_target_blocks = 256
+#: and at least this many splits while a split has at most 64 blocks
+decode_min_splits = 8
 #: portions of prompts with fewer query blocks than this have their keys split over blocks (1: never)
 portion_target_blocks = 1024
 #: in parts of at least this many keys
@@ -562,7 +564,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         blocks_per_split = num_single * kvh * ((heads // kvh + 15) // 16)
         want = -(-decode_target_blocks // blocks_per_split)
         if blocks_per_split <= 64:
-            want = max(want, 8)     # (batch 8 of the 8B shape: eight splits 3.87 ms a step, four 3.94)
+            want = max(want, decode_min_splits)     # (batch 8 of the 8B shape: eight splits 3.87 ms a step, four 3.94)
         splits = max(1, min(64, want, max(1, max_context_len // 128)))
         if splits > 1:
             scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)

@@ -582,6 +582,21 @@ def test_attention_ignores_what_lies_past_the_last_key(dtype, fast, heads, kv, d
         assert bool(torch.isfinite(got.float()).all())
 
 
+@pytest.mark.parametrize("heads,kv,d,page", [(5, 1, 32, 8), (6, 2, 96, 16), (4, 2, 64, 16), (8, 2, 128, 16)])
+def test_attention_decode_with_more_than_32_splits(heads, kv, d, page):
+    """One request of 5,000 keys is cut into 39 splits (one for every 128 keys) where few blocks would otherwise run:
+    the kernel that adds the splits hands each split's weight from lane to lane, which every lane has to take part
+    in also for head sizes below 64 (a lane that sat out once left the later splits' weights undefined)."""
+    ops = _ops()
+    keep = ops.decode_target_blocks
+    try:
+        ops.decode_target_blocks = 4096
+        _attention_case(torch.bfloat16, heads, kv, d, page, [1], [5000], 0, seed=24)
+        _attention_case(torch.bfloat16, heads, kv, d, page, [1, 1], [4999, 2300], 700, seed=25)
+    finally:
+        ops.decode_target_blocks = keep
+
+
 def test_attention_mfma_long_decode():
     _attention_case(torch.bfloat16, 8, 2, 128, 16, [1, 1], [3000, 2049], 0, seed=16)
 
