@@ -82,7 +82,10 @@ class Engine:
             return pages_cap
         free, _total = torch.cuda.mem_get_info(self.device)
         workspace = 2 << 30            # activations of the largest step, logits, sampler scratch
-        budget = int(free * utilization) - workspace
+        # the fixed-size state of every request slot comes out of the same memory
+        state_bytes = sum((max_batch_size + 1) * torch.Size(s.shape).numel() * torch.empty((), dtype=s.dtype).element_size()
+                          for s in m.state_specs.values())
+        budget = int(free * utilization) - workspace - state_bytes
         return max(1, min(pages_cap, budget // per_page))
 
     # ---- requests ------------------------------------------------------------

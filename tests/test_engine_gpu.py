@@ -50,6 +50,72 @@ def test_bfloat16_greedy_generation_runs_and_is_repeatable(tiny_dirs):
     assert a == b and all(len(o) == 20 for o in a)
 
 
+def test_bfloat16_greedy_generation_against_plain(tiny_dirs):
+    """The bfloat16 engine generates greedily; at every step the plain implementation (float64, on the same
+    bfloat16 weights, fed the engine's own tokens so far) must rank the engine's token first, or within the
+    rounding noise of bfloat16 storage of its own first: the token's plain logit may lie below the plain maximum
+    by no more than twice that noise (``helpers.plain_reference``'s bound, in logit units)."""
+    from tempura_amd.sampling import SamplingParams
+    for name in ("C", "D"):
+        cfg, W = tiny_dirs.plain_model(name, "bfloat16")
+        prompts = [helpers.random_tokens(cfg["vocab_size"], n, seed=300 + n) for n in (3, 50, 21)]
+        outs = _engine(tiny_dirs, name, "bfloat16").generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=20))
+        agree = total = 0
+        for p, o in zip(prompts, outs):
+            assert len(o) == 20
+            exact, bound = helpers.plain_reference(cfg, W, p + o, "bfloat16")
+            slack = bound * float(exact.abs().max())
+            for i, tok in enumerate(o):
+                row = exact[len(p) + i - 1]
+                assert float(row.max() - row[tok]) <= slack, \
+                    f"{name}: token {i} of the bfloat16 engine is {float(row.max() - row[tok]):.3e} below the plain maximum (slack {slack:.3e})"
+                agree += int(tok == int(torch.nonzero(row == row.max()).max()))
+                total += 1
+        assert agree >= 0.9 * total, f"{name}: only {agree} of {total} tokens are the plain implementation's first choice"
+
+
+def test_baseline_tiny_workloads(tmp_path):
+    """The two tiny workloads as they are specified: configuration A with a position limit of 128 (prompts of 5, 17
+    and 33 ids, 16 greedy steps, pages of 16) and B with a limit of 256 (prompts of 1, 9, 40, 63 and 120 ids, 24
+    steps at temperature 0.8 from seed 2, pages of 8), float32, weights N(0, 0.02) from seeds 0 and 1 with norm
+    weights 1.  Greedy tokens equal the plain implementation's; sampled tokens are the same alone and in the
+    batch and every one of them lies in the plain implementation's top 50; and a request that reaches the position
+    limit ends there with the reason max_model_len."""
+    from tempura_amd.config import LlamaConfig
+    from tempura_amd.engine import Engine
+    from tempura_amd.kernels import ops
+    from tempura_amd.sampling import SamplingParams
+    from tempura_amd.weights import write_random_model
+    ops.set_backend(None)
+    a = LlamaConfig.from_dict({**helpers.CONFIGS["A"].to_dict(), "max_position_embeddings": 128})
+    b = LlamaConfig.from_dict({**helpers.CONFIGS["B"].to_dict(), "max_position_embeddings": 256})
+    da = write_random_model(a, str(tmp_path / "a"), seed=0, std=0.02, dtype="float32")
+    db = write_random_model(b, str(tmp_path / "b"), seed=1, std=0.02, dtype="float32")
+    ca, Wa = plain.read_model_dir(da)
+    prompts = [helpers.random_tokens(256, n, seed=i) for i, n in enumerate((5, 17, 33))]
+    eng = Engine(da, dtype="float32", page_size=16, kv_pages=24, max_batch_size=3)
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=16))
+    assert outs == [plain.greedy_generate(ca, Wa, p, 16) for p in prompts]
+    # 120 prompt ids and room for 8 more: the request ends at the limit of 128 positions
+    rid = eng.add_request(helpers.random_tokens(256, 120, seed=9), SamplingParams(temperature=0.0, max_new_tokens=50, ignore_eos=True))
+    while eng.has_unfinished():
+        eng.step()
+    assert eng.request(rid).finish_reason == "max_model_len" and len(eng.request(rid).output) == 8
+    with pytest.raises(ValueError, match="no room"):
+        eng.add_request(helpers.random_tokens(256, 128, seed=9), SamplingParams(max_new_tokens=1))
+    cb, Wb = plain.read_model_dir(db)
+    prompts = [helpers.random_tokens(384, n, seed=10 + i) for i, n in enumerate((1, 9, 40, 63, 120))]
+    params = SamplingParams(temperature=0.8, seed=2, max_new_tokens=24)
+    eng = Engine(db, dtype="float32", page_size=8, kv_pages=96, max_batch_size=5)
+    outs = eng.generate(prompts, params)
+    assert all(len(o) == 24 for o in outs)
+    assert outs[3] == Engine(db, dtype="float32", page_size=8, kv_pages=32, max_batch_size=1).generate([prompts[3]], params)[0]
+    for p, o in zip(prompts[:3], outs[:3]):
+        logits = plain.forward(cb, Wb, p + o)
+        for i, tok in enumerate(o):
+            assert tok in torch.topk(logits[len(p) + i - 1], 50).indices.tolist(), "a sampled token outside the top 50 (top_k's default)"
+
+
 def test_preemption_by_recompute_keeps_tokens(tiny_dirs):
     """So few pages that running requests are preempted: every request still gets exactly the tokens it gets
     with plenty of pages, in greedy and in seeded temperature sampling."""
