@@ -330,7 +330,8 @@ def main() -> int:
             points[f"decode_b{b}_hbm_frac"] = round(r["bytes"] / (r["ms"] / 1e3) / 1e9 / HBM_PEAK_GBS, 4)
             say(f"engine decode b{b}: {r['tps']:.1f} tok/s, {r['ms']:.3f} ms/step")
         for b in sorted({1, args.batch, 64}):
-            tps, ms = runner_decode(eng, cfg, b, args.prompt_len, 8, ps)
+            # (the same number of steps, so the same range of context lengths, as the engine's figure it stands beside)
+            tps, ms = runner_decode(eng, cfg, b, args.prompt_len, warmup if b == args.batch else 8, steps if b == args.batch else ps)
             points[f"runner_b{b}"] = round(tps, 1)
             say(f"step function alone b{b}: {tps:.1f} tok/s, {ms:.3f} ms/step")
         if not args.no_long:
