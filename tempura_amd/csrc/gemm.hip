@@ -181,7 +181,8 @@ extern "C" int tp_linear_rope(const void* x, const void* w, int w_tiled, int M, 
 // multiplied by rsqrt(sum of squares / K + pre_eps): x is then that product's post_xg.
 //
 // `layout` (bfloat16, at most 16 rows): bit 0, x is k-blocked [K / 8, M, 8] instead of [M, K]; bit 1, the
-// gated output (accumulate == 2) is written k-blocked [N / 16, M, 8] for a product that reads it so.
+// gated output (accumulate == 2) is written k-blocked [N / 16, M, 8] for a product that reads it so; bit 3, post_xg
+// is written k-blocked [N / 8, M, 8].
 // Bit 2 (bfloat16, any number of rows, N % 16 == 0, K % 64 == 0): w is tiled, [N / 16][K / 32][64][8]: the 16 x 32
 // block of rows 16 i.. and columns 32 j.. as 1,024 contiguous bytes, element (r, c) of the block at
 // ((c / 8) * 16 + r) * 8 + c % 8 (the matrix cores' operand order), blocks of a row group side by side.
@@ -197,7 +198,7 @@ extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* ou
   TP_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   TP_REQUIRE(accumulate != 1 || out_dt == TP_F32, "linear: accumulating output must be float32");
   const bool split_norm = pre_ss != nullptr || post_w != nullptr || (layout & 3) != 0;
-  TP_REQUIRE((layout & ~7) == 0 && (!(layout & 2) || accumulate == 2) && (!(layout & 1) || pre_ss == nullptr),
+  TP_REQUIRE((layout & ~15) == 0 && (!(layout & 2) || accumulate == 2) && (!(layout & 8) || post_w != nullptr),
              "linear: bad layout flags %d", layout);
   TP_REQUIRE(!(layout & 4) || (in_dt == TP_BF16 && allow_mfma && N % 16 == 0 && K % 64 == 0),
              "linear: tiled weights are bfloat16 with N %% 16 == 0 and K %% 64 == 0 (N=%d K=%d)", N, K);

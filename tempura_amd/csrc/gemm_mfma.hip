@@ -50,7 +50,7 @@ __device__ inline bf16x8_t as_frag(u32x4_t v) { return __builtin_bit_cast(bf16x8
 // k group l / 16) at l * 16.  A wave's load of a fragment then covers eight whole cache lines instead of 64-byte
 // pieces of sixteen rows, which is what the address path of a CU can keep up with when the weights stream from HBM
 // (the down projection of 8 rows: 26.0 -> 23.4 us), and a stage of the pipelined kernels is a plain copy.
-enum { X_KBLOCKED = 1, OUT_KBLOCKED = 2, W_TILED = 4 };
+enum { X_KBLOCKED = 1, OUT_KBLOCKED = 2, W_TILED = 4, XG_KBLOCKED = 8 };
 
 __device__ inline void store_gated(void* out, int layout, int M, int width, int m, int col, float v) {
   const size_t idx = (layout & OUT_KBLOCKED) ? ((size_t)(col >> 3) * M + m) * 8 + (col & 7) : (size_t)m * width + col;
@@ -261,7 +261,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_mfma_kernel(const bf16
         float* o = (float*)out + (size_t)m * N + n;
         const float h = *o + v;
         *o = h;
-        post.xg[(size_t)m * N + n] = float_to_bf16(h * post.w[n]);
+        // (k-blocked on request: the product that consumes these rows then reads them straight from memory as operands)
+        post.xg[(layout & XG_KBLOCKED) ? ((size_t)(n >> 3) * M + m) * 8 + (n & 7) : (size_t)m * N + n] = float_to_bf16(h * post.w[n]);
         sq = h * h;
       }
       sq += __shfl_xor(sq, 1, 64);      // the four columns r = 0..3 of this row
@@ -416,7 +417,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const bf16_
         float* o = (float*)out + (size_t)m * N + n;
         const float h = *o + v;
         *o = h;
-        post.xg[(size_t)m * N + n] = float_to_bf16(h * post.w[n]);
+        // (k-blocked on request: the product that consumes these rows then reads them straight from memory as operands)
+        post.xg[(layout & XG_KBLOCKED) ? ((size_t)(n >> 3) * M + m) * 8 + (n & 7) : (size_t)m * N + n] = float_to_bf16(h * post.w[n]);
         sq = h * h;
       }
       sq += __shfl_xor(sq, 1, 64);
@@ -766,7 +768,9 @@ int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N,
   if (M < 1 || (M > 16 && M <= 128) || K % 32 != 0 || head_dim % 16 != 0 || rotary_dim % 2 != 0 || rotary_dim > head_dim) return -1;
   if (N != (n_heads + 2 * n_kv) * head_dim || page_size < 1) return -1;
   if (((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return -1;
-  if (w_tiled && (N % 16 != 0 || K % 64 != 0)) return -1;
+  // w_tiled: bit 0, the weight is tiled; bit 1 (at most 16 rows), x is k-blocked [K / 8, M, 8]
+  if ((w_tiled & 1) && (N % 16 != 0 || K % 64 != 0)) return -1;
+  if ((w_tiled & 2) && M > 16) return -1;
   const RowScale pre = {pre_ss, pre_count, 1.0f / (float)K, pre_eps};
   const NormPrep post = {nullptr, nullptr, nullptr};
   const RopeOut rp = {positions, slots, inv_freq, (const float2*)cos_sin, factor, rotary_dim, n_heads, n_kv, head_dim, page_size,
@@ -775,9 +779,10 @@ int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N,
     // long steps: the pipelined kernels, whose wave tiles (64 or 128 columns) must lie inside one head, with the
     // step's table of cosines and sines
     if (head_dim != 128 || rotary_dim % 8 != 0 || cos_sin == nullptr || pre_ss != nullptr || page_size % 8 != 0) return -1;
-    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, s);
+    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled & 1, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, s);
   }
-  launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, w_tiled ? W_TILED : 0, pre, post, rp, s);
+  launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, (w_tiled & 1 ? W_TILED : 0) | (w_tiled & 2 ? X_KBLOCKED : 0),
+                   pre, post, rp, s);
   return 0;
 }
 
@@ -791,7 +796,8 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   if (K % 32 != 0) return -1;
   const int w_tiled = (layout & W_TILED) != 0;
   if (w_tiled && (N % 16 != 0 || K % 64 != 0)) return -1;
-  if ((layout & (X_KBLOCKED | OUT_KBLOCKED)) != 0 && M > 16) return -1;
+  if ((layout & (X_KBLOCKED | OUT_KBLOCKED | XG_KBLOCKED)) != 0 && M > 16) return -1;
+  if ((layout & XG_KBLOCKED) && (post_w == nullptr || N % 8 != 0)) return -1;
   if ((layout & OUT_KBLOCKED) && accumulate != 2) return -1;
   if ((pre_ss != nullptr || post_w != nullptr) && M > 16) return -1;
   if (post_w != nullptr && accumulate != 1) return -1;

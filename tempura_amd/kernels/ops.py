@@ -165,14 +165,23 @@ class Prenormed:
     bfloat16(h * norm weight) [m, k]; ``ss`` [ceil(k / 16), 16] float32 holds, per block of 16 columns
     and row, the sum of squares of h; the consumer multiplies its float32 result rows by
     rsqrt(sum(ss) / k + eps).  Made by ``linear(..., residual=h, next_norm=(weight, eps))``."""
-    __slots__ = ("x", "ss", "eps")
+    __slots__ = ("x", "ss", "eps", "blocked")
 
-    def __init__(self, x, ss, eps):
+    def __init__(self, x, ss, eps, blocked=None):
         self.x, self.ss, self.eps = x, ss, float(eps)
+        #: None: ``x`` is row-major [m, k]; (m, k): ``x`` is stored k-blocked, [k / 8, m, 8] (see ``KBlocked``)
+        self.blocked = blocked
 
     @property
     def shape(self):
-        return self.x.shape
+        return self.x.shape if self.blocked is None else self.blocked
+
+    def rows(self):
+        """``x`` as a row-major [m, k] tensor (a copy when it is stored k-blocked)."""
+        if self.blocked is None:
+            return self.x
+        m, k = self.blocked
+        return self.x.permute(1, 0, 2).reshape(m, k)
 
 
 class KBlocked:
@@ -280,12 +289,15 @@ def split_norm_ok(m: int, width: int, dtype: torch.dtype) -> bool:
 
 
 def _pre_args(x):
+    """(the tensor a product reads, the arguments of its row scale, its rows and columns, layout bit 1 when the
+    tensor is k-blocked) of plain rows or of ``Prenormed`` rows."""
     if isinstance(x, Prenormed):
         _dev_ok(x.x, x.ss)
-        _need(x.x.dtype == torch.bfloat16 and x.ss.dtype == torch.float32 and
-              tuple(x.ss.shape) == ((x.x.shape[1] + 15) // 16, 16), "linear: malformed handed-over rows")
-        return x.x, (_ptr(x.ss), x.ss.shape[0], ctypes.c_float(x.eps))
-    return x, (_ptr(None), 0, ctypes.c_float(0.0))
+        m, k = x.shape
+        _need(x.x.dtype == torch.bfloat16 and x.ss.dtype == torch.float32 and x.x.numel() == m * k and
+              tuple(x.ss.shape) == ((k + 15) // 16, 16), "linear: malformed handed-over rows")
+        return x.x, (_ptr(x.ss), x.ss.shape[0], ctypes.c_float(x.eps)), (m, k), (1 if x.blocked is not None else 0)
+    return x, (_ptr(None), 0, ctypes.c_float(0.0)), (tuple(x.shape) if x.dim() == 2 else None), 0
 
 
 def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
@@ -294,12 +306,12 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     With ``blocked_out`` the result comes as ``KBlocked`` when there are at most 16 rows and i % 32 == 0 (else as a tensor)."""
     if _backend is not None:
         return _backend.linear_swiglu(x, w, blocked_out) if blocked_out else _backend.linear_swiglu(x, w)
-    x, pre = _pre_args(x)
+    x, pre, mk, xl = _pre_args(x)
     wd, wl = _w_args(w)
     _dev_ok(x, wd)
-    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_swiglu: shapes {tuple(x.shape)} x {tuple(w.shape)}")
+    _need(mk is not None and w.dim() == 2 and mk[1] == w.shape[1], f"linear_swiglu: shapes {mk} x {tuple(w.shape)}")
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "linear_swiglu: operands must be bfloat16")
-    m, k = x.shape
+    m, k = mk
     n = w.shape[0]
     _need(n % 16 == 0 and k % 32 == 0, "linear_swiglu: needs 2i % 16 == 0 and k % 32 == 0")
     # (the product that takes such rows is an MFMA kernel over K in steps of 32)
@@ -310,7 +322,7 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     scratch, nscratch = _splitk_scratch(x, m, n)
     _call("tp_linear_fused", _ptr(x), _ptr(wd), _BF16, _ptr(out.data if blocked_out else out), _BF16, 2, m, n, k, 1,
-          _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), (2 if blocked_out else 0) | wl,
+          _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), (2 if blocked_out else 0) | wl | xl,
           0, _ptr(None), _stream())
     return out
 
@@ -355,11 +367,11 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
         _dev_ok(x, wd, residual)
         _need(w.dim() == 2 and w.shape[1] == k and w.dtype == torch.bfloat16, f"linear: shapes {(m, k)} x {tuple(w.shape)}")
     else:
-        x, pre = _pre_args(x)
+        x, pre, mk, layout = _pre_args(x)
         _dev_ok(x, wd, residual)
-        _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}")
+        _need(mk is not None and w.dim() == 2 and mk[1] == w.shape[1], f"linear: shapes {mk} x {tuple(w.shape)}")
         _need(x.dtype == w.dtype, f"linear: operand dtypes differ ({x.dtype}, {w.dtype})")
-        m, k = x.shape
+        m, k = mk
     n = w.shape[0]
     if residual is not None:
         _need(residual.dtype == torch.float32 and tuple(residual.shape) == (m, n), "linear: residual must be float32 [m, n]")
@@ -372,9 +384,15 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
         _dev_ok(weight)
         _need(residual is not None, "linear: next_norm needs a residual")
         _need(weight.dtype == torch.float32 and weight.numel() == n, "linear: norm weight must be float32 [n]")
-        handed = Prenormed(torch.empty((m, n), dtype=torch.bfloat16, device=x.device),
-                           torch.empty(((n + 15) // 16, 16), dtype=torch.float32, device=x.device), eps)
+        # (the rows go on k-blocked where the consumer can read them so: a product of a few rows then takes its
+        # activations straight from memory as operands instead of staging them through LDS)
+        hand_blocked = handoff_blocked and n % 32 == 0
+        handed = Prenormed(torch.empty((n // 8, m, 8) if hand_blocked else (m, n), dtype=torch.bfloat16, device=x.device),
+                           torch.empty(((n + 15) // 16, 16), dtype=torch.float32, device=x.device), eps,
+                           (m, n) if hand_blocked else None)
         post = (_ptr(weight), _ptr(handed.x), _ptr(handed.ss))
+        if hand_blocked:
+            layout |= 8
     scratch, nscratch = _splitk_scratch(x, m, n) if allow_mfma else (None, 0)
     # 17..128 rows: the partial sums of a split K may stay unadded for the kernel that consumes the rows
     layout |= wl
@@ -397,6 +415,8 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
     return out if next_norm is None else (out, handed)
 
 
+#: rows handed from one product to the next with a norm between them travel k-blocked (up to 16 rows)
+handoff_blocked = True
 #: long steps may rotate and store in the projection's epilogue too (False: only the few rows of decoding)
 rope_in_long_products = True
 
@@ -421,11 +441,11 @@ def linear_rope_kv(x, w: torch.Tensor, positions: torch.Tensor, slots: torch.Ten
     ``linear_rope_ok``) with the rotation and the cache write in its epilogue: the same result as ``linear``
     to float32 followed by ``rope_kv_write`` (w's q and k heads in paired order), without the kernel and the
     rows in between.  Returns q as bfloat16 [m, heads, head_dim]."""
-    x, pre = _pre_args(x)
+    x, pre, mk, xl = _pre_args(x)
     wd, wl = _w_args(w)
     _dev_ok(x, wd, positions, slots, inv_freq, k_cache, v_cache)
-    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear_rope_kv: shapes {tuple(x.shape)} x {tuple(w.shape)}")
-    m, k = x.shape
+    _need(mk is not None and w.dim() == 2 and mk[1] == w.shape[1], f"linear_rope_kv: shapes {mk} x {tuple(w.shape)}")
+    m, k = mk
     n = w.shape[0]
     _need(linear_rope_ok(m, n, k, head_dim, rotary_dim, k_cache.shape[2] if k_cache.dim() == 4 else 0, x.dtype, k_cache.dtype,
                          pre[1] != 0) and w.dtype == torch.bfloat16,
@@ -446,7 +466,7 @@ def linear_rope_kv(x, w: torch.Tensor, positions: torch.Tensor, slots: torch.Ten
         _need(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and tuple(cos_sin.shape) == (m, rotary_dim // 2, 2),
               "linear_rope_kv: table must be float32 [m, rotary_dim / 2, 2]")
     q = torch.empty((m, num_heads, head_dim), dtype=torch.bfloat16, device=x.device)
-    _call("tp_linear_rope", _ptr(x), _ptr(wd), int(wl != 0), m, n, k, *pre, _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
+    _call("tp_linear_rope", _ptr(x), _ptr(wd), int(wl != 0) | (2 if xl else 0), m, n, k, *pre, _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
           ctypes.c_float(factor), num_heads, num_kv_heads, head_dim, _ptr(q), _ptr(k_cache), _ptr(v_cache),
           k_cache.shape[2], _ptr(cos_sin), _stream())
     return q

@@ -86,7 +86,7 @@ class PagedAttention(Mixer):
         q = None
         if rot is not None and cache.writes:
             rows = x.x if isinstance(x, ops.Prenormed) else x
-            if ops.linear_rope_ok(rows.shape[0], self.wqkv.shape[0], rows.shape[1], self.head_dim, rot[1], cache.k.shape[2],
+            if ops.linear_rope_ok(x.shape[0], self.wqkv.shape[0], x.shape[1], self.head_dim, rot[1], cache.k.shape[2],
                                   rows.dtype, cache.k.dtype, isinstance(x, ops.Prenormed)):
                 # a few rows (decoding) or a long step: the projection rotates and stores its rows itself
                 table = self.position.table(ctx, always=True) if hasattr(self.position, "table") else None

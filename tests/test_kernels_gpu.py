@@ -458,7 +458,7 @@ def test_linear_split_norm(m, hidden, kp, nc):
     out, pre = ops.linear(a.to(DEV), wo.to(DEV), torch.float32, residual=hd, next_norm=(nw.to(DEV), eps))
     assert out is hd and pre is not None
     _close(hd, h2_ref, 2e-5, "residual")
-    assert torch.equal(pre.x.cpu(), (hd.cpu() * nw).to(torch.bfloat16)), "rows times norm weight, rounded once"
+    assert torch.equal(pre.rows().cpu(), (hd.cpu() * nw).to(torch.bfloat16)), "rows times norm weight, rounded once"
     ss = pre.ss.cpu().double().sum(0)[:m]
     assert float(((ss - (hd.cpu().double() ** 2).sum(1)).abs() / ss).max()) < 1e-5
     normed = h2_ref * torch.rsqrt((h2_ref ** 2).mean(1, keepdim=True) + eps) * nw.double()
