@@ -332,12 +332,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int skip_
 // ---- prefill, keys and values through LDS ---------------------------------------------------
 // The four waves of a block (four heads of one kv group) need the same keys and values.  Here a
 // step's 32 keys and values are copied once per block into LDS by the direct global-to-LDS load,
-// three steps ahead of their use (a ring of four stages, one barrier per step), and every wave reads
+// NS - 1 steps ahead of their use (a ring of NS stages, three or four; one barrier per step), and every wave reads
 // its operand fragments from there: a quarter of the global load instructions, and none of their
-// latency in the way.  Head sizes 32, 64, 128 (a power-of-two number of 16-byte chunks per key row).
+// latency in the way.  Head sizes 32, 64, 128 (a power-of-two number of 16-byte chunks per key row); pages of
+// at least 16 keys (a power of two), so that each half of a step lies in one page.
 // LDS layout of a stage: the key tile as 32 rows of D elements, chunk c of row r stored at
 // (c + f(r)) mod (D / 8) so that the 16 rows a quarter wave reads fall into different banks; the
-// value tile as D rows of 32 keys (64 bytes), chunk g of row d at g ^ ((d >> 2) & 3).
+// value tile in pieces of 1 KB, one per (32 elements, half of the step's keys), the eight keys 8 e.. of
+// element d at place 32 e + d % 32 of its piece.
 #define GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define ATTN_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
@@ -354,14 +356,13 @@ __device__ __host__ inline int portion_parts(int steps, int max_parts, int min_s
   return max_parts <= 1 ? 1 : min(max_parts, max(1, steps / min_steps));
 }
 
-template <int D, int NQ>
-__global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, int skip_single) {
+template <int D, int NQ, int NS = 4, int OCC = 2>
+__global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, int skip_single) {
   constexpr int C = D / 8;             // 16-byte chunks per key row
   constexpr int SH = C == 16 ? 0 : (C == 8 ? 1 : 2);
   constexpr int KI = D / 16;           // 1 KB loads per key tile (32 rows of 2 D bytes), and per value tile
   constexpr int LP = 2 * KI / 4;       // loads per wave and step
   constexpr int STAGE = 2 * KI * 1024;
-  constexpr int NS = 4;
   static_assert(D == 32 || D == 64 || D == 128, "head size");
   __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -418,82 +419,82 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
   }
   const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this block
 
-  // what this lane fetches in each of its loads of a step: load t = wave + 4 i; t < KI is a piece of
-  // the key tile (64 chunk slots: 64 / C whole rows, all in one page), else of the value tile (16 rows
-  // of four chunks of eight keys, up to four pages).  Page numbers are read with wave-uniform (scalar)
-  // loads: a vector load here would have to wait for every outstanding copy into LDS.
+  // What this lane fetches in each of its loads of a step: load t = wave + 4 i.  t < KI is a piece of the key tile
+  // (64 chunk slots: 64 / C whole rows of one group of eight keys), else a piece of the value tile: the step's keys
+  // are two halves of 16 (each inside one page: pages hold at least 16 keys), and value load tv = t - KI covers half
+  // tv % 2 for the 32 elements 32 (tv / 2)..: lane L takes the eight keys L / 32 of element L % 32.  So every load
+  // has ONE page, and its address is a uniform part (scalar arithmetic, no branches) plus the lane's constant
+  // offset.  Page numbers are read with wave-uniform (scalar) loads, one step ahead: a vector load here would have
+  // to wait for every outstanding copy into LDS.
   const int psh = a.page_shift, pmask = ps - 1;
+  __builtin_assume(wave >= 0 && wave < 4);
   // the block table through the constant address space: uniform loads from it are scalar loads
   const __attribute__((address_space(4))) int* ctab = (const __attribute__((address_space(4))) int*)(uintptr_t)table;
-  // (load t = wave + 4 i; t < KI: slot 64 t + lane of the key tile, row = slot / C, chunk slot % C rotated
-  // by the row; else value row d = 16 (t - KI) + lane / 4 and the group of eight keys vgroup)
-  const int vgroup = (lane & 3) ^ ((lane >> 4) & 3);
+  // (key load t: slot 64 t + lane of the key tile, row = slot / C, chunk slot % C rotated by the row)
   auto key_row = [&](int t) { return (64 * t + lane) / C; };
   auto key_byte = [&](int t) {
     const int row = (64 * t + lane) / C, pc = (64 * t + lane) % C;
     const int f = ((((row >> 3) << 2) | (row & 3)) >> SH);
     return ((pc - f) & (C - 1)) * 16;
   };
-  auto value_row = [&](int t) { return 16 * (t - KI) + (lane >> 2); };
+  auto value_row = [&](int t) { return 32 * ((t - KI) >> 1) + (lane & 31); };
   unsigned lane_off[LP];   // byte offset of this lane's 16 bytes from the uniform part of a load's address
+  bool second[LP];         // the load's keys lie in the second half of the step (keys j0 + 16..)
+  unsigned row8[LP];       // key loads: the first key of the load's group of eight, from j0
 #pragma unroll
   for (int i = 0; i < LP; ++i) {
     const int t = wave + 4 * i;
-    if (t < KI)
-      lane_off[i] = (unsigned)((key_row(t) - 8 * (((64 * t) / C) >> 3)) * D * 2 + key_byte(t));
-    else
-      lane_off[i] = (unsigned)(((kvh * D + value_row(t)) * ps + ((8 * vgroup) & pmask)) * 2);
+    if (t < KI) {
+      const int gr = ((64 * t) / C) >> 3;
+      lane_off[i] = (unsigned)((key_row(t) - 8 * gr) * D * 2 + key_byte(t));
+      second[i] = gr >= 2;
+      row8[i] = 8 * gr;
+    } else {
+      lane_off[i] = (unsigned)((value_row(t) * ps + 8 * (lane >> 5)) * 2);
+      second[i] = ((t - KI) & 1) != 0;
+      row8[i] = 0;
+    }
   }
-  const unsigned vpage_bytes = (unsigned)(a.n_kv * D * ps * 2);
-  // the pages of the four groups of eight keys of a step (clamped to the last key that exists); a key
-  // load's rows lie in one of these groups, or past the end in the last key's page
-  auto pages_of = [&](int step, int (&pg)[4]) {
+  const unsigned page_bytes = (unsigned)(a.n_kv * D * ps * 2);   // of a key page, and of a value page
+  const unsigned char* kbase = (const unsigned char*)a.k_cache + (size_t)kvh * ps * D * 2;
+  const unsigned char* vbase = (const unsigned char*)a.v_cache + (size_t)kvh * D * ps * 2;
+  // the pages of the two halves of the step that is issued next (the second clamped to the last key that exists)
+  int pp0 = 0, pp1 = 0;
+  auto pages_of = [&](int step) {
     const int j0 = first + step * 32;
-#pragma unroll
-    for (int gg = 0; gg < 4; ++gg) pg[gg] = ctab[min(j0 + 8 * gg, (ctx - 1) & ~7) >> psh];
+    pp0 = ctab[j0 >> psh];
+    pp1 = ctab[min(j0 + 16, (ctx - 1) & ~7) >> psh];
   };
-  auto issue = [&](int step, int stage, const int (&pg)[4]) {
+  auto issue = [&](int step, int stage) {
     const int j0 = first + step * 32;
     unsigned char* buf = stages + stage * STAGE;
-    if (j0 + 32 <= ctx) {
-      // all 32 keys exist: a load's address is a uniform part (page, kv head, place in the page; scalar
-      // arithmetic) plus the lane's constant offset; only the page of a value load differs by lane
-      const unsigned in_page = (unsigned)(j0 & pmask);
-      // (opaque copies: the compiler otherwise turns the selection by lane into an indexed load from a
-      // copy of pg in scratch memory)
-      int p0 = pg[0], p1 = pg[1], p2 = pg[2], p3 = pg[3];
-      asm volatile("" : "+s"(p0), "+s"(p1), "+s"(p2), "+s"(p3));
-      const int vpage = vgroup == 0 ? p0 : (vgroup == 1 ? p1 : (vgroup == 2 ? p2 : p3));
-      const unsigned char* vsrc = (const unsigned char*)a.v_cache + (size_t)(unsigned)vpage * vpage_bytes + in_page * 2;
+    if (j0 + 32 <= ctx) {   // all 32 keys exist
 #pragma unroll
       for (int i = 0; i < LP; ++i) {
         const int t = wave + 4 * i;
+        const unsigned page = (unsigned)(second[i] ? pp1 : pp0);
         const unsigned char* src;
-        if (t < KI) {
-          const int gr = ((64 * t) / C) >> 3;
-          const int page = gr == 0 ? pg[0] : (gr == 1 ? pg[1] : (gr == 2 ? pg[2] : pg[3]));
-          const unsigned char* kb = (const unsigned char*)(a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + ((j0 + 8 * gr) & pmask)) * D);
-          src = kb + lane_off[i];
-        } else {
-          src = vsrc + lane_off[i];
-        }
-        __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+        if (t < KI)
+          src = kbase + (size_t)page * page_bytes + (unsigned)(((j0 + row8[i]) & pmask) * D * 2);
+        else
+          src = vbase + (size_t)page * page_bytes + (unsigned)(((j0 + (second[i] ? 16 : 0)) & pmask) * 2);
+        __builtin_amdgcn_global_load_lds(GPTR(src + lane_off[i]), LPTR(buf + t * 1024), 16, 0, 0);
       }
       return;
     }
+    // the step that holds the last key: rows and groups past it are clamped to it (their scores are masked, their
+    // values cleared when they are read)
 #pragma unroll
     for (int i = 0; i < LP; ++i) {
       const int t = wave + 4 * i;
       const unsigned char* src;
       if (t < KI) {
-        const int gr = ((64 * t) / C) >> 3;                  // the group of eight keys this load lies in
-        const int page = gr == 0 ? pg[0] : (gr == 1 ? pg[1] : (gr == 2 ? pg[2] : pg[3]));
         const int key = min(j0 + key_row(t), ctx - 1);
+        const int page = second[i] ? pp1 : pp0;
         src = (const unsigned char*)(a.k_cache + ((size_t)(page * a.n_kv + kvh) * ps + (key & pmask)) * D) + key_byte(t);
       } else {
-        const int gg = vgroup;
-        const int kb = min(j0 + 8 * gg, (ctx - 1) & ~7);
-        const int page = gg == 0 ? pg[0] : (gg == 1 ? pg[1] : (gg == 2 ? pg[2] : pg[3]));
+        const int kb = min(j0 + (second[i] ? 16 : 0) + 8 * (lane >> 5), (ctx - 1) & ~7);
+        const int page = second[i] ? pp1 : pp0;
         src = (const unsigned char*)(a.v_cache + ((size_t)(page * a.n_kv + kvh) * D + value_row(t)) * ps + (kb & pmask));
       }
       __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
@@ -508,16 +509,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
 #pragma unroll
     for (int dk = 0; dk < D / 32; ++dk) kaddr[t2][dk] = (row * C + ((dk * 4 + g + (c >> SH)) & (C - 1))) * 16;
   }
-  const unsigned vaddr = KI * 1024 + (c * 4 + (g ^ ((c >> 2) & 3))) * 16;
+  // value fragment dt of lane (g, c): element 16 dt + c, keys 8 g..: load 2 (dt / 2) + g / 2, place 32 (g % 2) + 16 (dt % 2) + c;
+  // eight neighbouring lanes read 128 contiguous bytes
+  const unsigned vaddr = KI * 1024 + (g >> 1) * 1024 + (g & 1) * 512 + c * 16;
 
-  int pg[4];          // page numbers of the step that is issued next, fetched one step ahead (scalar loads)
 #pragma unroll
   for (int p = 0; p < NS; ++p)
     if (p < nsteps) {
-      pages_of(p, pg);
-      issue(p, p, pg);
+      pages_of(p);
+      issue(p, p);
     }
-  if (NS < nsteps) pages_of(NS, pg);
+  if (NS < nsteps) pages_of(NS);
   // The scores of step s + 1 are multiplied while the softmax of step s runs on the vector ALU (two
   // independent instruction streams for the scheduler to interleave); so step s reads the values of
   // stage s and the keys of stage s + 1, and a stage is free again one step later than it would be.
@@ -556,8 +558,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     if (ahead >= 1) ATTN_WAIT_VM(LP); else ATTN_WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
     if (s >= 1 && s + NS - 1 < nsteps) {
-      issue(s + NS - 1, stage == 0 ? NS - 1 : stage - 1, pg);
-      if (s + NS < nsteps) pages_of(s + NS, pg);
+      issue(s + NS - 1, stage == 0 ? NS - 1 : stage - 1);
+      if (s + NS < nsteps) pages_of(s + NS);
     }
     const unsigned base = lds0 + stage * STAGE;
     // the keys of the following stage are multiplied into the next step's scores before this step's
@@ -569,7 +571,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_lds_kernel(AttnArgs a, in
     }
     // the value fragments travel while the softmax runs
     u32x4_t vv[D / 16];
-#define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<dt * 1024>(base + vaddr)
+#define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<(dt >> 1) * 2048 + (dt & 1) * 256>(base + vaddr)
     ATTN_RV(0); ATTN_RV(1); ATTN_RV(2); ATTN_RV(3); ATTN_RV(4); ATTN_RV(5); ATTN_RV(6); ATTN_RV(7);
 #undef ATTN_RV
     bf16x8_t pf[NQ];
@@ -809,16 +811,19 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     }
   }
   if (has_multi) {
-    // A wave owns 32 query rows (two tiles: half the key and value reads per product) when that still gives
-    // every CU its two blocks; otherwise 16 rows and twice the blocks (a portion of 512 tokens behind a long
-    // prefix: a fifth faster).  Both give the same bits: a query column never sees another's values.
+    // A wave owns 16 query rows, three blocks to a CU, or 32 rows (two tiles: half the key and value reads per
+    // product, more registers), two blocks to a CU.  A step's time is set by how many instructions a wave has to
+    // issue, so more waves help while there are few blocks: measured with 32 heads of 128 in 8 groups, 16 rows are
+    // faster up to about 2,500 query rows (1,024: 31 against 42 us; 2,048: 60 against 78; 3,072: 125 against 118;
+    // 8,192: 733 against 674; 32,768: 10.9 against 9.4 ms).  Both give the same bits: a query column never sees
+    // another's values.
     const int kv_groups = a.n_kv * ((group + 3) / 4);
     const long blocks2 = (long)((max_q_len + 31) / 32) * kv_groups * n_req;
-    const bool two = g_attn_tune == 2 || (g_attn_tune != 3 && blocks2 >= 512);
+    const bool two = g_attn_tune == 2 || (g_attn_tune != 3 && blocks2 >= 768);
     const int rows = two ? 32 : 16;
     const int skip = num_single > 0 ? 1 : 0;
     if constexpr (D == 32 || D == 64 || D == 128) {
-      if (a.portion_splits > 1 && g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
+      if (a.portion_splits > 1 && g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D) {
         // few query blocks under a long context: the keys of each are split over blocks (of 32 query rows)
         const dim3 sgrid((max_q_len + 31) / 32, kv_groups, n_req * a.portion_splits);
         hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), sgrid, dim3(256), 0, s, a, skip);
@@ -832,11 +837,11 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
-      if (g_attn_tune != 1 && a.page_shift >= 3 && a.page_size >= 512 / D) {
+      if (g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D) {
         if (two)
           hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), grid, dim3(256), 0, s, a, skip);
         else
-          hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 1>), grid, dim3(256), 0, s, a, skip);
+          hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 1, 3, 3>), grid, dim3(256), 0, s, a, skip);
         return 0;
       }
     }
