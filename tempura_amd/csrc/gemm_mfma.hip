@@ -668,9 +668,10 @@ int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, i
                      size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s);
 
 extern int g_pipe_big;
-// order: 1 tiled plain, 2 tiled XCD-aware, 3 pipelined; 5 / 6: pipelined with 256 x 256 tiles always / never
+// order: 1 tiled plain, 2 tiled XCD-aware, 3 pipelined; 5 / 6: pipelined with 256 x 256 tiles always / never;
+// 7 / 8: with 256 x 192 tiles wherever N is a multiple of 192 / never
 extern "C" void tp_linear_tune_tile(int order) {
-  g_pipe_big = order == 5 ? 1 : (order == 6 ? 2 : 0);
+  g_pipe_big = order == 5 ? 1 : (order == 6 ? 2 : (order == 7 ? 3 : (order == 8 ? 4 : 0)));
   g_tune_order = order >= 5 ? 0 : order;
 }
 

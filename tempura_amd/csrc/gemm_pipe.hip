@@ -615,49 +615,57 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
 // the CUs; the columns that are left go to the kernel above.
 namespace {
 
-constexpr int BNB = 256, STAGE_BIG = (BM + BNB) * ROWB, NSB = 2, LPWB = 16;
+constexpr int BNB = 256, NSB = 2;
 constexpr int CLDB = 128 + 4;   // padded row of a quarter (32 rows) of a wave's result tile in LDS, in floats
+constexpr int CLDS = 32 + 4;    // padded row of a strip (32 columns) of a wave's result tile in LDS, in floats
 
-// Operand fragments of a half step (32 of K): eight 16-row tiles of x, eight of w.  The w fragments are
-// double-buffered, and so are the last two x fragments; x fragments 0..5 are used by one row of MFMAs each,
+// Operand fragments of a half step (32 of K): eight 16-row tiles of x, NJ (eight or six) of w.  The w fragments
+// are double-buffered, and so are the last two x fragments; x fragments 0..5 are used by one row of MFMAs each,
 // so the next half step's takes the register as soon as that row has been issued (the LDS read takes far
 // longer than an MFMA needs to fetch its operands).
+template <int NJ>
 struct FragsBig {
-  u32x4_t a[6], a6[2], a7[2], b[2][8];
+  u32x4_t a[6], a6[2], a7[2], b[2][NJ];
 };
-#define TIE_FRAGS(f, p)                                                                                                  \
-  asm volatile("s_waitcnt lgkmcnt(0)"                                                                                   \
-               : "+v"(f.b[p][0]), "+v"(f.b[p][1]), "+v"(f.b[p][2]), "+v"(f.b[p][3]), "+v"(f.b[p][4]), "+v"(f.b[p][5]),    \
-                 "+v"(f.b[p][6]), "+v"(f.b[p][7]), "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), \
-                 "+v"(f.a[5]), "+v"(f.a6[p]), "+v"(f.a7[p]))
-// load I (0..15) of this wave into stage `buf`: 0..7 are x rows, 8..15 w rows; one load covers 8 rows
-template <int I>
+template <int NJ, int p>
+__device__ inline void tie_frags(FragsBig<NJ>& f) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(f.b[p][0]), "+v"(f.b[p][1]), "+v"(f.b[p][2]), "+v"(f.b[p][3]), "+v"(f.b[p][4]), "+v"(f.b[p][5]),
+                 "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), "+v"(f.a[5]), "+v"(f.a6[p]),
+                 "+v"(f.a7[p]));
+  if constexpr (NJ == 8) asm volatile("" : "+v"(f.b[p][6]), "+v"(f.b[p][7]));
+}
+// load I (0..7 + NJ) of this wave into stage `buf`: 0..7 are x rows, the others w rows; one load covers 8 rows
+template <int I, int NJ>
 __device__ inline void issue_big(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
-                                 const unsigned (&voff)[LPWB], int wave) {
-  const int t = I < 8 ? wave * 8 + I : 32 + wave * 8 + (I - 8);
-  const unsigned char* src = (I < 8 ? xk : wk) + voff[I];
-  __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+                                 const unsigned (&voff)[8 + NJ], int wave) {
+  if constexpr (I < 8 + NJ) {
+    const int t = I < 8 ? wave * 8 + I : 32 + wave * NJ + (I - 8);
+    const unsigned char* src = (I < 8 ? xk : wk) + voff[I];
+    __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+  }
 }
+template <int NJ>
 __device__ inline void issue_stage_big(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
-                                       const unsigned (&voff)[LPWB], int wave) {
-  issue_big<0>(buf, xk, wk, voff, wave); issue_big<1>(buf, xk, wk, voff, wave); issue_big<2>(buf, xk, wk, voff, wave);
-  issue_big<3>(buf, xk, wk, voff, wave); issue_big<4>(buf, xk, wk, voff, wave); issue_big<5>(buf, xk, wk, voff, wave);
-  issue_big<6>(buf, xk, wk, voff, wave); issue_big<7>(buf, xk, wk, voff, wave); issue_big<8>(buf, xk, wk, voff, wave);
-  issue_big<9>(buf, xk, wk, voff, wave); issue_big<10>(buf, xk, wk, voff, wave); issue_big<11>(buf, xk, wk, voff, wave);
-  issue_big<12>(buf, xk, wk, voff, wave); issue_big<13>(buf, xk, wk, voff, wave); issue_big<14>(buf, xk, wk, voff, wave);
-  issue_big<15>(buf, xk, wk, voff, wave);
+                                       const unsigned (&voff)[8 + NJ], int wave) {
+  issue_big<0, NJ>(buf, xk, wk, voff, wave); issue_big<1, NJ>(buf, xk, wk, voff, wave); issue_big<2, NJ>(buf, xk, wk, voff, wave);
+  issue_big<3, NJ>(buf, xk, wk, voff, wave); issue_big<4, NJ>(buf, xk, wk, voff, wave); issue_big<5, NJ>(buf, xk, wk, voff, wave);
+  issue_big<6, NJ>(buf, xk, wk, voff, wave); issue_big<7, NJ>(buf, xk, wk, voff, wave); issue_big<8, NJ>(buf, xk, wk, voff, wave);
+  issue_big<9, NJ>(buf, xk, wk, voff, wave); issue_big<10, NJ>(buf, xk, wk, voff, wave); issue_big<11, NJ>(buf, xk, wk, voff, wave);
+  issue_big<12, NJ>(buf, xk, wk, voff, wave); issue_big<13, NJ>(buf, xk, wk, voff, wave); issue_big<14, NJ>(buf, xk, wk, voff, wave);
+  issue_big<15, NJ>(buf, xk, wk, voff, wave);
 }
-// The 64 MFMAs of a half step with the fragments of parity P, row by row.  READ: the next half step's
+// The 8 x NJ MFMAs of a half step with the fragments of parity P, row by row.  READ: the next half step's
 // fragments are requested between them (w and the last two x fragments into the other set, x fragment i into
-// a[i] after row i).  LOAD: one global load per group of four MFMAs.
-template <int P, bool READ, bool LOAD>
-__device__ inline void half_step_big(f32x4_t (&acc)[8][8], FragsBig& f, unsigned aaddr, unsigned baddr, unsigned char* buf,
-                                     const unsigned char* xk, const unsigned char* wk, const unsigned (&voff)[LPWB],
+// a[i] after row i).  LOAD: one global load per group of MFMAs.
+template <int P, bool READ, bool LOAD, int NJ>
+__device__ inline void half_step_big(f32x4_t (&acc)[8][NJ], FragsBig<NJ>& f, unsigned aaddr, unsigned baddr, unsigned char* buf,
+                                     const unsigned char* xk, const unsigned char* wk, const unsigned (&voff)[8 + NJ],
                                      int wave) {
 #define SB() __builtin_amdgcn_sched_barrier(0)
 #define AF(I) (I < 6 ? f.a[I < 6 ? I : 0] : (I == 6 ? f.a6[P] : f.a7[P]))
 // (written as assembly with the accumulator tied to an AGPR: left to itself the register allocator keeps
-// part of the 256 accumulator registers in VGPRs and copies them back and forth inside the loop)
+// part of the accumulator registers in VGPRs and copies them back and forth inside the loop)
 #define M1(I, J) \
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[I][J]) : "v"(AF(I)), "v"(f.b[P][J])); \
   SB()
@@ -673,26 +681,44 @@ __device__ inline void half_step_big(f32x4_t (&acc)[8][8], FragsBig& f, unsigned
   if (READ) f.a7[P ^ 1] = lds_read16<7 * 16 * ROWB>(aaddr);    \
   SB()
 #define LD(G) \
-  if (LOAD) issue_big<G>(buf, xk, wk, voff, wave); \
+  if (LOAD) issue_big<G, NJ>(buf, xk, wk, voff, wave); \
   SB()
+  if constexpr (NJ == 8) {
 #define ROW(I, PRE0, PRE1)                             \
   PRE0;                                                \
   M1(I, 0); M1(I, 1); LD(2 * (I)); M1(I, 2); M1(I, 3); \
   PRE1;                                                \
   M1(I, 4); M1(I, 5); LD(2 * (I) + 1); M1(I, 6); M1(I, 7)
-  ROW(0, RB(0), RB(1));
-  ROW(1, RB(2); RA(0), RB(3));
-  ROW(2, RB(4); RA(1), RB(5));
-  ROW(3, RB(6); RA(2), RB(7));
-  ROW(4, RA(3), R67());
-  ROW(5, RA(4), (void)0);
-  ROW(6, RA(5), (void)0);
-  ROW(7, (void)0, (void)0);
+    ROW(0, RB(0), RB(1));
+    ROW(1, RB(2); RA(0), RB(3));
+    ROW(2, RB(4); RA(1), RB(5));
+    ROW(3, RB(6); RA(2), RB(7));
+    ROW(4, RA(3), R67());
+    ROW(5, RA(4), (void)0);
+    ROW(6, RA(5), (void)0);
+    ROW(7, (void)0, (void)0);
+#undef ROW
+  } else {
+    static_assert(NJ == 6 || NJ == 8, "w tiles per wave");
+#define ROW(I, PRE0, PRE1)                   \
+  PRE0;                                      \
+  M1(I, 0); M1(I, 1); LD(2 * (I)); M1(I, 2); \
+  PRE1;                                      \
+  M1(I, 3); M1(I, 4); LD(2 * (I) + 1); M1(I, 5)
+    ROW(0, RB(0), RB(1));
+    ROW(1, RB(2); RA(0), RB(3));
+    ROW(2, RB(4); RA(1), RB(5));
+    ROW(3, RA(2), (void)0);
+    ROW(4, RA(3), R67());
+    ROW(5, RA(4), (void)0);
+    ROW(6, RA(5), (void)0);
+    ROW(7, (void)0, (void)0);
+#undef ROW
+  }
   if (READ) {
-    TIE_FRAGS(f, P ^ 1);
+    tie_frags<NJ, (P ^ 1)>(f);
     SB();
   }
-#undef ROW
 #undef LD
 #undef R67
 #undef RA
@@ -701,8 +727,9 @@ __device__ inline void half_step_big(f32x4_t (&acc)[8][8], FragsBig& f, unsigned
 #undef AF
 #undef SB
 }
-__device__ inline void read_all_big(FragsBig& f, unsigned aaddr, unsigned baddr) {
-#define RB0(J) f.b[0][J] = lds_read16<(J) * 16 * ROWB>(baddr)
+template <int NJ>
+__device__ inline void read_all_big(FragsBig<NJ>& f, unsigned aaddr, unsigned baddr) {
+#define RB0(J) if constexpr (J < NJ) f.b[0][J < NJ ? J : 0] = lds_read16<(J) * 16 * ROWB>(baddr)
 #define RA0(I) f.a[I] = lds_read16<(I) * 16 * ROWB>(aaddr)
   RB0(0); RB0(1); RB0(2); RB0(3); RB0(4); RB0(5); RB0(6); RB0(7);
   RA0(0); RA0(1); RA0(2); RA0(3); RA0(4); RA0(5);
@@ -710,21 +737,25 @@ __device__ inline void read_all_big(FragsBig& f, unsigned aaddr, unsigned baddr)
   f.a7[0] = lds_read16<7 * 16 * ROWB>(aaddr);
 #undef RB0
 #undef RA0
-  TIE_FRAGS(f, 0);
+  tie_frags<NJ, 0>(f);
 }
 
 }  // namespace
 
-// No split of K here.  N: the columns of this launch (a multiple of 256); ldo as above.
+// No split of K here.  A block tile is 256 rows x 32 NJ columns (NJ = 8: 256, a wave owns 128 x 128; NJ = 6: 192, a
+// wave owns 128 x 96: for an N where that many more tiles make whole rounds of the CUs).  N: the columns of this
+// launch (a multiple of the tile's); ldo as above.
+template <int NJ>
 __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                             void* __restrict__ out, int mode, int M, int N, int K,
                                                             int pm, int ldo, RopeOut rp, int wt) {
-  __shared__ __attribute__((aligned(1024))) unsigned char stages[NSB * STAGE_BIG];
+  constexpr int BNT = 32 * NJ, WN = 16 * NJ, STAGE = (BM + BNT) * ROWB, LPWT = 8 + NJ;
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[NSB * STAGE];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   int bm, bn;
   {
-    const int MB = (M + BM - 1) / BM, NB = N / BNB;
+    const int MB = (M + BM - 1) / BM, NB = N / BNT;
     const int pq = 32 / pm;
     const int MS = (MB + pm - 1) / pm;
     const int c = blockIdx.x % 8, j = blockIdx.x / 8;
@@ -733,27 +764,27 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
     bn = c + 8 * ((t / MS) * pq + r / pm);
     if (bm >= MB || bn >= NB) return;
   }
-  const int m0 = bm * BM, n0 = bn * BNB;
-  f32x4_t acc[8][8];
+  const int m0 = bm * BM, n0 = bn * BNT;
+  f32x4_t acc[8][NJ];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NJ; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   const int KT = K / BK;
   const int g = lane >> 4, c = lane & 15;
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
   const unsigned off0 = c * ROWB + (((0 * 4 + g) ^ ((c >> 1) & 7)) << 4);
   const unsigned off1 = c * ROWB + (((1 * 4 + g) ^ ((c >> 1) & 7)) << 4);
-  const unsigned arow = wm * 128 * ROWB, brow = (BM + wn * 128) * ROWB;
-  unsigned voff[LPWB];
+  const unsigned arow = wm * 128 * ROWB, brow = (BM + wn * WN) * ROWB;
+  unsigned voff[LPWT];
 #pragma unroll
-  for (int i = 0; i < LPWB; ++i) {
-    const int row = (wave * 8 + (i & 7)) * 8 + (lane >> 3);
+  for (int i = 0; i < LPWT; ++i) {
+    const int row = (i < 8 ? wave * 8 + i : wave * NJ + (i - 8)) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     const int grow = i < 8 ? min(row, M - 1 - m0) : row;   // (every w row of the launch exists)
     voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
     if (wt && i >= 8) {   // block u of the stage's weights: row group u / 2 of the block tile, first or second 32 of k
-      const int u = wave * 8 + (i & 7);
+      const int u = wave * NJ + (i - 8);
       voff[i] = ((unsigned)(u / 2) * (unsigned)(K / 32) + (u & 1)) * 1024u + lane * 16;
     }
   }
@@ -763,59 +794,61 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
   const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2;
 #pragma unroll
   for (int p = 0; p < NSB; ++p)
-    if (p < KT) issue_stage_big(stages + p * STAGE_BIG, xk + p * BK * 2, wk + p * wkstep, voff, wave);
+    if (p < KT) issue_stage_big<NJ>(stages + p * STAGE, xk + p * BK * 2, wk + p * wkstep, voff, wave);
   xk += NSB * BK * 2;
   wk += NSB * wkstep;
-  FragsBig f;
-  if (KT > 1) WAIT_VM(LPWB); else WAIT_VM(0);
+  FragsBig<NJ> f;
+  if (KT > 1) WAIT_VM(LPWT); else WAIT_VM(0);
   __builtin_amdgcn_s_barrier();
-  read_all_big(f, lds0 + arow + off0, lds0 + brow + boff0);
+  read_all_big<NJ>(f, lds0 + arow + off0, lds0 + brow + boff0);
   // Tile kt: the first half step multiplies the fragments of its first 32 of K and reads those of the second;
   // then tile kt + 1 must have landed for every wave (barrier), which also means that every wave is done
   // reading tile kt's stage: the second half step refills it with tile kt + 2 while it multiplies and reads
   // the first fragments of tile kt + 1.
   int st = 0, kt = 0;
   for (; kt + NSB < KT; ++kt) {
-    const unsigned cur = lds0 + st * STAGE_BIG, nxt = lds0 + (st ^ 1) * STAGE_BIG;
-    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    const unsigned cur = lds0 + st * STAGE, nxt = lds0 + (st ^ 1) * STAGE;
+    half_step_big<0, true, false, NJ>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
-    half_step_big<1, true, true>(acc, f, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE_BIG, xk, wk, voff, wave);
+    half_step_big<1, true, true, NJ>(acc, f, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE, xk, wk, voff, wave);
     xk += BK * 2;
     wk += wkstep;
     st ^= 1;
   }
   for (; kt + 1 < KT; ++kt) {  // nothing left to load
-    const unsigned cur = lds0 + st * STAGE_BIG, nxt = lds0 + (st ^ 1) * STAGE_BIG;
-    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    const unsigned cur = lds0 + st * STAGE, nxt = lds0 + (st ^ 1) * STAGE;
+    half_step_big<0, true, false, NJ>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
     WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
-    half_step_big<1, true, false>(acc, f, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
+    half_step_big<1, true, false, NJ>(acc, f, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
     st ^= 1;
   }
   {
-    const unsigned cur = lds0 + st * STAGE_BIG;
-    half_step_big<0, true, false>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
-    half_step_big<1, false, false>(acc, f, 0, 0, nullptr, nullptr, nullptr, voff, wave);
+    const unsigned cur = lds0 + st * STAGE;
+    half_step_big<0, true, false, NJ>(acc, f, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    half_step_big<1, false, false, NJ>(acc, f, 0, 0, nullptr, nullptr, nullptr, voff, wave);
   }
   // The MFMAs are assembly, so the compiler does not know that their results take time: wait out the last ones
   // (eight passes of the matrix core and the write-back).  The wait is tied to their accumulators, or the
   // compiler may read them (a register copy on the way into the epilogue) before it.
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15"
-               : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]), "+a"(acc[7][4]), "+a"(acc[7][5]),
-                 "+a"(acc[7][6]), "+a"(acc[7][7])
+               : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]), "+a"(acc[7][4]), "+a"(acc[7][5])
                :
                : "memory");
+  if constexpr (NJ == 8) asm volatile("" : "+a"(acc[7][6]), "+a"(acc[7][7]));
   // (and every other accumulator passes through an ordered statement after it)
 #pragma unroll
-  for (int i = 0; i < 7; ++i)
-    asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]), "+a"(acc[i][5]),
-                 "+a"(acc[i][6]), "+a"(acc[i][7]));
+  for (int i = 0; i < 7; ++i) {
+    asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]), "+a"(acc[i][5]));
+    if constexpr (NJ == 8) asm volatile("" : "+a"(acc[i][6]), "+a"(acc[i][7]));
+  }
 
-  // ---- the result leaves through LDS, 32 rows of the wave's 128 x 128 at a time ---------------------------
   __syncthreads();
+  const int mw = m0 + wm * 128, nw = n0 + wn * WN;
+  if constexpr (NJ == 8) {
+  // ---- the result leaves through LDS, 32 rows of the wave's 128 x 128 at a time ---------------------------
   float* ct = (float*)stages + wave * (32 * CLDB);
-  const int mw = m0 + wm * 128, nw = n0 + wn * 128;
   // (written out four times: were the loop over the quarters not unrolled, the accumulators would be indexed at
   // run time and live in scratch memory)
 #define QUARTER(Q)                                                                                              \
@@ -837,6 +870,51 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
   QUARTER(2)
   QUARTER(3)
 #undef QUARTER
+  } else {
+  // ---- the wave's 128 x 96 leaves as a strip of 64 columns (two halves of 64 rows) and one of 32.  A strip
+  // must lie inside one head of the q/k/v projection (heads of 128 begin at multiples of 128): the wave's first
+  // column is 0, 32, 64 or 96 past such a multiple, and only from 96 the strip of 32 has to come first.  (Both
+  // orders are written out: the accumulators are indexed by constants only.) -----------------------------------
+  float* ct = (float*)stages + wave * (128 * CLDS);
+#define STRIP32(JB)                                                                                             \
+  {                                                                                                             \
+    RopeFetch<128, 32> fetched;                                                                                 \
+    if (mode == OUT_ROPE) rope_fetch(fetched, lane, mw, nw + (JB) * 16, rp, M);                                 \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i) _Pragma("unroll") for (int j = 0; j < 2; ++j)                 \
+        _Pragma("unroll") for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLDS + j * 16 + c] = acc[i][(JB) + j][r]; \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
+    if (mode == OUT_ROPE)                                                                                       \
+      emit_tile_rope<128, 32, CLDS>(ct, lane, mw, nw + (JB) * 16, rp, M, fetched);                              \
+    else                                                                                                        \
+      emit_tile<128, 32, CLDS>(ct, lane, mw, nw + (JB) * 16, out, mode, M, N, ldo);                             \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
+  }
+#define STRIP64(JB, H)                                                                                          \
+  {                                                                                                             \
+    RopeFetch<64, 64> fetched;                                                                                  \
+    if (mode == OUT_ROPE) rope_fetch(fetched, lane, mw + (H) * 64, nw + (JB) * 16, rp, M);                      \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)                 \
+        _Pragma("unroll") for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[(H) * 4 + i][(JB) + j][r]; \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
+    if (mode == OUT_ROPE)                                                                                       \
+      emit_tile_rope<64, 64, CLD>(ct, lane, mw + (H) * 64, nw + (JB) * 16, rp, M, fetched);                     \
+    else                                                                                                        \
+      emit_tile<64, 64, CLD>(ct, lane, mw + (H) * 64, nw + (JB) * 16, out, mode, M, N, ldo);                    \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                          \
+  }
+  static_assert(128 * CLDS >= 64 * CLD, "room for either strip");
+  if ((rp.col0 + nw) % 128 == 96) {
+    STRIP32(0)
+    STRIP64(2, 0)
+    STRIP64(2, 1)
+  } else {
+    STRIP64(0, 0)
+    STRIP64(0, 1)
+    STRIP32(4)
+  }
+#undef STRIP64
+#undef STRIP32
+  }
 }
 
 // ---- the same pipeline for 17..128 rows -----------------------------------------------------------
@@ -1007,7 +1085,7 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
 
 // Returns 0 when launched, -1 when the sizes are not this kernel's.  `scratch` (optional) is room for
 // float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
-int g_pipe_big = 0;   // tuning: 1 = 256 x 256 tiles for every whole block of 256 columns, 2 = never
+int g_pipe_big = 0;   // tuning: 1 = 256 x 256 tiles for every whole block of 256 columns, 2 = never; 3 = 256 x 192 wherever N allows, 4 = never
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
                    size_t scratch_floats, int tune_splits, const RopeOut* rope, hipStream_t s) {
   if ((mode == OUT_ROPE) != (rope != nullptr)) return -1;
@@ -1054,11 +1132,24 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
         nb_big = (int)cand;
       }
     if (g_pipe_big == 1) nb_big = (int)NB2;
+    // Tiles of 256 x 192 where N is a multiple of 192 and that many more tiles fill whole rounds: priced at 1.35
+    // small tiles (the q/k/v projection of 2,048 rows, N = 6,144: 256 tiles in one round instead of 192 of 256 x 256
+    // on three quarters of the CUs, 109 -> 8x us).
+    if (N % 192 == 0 && mode != OUT_SWIGLU && g_pipe_big != 4) {
+      const long t192 = (long)MB * (N / 192);
+      if (1.35 * (double)((t192 + 255) / 256) < best - 1e-9 || g_pipe_big == 3) {
+        const long Q3 = (N / 192 + 7) / 8, QS3 = (Q3 + pq - 1) / pq;
+        const long blocks3 = 8 * QS3 * MS * 32;
+        hipLaunchKernelGGL(gemm_pipe_big_kernel<6>, dim3((unsigned)blocks3), dim3(256), 0, s, x, w, out, mode, M, N, K, pm, ldo,
+                           rp, w_tiled);
+        return 0;
+      }
+    }
   }
   if (nb_big > 0) {
     const long Q2 = (nb_big + 7) / 8, QS2 = (Q2 + pq - 1) / pq;
     const long blocks2 = 8 * QS2 * MS * 32;
-    hipLaunchKernelGGL(gemm_pipe_big_kernel, dim3((unsigned)blocks2), dim3(256), 0, s, x, w, out, mode, M, nb_big * BNB, K,
+    hipLaunchKernelGGL(gemm_pipe_big_kernel<8>, dim3((unsigned)blocks2), dim3(256), 0, s, x, w, out, mode, M, nb_big * BNB, K,
                        pm, ldo, rp, w_tiled);
     const int n_done = nb_big * BNB;
     if (n_done == N) return 0;

@@ -113,7 +113,7 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
 @pytest.mark.parametrize("m,heads,kv,d,rot,k,page", [(1, 4, 2, 64, 64, 256, 16), (8, 32, 8, 128, 128, 4096, 16),
                                                     (16, 3, 1, 48, 32, 96, 8), (5, 6, 3, 16, 16, 2048, 32),
                                                     (2100, 32, 8, 128, 128, 128, 16), (3000, 24, 8, 128, 64, 192, 8),
-                                                    (4300, 4, 2, 128, 128, 64, 16)])
+                                                    (4300, 4, 2, 128, 128, 64, 16), (2900, 10, 1, 128, 128, 320, 16)])
 def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
     """The projection of a few rows that rotates and stores its rows in its epilogue gives the bits of the
     plain product followed by the rotation and cache-write kernel; and both agree with float64."""
@@ -154,6 +154,15 @@ def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
         q4 = ops.linear_rope_kv(xd, ops.tile_weight(wd), pd, sd, invd, rot, 1.0, heads, kv, d, k4, v4,
                                 ops.rope_table(pd, invd, rot, 1.0) if m > 16 else None)
         assert torch.equal(q4, q1) and torch.equal(k4, k1) and torch.equal(v4, v1)
+    if m > 16 and n % 192 == 0:       # tiles of 256 x 192, whose columns span two heads: the same bits
+        ops.library().tp_linear_tune_tile(7)
+        try:
+            for wv in (wd, ops.tile_weight(wd)):
+                k5, v5 = kc.to(DEV), vc.to(DEV)
+                q5 = ops.linear_rope_kv(xd, wv, pd, sd, invd, rot, 1.0, heads, kv, d, k5, v5, ops.rope_table(pd, invd, rot, 1.0))
+                assert torch.equal(q5, q1) and torch.equal(k5, k1) and torch.equal(v5, v1)
+        finally:
+            ops.library().tp_linear_tune_tile(0)
     kr, vr = kc.clone(), vc.clone()
     qr = emu.rope_kv_write(x.double() @ w.double().T, pos, slots, inv, rot, 1.0, heads, kv, d, kr, vr, torch.float64)
     _close(q2, qr, 1e-2, "q")
@@ -409,13 +418,14 @@ def test_tiled_weights_give_the_same_bits(m, n, k):
         assert torch.equal(ops.linear(kb, t, torch.float32), ops.linear(kb, w, torch.float32))
 
 
-@pytest.mark.parametrize("m,n,k", [(300, 512, 128), (1000, 816, 192), (257, 256, 64), (2048, 8448, 128), (2100, 6144, 128)])
+@pytest.mark.parametrize("m,n,k", [(300, 512, 128), (1000, 816, 192), (257, 256, 64), (2048, 8448, 128), (2100, 6144, 128),
+                                   (600, 1152, 320)])
 def test_linear_big_tiles(m, n, k):
     """The 256 x 256 block tiles, forced for every whole block of 256 columns (the columns that are left take
-    the 256 x 128 tiles in a second launch): every output mode against float64, with rows and columns that
-    fill no whole tile; and the choice the library makes by itself at a size where it mixes both.  (The last size,
-    many tiles with a K loop of two steps, is the one at which accumulators read too soon after the last MFMA
-    showed as wrong tiles.)"""
+    the 256 x 128 tiles in a second launch), and the 256 x 192 tiles, forced wherever N is a multiple of 192:
+    every output mode against float64, with rows and columns that fill no whole tile; and the choice the library
+    makes by itself at a size where it mixes tiles.  (The size with many tiles and a K loop of two steps is the
+    one at which accumulators read too soon after the last MFMA showed as wrong tiles.)"""
     ops = _ops()
     lib = ops.library()
     g = torch.Generator().manual_seed(12)
@@ -426,7 +436,7 @@ def test_linear_big_tiles(m, n, k):
     xd, wd = x.to(DEV), w.to(DEV)
     gate_up = ref.view(m, n // 16, 2, 8)
     gated = (torch.nn.functional.silu(gate_up[:, :, 0]) * gate_up[:, :, 1]).reshape(m, n // 2)
-    for mode in (5, 0):
+    for mode in (5, 7, 0):
         lib.tp_linear_tune_tile(mode)
         try:
             _close(ops.linear(xd, wd, torch.float32), ref, 2e-5, f"f32 out, tile mode {mode}")
