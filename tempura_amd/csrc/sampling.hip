@@ -224,11 +224,16 @@ __device__ inline unsigned int select_key(float v, float maxv, float mean_d) {
 // After the first pass the elements of the chosen bin are copied to `cand` (LDS, SMP_CAND entries) when they fit,
 // and the other three passes run over those few instead of the whole row: the k-th largest of 128,256 logits
 // shares its first byte (sign and seven exponent bits) with a few thousand others at most.
+// Logits crowd into a few bins of the first pass (one binade, one bin), and additions to one LDS address from the lanes
+// of a wave go one after the other: every bin therefore has SMP_REP counters side by side, a lane adds to the one of
+// its number, and the copies are summed when the pass is over (8 copies, a row of 128,256 logits, timed from the host: top-k 50
+// 182 -> 143 us, top-p 0.9 256 -> 199 us, typical-p 623 -> 465 us).
 #define SMP_CAND 4096
+#define SMP_REP 8
 template <bool MASS, bool TYP = false>
 __device__ unsigned int radix_select(const float* __restrict__ x, int n, float maxv, unsigned int floor_key,
-                                     unsigned long long target, unsigned long long* hist /*256*/,
-                                     unsigned int* cnt /*256*/, unsigned long long* sh /*4*/, float* cand /*SMP_CAND*/,
+                                     unsigned long long target, unsigned long long* hist /*256 * SMP_REP*/,
+                                     unsigned int* cnt /*256 * SMP_REP*/, unsigned long long* sh /*4*/, float* cand /*SMP_CAND*/,
                                      unsigned long long* gt_out, unsigned int* eq_count, float mean_d = 0.f) {
   unsigned int prefix = 0;
   unsigned long long gt = 0;
@@ -236,18 +241,19 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 24 - 8 * pass;
     __syncthreads();
-    for (int i = threadIdx.x; i < 256; i += blockDim.x) {
+    for (int i = threadIdx.x; i < 256 * SMP_REP; i += blockDim.x) {
       hist[i] = 0;
       cnt[i] = 0;
     }
     __syncthreads();
+    const unsigned int copy = threadIdx.x % SMP_REP;
     auto take = [&](float v) {
       if (float_key(v) < floor_key) return;
       const unsigned int key = select_key<TYP>(v, maxv, mean_d);
       if (pass > 0 && (key >> (shift + 8)) != prefix) return;
-      const unsigned int bin = (key >> shift) & 255u;
-      atomicAdd(&cnt[bin], 1u);
-      if (MASS) atomicAdd(&hist[bin], fix_mass(v, maxv));   // (counting: the weight of a bin is its count)
+      const unsigned int slot = ((key >> shift) & 255u) * SMP_REP + copy;
+      atomicAdd(&cnt[slot], 1u);
+      if (MASS) atomicAdd(&hist[slot], fix_mass(v, maxv));   // (counting: the weight of a bin is its count)
     };
     if (n_cand >= 0) {
       for (int j = threadIdx.x; j < n_cand; j += blockDim.x) take(cand[j]);
@@ -264,17 +270,29 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
       for (; j < n; j += bd) take(x[j]);
     }
     __syncthreads();
+    for (int b = threadIdx.x; b < 256; b += blockDim.x) {   // a bin's copies into its first (integers: any order)
+      unsigned long long hs = 0;
+      unsigned int cs = 0;
+#pragma unroll
+      for (int r = 0; r < SMP_REP; ++r) {
+        hs += hist[b * SMP_REP + r];
+        cs += cnt[b * SMP_REP + r];
+      }
+      hist[b * SMP_REP] = hs;
+      cnt[b * SMP_REP] = cs;
+    }
+    __syncthreads();
     if (threadIdx.x == 0) {
       unsigned long long run = gt;
       int b = 255;
       for (; b > 0; --b) {
-        const unsigned long long w = MASS ? hist[b] : (unsigned long long)cnt[b];
+        const unsigned long long w = MASS ? hist[b * SMP_REP] : (unsigned long long)cnt[b * SMP_REP];
         if (run + w >= target) break;
         run += w;
       }
       sh[0] = run;
       sh[1] = (unsigned long long)b;
-      sh[2] = (unsigned long long)cnt[b];
+      sh[2] = (unsigned long long)cnt[b * SMP_REP];
       sh[3] = 0;            // (the candidates' counter)
     }
     __syncthreads();
@@ -434,8 +452,8 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
     const float* __restrict__ typical_p, const float* __restrict__ rnd, int* __restrict__ out,
     float* __restrict__ info, const float* __restrict__ part_max, const unsigned long long* __restrict__ part_mass) {
-  __shared__ unsigned long long hist[256];
-  __shared__ unsigned int cnt[256];
+  __shared__ unsigned long long hist[256 * SMP_REP];
+  __shared__ unsigned int cnt[256 * SMP_REP];
   __shared__ unsigned long long sh[4];
   __shared__ float cand[SMP_CAND];
   __shared__ unsigned long long scan[SMP_WAVES];
