@@ -99,6 +99,29 @@ def cmd_run(args) -> int:
     return 0
 
 
+def cmd_profile(args) -> int:
+    """Per-entry-point times of one step of prompts and of a few decode steps, run eagerly with events around every
+    call into the kernel library; with --layer-stats the residual stream's mean, variance and largest magnitude
+    before every layer."""
+    eng = _engine_from_args(args)
+    rep = eng.profile(prompt_len=args.prompt_len, batch=args.batch, decode_steps=args.decode_steps,
+                      layer_stats=args.layer_stats, seed=args.seed)
+    if args.json:
+        print(json.dumps(rep))
+        return 0
+    for phase, what in (("prefill", f"{args.batch} prompts of {args.prompt_len} tokens, one step"),
+                        ("decode", f"{args.decode_steps} steps of {args.batch} tokens")):
+        total = sum(r[2] for r in rep[phase])
+        print(f"{phase} ({what}): {total / 1e3:.3f} ms in the kernel library")
+        for name, calls, us, share in rep[phase]:
+            print(f"  {name:40s} {calls:6d} calls {us:12.1f} us {100 * share:5.1f} %")
+    if args.layer_stats:
+        print("residual stream before each layer (and after the last): mean, variance, largest magnitude")
+        for i, mean, var, top in rep["layers"]:
+            print(f"  {i:4d} {mean: .4e} {var:.4e} {top:.4e}")
+    return 0
+
+
 def cmd_inspect(args) -> int:
     from .inspect import format_report, inspect
     info = inspect(args.path)
@@ -167,6 +190,15 @@ def main(argv=None) -> int:
     p.add_argument("--out")
     p.add_argument("--list", action="store_true")
     p.set_defaults(fn=cmd_random_model)
+
+    p = sub.add_parser("profile", help="time every kernel-library call of a prompt step and of decode steps (eager)")
+    _add_engine_args(p)
+    p.add_argument("--prompt-len", type=int, default=128)
+    p.add_argument("--batch", type=int, default=1, help="requests, all in one step")
+    p.add_argument("--decode-steps", type=int, default=4)
+    p.add_argument("--layer-stats", action="store_true", help="also the residual stream's statistics per layer")
+    p.add_argument("--json", action="store_true")
+    p.set_defaults(fn=cmd_profile)
 
     p = sub.add_parser("replay", help="trace replay (same as bin/trace_run)", add_help=False)
     p.set_defaults(fn=None)

@@ -267,6 +267,60 @@ class Engine:
             self.runner.end_request(rid)
         return logits[0].cpu()
 
+    def profile(self, prompt_len: int = 128, batch: int = 1, decode_steps: int = 4, layer_stats: bool = False,
+                seed: int = 0) -> Dict[str, object]:
+        """Where a step's time goes: ``batch`` fresh requests with prompts of ``prompt_len`` seeded random tokens,
+        one eager step for all prompts and ``decode_steps`` eager steps of one token each, every call into the
+        kernel library between a pair of stream events (``ops.KernelTimer``; the reference times layers and prints
+        per-tick times behind environment switches, /root/reference/engine/src/model.rs:1342-1345,
+        /root/reference/server/src/engine_task.rs:530-553).  Returns ``{"prefill": rows, "decode": rows}`` with rows
+        (entry point, calls, microseconds, share), the decode rows summed over the steps; with ``layer_stats`` also
+        ``"layers"``: mean, variance and largest magnitude of the residual stream before every layer and after the
+        last, for the prompts' step (the reference's summary trace, /root/reference/engine/src/pipeline.rs:149-187).
+        The requests are ended afterwards; nothing of the engine's own queue is touched."""
+        import random as _random
+        if self._ahead is not None:
+            self._ahead = (self._ahead[0], ops.take_rows(self._ahead[1]))
+        g = _random.Random(seed)
+        vocab = self.model.spec.vocab_size
+        rids = [("profile", next(self._ids)) for _ in range(batch)]
+        prompts = [[g.randrange(vocab) for _ in range(prompt_len)] for _ in rids]
+        runner = self.runner
+        keep_graph, runner.use_graph = runner.use_graph, False
+        stats: List[tuple] = []
+
+        def observe(i, h):
+            hd = h.double()
+            stats.append((i, float(hd.mean()), float(hd.var(unbiased=False)), float(hd.abs().max())))
+
+        def rows_of(timer):
+            table = timer.table()
+            total = sum(r[3] for r in table) or 1.0
+            return [(name, calls, round(us, 1), round(us / total, 4)) for name, _, calls, us in table]
+
+        out: Dict[str, object] = {}
+        for rid in rids:
+            runner.add_request(rid)
+        try:
+            self.model.observer = observe if layer_stats else None
+            with ops.KernelTimer() as timer:
+                logits = runner.step([StepEntry(rid, p, [prompt_len - 1]) for rid, p in zip(rids, prompts)])
+            self.model.observer = None
+            out["prefill"] = rows_of(timer)
+            if layer_stats:
+                out["layers"] = stats
+            with ops.KernelTimer() as timer:
+                for _ in range(decode_steps):
+                    nxt = ops.argmax(logits).tolist()
+                    logits = runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, nxt)])
+            out["decode"] = rows_of(timer)
+        finally:
+            self.model.observer = None
+            runner.use_graph = keep_graph
+            for rid in rids:
+                runner.end_request(rid)
+        return out
+
     def request(self, rid) -> Request:
         return self._requests[rid]
 

@@ -32,6 +32,9 @@ class CausalLM:
         self.final_norm = build_part("norm", spec.final_norm, h, dtype, device)
         self.lm_head = part_class("lm_head", spec.lm_head.kind)(spec.lm_head, h, dtype, device, spec.vocab_size)
         self.order = spec.resolved_order()
+        #: None, or a callable (i, h) called before run-order entry i and once after the last with the residual
+        #: stream as it stands (eager passes only; see ``Engine.profile``)
+        self.observer = None
         self._plan_caches()
 
     # ---- caches --------------------------------------------------------
@@ -118,7 +121,10 @@ class CausalLM:
         h = self.embedding.forward(tokens)
         m = h.shape[0]
         x = None      # rows handed from one block to the next (a norm carried by the products around it)
+        observe = self.observer
         for i, call in enumerate(self.order):
+            if observe is not None:
+                observe(i, h)
             layer = self.layers[call.layer]
             if not hasattr(layer, "entry_norm"):
                 layer.forward(h, ctx, caches[i])
@@ -127,5 +133,7 @@ class CausalLM:
             after = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else None
             next_norm = after.entry_norm(m) if hasattr(after, "entry_norm") else None
             x = layer.forward(h, ctx, caches[i], x, next_norm)
+        if observe is not None:
+            observe(len(self.order), h)
         x = self.final_norm.forward(h, ctx.logit_rows)
         return self.lm_head.forward(x)

@@ -57,11 +57,53 @@ def library():
     return _Library.get()
 
 
-def _call(name: str, *args) -> None:
+class KernelTimer:
+    """Times every call into the kernel library made while it is active (``with KernelTimer() as t:``), with a pair
+    of events on the current stream around each call: eager steps only (events cannot be recorded into a graph
+    that is replayed), and the pairs serialise nothing, so a call's time includes what its kernels wait for.
+    ``label`` (settable at any time) is stored with every call; ``table()`` waits for the device and returns
+    rows (entry point, label, calls, total microseconds), largest first."""
+
+    def __init__(self):
+        self.label = ""
+        self._events = []
+
+    def __enter__(self):
+        global _timer
+        self._before, _timer = _timer, self
+        return self
+
+    def __exit__(self, *exc):
+        global _timer
+        _timer = self._before
+        return False
+
+    def table(self, by_label: bool = False):
+        torch.cuda.synchronize()
+        total = {}
+        for name, label, e0, e1 in self._events:
+            key = (name, label if by_label else "")
+            calls, us = total.get(key, (0, 0.0))
+            total[key] = (calls + 1, us + 1e3 * e0.elapsed_time(e1))
+        return sorted(((k[0], k[1], c, us) for k, (c, us) in total.items()), key=lambda r: -r[3])
+
+
+_timer: Optional[KernelTimer] = None
+
+
+def _call(name: str, *args, tag: Optional[tuple] = None) -> None:
+    """``tag``: what distinguishes this call in a ``KernelTimer``'s table (a product's sizes)."""
     lib = _Library.get()
+    t = _timer
+    if t is not None:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise KernelError(f"{name}: {lib.tp_last_error().decode()}")
+    if t is not None:
+        e1.record()
+        t._events.append((name if tag is None else name + " " + "x".join(map(str, tag)), t.label, e0, e1))
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -323,7 +365,7 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
     scratch, nscratch = _splitk_scratch(x, m, n)
     _call("tp_linear_fused", _ptr(x), _ptr(wd), _BF16, _ptr(out.data if blocked_out else out), _BF16, 2, m, n, k, 1,
           _ptr(scratch), ctypes.c_size_t(nscratch), *pre, _ptr(None), _ptr(None), _ptr(None), (2 if blocked_out else 0) | wl | xl,
-          0, _ptr(None), _stream())
+          0, _ptr(None), _stream(), tag=(m, n, k))
     return out
 
 
@@ -401,7 +443,7 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
          (partial_ok and residual is None and out_dtype == torch.float32))
     splits = ctypes.c_int(1)
     _call("tp_linear_fused", _ptr(x), _ptr(wd), _dt(x), _ptr(out), _dt(out), acc, m, n, k, int(allow_mfma), _ptr(scratch),
-          ctypes.c_size_t(nscratch), *pre, *post, layout, int(defer), ctypes.byref(splits), _stream())
+          ctypes.c_size_t(nscratch), *pre, *post, layout, int(defer), ctypes.byref(splits), _stream(), tag=(m, n, k))
     if defer and splits.value > 1:
         if next_norm is None:
             return Partials(scratch[: splits.value * m * n].view(splits.value, m, n))
@@ -468,7 +510,7 @@ def linear_rope_kv(x, w: torch.Tensor, positions: torch.Tensor, slots: torch.Ten
     q = torch.empty((m, num_heads, head_dim), dtype=torch.bfloat16, device=x.device)
     _call("tp_linear_rope", _ptr(x), _ptr(wd), int(wl != 0) | (2 if xl else 0), m, n, k, *pre, _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim,
           ctypes.c_float(factor), num_heads, num_kv_heads, head_dim, _ptr(q), _ptr(k_cache), _ptr(v_cache),
-          k_cache.shape[2], _ptr(cos_sin), _stream())
+          k_cache.shape[2], _ptr(cos_sin), _stream(), tag=(m, n, k))
     return q
 
 

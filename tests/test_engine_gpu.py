@@ -278,6 +278,52 @@ def test_command_line(tiny_dirs, tmp_path):
     rec = json.loads(p.stdout.strip().splitlines()[-1])
     assert rec["output_ids"] == plain.greedy_generate(cfg, W, prompt, 6) and rec["finish_reason"] == "length"
     assert '"stats"' in p.stderr
+    p = subprocess.run([sys.executable, tempura, "profile", "--model", model, "--dtype", "float32", "--prompt-len", "12",
+                        "--batch", "2", "--decode-steps", "2", "--kv-blocks", "16", "--max-batch-size", "2", "--json"],
+                       capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    rep = json.loads(p.stdout.strip().splitlines()[-1])
+    assert rep["prefill"] and rep["decode"] and any(r[0] == "tp_paged_attention" for r in rep["decode"])
+
+
+def test_profile_times_every_call_and_reports_the_residual_stream(tiny_dirs):
+    """``Engine.profile``: the step of the prompts makes the calls the model's layers make (one attention call a
+    layer), the statistics of the residual stream before every layer are the plain implementation's, and the
+    engine generates afterwards as if nothing had happened."""
+    import math
+    from tempura_amd.engine import Engine
+    from tempura_amd.sampling import SamplingParams
+    cfg, W = tiny_dirs.plain_model("A")
+    eng = Engine(tiny_dirs.path("A", "float32"), dtype="float32", page_size=16, kv_pages=24, max_batch_size=3)
+    prompt = helpers.random_tokens(cfg["vocab_size"], 9, seed=77)
+    params = SamplingParams(temperature=0.0, max_new_tokens=5)
+    before = eng.generate([prompt], params)
+    rep = eng.profile(prompt_len=21, batch=2, decode_steps=3, layer_stats=True, seed=5)
+    L = cfg["num_hidden_layers"]
+    calls = {name: n for name, n, _, _ in rep["prefill"]}
+    assert calls["tp_paged_attention"] == L and sum(n for name, n in calls.items() if name.startswith("tp_linear")) >= 4 * L and all(us > 0 for _, _, us, _ in rep["prefill"])
+    assert abs(sum(share for *_, share in rep["prefill"]) - 1.0) < 1e-2
+    assert {name: n for name, n, _, _ in rep["decode"]}["tp_paged_attention"] == 3 * L
+    # the residual stream of both prompts, from the plain implementation's formulas
+    import random
+    g = random.Random(5)
+    prompts = [[g.randrange(cfg["vocab_size"]) for _ in range(21)] for _ in range(2)]
+    get = lambda name: W[name].double()
+    inv = plain.rope_inv_freq(cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"],
+                              cfg.get("rope_theta", 10000.0), cfg.get("rope_scaling"))
+    hs = [get("model.embed_tokens.weight")[torch.tensor(p)] for p in prompts]
+    assert len(rep["layers"]) == L + 1
+    for l in range(L + 1):
+        h = torch.cat(hs)
+        i, mean, var, top = rep["layers"][l]
+        assert i == l
+        assert math.isclose(mean, float(h.mean()), rel_tol=1e-3, abs_tol=1e-6)
+        assert math.isclose(var, float(h.var(unbiased=False)), rel_tol=1e-3)
+        assert math.isclose(top, float(h.abs().max()), rel_tol=1e-3)
+        if l < L:
+            hs = [plain.decoder_layer(cfg, get, l, h1, torch.arange(21), inv) for h1 in hs]
+    assert eng.generate([prompt], params) == before
+    assert eng.runner.cache.free_pages() == [p.num_pages for p in eng.runner.cache.pools]
 
 
 def test_model_width_layer_against_plain(tmp_path):
