@@ -818,7 +818,9 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     // 8,192: 733 against 674; 32,768: 10.9 against 9.4 ms).  Both give the same bits: a query column never sees
     // another's values.
     const int kv_groups = a.n_kv * ((group + 3) / 4);
-    const long blocks2 = (long)((max_q_len + 31) / 32) * kv_groups * n_req;
+    // (blocks of 32 rows that have work: from the rows of the portions, not from the grid, which spans the longest
+    // portion for every request; single tokens take the decode kernel)
+    const long blocks2 = (long)((n_tokens - num_single + 31) / 32 + (n_req - num_single - 1)) * kv_groups;
     const bool two = g_attn_tune == 2 || (g_attn_tune != 3 && blocks2 >= 768);
     const int rows = two ? 32 : 16;
     const int skip = num_single > 0 ? 1 : 0;

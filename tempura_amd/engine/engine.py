@@ -132,6 +132,10 @@ class Engine:
             items = self.scheduler.schedule()
             if not items:
                 return []
+            # Prompt portions go first in the batch, single tokens last: a portion that starts at a multiple of
+            # eight positions then also starts at a multiple of eight rows, which is what lets the projection's
+            # epilogue store eight tokens' values as one piece of the transposed value cache.
+            items.sort(key=lambda it: it.count == 1)
             entries = []
             for it in items:
                 toks = it.request.step_tokens(it.start, it.count)

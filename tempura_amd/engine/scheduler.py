@@ -83,6 +83,7 @@ class SchedulerConfig:
     max_num_batched_tokens: int = 2048      # token budget of one step
     prefill_chunk_size: int = 512           # largest prompt portion (engine_task.rs:11)
     max_model_len: int = 4096               # the reference's --max-seq-len
+    portion_align: int = 8                  # a prompt portion that is not the last ends at a multiple of this
 
 
 @dataclass
@@ -144,9 +145,22 @@ class Scheduler:
         return bool(self.waiting or self.running)
 
     # ---- one step's plan -------------------------------------------------
-    def _portion(self, req: Request, budget: int) -> int:
+    def _portion(self, req: Request, budget: int, alone: bool) -> int:
+        """Tokens of the request's prompt for this step: what is left, at most a chunk, at most the budget.  A
+        portion that is cut short of the prompt's end is cut at a multiple of ``portion_align`` positions, so that
+        the next one starts there (cache rows are written in aligned groups of eight where they can be); when
+        not even one such multiple is in reach the request waits for the next step (0), unless the step has no
+        other work (``alone``): then it takes what it can get."""
         rest = req.num_tokens - req.num_computed
-        return min(rest, self.config.prefill_chunk_size, budget)
+        count = min(rest, self.config.prefill_chunk_size, budget)
+        align = self.config.portion_align
+        if count < rest and align > 1:
+            over = (req.num_computed + count) % align
+            if over < count:
+                count -= over
+            elif not alone:
+                count = 0
+        return count
 
     def _fits(self, req: Request, count: int, planned: List[int]) -> bool:
         need = self.cache.pages_needed(req.rid, count)
@@ -183,7 +197,9 @@ class Scheduler:
                 continue
             if budget <= 0:
                 break
-            count = 1 if req.is_decoding else self._portion(req, budget)
+            count = 1 if req.is_decoding else self._portion(req, budget, not items)
+            if count == 0:
+                continue
             while not self._fits(req, count, planned):
                 # give back the pages of the most recently admitted request that is not in the plan yet
                 victims = [r for r in reversed(self.running) if r is not req and all(it.request is not r for it in items)]
@@ -204,8 +220,8 @@ class Scheduler:
                 if len(self.cache.live_requests()) >= self.cache.max_requests:
                     break
                 self.cache.add(req.rid)
-            count = self._portion(req, budget)
-            if not self._fits(req, count, planned):
+            count = self._portion(req, budget, not items)
+            if count == 0 or not self._fits(req, count, planned):
                 self.cache.release(req.rid)
                 break
             self.waiting.popleft()

@@ -78,8 +78,29 @@ def test_mixed_steps_decoding_first_and_budget():
     assert seen_mixed, "prompt portions ran beside decoded tokens"
     assert sorted(r.rid for r in sched.finished) == ["a", "b", "c"]
     assert [len(r.output) for r in sorted(sched.finished, key=lambda r: r.rid)] == [30, 2, 2]
-    # first step: a's whole prompt (5) then 15 of b's tokens fill the budget of 20
-    assert steps[0] == [("a", 0, 5, True), ("b", 0, 15, False)]
+    # first step: a's whole prompt (5); b gets what is left of the budget of 20, cut at a multiple of 8 positions;
+    # the 7 that remain reach no multiple of 8 of c's 9 tokens: c waits
+    assert steps[0] == [("a", 0, 5, True), ("b", 0, 8, False)]
+
+
+def test_portions_end_at_aligned_positions():
+    """A portion that the budget or the chunk size cuts short of the prompt's end stops at a multiple of
+    ``portion_align`` positions (when it has more than that many tokens), the last portion takes what is left;
+    with an alignment of 1 the budget is used to the last token."""
+    sched, cache = make(max_num_batched_tokens=21, prefill_chunk_size=13)
+    sched.add_request(req("a", 50, max_new=1))
+    steps = run(sched, cache)
+    portions = [(start, count) for step in steps for _, start, count, _ in step if start < 50]
+    assert portions == [(0, 8), (8, 8), (16, 8), (24, 8), (32, 8), (40, 10)]
+    sched, cache = make(max_num_batched_tokens=21, prefill_chunk_size=13, portion_align=1)
+    sched.add_request(req("a", 50, max_new=1))
+    steps = run(sched, cache)
+    assert [(start, count) for step in steps for _, start, count, _ in step if start < 50] == [(0, 13), (13, 13), (26, 13), (39, 11)]
+    # a budget below the alignment is still used by a request that runs alone (and reaches a multiple when it can)
+    sched, cache = make(max_num_batched_tokens=5, prefill_chunk_size=13)
+    sched.add_request(req("a", 12, max_new=1))
+    steps = run(sched, cache)
+    assert [(start, count) for step in steps for _, start, count, _ in step if start < 12] == [(0, 5), (5, 3), (8, 4)]
 
 
 def test_eos_stops_and_is_kept():
