@@ -135,7 +135,10 @@ class Engine:
             # Prompt portions go first in the batch, single tokens last: a portion that starts at a multiple of
             # eight positions then also starts at a multiple of eight rows, which is what lets the projection's
             # epilogue store eight tokens' values as one piece of the transposed value cache.
-            items.sort(key=lambda it: it.count == 1)
+            # Among the single tokens the longest contexts go first: attention hands its blocks out in this order,
+            # and a batch of short and long contexts ends sooner when the long ones start first (60 requests of
+            # 128 to 2,304 keys: 77 -> 74 us a layer).
+            items.sort(key=lambda it: (it.count == 1, -it.start))
             entries = []
             for it in items:
                 toks = it.request.step_tokens(it.start, it.count)
