@@ -395,22 +395,22 @@ __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0
   if (mode == OUT_SWIGLU) {
     // the weight rows alternate eight gate rows and eight up rows: output column 8 b + i pairs columns
     // 16 b + i and 16 b + 8 + i; COLS / 2 outputs per row, four per lane
-    constexpr int LPR = COLS / 8, RPP = 64 / LPR, PASSES = ROWS / RPP;
+    constexpr int LPR = COLS / 8, RPP = 64 / LPR, PASSES = ROWS / RPP, B = PASSES < 4 ? PASSES : 4;
     const int o = (lane % LPR) * 4, rr = lane / LPR;
     const int cg = (o / 8) * 16 + o % 8;
     bf16_t* ob = (bf16_t*)out;
     if (ncol0 + cg >= N) return;   // N is a multiple of 16: the whole group is inside or outside
 #pragma unroll
-    for (int p0 = 0; p0 < PASSES; p0 += 4) {
-      f32x4_t gt[4], up[4];
+    for (int p0 = 0; p0 < PASSES; p0 += B) {
+      f32x4_t gt[B], up[B];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < B; ++u) {
         const int row = (p0 + u) * RPP + rr;
         gt[u] = *(const f32x4_t*)(ct + row * LD + cg);
         up[u] = *(const f32x4_t*)(ct + row * LD + cg + 8);
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < B; ++u) {
         const int m = mrow0 + (p0 + u) * RPP + rr;
         u32x2_t pk;
         pk[0] = pack_bf16(silu_mul(gt[u][0], up[u][0]), silu_mul(gt[u][1], up[u][1]));
@@ -421,6 +421,7 @@ __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0
     return;
   }
   constexpr int LPR = COLS / 4, RPP = 64 / LPR, PASSES = ROWS / RPP;
+  static_assert(PASSES % 4 == 0, "the loop below takes four passes at a time");
   const int col = (lane % LPR) * 4, rr = lane / LPR;
   if (ldo % 4 == 0 && ncol0 + col + 3 < N) {
 #pragma unroll
@@ -921,48 +922,60 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
 // Here the weights are the traffic and the matrix core has little to do: a block owns 64 x 128 of the
 // result (a wave 32 x 64), three stages of (64 + 128) rows (72 KB: two blocks per CU), K split over
 // blockIdx.y until there are about two blocks for every CU.  Loads, LDS reads and MFMAs interleave as above.
+// NJ = 2 instead of 4: 64 x 64 blocks (a wave 32 x 32, 48 KB of stages), for products whose N gives too few blocks
+// of 128 columns to put one on every CU without cutting K into short pieces.
 namespace {
 
-constexpr int BM64 = 64, STAGE64 = (BM64 + BN) * ROWB, LPW64 = 6;
+constexpr int BM64 = 64;
 
+template <int NJ>
 struct Frags64 {
-  u32x4_t a[2], b[4];
+  u32x4_t a[2], b[NJ];
 };
-__device__ inline void wait_frags(Frags64& f) {
-  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3]));
+template <int NJ>
+__device__ inline void wait_frags(Frags64<NJ>& f) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.b[0]), "+v"(f.b[1]));
+  if constexpr (NJ == 4) asm volatile("" : "+v"(f.b[2]), "+v"(f.b[3]));
 }
-template <int R>
-__device__ inline void read_one(Frags64& f, unsigned aaddr, unsigned baddr) {
-  if constexpr (R < 4)
+// read R of a half step: the NJ w fragments, then the two x fragments
+template <int R, int NJ>
+__device__ inline void read_one(Frags64<NJ>& f, unsigned aaddr, unsigned baddr) {
+  if constexpr (R < NJ)
     f.b[R] = lds_read16<R * 16 * ROWB>(baddr);
   else
-    f.a[R - 4] = lds_read16<(R - 4) * 16 * ROWB>(aaddr);
+    f.a[R - NJ] = lds_read16<(R - NJ) * 16 * ROWB>(aaddr);
 }
-// load I (0..5) of this wave: 0..1 are x rows, 2..5 w rows
-template <int I>
+// load I (0..1 + NJ) of this wave: 0..1 are x rows, the others w rows
+template <int I, int NJ>
 __device__ inline void issue_one64(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
-                                   const unsigned (&voff)[LPW64], int wave) {
-  const int t = I < 2 ? wave * 2 + I : 8 + wave * 4 + (I - 2);
+                                   const unsigned (&voff)[2 + NJ], int wave) {
+  const int t = I < 2 ? wave * 2 + I : 8 + wave * NJ + (I - 2);
   const unsigned char* src = (I < 2 ? xk : wk) + voff[I];
   // (the weights are read once per step: nontemporal, aux bit 1; the few activation rows stay cached)
   __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, I < 2 ? 0 : 2);
 }
-template <bool READ, bool LOAD>
-__device__ inline void half_step64(f32x4_t (&acc)[2][4], const Frags64& cur, Frags64& nxt, unsigned aaddr, unsigned baddr,
+template <bool READ, bool LOAD, int NJ>
+__device__ inline void half_step64(f32x4_t (&acc)[2][NJ], const Frags64<NJ>& cur, Frags64<NJ>& nxt, unsigned aaddr, unsigned baddr,
                                    unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
-                                   const unsigned (&voff)[LPW64], int wave) {
+                                   const unsigned (&voff)[2 + NJ], int wave) {
 #define SB() __builtin_amdgcn_sched_barrier(0)
 #define RD(R) \
-  if (READ) read_one<R>(nxt, aaddr, baddr); \
+  if (READ) read_one<R, NJ>(nxt, aaddr, baddr); \
   SB()
 #define LD(I) \
-  if (LOAD) issue_one64<I>(buf, xk, wk, voff, wave); \
+  if (LOAD) issue_one64<I, NJ>(buf, xk, wk, voff, wave); \
   SB()
 #define M1(I, J) \
   acc[I][J] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(cur.a[I]), as_frag(cur.b[J]), acc[I][J], 0, 0, 0); \
   SB()
-  RD(0); M1(0, 0); LD(0); RD(1); M1(0, 1); LD(1); RD(2); M1(0, 2); LD(2); RD(3); M1(0, 3); LD(3);
-  RD(4); M1(1, 0); LD(4); RD(5); M1(1, 1); LD(5); M1(1, 2); M1(1, 3);
+  if constexpr (NJ == 4) {
+    RD(0); M1(0, 0); LD(0); RD(1); M1(0, 1); LD(1); RD(2); M1(0, 2); LD(2); RD(3); M1(0, 3); LD(3);
+    RD(4); M1(1, 0); LD(4); RD(5); M1(1, 1); LD(5); M1(1, 2); M1(1, 3);
+  } else {
+    static_assert(NJ == 2 || NJ == 4, "w tiles per wave");
+    RD(0); M1(0, 0); LD(0); RD(1); M1(0, 1); LD(1);
+    RD(2); M1(1, 0); LD(2); RD(3); M1(1, 1); LD(3);
+  }
 #undef RD
 #undef LD
 #undef M1
@@ -971,20 +984,22 @@ __device__ inline void half_step64(f32x4_t (&acc)[2][4], const Frags64& cur, Fra
 
 }  // namespace
 
+template <int NJ>
 __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              void* __restrict__ out, float* __restrict__ partial,
                                                              int mode, int M, int N, int K, int wt) {
-  __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE64];
+  constexpr int BNT = 32 * NJ, STAGE = (BM64 + BNT) * ROWB, LPWT = 2 + NJ;
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[NS * STAGE];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int MB = (M + BM64 - 1) / BM64;
   const int bm = blockIdx.x % MB, bn = blockIdx.x / MB;     // the row blocks of a column block run side by side
-  const int m0 = bm * BM64, n0 = bn * BN;
-  f32x4_t acc[2][4];
+  const int m0 = bm * BM64, n0 = bn * BNT;
+  f32x4_t acc[2][NJ];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NJ; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   const int kt_per = (K / BK + gridDim.y - 1) / gridDim.y;
   const int kt_first = blockIdx.y * kt_per;
   const int KT = min(K / BK, kt_first + kt_per) - kt_first;
@@ -996,16 +1011,16 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
   const unsigned off0 = c * ROWB + (((0 * 4 + g) ^ ((c >> 1) & 7)) << 4);
   const unsigned off1 = c * ROWB + (((1 * 4 + g) ^ ((c >> 1) & 7)) << 4);
-  const unsigned arow = wm * 32 * ROWB, brow = (BM64 + wn * 64) * ROWB;
-  unsigned voff[LPW64];
+  const unsigned arow = wm * 32 * ROWB, brow = (BM64 + wn * 16 * NJ) * ROWB;
+  unsigned voff[LPWT];
 #pragma unroll
-  for (int i = 0; i < LPW64; ++i) {
-    const int row = (i < 2 ? (wave * 2 + i) * 8 : (wave * 4 + i - 2) * 8) + (lane >> 3);
+  for (int i = 0; i < LPWT; ++i) {
+    const int row = (i < 2 ? (wave * 2 + i) * 8 : (wave * NJ + i - 2) * 8) + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     const int grow = i < 2 ? min(row, M - 1 - m0) : min(row, N - 1 - n0);
     voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
     if (wt && i >= 2) {   // block u of the stage's weights: row group u / 2 of the block tile, first or second 32 of k
-      const int u = wave * 4 + i - 2;
+      const int u = wave * NJ + i - 2;
       const int grp = min(u / 2, (N - n0) / 16 - 1);
       voff[i] = ((unsigned)grp * (unsigned)(K / 32) + (u & 1)) * 1024u + lane * 16;
     }
@@ -1015,68 +1030,74 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
   const unsigned char* xk = (const unsigned char*)x + ((size_t)m0 * K + (size_t)kt_first * BK) * 2;
   const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2 + (size_t)kt_first * wkstep;
   auto issue_stage64 = [&](unsigned char* buf, const unsigned char* xs, const unsigned char* ws) {
-    issue_one64<0>(buf, xs, ws, voff, wave);
-    issue_one64<1>(buf, xs, ws, voff, wave);
-    issue_one64<2>(buf, xs, ws, voff, wave);
-    issue_one64<3>(buf, xs, ws, voff, wave);
-    issue_one64<4>(buf, xs, ws, voff, wave);
-    issue_one64<5>(buf, xs, ws, voff, wave);
+    issue_one64<0, NJ>(buf, xs, ws, voff, wave);
+    issue_one64<1, NJ>(buf, xs, ws, voff, wave);
+    issue_one64<2, NJ>(buf, xs, ws, voff, wave);
+    issue_one64<3, NJ>(buf, xs, ws, voff, wave);
+    if constexpr (NJ == 4) {
+      issue_one64<4, NJ>(buf, xs, ws, voff, wave);
+      issue_one64<5, NJ>(buf, xs, ws, voff, wave);
+    }
   };
 #pragma unroll
   for (int p = 0; p < NS; ++p)
-    if (p < KT) issue_stage64(stages + p * STAGE64, xk + p * BK * 2, wk + p * wkstep);
+    if (p < KT) issue_stage64(stages + p * STAGE, xk + p * BK * 2, wk + p * wkstep);
   xk += NS * BK * 2;
   wk += NS * wkstep;
-  Frags64 fa, fb;
-  if (KT > 2) WAIT_VM(2 * LPW64); else WAIT_VM(0);
+  Frags64<NJ> fa, fb;
+  if (KT > 2) WAIT_VM(2 * LPWT); else WAIT_VM(0);
   __builtin_amdgcn_s_barrier();
-#define READ_ALL64(f, aaddr, baddr) \
-  read_one<0>(f, aaddr, baddr); read_one<1>(f, aaddr, baddr); read_one<2>(f, aaddr, baddr); \
-  read_one<3>(f, aaddr, baddr); read_one<4>(f, aaddr, baddr); read_one<5>(f, aaddr, baddr)
-  READ_ALL64(fa, lds0 + arow + off0, lds0 + brow + boff0);
-  wait_frags(fa);
+  auto read_all = [&](Frags64<NJ>& f, unsigned aaddr, unsigned baddr) {
+    read_one<0, NJ>(f, aaddr, baddr); read_one<1, NJ>(f, aaddr, baddr); read_one<2, NJ>(f, aaddr, baddr);
+    read_one<3, NJ>(f, aaddr, baddr);
+    if constexpr (NJ == 4) {
+      read_one<4, NJ>(f, aaddr, baddr); read_one<5, NJ>(f, aaddr, baddr);
+    }
+  };
+  read_all(fa, lds0 + arow + off0, lds0 + brow + boff0);
+  wait_frags<NJ>(fa);
   int st = 0, kt = 0;
   for (; kt + NS < KT; ++kt) {
     const int sn = st + 1 == NS ? 0 : st + 1;
-    const unsigned cur = lds0 + st * STAGE64, nxt = lds0 + sn * STAGE64;
-    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
-    wait_frags(fb);
-    WAIT_VM(LPW64);
+    const unsigned cur = lds0 + st * STAGE, nxt = lds0 + sn * STAGE;
+    half_step64<true, false, NJ>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags<NJ>(fb);
+    WAIT_VM(LPWT);
     __builtin_amdgcn_s_barrier();
-    half_step64<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE64, xk, wk, voff, wave);
-    wait_frags(fa);
+    half_step64<true, true, NJ>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE, xk, wk, voff, wave);
+    wait_frags<NJ>(fa);
     xk += BK * 2;
     wk += wkstep;
     st = sn;
   }
   for (; kt + 1 < KT; ++kt) {
     const int sn = st + 1 == NS ? 0 : st + 1;
-    const unsigned cur = lds0 + st * STAGE64, nxt = lds0 + sn * STAGE64;
-    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
-    wait_frags(fb);
+    const unsigned cur = lds0 + st * STAGE, nxt = lds0 + sn * STAGE;
+    half_step64<true, false, NJ>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags<NJ>(fb);
     WAIT_VM(0);
     __builtin_amdgcn_s_barrier();
-    half_step64<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
-    wait_frags(fa);
+    half_step64<true, false, NJ>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags<NJ>(fa);
     st = sn;
   }
   {
-    const unsigned cur = lds0 + st * STAGE64;
-    half_step64<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
-    wait_frags(fb);
-    half_step64<false, false>(acc, fb, fa, 0, 0, nullptr, nullptr, nullptr, voff, wave);
+    const unsigned cur = lds0 + st * STAGE;
+    half_step64<true, false, NJ>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags<NJ>(fb);
+    half_step64<false, false, NJ>(acc, fb, fa, 0, 0, nullptr, nullptr, nullptr, voff, wave);
   }
-  // the result leaves through LDS, as above: 32 x 64 per wave
+  // the result leaves through LDS, as above: 32 x 16 NJ per wave
   __syncthreads();
   float* ct = (float*)stages + wave * (32 * CLD);
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  emit_tile<32, 64, CLD>(ct, lane, m0 + wm * 32, n0 + wn * 64, out, mode, M, N, mode == OUT_SWIGLU ? N / 2 : N);
+  emit_tile<32, 16 * NJ, CLD>(ct, lane, m0 + wm * 32, n0 + wn * 16 * NJ, out, mode, M, N, mode == OUT_SWIGLU ? N / 2 : N);
 }
 
 // Defined in gemm_mfma.hip.
@@ -1175,6 +1196,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   return 0;
 }
 
+int g_pipe64_narrow = 0;   // tuning: 1 = blocks of 64 columns always, 2 = never
 // The 64-row pipeline (17..128 rows).  `defer`: when K is split, leave the partial sums in `scratch` for the
 // caller's next kernel and report their number through *splits_out.
 int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
@@ -1183,23 +1205,44 @@ int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, i
   if (w_tiled && N % 16 != 0) return -1;
   if ((size_t)(BM64 - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;
   if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
-  const int MB = (M + BM64 - 1) / BM64, NB = (N + BN - 1) / BN;
-  const long tiles = (long)MB * NB;
-  if (tiles > 0x7fffffffL) return -1;
+  const int MB = (M + BM64 - 1) / BM64;
+  const int KT = K / BK;
   // a block for every CU, at least sixteen tiles of K each (measured at 24, 64 and 128 rows of the 8B
   // shapes: more splits than that cost more in partial sums than they gain)
-  int splits = 1;
-  const int KT = K / BK;
-  if (scratch != nullptr) {
-    splits = tune_splits > 0 ? tune_splits : (int)(256 / tiles);
-    splits = std::max(1, std::min(splits, std::min(16, KT / 16)));
-    while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
-    const int per = (KT + splits - 1) / splits;
-    splits = (KT + per - 1) / per;
+  auto plan = [&](int bn, long& tiles) {
+    tiles = (long)MB * ((N + bn - 1) / bn);
+    int splits = 1;
+    if (scratch != nullptr) {
+      splits = tune_splits > 0 ? tune_splits : (int)(256 / std::max(1L, tiles));
+      splits = std::max(1, std::min(splits, std::min(16, KT / 16)));
+      while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
+      const int per = (KT + splits - 1) / splits;
+      splits = (KT + per - 1) / per;
+    }
+    return splits;
+  };
+  long tiles = 0, tiles_narrow = 0;
+  int splits = plan(BN, tiles);
+  const int splits_narrow = plan(64, tiles_narrow);
+  if (tiles > 0x7fffffffL || tiles_narrow > 0x7fffffffL) return -1;
+  // blocks of 64 columns where those of 128 leave a fifth of the CUs or more without one, or where they give
+  // every CU a block without any split of K (measured at 64 rows: 4096 x 4096 15.7 -> 15.0 us with the kernel
+  // that adds the partial sums, 5120 x 3072 11.0 -> 9.1, 3072 x 3072 14.1 -> 12.3, 16384 x 3072 gated 25.1 -> 21.1;
+  // 6144 x 4096, which has 192 blocks of 128 columns, 12.4 -> 14.9: left as it is)
+  const bool narrow = g_pipe64_narrow == 1 ||
+                      (g_pipe64_narrow == 0 && tiles_narrow * splits_narrow >= tiles * splits &&
+                       ((tiles * splits < 192 && tiles_narrow * splits_narrow > tiles * splits) || (splits > 1 && splits_narrow == 1)));
+  if (narrow) {
+    tiles = tiles_narrow;
+    splits = splits_narrow;
   }
   const bool leave = defer && splits > 1 && splits_out != nullptr && mode != OUT_SWIGLU;
-  hipLaunchKernelGGL(gemm_pipe64_kernel, dim3((unsigned)tiles, splits), dim3(256), 0, s, x, w, out,
-                     splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled);
+  if (narrow)
+    hipLaunchKernelGGL(gemm_pipe64_kernel<2>, dim3((unsigned)tiles, splits), dim3(256), 0, s, x, w, out,
+                       splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled);
+  else
+    hipLaunchKernelGGL(gemm_pipe64_kernel<4>, dim3((unsigned)tiles, splits), dim3(256), 0, s, x, w, out,
+                       splits > 1 ? scratch : nullptr, mode, M, N, K, w_tiled);
   if (leave) {
     *splits_out = splits;
   } else if (splits > 1) {

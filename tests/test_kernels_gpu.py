@@ -418,6 +418,51 @@ def test_tiled_weights_give_the_same_bits(m, n, k):
         assert torch.equal(ops.linear(kb, t, torch.float32), ops.linear(kb, w, torch.float32))
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 48, 64), (33, 1008, 320), (64, 3072, 3072), (100, 16400, 128), (128, 528, 2048), (60, 4096, 4096)])
+def test_linear_mid_rows_both_block_widths(m, n, k):
+    """The pipelined product for 17..128 rows with blocks of 128 and of 64 columns, each forced: every output mode
+    against float64 (columns that fill no whole block, K split over blocks or not), the partial sums left to the
+    next kernel, tiled weights; and the two widths give the same bits (each element's sum runs over K in the
+    same order)."""
+    ops = _ops()
+    lib = ops.library()
+    g = torch.Generator().manual_seed(14)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    ref = x.double() @ w.double().T
+    res = torch.randn(m, n, generator=g)
+    nw = (1 + 0.3 * torch.randn(n, generator=g)).float()
+    xd, wd = x.to(DEV), w.to(DEV)
+    gate_up = ref.view(m, n // 16, 2, 8)
+    gated = (torch.nn.functional.silu(gate_up[:, :, 0]) * gate_up[:, :, 1]).reshape(m, n // 2)
+    got = {}
+    for width in (2, 1):        # 128 columns, 64 columns
+        lib.tp_linear_tune_narrow(width)
+        try:
+            outs = []
+            for wv in (wd, ops.tile_weight(wd)):
+                outs.append(ops.linear(xd, wv, torch.float32))
+                _close(outs[-1], ref, 2e-5, f"f32 out, width code {width}")
+                outs.append(ops.linear(xd, wv, torch.bfloat16))
+                _close(outs[-1], ref, 1e-2, f"bf16 out, width code {width}")
+                outs.append(ops.linear(xd, wv, torch.float32, residual=res.clone().to(DEV)))
+                _close(outs[-1], ref + res.double(), 2e-5, f"residual, width code {width}")
+                outs.append(ops.linear_swiglu(xd, wv))
+                _close(outs[-1], gated, 1e-2, f"gated, width code {width}")
+                h = res.clone().to(DEV)
+                handed = ops.linear(xd, wv, torch.float32, residual=h, next_norm=(nw.to(DEV), 1e-5))
+                _close(h, ref + res.double(), 2e-5, f"residual with the next norm, width code {width}")
+                outs.append(h)
+                p = ops.linear(xd, wv, torch.float32, partial_ok=True)
+                p = p.data.sum(0)[:m] if isinstance(p, ops.Partials) else p
+                _close(p, ref, 2e-5, f"partial sums, width code {width}")
+            got[width] = outs
+        finally:
+            lib.tp_linear_tune_narrow(0)
+    for a, b in zip(got[1], got[2]):
+        assert torch.equal(a, b), "blocks of 64 and of 128 columns give the same bits"
+
+
 @pytest.mark.parametrize("m,n,k", [(300, 512, 128), (1000, 816, 192), (257, 256, 64), (2048, 8448, 128), (2100, 6144, 128),
                                    (600, 1152, 320)])
 def test_linear_big_tiles(m, n, k):
