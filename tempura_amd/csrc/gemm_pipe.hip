@@ -292,9 +292,12 @@ __device__ inline void rope_fetch(RopeFetch<ROWS, COLS>& f, int lane, int mrow0,
         int sl[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) sl[i] = rp.slots[m0 + i];
-        bool run = (sl[0] & 7) == 0;
+        // a run: every place follows the one before, or begins a group of eight where that one ended a group
+        // (eight tokens in a row of one request, whose next page may lie anywhere); from a multiple of eight it is
+        // one piece of the value cache, otherwise the ends of two
+        bool run = true;
 #pragma unroll
-        for (int i = 1; i < 8; ++i) run = run && sl[i] == sl[0] + i;
+        for (int i = 1; i < 8; ++i) run = run && (sl[i] == sl[i - 1] + 1 || ((sl[i] & 7) == 0 && (sl[i - 1] & 7) == 7));
         if (run) s0 = sl[0];
       }
     }
@@ -365,7 +368,7 @@ __device__ inline void emit_tile_rope(const float* ct, int lane, int mrow0, int 
     float y[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) y[i] = ct[(rg * 8 + i) * LD + colv];
-    if (s0 >= 0) {
+    if (s0 >= 0 && (s0 & 7) == 0) {
       const size_t page = (size_t)(s0 / rp.page_size), off = (size_t)(s0 % rp.page_size);
       u32x4_t pk;
       pk[0] = pack_bf16(y[0], y[1]);
@@ -373,6 +376,17 @@ __device__ inline void emit_tile_rope(const float* ct, int lane, int mrow0, int 
       pk[2] = pack_bf16(y[4], y[5]);
       pk[3] = pack_bf16(y[6], y[7]);
       *(u32x4_t*)(rp.v_cache + ((page * rp.n_kv + kh) * rp.head_dim + d0 + colv) * rp.page_size + off) = pk;
+    } else if (s0 >= 0) {
+      // a run that starts inside a group of eight places: the end of that group, then the start of the group that
+      // holds the next token (two addresses worked out instead of eight)
+      const int n0 = 8 - (s0 & 7);
+      const int s1 = rp.slots[m0 + n0];
+      const size_t page0 = (size_t)(s0 / rp.page_size), off0 = (size_t)(s0 % rp.page_size);
+      const size_t page1 = (size_t)(s1 / rp.page_size), off1 = (size_t)(s1 % rp.page_size);
+      bf16_t* p0 = rp.v_cache + ((page0 * rp.n_kv + kh) * rp.head_dim + d0 + colv) * rp.page_size + off0;
+      bf16_t* p1 = rp.v_cache + ((page1 * rp.n_kv + kh) * rp.head_dim + d0 + colv) * rp.page_size + off1 - n0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) (i < n0 ? p0 : p1)[i] = float_to_bf16(y[i]);
     } else {
       for (int i = 0; i < 8 && m0 + i < M; ++i) {
         const int sl = rp.slots[m0 + i];
