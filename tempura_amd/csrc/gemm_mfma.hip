@@ -675,6 +675,10 @@ extern "C" void tp_linear_tune_tile(int order) {
   g_tune_order = order >= 5 ? 0 : order;
 }
 
+extern int g_pipe_mid;
+// the pipelined product's 128 x 128 blocks: 0 chosen by shape, 1 for every product of more than 128 rows, 2 never
+extern "C" void tp_linear_tune_mid_tile(int v) { g_pipe_mid = v; }
+
 extern int g_pipe64_narrow;
 // the 64-row pipeline's blocks: 0 chosen by shape, 1 always 64 columns wide, 2 always 128
 extern "C" void tp_linear_tune_narrow(int v) { g_pipe64_narrow = v; }

@@ -490,9 +490,29 @@ __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0
 
 }  // namespace
 
+// Which tile a block takes.  Blocks go to the 8 XCDs in turn and each XCD has an L2 of its own: XCD c takes the
+// column blocks c, c + 8, ... (at most Q of them) and all MB row blocks, as a list without gaps (a block that
+// finds no tile and leaves at once still held up the ones behind it: a product with a fifth of such blocks
+// took twice its time).  The list walks groups of pq column blocks; inside a group, strips of pm row blocks;
+// inside a strip, row blocks fastest: the 32 blocks that an XCD runs at a time share pm row blocks of x and
+// about 32 / pm column blocks of w.  False for the few blocks past an XCD's last column block.
+__device__ inline bool tile_of_block(unsigned block, int MB, int NB, int pm, int& bm, int& bn) {
+  const int c = block % 8, j = block / 8;
+  const int pq = max(1, 32 / pm), Q = (NB + 7) / 8;
+  const int group = MB * pq;
+  const int k = j / group, rem = j - k * group;
+  const int wk = min(pq, Q - k * pq);
+  const int strip = pm * wk;
+  const int sidx = rem / strip, r = rem - sidx * strip;
+  const int hs = min(pm, MB - sidx * pm);
+  bm = sidx * pm + r % hs;
+  bn = c + 8 * (k * pq + r / hs);
+  return bn < NB;
+}
+
 // ldo: row stride of `out` in elements (N, or N / 2 for the gated mode, when the launch covers all columns;
 // a launch may cover a range of columns with `w` and `out` pointing at its first).
-// pm: row blocks of a patch (a power of two up to 8); a patch holds 32 blocks.  blockIdx.y splits K:
+// pm: row blocks of a strip (see tile_of_block).  blockIdx.y splits K:
 // with more than one split every block writes its float32 partial tile to `partial` [split, M, N]
 // and a second kernel adds the splits in ascending order and applies the epilogue.
 __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
@@ -503,16 +523,8 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(const bf16_t* __restrict
   const int wm = wave >> 1, wn = wave & 1;
   int bm, bn;
   {
-    // XCD c takes the column blocks c, c + 8, ...; its blocks j = 0, 1, ... walk patches of pm row
-    // blocks x (32 / pm) of its column blocks, row blocks fastest
     const int MB = (M + BM - 1) / BM, NB = (N + BN - 1) / BN;
-    const int pq = 32 / pm;
-    const int MS = (MB + pm - 1) / pm;
-    const int c = blockIdx.x % 8, j = blockIdx.x / 8;
-    const int t = j / 32, r = j % 32;
-    bm = (t % MS) * pm + r % pm;
-    bn = c + 8 * ((t / MS) * pq + r / pm);
-    if (bm >= MB || bn >= NB) return;
+    if (!tile_of_block(blockIdx.x, MB, NB, pm, bm, bn)) return;
   }
   const int m0 = bm * BM, n0 = bn * BN;
   f32x4_t acc[8][4];
@@ -771,13 +783,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
   int bm, bn;
   {
     const int MB = (M + BM - 1) / BM, NB = N / BNT;
-    const int pq = 32 / pm;
-    const int MS = (MB + pm - 1) / pm;
-    const int c = blockIdx.x % 8, j = blockIdx.x / 8;
-    const int t = j / 32, r = j % 32;
-    bm = (t % MS) * pm + r % pm;
-    bn = c + 8 * ((t / MS) * pq + r / pm);
-    if (bm >= MB || bn >= NB) return;
+    if (!tile_of_block(blockIdx.x, MB, NB, pm, bm, bn)) return;
   }
   const int m0 = bm * BM, n0 = bn * BNT;
   f32x4_t acc[8][NJ];
@@ -1114,9 +1120,249 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe64_kernel(const bf16_t* __res
   emit_tile<32, 16 * NJ, CLD>(ct, lane, m0 + wm * 32, n0 + wn * 16 * NJ, out, mode, M, N, mode == OUT_SWIGLU ? N / 2 : N);
 }
 
+// ---- the same pipeline on 128 x 128 blocks ------------------------------------------------------------
+// For steps of a few hundred rows (a prompt portion of 512) times a narrow weight: 256 x 128 blocks then make
+// fewer than 128 tiles, K has to be split over blocks, and a kernel has to add the partial sums.  Here a block
+// owns 128 x 128 (a wave 64 x 64: sixteen MFMAs per eight fragment reads), three stages of (128 + 128) rows
+// (96 KB).  The row blocks of a column block run side by side (they share its weights in L2); K is split only when
+// even these tiles are too few.  Epilogues as above, the rotating one included (a wave's 64 columns lie in one head).
+namespace {
+
+constexpr int BM128 = 128, BN128 = 128, STAGE128 = (BM128 + BN128) * ROWB, LPW128 = 8;
+// five stages of 32 KB: a step of 128 x 128 x 64 is short (512 cycles of MFMA a wave), and a load has to be four
+// steps ahead to have arrived from L2 when its turn comes
+constexpr int NS128 = 5;
+
+struct Frags128 {
+  u32x4_t a[4], b[4];
+};
+__device__ inline void wait_frags128(Frags128& f) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3]));
+}
+// read R (0..7) of a half step: the four w fragments, then the four x fragments
+template <int R>
+__device__ inline void read_one128(Frags128& f, unsigned aaddr, unsigned baddr) {
+  if constexpr (R < 4)
+    f.b[R] = lds_read16<R * 16 * ROWB>(baddr);
+  else
+    f.a[R - 4] = lds_read16<(R - 4) * 16 * ROWB>(aaddr);
+}
+// load I (0..7) of this wave: 0..3 are x rows, 4..7 w rows; one load covers 8 rows
+template <int I>
+__device__ inline void issue_one128(unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                    const unsigned (&voff)[LPW128], int wave) {
+  const int t = I < 4 ? wave * 4 + I : 16 + wave * 4 + (I - 4);
+  const unsigned char* src = (I < 4 ? xk : wk) + voff[I];
+  __builtin_amdgcn_global_load_lds(GPTR(src), LPTR(buf + t * 1024), 16, 0, 0);
+}
+template <bool READ, bool LOAD>
+__device__ inline void half_step128(f32x4_t (&acc)[4][4], const Frags128& cur, Frags128& nxt, unsigned aaddr, unsigned baddr,
+                                    unsigned char* buf, const unsigned char* xk, const unsigned char* wk,
+                                    const unsigned (&voff)[LPW128], int wave) {
+#define SB() __builtin_amdgcn_sched_barrier(0)
+#define RD(R) \
+  if (READ) read_one128<R>(nxt, aaddr, baddr); \
+  SB()
+#define LD(I) \
+  if (LOAD) issue_one128<I>(buf, xk, wk, voff, wave); \
+  SB()
+// (assembly with the accumulator as an AGPR operand that is read and written in place: left to the compiler,
+// the sixteen accumulators were moved between register files around every MFMA)
+#define M1(I, J) \
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[I][J]) : "v"(cur.a[I]), "v"(cur.b[J])); \
+  SB()
+  RD(0); M1(0, 0); LD(0); RD(1); M1(0, 1); LD(1); RD(2); M1(0, 2); LD(2); RD(3); M1(0, 3); LD(3);
+  RD(4); M1(1, 0); LD(4); RD(5); M1(1, 1); LD(5); RD(6); M1(1, 2); LD(6); RD(7); M1(1, 3); LD(7);
+  M1(2, 0); M1(2, 1); M1(2, 2); M1(2, 3); M1(3, 0); M1(3, 1); M1(3, 2); M1(3, 3);
+#undef RD
+#undef LD
+#undef M1
+#undef SB
+}
+
+}  // namespace
+
+__global__ __launch_bounds__(256) void gemm_pipe128_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                           void* __restrict__ out, float* __restrict__ partial, int mode,
+                                                           int M, int N, int K, int ldo, RopeOut rp, int wt, int splits) {
+  __shared__ __attribute__((aligned(1024))) unsigned char stages[NS128 * STAGE128];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  // Blocks go to the 8 XCDs in turn, and each XCD has an L2 of its own: XCD j takes the j-th eighth of the list
+  // of (part of K, column block, row block), row blocks fastest, so that what it holds at a time is a few column
+  // blocks of the weights and the rows of x over one part of K, and the weights cross the fabric once.
+  const int MB = (M + BM128 - 1) / BM128;
+  const int tiles = MB * ((N + BN128 - 1) / BN128);
+  const int total = tiles * splits;
+  const int per_xcd = (total + 7) / 8;
+  const int item = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= per_xcd || item >= total) return;
+  const int split = item / tiles, tile = item - split * tiles;
+  const int bm = tile % MB, bn = tile / MB;
+  const int m0 = bm * BM128, n0 = bn * BN128;
+  f32x4_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const int kt_per = (K / BK + splits - 1) / splits;
+  const int kt_first = split * kt_per;
+  const int KT = min(K / BK, kt_first + kt_per) - kt_first;
+  if (partial != nullptr) {   // K is split: float32 partial sums, added by a kernel of their own
+    mode = OUT_F32;
+    out = partial + (size_t)split * M * N;
+    ldo = N;
+  }
+  const int g = lane >> 4, c = lane & 15;
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)&stages[0];
+  const unsigned off0 = c * ROWB + (((0 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned off1 = c * ROWB + (((1 * 4 + g) ^ ((c >> 1) & 7)) << 4);
+  const unsigned arow = wm * 64 * ROWB, brow = (BM128 + wn * 64) * ROWB;
+  unsigned voff[LPW128];
+#pragma unroll
+  for (int i = 0; i < LPW128; ++i) {
+    const int row = (wave * 4 + (i & 3)) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    const int grow = i < 4 ? min(row, M - 1 - m0) : min(row, N - 1 - n0);
+    voff[i] = (unsigned)grow * (unsigned)K * 2u + chunk * 16;
+    if (wt && i >= 4) {   // block u of the stage's weights: row group u / 2 of the block tile, first or second 32 of k
+      const int u = wave * 4 + (i - 4);
+      const int grp = min(u / 2, (N - n0) / 16 - 1);
+      voff[i] = ((unsigned)grp * (unsigned)(K / 32) + (u & 1)) * 1024u + lane * 16;
+    }
+  }
+  const int wkstep = wt ? 2048 : BK * 2;
+  const unsigned boff0 = wt ? lane * 16 : off0, boff1 = wt ? 1024 + lane * 16 : off1;
+  const unsigned char* xk = (const unsigned char*)x + ((size_t)m0 * K + (size_t)kt_first * BK) * 2;
+  const unsigned char* wk = (const unsigned char*)w + (size_t)n0 * K * 2 + (size_t)kt_first * wkstep;
+  auto issue_stage = [&](unsigned char* buf, const unsigned char* xs, const unsigned char* ws) {
+    issue_one128<0>(buf, xs, ws, voff, wave); issue_one128<1>(buf, xs, ws, voff, wave);
+    issue_one128<2>(buf, xs, ws, voff, wave); issue_one128<3>(buf, xs, ws, voff, wave);
+    issue_one128<4>(buf, xs, ws, voff, wave); issue_one128<5>(buf, xs, ws, voff, wave);
+    issue_one128<6>(buf, xs, ws, voff, wave); issue_one128<7>(buf, xs, ws, voff, wave);
+  };
+#pragma unroll
+  for (int p = 0; p < NS128; ++p)
+    if (p < KT) issue_stage(stages + p * STAGE128, xk + p * BK * 2, wk + p * wkstep);
+  xk += NS128 * BK * 2;
+  wk += NS128 * wkstep;
+  Frags128 fa, fb;
+  if (KT >= NS128) WAIT_VM((NS128 - 1) * LPW128); else WAIT_VM(0);
+  __builtin_amdgcn_s_barrier();
+  auto read_all = [&](Frags128& f, unsigned aaddr, unsigned baddr) {
+    read_one128<0>(f, aaddr, baddr); read_one128<1>(f, aaddr, baddr); read_one128<2>(f, aaddr, baddr);
+    read_one128<3>(f, aaddr, baddr); read_one128<4>(f, aaddr, baddr); read_one128<5>(f, aaddr, baddr);
+    read_one128<6>(f, aaddr, baddr); read_one128<7>(f, aaddr, baddr);
+  };
+  read_all(fa, lds0 + arow + off0, lds0 + brow + boff0);
+  wait_frags128(fa);
+  int st = 0, kt = 0;
+  for (; kt + NS128 < KT; ++kt) {
+    const int sn = st + 1 == NS128 ? 0 : st + 1;
+    const unsigned cur = lds0 + st * STAGE128, nxt = lds0 + sn * STAGE128;
+    half_step128<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags128(fb);
+    WAIT_VM((NS128 - 2) * LPW128);
+    __builtin_amdgcn_s_barrier();
+    half_step128<true, true>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, stages + st * STAGE128, xk, wk, voff, wave);
+    wait_frags128(fa);
+    xk += BK * 2;
+    wk += wkstep;
+    st = sn;
+  }
+  for (; kt + 1 < KT; ++kt) {   // nothing left to load
+    const int sn = st + 1 == NS128 ? 0 : st + 1;
+    const unsigned cur = lds0 + st * STAGE128, nxt = lds0 + sn * STAGE128;
+    half_step128<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags128(fb);
+    WAIT_VM(0);
+    __builtin_amdgcn_s_barrier();
+    half_step128<true, false>(acc, fb, fa, nxt + arow + off0, nxt + brow + boff0, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags128(fa);
+    st = sn;
+  }
+  {
+    const unsigned cur = lds0 + st * STAGE128;
+    half_step128<true, false>(acc, fa, fb, cur + arow + off1, cur + brow + boff1, nullptr, nullptr, nullptr, voff, wave);
+    wait_frags128(fb);
+    half_step128<false, false>(acc, fb, fa, 0, 0, nullptr, nullptr, nullptr, voff, wave);
+  }
+  // The MFMAs are assembly, so the compiler does not know that their results take time: wait out the last ones,
+  // tied to their accumulators, and pass every other accumulator through an ordered statement after the wait.
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15"
+               : "+a"(acc[3][0]), "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3])
+               :
+               : "memory");
+#pragma unroll
+  for (int i = 0; i < 3; ++i) asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]));
+  // the result leaves through LDS: 64 x 64 per wave
+  __syncthreads();
+  float* ct = (float*)stages + wave * (64 * CLD);
+  const int mw = m0 + wm * 64, nw = n0 + wn * 64;
+  RopeFetch<64, 64> fetched;
+  if (mode == OUT_ROPE) rope_fetch(fetched, lane, mw, nw, rp, M);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ct[(i * 16 + g * 4 + r) * CLD + j * 16 + c] = acc[i][j][r];
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  if (mode == OUT_ROPE)
+    emit_tile_rope<64, 64, CLD>(ct, lane, mw, nw, rp, M, fetched);
+  else
+    emit_tile<64, 64, CLD>(ct, lane, mw, nw, out, mode, M, N, ldo);
+}
+
 // Defined in gemm_mfma.hip.
 __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ out, int mode,
                                           int splits, int M, int N);
+
+int g_pipe_mid = 0;   // tuning: 1 = 128 x 128 blocks for every product of more than 128 rows, 2 = never
+
+// Into how many parts the 128 x 128 blocks cut K: whole parts of at least sixteen steps, no more blocks than CUs.
+static int splits128(int M, int N, int K, bool can_split, size_t scratch_floats) {
+  const long tiles = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
+  const int KT = K / BK;
+  int splits = 1;
+  if (can_split) {   // (the rotating epilogue takes whole sums)
+    splits = std::max(1, std::min((int)(256 / tiles), std::min(16, KT / 16)));
+    while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
+    const int per = (KT + splits - 1) / splits;
+    splits = (KT + per - 1) / per;
+  }
+  return splits;
+}
+
+// What a product costs in microseconds, roughly, as `blocks` blocks that take `steps` steps of K each at
+// `step_us` a step, one block on a CU at a time, and a kernel that adds the parts if K is split.  Measured:
+// 0.44 us a step for a block of 128 x 128, 0.71 us for one of 256 x 128; the parts are written and read
+// again at about 3 TB/s.
+static double pipe_cost(long blocks, int steps, double step_us, int splits, int M, int N) {
+  const double rounds = (double)((blocks + 255) / 256);
+  return rounds * steps * step_us + (splits > 1 ? 3.0 + (splits + 2.0) * M * N * 4.0 / 3e6 : 0.0);
+}
+// The 128 x 128 blocks.  Returns 0 when launched.
+static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K,
+                             float* scratch, size_t scratch_floats, const RopeOut* rope, hipStream_t s) {
+  const int MB = (M + BM128 - 1) / BM128, NB = (N + BN128 - 1) / BN128;
+  const long tiles = (long)MB * NB;
+  const int splits = splits128(M, N, K, scratch != nullptr && rope == nullptr, scratch_floats);
+  RopeOut rp = {};
+  if (rope != nullptr) rp = *rope;
+  const int ldo = mode == OUT_SWIGLU ? N / 2 : N;
+  const long per_xcd = (tiles * splits + 7) / 8;
+  if (8 * per_xcd > 0x7fffffffL) return -1;
+  hipLaunchKernelGGL(gemm_pipe128_kernel, dim3((unsigned)(8 * per_xcd)), dim3(256), 0, s, x, w, out,
+                     splits > 1 ? scratch : nullptr, mode, M, N, K, ldo, rp, w_tiled, splits);
+  if (splits > 1) {
+    const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
+                       splits, M, N);
+  }
+  return 0;
+}
 
 // Returns 0 when launched, -1 when the sizes are not this kernel's.  `scratch` (optional) is room for
 // float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
@@ -1129,10 +1375,30 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   if ((size_t)(BM - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;  // a lane's source offset is 32 bits
   if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
   const int MB = (M + BM - 1) / BM, NB = (N + BN - 1) / BN;
-  const int pm = MB >= 5 ? 8 : (MB >= 3 ? 4 : MB);
-  const int pq = 32 / pm;
-  const long Q = (NB + 7) / 8, MS = (MB + pm - 1) / pm, QS = (Q + pq - 1) / pq;
-  const long blocks = 8 * QS * MS * 32;
+  // Steps of a few hundred rows, with at most one round of 256 x 128 blocks: blocks of 128 x 128 where they
+  // are cheaper (more of them, so more CUs at work and K in fewer parts).
+  bool mid = g_pipe_mid == 1;
+  if (g_pipe_mid == 0 && M > 128 && (long)MB * NB <= 256) {
+    const int KT = K / BK;
+    const bool can_split = scratch != nullptr && rope == nullptr;
+    const long tiles = (long)MB * NB, tiles128 = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
+    int s256 = 1;
+    if (scratch != nullptr) {   // (as below)
+      s256 = tune_splits > 0 ? tune_splits : (tiles >= 128 ? 1 : (int)((256 + tiles - 1) / tiles));
+      s256 = std::max(1, std::min(s256, std::min(16, KT / 16)));
+      while (s256 > 1 && (size_t)s256 * M * N > scratch_floats) --s256;
+    }
+    const int s128 = splits128(M, N, K, can_split, scratch_floats);
+    mid = pipe_cost(tiles128 * s128, (KT + s128 - 1) / s128, 0.44, s128, M, N) <
+          pipe_cost(tiles * s256, (KT + s256 - 1) / s256, 0.71, s256, M, N);
+  }
+  if (mid) return tp_linear_pipe128(x, w, w_tiled, out, mode, M, N, K, scratch, scratch_floats, rope, s);
+  // (see tile_of_block) strips of at most eight row blocks, all about as tall; a launch of nb column blocks has
+  // 8 x MB x ceil(nb / 8) blocks
+  const int strips = (MB + 7) / 8;
+  const int pm = (MB + strips - 1) / strips;
+  auto blocks_for = [&](long nb) { return 8L * MB * ((nb + 7) / 8); };
+  const long blocks = blocks_for(NB);
   if (blocks > 0x7fffffffL) return -1;
   // splits: enough blocks for the 256 CUs, at least sixteen tiles of K each (measured: more splits than
   // that cost more in partial sums than they gain)
@@ -1173,8 +1439,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     if (N % 192 == 0 && mode != OUT_SWIGLU && g_pipe_big != 4) {
       const long t192 = (long)MB * (N / 192);
       if (1.35 * (double)((t192 + 255) / 256) < best - 1e-9 || g_pipe_big == 3) {
-        const long Q3 = (N / 192 + 7) / 8, QS3 = (Q3 + pq - 1) / pq;
-        const long blocks3 = 8 * QS3 * MS * 32;
+        const long blocks3 = blocks_for(N / 192);
         hipLaunchKernelGGL(gemm_pipe_big_kernel<6>, dim3((unsigned)blocks3), dim3(256), 0, s, x, w, out, mode, M, N, K, pm, ldo,
                            rp, w_tiled);
         return 0;
@@ -1182,8 +1447,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     }
   }
   if (nb_big > 0) {
-    const long Q2 = (nb_big + 7) / 8, QS2 = (Q2 + pq - 1) / pq;
-    const long blocks2 = 8 * QS2 * MS * 32;
+    const long blocks2 = blocks_for(nb_big);
     hipLaunchKernelGGL(gemm_pipe_big_kernel<8>, dim3((unsigned)blocks2), dim3(256), 0, s, x, w, out, mode, M, nb_big * BNB, K,
                        pm, ldo, rp, w_tiled);
     const int n_done = nb_big * BNB;
@@ -1191,8 +1455,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     // the rest of the columns
     const int N2 = N - n_done;
     const int NBr = (N2 + BN - 1) / BN;
-    const long Qr = (NBr + 7) / 8, QSr = (Qr + pq - 1) / pq;
-    const long blocksr = 8 * QSr * MS * 32;
+    const long blocksr = blocks_for(NBr);
     const size_t esz = mode == OUT_BF16 || mode == OUT_SWIGLU ? 2 : 4;
     void* out2 = out == nullptr ? nullptr : (char*)out + (size_t)(mode == OUT_SWIGLU ? n_done / 2 : n_done) * esz;
     rp.col0 = n_done;

@@ -14,7 +14,7 @@ from tempura_amd.csrc import build
 
 # kernels that must not spill, by a piece of their (mangled) name
 NO_SCRATCH = {
-    "gemm_pipe.hip": ["gemm_pipe_kernel", "gemm_pipe_big_kernel", "gemm_pipe64_kernel"],
+    "gemm_pipe.hip": ["gemm_pipe_kernel", "gemm_pipe_big_kernel", "gemm_pipe64_kernel", "gemm_pipe128_kernel"],
     "gemm_mfma.hip": ["gemm_skinny_mfma_kernel", "gemm_skinny_lds_kernel"],
     "attention_mfma.hip": ["attn_prefill_lds_kernel", "attn_decode_kernel"],
 }

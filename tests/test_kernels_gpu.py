@@ -113,7 +113,8 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
 @pytest.mark.parametrize("m,heads,kv,d,rot,k,page", [(1, 4, 2, 64, 64, 256, 16), (8, 32, 8, 128, 128, 4096, 16),
                                                     (16, 3, 1, 48, 32, 96, 8), (5, 6, 3, 16, 16, 2048, 32),
                                                     (2100, 32, 8, 128, 128, 128, 16), (3000, 24, 8, 128, 64, 192, 8),
-                                                    (4300, 4, 2, 128, 128, 64, 16), (2900, 10, 1, 128, 128, 320, 16)])
+                                                    (4300, 4, 2, 128, 128, 64, 16), (2900, 10, 1, 128, 128, 320, 16),
+                                                    (520, 32, 8, 128, 128, 256, 16)])
 def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
     """The projection of a few rows that rotates and stores its rows in its epilogue gives the bits of the
     plain product followed by the rotation and cache-write kernel; and both agree with float64."""
@@ -154,6 +155,15 @@ def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
         q4 = ops.linear_rope_kv(xd, ops.tile_weight(wd), pd, sd, invd, rot, 1.0, heads, kv, d, k4, v4,
                                 ops.rope_table(pd, invd, rot, 1.0) if m > 16 else None)
         assert torch.equal(q4, q1) and torch.equal(k4, k1) and torch.equal(v4, v1)
+    if m > 128:                        # blocks of 128 x 128 (steps of a few hundred rows): the same bits
+        ops.library().tp_linear_tune_mid_tile(1)
+        try:
+            for wv in (wd, ops.tile_weight(wd)):
+                k6, v6 = kc.to(DEV), vc.to(DEV)
+                q6 = ops.linear_rope_kv(xd, wv, pd, sd, invd, rot, 1.0, heads, kv, d, k6, v6, ops.rope_table(pd, invd, rot, 1.0))
+                assert torch.equal(q6, q1) and torch.equal(k6, k1) and torch.equal(v6, v1)
+        finally:
+            ops.library().tp_linear_tune_mid_tile(0)
     if m > 16 and n % 192 == 0:       # tiles of 256 x 192, whose columns span two heads: the same bits
         ops.library().tp_linear_tune_tile(7)
         try:
@@ -461,6 +471,44 @@ def test_linear_mid_rows_both_block_widths(m, n, k):
             lib.tp_linear_tune_narrow(0)
     for a, b in zip(got[1], got[2]):
         assert torch.equal(a, b), "blocks of 64 and of 128 columns give the same bits"
+
+
+@pytest.mark.parametrize("m,n,k", [(129, 128, 64), (300, 528, 128), (512, 3072, 3072), (700, 1040, 448), (1000, 816, 192),
+                                   (260, 4096, 4096)])
+def test_linear_blocks_of_128(m, n, k):
+    """The pipelined product on 128 x 128 blocks (what steps of a few hundred rows take when 256 x 128 blocks would
+    be too few), forced: every output mode against float64, rows and columns that fill no whole block, K split
+    over blocks or not, tiled weights; the bits of the 256 x 128 blocks wherever neither splits K."""
+    ops = _ops()
+    lib = ops.library()
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = torch.randn(n, k, generator=g).to(torch.bfloat16)
+    ref = x.double() @ w.double().T
+    res = torch.randn(m, n, generator=g)
+    xd, wd = x.to(DEV), w.to(DEV)
+    gate_up = ref.view(m, n // 16, 2, 8)
+    gated = (torch.nn.functional.silu(gate_up[:, :, 0]) * gate_up[:, :, 1]).reshape(m, n // 2)
+    got = {}
+    for code in (1, 2):          # 128 x 128 always, never
+        lib.tp_linear_tune_mid_tile(code)
+        try:
+            outs = []
+            for wv in (wd, ops.tile_weight(wd)):
+                outs.append(ops.linear(xd, wv, torch.float32))
+                _close(outs[-1], ref, 2e-5, f"f32 out, code {code}")
+                outs.append(ops.linear(xd, wv, torch.bfloat16))
+                _close(outs[-1], ref, 1e-2, f"bf16 out, code {code}")
+                outs.append(ops.linear(xd, wv, torch.float32, residual=res.clone().to(DEV)))
+                _close(outs[-1], ref + res.double(), 2e-5, f"residual, code {code}")
+                outs.append(ops.linear_swiglu(xd, wv))
+                _close(outs[-1], gated, 1e-2, f"gated, code {code}")
+            got[code] = outs
+        finally:
+            lib.tp_linear_tune_mid_tile(0)
+    if k // 64 < 32:             # (neither kernel splits a K of fewer than 32 steps)
+        for a, b in zip(got[1], got[2]):
+            assert torch.equal(a, b), "blocks of 128 x 128 and of 256 x 128 give the same bits"
 
 
 @pytest.mark.parametrize("m,n,k", [(300, 512, 128), (1000, 816, 192), (257, 256, 64), (2048, 8448, 128), (2100, 6144, 128),
