@@ -279,10 +279,10 @@ class Engine:
     def profile(self, prompt_len: int = 128, batch: int = 1, decode_steps: int = 4, layer_stats: bool = False,
                 seed: int = 0) -> Dict[str, object]:
         """Where a step's time goes: ``batch`` fresh requests with prompts of ``prompt_len`` seeded random tokens,
-        one eager step for all prompts and ``decode_steps`` eager steps of one token each, every call into the
-        kernel library between a pair of stream events (``ops.KernelTimer``; the reference times layers and prints
-        per-tick times behind environment switches, /root/reference/engine/src/model.rs:1342-1345,
-        /root/reference/server/src/engine_task.rs:530-553).  Returns ``{"prefill": rows, "decode": rows}`` with rows
+        one eager step for all prompts and ``decode_steps`` eager steps of one token each (after one untimed pass of
+        the same shapes), every call into the kernel library between a pair of stream events (``ops.KernelTimer``;
+        the reference times layers and prints per-tick times behind environment switches,
+        /root/reference/engine/src/model.rs:1342-1345, /root/reference/server/src/engine_task.rs:530-553).  Returns ``{"prefill": rows, "decode": rows}`` with rows
         (entry point, calls, microseconds, share), the decode rows summed over the steps; with ``layer_stats`` also
         ``"layers"``: mean, variance and largest magnitude of the residual stream before every layer and after the
         last, for the prompts' step (the reference's summary trace, /root/reference/engine/src/pipeline.rs:149-187).
@@ -308,6 +308,18 @@ class Engine:
             return [(name, calls, round(us, 1), round(us / total, 4)) for name, _, calls, us in table]
 
         out: Dict[str, object] = {}
+        # Once untimed: a pair of events also spans what the host does between them while the GPU waits, and the
+        # first step of a new size allocates its buffers (the q/k/v projection of 2,048 rows showed as 117 us
+        # cold, 39 us after).
+        for rid in rids:
+            runner.add_request(rid)
+        try:
+            logits = runner.step([StepEntry(rid, p, [prompt_len - 1]) for rid, p in zip(rids, prompts)])
+            if decode_steps > 0:
+                runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, ops.argmax(logits).tolist())])
+        finally:
+            for rid in rids:
+                runner.end_request(rid)
         for rid in rids:
             runner.add_request(rid)
         try:
