@@ -785,9 +785,10 @@ int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N,
   const RopeOut rp = {positions, slots, inv_freq, (const float2*)cos_sin, factor, rotary_dim, n_heads, n_kv, head_dim, page_size,
                       0, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache};
   if (M > 16) {
-    // long steps: the pipelined kernels, whose wave tiles (64 or 128 columns) must lie inside one head, with the
-    // step's table of cosines and sines
-    if (head_dim != 128 || rotary_dim % 8 != 0 || cos_sin == nullptr || pre_ss != nullptr || page_size % 8 != 0) return -1;
+    // long steps: the pipelined kernels, whose wave tiles of 64 columns must each lie inside q, k or v (heads of a
+    // multiple of 64; the wider tiles are left out unless the heads are multiples of 128), with the step's table
+    // of cosines and sines
+    if (head_dim % 64 != 0 || rotary_dim % 8 != 0 || cos_sin == nullptr || pre_ss != nullptr || page_size % 8 != 0) return -1;
     return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled & 1, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, s);
   }
   launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, (w_tiled & 1 ? W_TILED : 0) | (w_tiled & 2 ? X_KBLOCKED : 0),

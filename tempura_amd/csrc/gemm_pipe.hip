@@ -264,6 +264,7 @@ __device__ inline void rope_fetch(RopeFetch<ROWS, COLS>& f, int lane, int mrow0,
   using F = RopeFetch<ROWS, COLS>;
   const int n0 = rp.col0 + ncol0;
   const int q_dim = rp.n_heads * rp.head_dim, kv_dim = rp.n_kv * rp.head_dim;
+  if (n0 >= q_dim + 2 * kv_dim) return;   // (a wave tile past the last column: N need be no multiple of the block's width)
   if (n0 < q_dim + kv_dim) {
     const int col = (lane % F::LPR) * 8, rr = lane / F::LPR;
     const int d = (n0 + col) % rp.head_dim;
@@ -311,11 +312,12 @@ __device__ inline void emit_tile_rope(const float* ct, int lane, int mrow0, int 
   using F = RopeFetch<ROWS, COLS>;
   const int n0 = rp.col0 + ncol0;                       // first column of the wave tile in the whole projection
   const int q_dim = rp.n_heads * rp.head_dim, kv_dim = rp.n_kv * rp.head_dim;
+  if (n0 >= q_dim + 2 * kv_dim) return;                 // a wave tile past the last column
   if (n0 < q_dim + kv_dim) {
     const int col = (lane % F::LPR) * 8, rr = lane / F::LPR;
     const bool is_q = n0 < q_dim;
     const int d = (n0 + col) % rp.head_dim;             // first of this lane's eight elements within its head
-    const int kh = is_q ? 0 : (n0 - q_dim) / rp.head_dim;
+    const int kh = is_q ? 0 : (n0 + col - q_dim) / rp.head_dim;   // (a wave tile may span two heads of 64)
     const bool rotate = d < rp.rotary_dim;
     const float* src = ct + rr * LD + col;
 #pragma unroll
@@ -357,11 +359,12 @@ __device__ inline void emit_tile_rope(const float* ct, int lane, int mrow0, int 
     return;
   }
   // values: COLS columns x ROWS / 8 groups of eight tokens, one (column, group) per lane and pass
-  const int kh = (n0 - q_dim - kv_dim) / rp.head_dim, d0 = (n0 - q_dim - kv_dim) % rp.head_dim;
 #pragma unroll
   for (int p = 0; p < 8; ++p) {
     const int it = lane + 64 * p;
     const int colv = it % COLS, rg = it / COLS;
+    const int kh = (n0 - q_dim - kv_dim + colv) / rp.head_dim;   // this column's head and its place in it
+    const int d0 = (n0 - q_dim - kv_dim + colv) % rp.head_dim - colv;
     const int m0 = mrow0 + rg * 8;
     const int s0 = f.slot[p];
     if (s0 == -2) continue;
@@ -1419,7 +1422,10 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   // needs the fewest rounds when a big tile is priced at 1.72 small ones (measured: 113 against 65 us at
   // K = 4096).
   int nb_big = 0;
-  if (splits == 1 && g_pipe_big != 2 && ldo % 4 == 0) {
+  // (with the rotating epilogue a wave's 128 columns of a big tile have to lie inside one of q, k and v: heads
+  // of a multiple of 128; the strips of the 192-column tile are ordered for heads of 128)
+  const bool big_ok = rope == nullptr || rope->head_dim % 128 == 0;
+  if (splits == 1 && g_pipe_big != 2 && ldo % 4 == 0 && big_ok) {
     const long NB2 = N / BNB;
     auto rounds = [&](long nb) {
       const long rest = (N - nb * BNB + BN - 1) / BN;
@@ -1436,7 +1442,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     // Tiles of 256 x 192 where N is a multiple of 192 and that many more tiles fill whole rounds: priced at 1.35
     // small tiles (the q/k/v projection of 2,048 rows, N = 6,144: 256 tiles in one round instead of 192 of 256 x 256
     // on three quarters of the CUs, 109 -> 8x us).
-    if (N % 192 == 0 && mode != OUT_SWIGLU && g_pipe_big != 4) {
+    if (N % 192 == 0 && mode != OUT_SWIGLU && g_pipe_big != 4 && (rope == nullptr || rope->head_dim == 128)) {
       const long t192 = (long)MB * (N / 192);
       if (1.35 * (double)((t192 + 255) / 256) < best - 1e-9 || g_pipe_big == 3) {
         const long blocks3 = blocks_for(N / 192);

@@ -466,13 +466,13 @@ rope_in_long_products = True
 def linear_rope_ok(m: int, n: int, k: int, head_dim: int, rotary_dim: int, page_size: int, x_dtype: torch.dtype,
                    cache_dtype: torch.dtype, prenormed: bool = False) -> bool:
     """Whether ``linear_rope_kv`` takes a projection of m rows onto n columns: a few rows (decoding), or a long
-    step with enough result tiles (128 x 128) to give half the CUs work without splitting K, heads of 128."""
+    step with enough result tiles (128 x 128) to give half the CUs work without splitting K, heads of a multiple of 64."""
     if not (_backend is None and allow_mfma and x_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16):
         return False
     if 0 < m <= 16:
         return k % 32 == 0 and head_dim % 16 == 0
     tiles = -(-m // 128) * -(-n // 128)      # (of 128 x 128, the smallest blocks of the pipelined products)
-    return (rope_in_long_products and m > 128 and tiles >= 128 and k % 64 == 0 and 255 * k * 2 + 128 < 2 ** 32 and head_dim == 128
+    return (rope_in_long_products and m > 128 and tiles >= 128 and k % 64 == 0 and 255 * k * 2 + 128 < 2 ** 32 and head_dim % 64 == 0
             and rotary_dim % 8 == 0 and page_size % 8 == 0 and not prenormed)
 
 

@@ -114,7 +114,9 @@ def test_rope_kv_write(dtype, heads, kv, d, rot, page):
                                                     (16, 3, 1, 48, 32, 96, 8), (5, 6, 3, 16, 16, 2048, 32),
                                                     (2100, 32, 8, 128, 128, 128, 16), (3000, 24, 8, 128, 64, 192, 8),
                                                     (4300, 4, 2, 128, 128, 64, 16), (2900, 10, 1, 128, 128, 320, 16),
-                                                    (520, 32, 8, 128, 128, 256, 16)])
+                                                    (520, 32, 8, 128, 128, 256, 16), (2100, 32, 8, 64, 64, 128, 16),
+                                                    (3000, 5, 3, 64, 32, 192, 8), (2600, 3, 1, 192, 192, 64, 16),
+                                                    (2200, 4, 2, 256, 256, 64, 16)])
 def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
     """The projection of a few rows that rotates and stores its rows in its epilogue gives the bits of the
     plain product followed by the rotation and cache-write kernel; and both agree with float64."""
@@ -164,8 +166,10 @@ def test_linear_rope_kv(m, heads, kv, d, rot, k, page):
                 assert torch.equal(q6, q1) and torch.equal(k6, k1) and torch.equal(v6, v1)
         finally:
             ops.library().tp_linear_tune_mid_tile(0)
-    if m > 16 and n % 192 == 0:       # tiles of 256 x 192, whose columns span two heads: the same bits
-        ops.library().tp_linear_tune_tile(7)
+    # tiles of 256 x 256 wherever the columns allow, and of 256 x 192 (whose columns span two heads of 128), asked
+    # for: the same bits (with heads that such a tile's strips would cut across, the narrower tiles are taken)
+    for code in ((5, 7) if m > 16 and n % 192 == 0 else (5,) if m > 16 else ()):
+        ops.library().tp_linear_tune_tile(code)
         try:
             for wv in (wd, ops.tile_weight(wd)):
                 k5, v5 = kc.to(DEV), vc.to(DEV)
