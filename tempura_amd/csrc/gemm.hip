@@ -187,7 +187,7 @@ extern "C" int tp_linear_rope(const void* x, const void* w, int w_tiled, int M, 
 // block of rows 16 i.. and columns 32 j.. as 1,024 contiguous bytes, element (r, c) of the block at
 // ((c / 8) * 16 + r) * 8 + c % 8 (the matrix cores' operand order), blocks of a row group side by side.
 //
-// `defer_reduce` (products of 17..128 rows whose K is split over blocks): the partial sums stay in `scratch`
+// `defer_reduce` (products of more than 16 rows whose K is split over blocks): the partial sums stay in `scratch`
 // as [*splits_out, M, N] float32 and `out` is not touched; the caller's next kernel adds them (ascending).
 // *splits_out == 1 means that the product wrote `out` itself.
 extern "C" int tp_linear_fused(const void* x, const void* w, int in_dt, void* out, int out_dt, int accumulate, int M,

@@ -662,7 +662,7 @@ static int g_tune_order = 0;   // large products: 1 tiled kernel, plain block or
 
 // Defined in gemm_pipe.hip; 0 when it took the product, -1 when the sizes are not its own.
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
-                   size_t scratch_floats, int tune_splits, const RopeOut* rope, hipStream_t s);
+                   size_t scratch_floats, int tune_splits, const RopeOut* rope, int defer, int* splits_out, hipStream_t s);
 
 int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
                      size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s);
@@ -789,7 +789,7 @@ int tp_linear_rope_mfma(const void* x, const void* w, int w_tiled, int M, int N,
     // multiple of 64; the wider tiles are left out unless the heads are multiples of 128), with the step's table
     // of cosines and sines
     if (head_dim % 64 != 0 || rotary_dim % 8 != 0 || cos_sin == nullptr || pre_ss != nullptr || page_size % 8 != 0) return -1;
-    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled & 1, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, s);
+    return tp_linear_pipe((const bf16_t*)x, (const bf16_t*)w, w_tiled & 1, nullptr, OUT_ROPE, M, N, K, nullptr, 0, 0, &rp, 0, nullptr, s);
   }
   launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, nullptr, OUT_ROPE, M, N, K, (w_tiled & 1 ? W_TILED : 0) | (w_tiled & 2 ? X_KBLOCKED : 0),
                    pre, post, rp, s);
@@ -836,7 +836,8 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
     // (measured at 128 rows: N = 28,672 59 us against 77 us, the narrow products a few us slower)
     const bool pipe = g_tune_order ? g_tune_order == 3 : (M > 128 || (M > 64 && N >= 16384));
     const bool pipe64 = !pipe && M <= 128 && scratch != nullptr && g_tune_mid != 2;
-    if (pipe && tp_linear_pipe(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, nullptr, s) == 0) {
+    if (pipe && tp_linear_pipe(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, nullptr, defer_reduce,
+                               splits_out, s) == 0) {
       // taken by the pipelined kernel
     } else if (pipe64 && tp_linear_pipe64(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits,
                                           defer_reduce, splits_out, s) == 0) {

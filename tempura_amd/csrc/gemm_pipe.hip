@@ -1348,7 +1348,8 @@ static double pipe_cost(long blocks, int steps, double step_us, int splits, int 
 }
 // The 128 x 128 blocks.  Returns 0 when launched.
 static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K,
-                             float* scratch, size_t scratch_floats, const RopeOut* rope, hipStream_t s) {
+                             float* scratch, size_t scratch_floats, const RopeOut* rope, int defer, int* splits_out,
+                             hipStream_t s) {
   const int MB = (M + BM128 - 1) / BM128, NB = (N + BN128 - 1) / BN128;
   const long tiles = (long)MB * NB;
   const int splits = splits128(M, N, K, scratch != nullptr && rope == nullptr, scratch_floats);
@@ -1359,7 +1360,9 @@ static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void
   if (8 * per_xcd > 0x7fffffffL) return -1;
   hipLaunchKernelGGL(gemm_pipe128_kernel, dim3((unsigned)(8 * per_xcd)), dim3(256), 0, s, x, w, out,
                      splits > 1 ? scratch : nullptr, mode, M, N, K, ldo, rp, w_tiled, splits);
-  if (splits > 1) {
+  if (splits > 1 && defer && splits_out != nullptr && mode != OUT_SWIGLU) {
+    *splits_out = splits;   // the parts stay unadded for the caller's next kernel
+  } else if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
                        splits, M, N);
@@ -1371,7 +1374,7 @@ static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void
 // float32 partial sums: with few result tiles K is split over blocks until there is work for every CU.
 int g_pipe_big = 0;   // tuning: 1 = 256 x 256 tiles for every whole block of 256 columns, 2 = never; 3 = 256 x 192 wherever N allows, 4 = never
 int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
-                   size_t scratch_floats, int tune_splits, const RopeOut* rope, hipStream_t s) {
+                   size_t scratch_floats, int tune_splits, const RopeOut* rope, int defer, int* splits_out, hipStream_t s) {
   if ((mode == OUT_ROPE) != (rope != nullptr)) return -1;
   if (w_tiled && N % 16 != 0) return -1;
   if (K % BK != 0 || K < BK) return -1;
@@ -1395,7 +1398,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     mid = pipe_cost(tiles128 * s128, (KT + s128 - 1) / s128, 0.44, s128, M, N) <
           pipe_cost(tiles * s256, (KT + s256 - 1) / s256, 0.71, s256, M, N);
   }
-  if (mid) return tp_linear_pipe128(x, w, w_tiled, out, mode, M, N, K, scratch, scratch_floats, rope, s);
+  if (mid) return tp_linear_pipe128(x, w, w_tiled, out, mode, M, N, K, scratch, scratch_floats, rope, defer, splits_out, s);
   // (see tile_of_block) strips of at most eight row blocks, all about as tall; a launch of nb column blocks has
   // 8 x MB x ceil(nb / 8) blocks
   const int strips = (MB + 7) / 8;
@@ -1471,7 +1474,9 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   }
   hipLaunchKernelGGL(gemm_pipe_kernel, dim3((unsigned)blocks, splits), dim3(256), 0, s, x, w, out, scratch, mode, M, N, K,
                      pm, ldo, rp, w_tiled);
-  if (splits > 1) {
+  if (splits > 1 && defer && splits_out != nullptr && mode != OUT_SWIGLU) {
+    *splits_out = splits;   // the parts stay unadded for the caller's next kernel
+  } else if (splits > 1) {
     const size_t n_out = mode == OUT_SWIGLU ? (size_t)M * (N / 2) : (size_t)M * N;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, s, scratch, out, mode,
                        splits, M, N);

@@ -323,11 +323,12 @@ class Partials:
 
 def split_norm_ok(m: int, width: int, dtype: torch.dtype) -> bool:
     """Whether the product before a norm over ``width`` columns of ``m`` rows can carry it (``linear`` with
-    ``next_norm``): up to 16 rows the two products around the norm share it, up to 128 rows the kernel
-    that adds the product's partial sums into the residual stream also norms the rows."""
+    ``next_norm``): up to 16 rows the two products around the norm share it; with more rows the kernel that
+    adds the product's partial sums into the residual stream also norms the rows, where the product splits K
+    (``linear`` says whether it did)."""
     if _backend is not None:
         return _backend.split_norm_ok(m, width, dtype)
-    return allow_mfma and dtype == torch.bfloat16 and 0 < m <= 128 and width % 32 == 0
+    return allow_mfma and dtype == torch.bfloat16 and 0 < m and width % 32 == 0
 
 
 def _pre_args(x):
@@ -391,7 +392,7 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
     [m, n]) the product is added into it in place and it is returned.
     With ``next_norm`` = (float32 weight [n], eps) (needs ``residual``) the result is the pair (residual, rows
     for the part behind that norm): ``Prenormed`` rows up to 16 rows of bfloat16, the normed rows themselves
-    up to 128 rows when the product's K was split (one kernel adds the partial sums into the residual and norms
+    from 17 rows on when the product's K was split (one kernel adds the partial sums into the residual and norms
     it), or None when the norm has to run on its own.
     With ``partial_ok`` (float32 output, no residual) the result may be ``Partials``."""
     if _backend is not None:
@@ -436,9 +437,9 @@ def linear(x, w: torch.Tensor, out_dtype: torch.dtype, residual: Optional[torch.
         if hand_blocked:
             layout |= 8
     scratch, nscratch = _splitk_scratch(x, m, n) if allow_mfma else (None, 0)
-    # 17..128 rows: the partial sums of a split K may stay unadded for the kernel that consumes the rows
+    # from 17 rows on: the partial sums of a split K may stay unadded for the kernel that consumes the rows
     layout |= wl
-    defer = scratch is not None and 16 < m <= 128 and (layout & 3) == 0 and \
+    defer = scratch is not None and 16 < m and (layout & 3) == 0 and \
         ((next_norm is not None and residual is not None and split_norm_ok(m, n, x.dtype) and n % 4 == 0 and n <= 16384) or
          (partial_ok and residual is None and out_dtype == torch.float32))
     splits = ctypes.c_int(1)

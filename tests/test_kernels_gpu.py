@@ -588,9 +588,10 @@ def test_linear_split_norm(m, hidden, kp, nc):
         _close(h3, hd.double().cpu() + a2.double() @ w2.double().T, 2e-5, "fallback product")
 
 
-@pytest.mark.parametrize("m,hidden,kp", [(17, 256, 1024), (64, 4096, 4096), (100, 160, 2048), (128, 512, 256)])
+@pytest.mark.parametrize("m,hidden,kp", [(17, 256, 1024), (64, 4096, 4096), (100, 160, 2048), (128, 512, 256),
+                                         (300, 1024, 2048), (512, 4096, 4096), (700, 3072, 8192), (1000, 512, 4096)])
 def test_linear_deferred_reduction(m, hidden, kp):
-    """Products of 17..128 rows split K over blocks; the partial sums may stay unadded for the next kernel:
+    """Products with few result tiles split K over blocks; the partial sums may stay unadded for the next kernel:
     the one that adds them into the residual stream and norms it, or the rotation and cache write."""
     ops = _ops()
     g = torch.Generator().manual_seed(31)
@@ -630,7 +631,7 @@ def test_linear_deferred_reduction(m, hidden, kp):
         kc = torch.zeros(pages, kvh, ps, d, dtype=torch.bfloat16, device=DEV)
         vc = torch.zeros(pages, kvh, d, ps, dtype=torch.bfloat16, device=DEV)
         qkv = ops.linear(xin.to(DEV), wqkv.to(DEV), torch.float32, partial_ok=partial_ok)
-        if partial_ok and hidden >= 1024:
+        if partial_ok and hidden >= 1024 and (m <= 128 or hidden >= 2048):
             assert isinstance(qkv, ops.Partials) and qkv.shape == (m, width)
         q = ops.rope_kv_write(qkv, pos.to(DEV), slots.to(DEV), inv_freq.to(DEV), d, 1.0, heads, kvh, d, kc, vc, torch.bfloat16)
         results.append((q, kc, vc))
