@@ -493,24 +493,27 @@ __device__ inline void emit_tile(const float* ct, int lane, int mrow0, int ncol0
 
 }  // namespace
 
-// Which tile a block takes.  Blocks go to the 8 XCDs in turn and each XCD has an L2 of its own: XCD c takes the
-// column blocks c, c + 8, ... (at most Q of them) and all MB row blocks, as a list without gaps (a block that
-// finds no tile and leaves at once still held up the ones behind it: a product with a fifth of such blocks
-// took twice its time).  The list walks groups of pq column blocks; inside a group, strips of pm row blocks;
-// inside a strip, row blocks fastest: the 32 blocks that an XCD runs at a time share pm row blocks of x and
-// about 32 / pm column blocks of w.  False for the few blocks past an XCD's last column block.
+// Which tile a block takes.  Blocks go to the 8 XCDs in turn and each XCD has an L2 of its own: XCD j takes the
+// j-th eighth of the list of tiles, all eighths equally long (with whole column blocks dealt out instead, 255 tiles
+// of three row blocks came to 33 on five XCDs of 32 CUs, a second round for one tile each: 170 us instead of 113),
+// and the list has no gaps (a block that finds no tile and leaves at once still held up the ones behind it: a
+// product with a fifth of such blocks took twice its time).  The list walks groups of pq column blocks; inside a
+// group, strips of pm row blocks; inside a strip, row blocks fastest: the 32 blocks that an XCD runs at a time
+// share pm row blocks of x and about 32 / pm column blocks of w.  False for the few blocks past the list's end.
 __device__ inline bool tile_of_block(unsigned block, int MB, int NB, int pm, int& bm, int& bn) {
-  const int c = block % 8, j = block / 8;
-  const int pq = max(1, 32 / pm), Q = (NB + 7) / 8;
+  const int total = MB * NB, per = (total + 7) / 8;
+  const int item = (int)(block % 8) * per + (int)(block / 8);
+  if ((int)(block / 8) >= per || item >= total) return false;
+  const int pq = max(1, 32 / pm);
   const int group = MB * pq;
-  const int k = j / group, rem = j - k * group;
-  const int wk = min(pq, Q - k * pq);
+  const int k = item / group, rem = item - k * group;
+  const int wk = min(pq, NB - k * pq);
   const int strip = pm * wk;
   const int sidx = rem / strip, r = rem - sidx * strip;
   const int hs = min(pm, MB - sidx * pm);
   bm = sidx * pm + r % hs;
-  bn = c + 8 * (k * pq + r / hs);
-  return bn < NB;
+  bn = k * pq + r / hs;
+  return true;
 }
 
 // ldo: row stride of `out` in elements (N, or N / 2 for the gated mode, when the launch covers all columns;
@@ -1324,20 +1327,6 @@ __global__ void gemm_splitk_reduce_kernel(const float* __restrict__ partial, voi
 
 int g_pipe_mid = 0;   // tuning: 1 = 128 x 128 blocks for every product of more than 128 rows, 2 = never
 
-// Into how many parts the 128 x 128 blocks cut K: whole parts of at least sixteen steps, no more blocks than CUs.
-static int splits128(int M, int N, int K, bool can_split, size_t scratch_floats) {
-  const long tiles = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
-  const int KT = K / BK;
-  int splits = 1;
-  if (can_split) {   // (the rotating epilogue takes whole sums)
-    splits = std::max(1, std::min((int)(256 / tiles), std::min(16, KT / 16)));
-    while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
-    const int per = (KT + splits - 1) / splits;
-    splits = (KT + per - 1) / per;
-  }
-  return splits;
-}
-
 // What a product costs in microseconds, roughly, as `blocks` blocks that take `steps` steps of K each at
 // `step_us` a step, one block on a CU at a time, and a kernel that adds the parts if K is split.  Measured:
 // 0.44 us a step for a block of 128 x 128, 0.71 us for one of 256 x 128; the parts are written and read
@@ -1346,6 +1335,46 @@ static double pipe_cost(long blocks, int steps, double step_us, int splits, int 
   const double rounds = (double)((blocks + 255) / 256);
   return rounds * steps * step_us + (splits > 1 ? 3.0 + (splits + 2.0) * M * N * 4.0 / 3e6 : 0.0);
 }
+
+// Into how many parts K (KT steps) is cut for `tiles` result tiles: the cheapest by pipe_cost among whole parts
+// of at least sixteen steps that the scratch memory holds (96 tiles of 256 x 128 and 224 steps: two parts,
+// 192 blocks in one round, not the three that make 288 blocks and a second round).
+static int best_splits(long tiles, int KT, double step_us, int M, int N, size_t scratch_floats) {
+  int best = 1;
+  double best_cost = pipe_cost(tiles, KT, step_us, 1, M, N);
+  const int cap = std::min(16, KT / 16);
+  for (int sp = 2; sp <= cap && (size_t)sp * M * N <= scratch_floats; ++sp) {
+    const int per = (KT + sp - 1) / sp;
+    if ((KT + per - 1) / per != sp) continue;   // (no part without a step)
+    const double c = pipe_cost(tiles * sp, per, step_us, sp, M, N);
+    if (c < best_cost - 1e-9) {
+      best_cost = c;
+      best = sp;
+    }
+  }
+  return best;
+}
+
+// The parts of K for blocks of 128 x 128 (the rotating epilogue takes whole sums: can_split false).
+static int splits128(int M, int N, int K, bool can_split, size_t scratch_floats) {
+  const long tiles = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
+  if (!can_split || tiles >= 256) return 1;
+  return best_splits(tiles, K / BK, 0.44, M, N, scratch_floats);
+}
+
+// The parts of K for blocks of 256 x 128: none with 128 tiles or more.
+static int splits256(long tiles, int KT, int M, int N, const float* scratch, size_t scratch_floats, int tune_splits) {
+  if (scratch == nullptr) return 1;
+  if (tune_splits > 0) {
+    int sp = std::max(1, std::min(tune_splits, std::min(16, KT / 16)));
+    while (sp > 1 && (size_t)sp * M * N > scratch_floats) --sp;
+    const int per = (KT + sp - 1) / sp;
+    return (KT + per - 1) / per;
+  }
+  if (tiles >= 128) return 1;
+  return best_splits(tiles, KT, 0.71, M, N, scratch_floats);
+}
+
 // The 128 x 128 blocks.  Returns 0 when launched.
 static int tp_linear_pipe128(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K,
                              float* scratch, size_t scratch_floats, const RopeOut* rope, int defer, int* splits_out,
@@ -1388,35 +1417,21 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     const int KT = K / BK;
     const bool can_split = scratch != nullptr && rope == nullptr;
     const long tiles = (long)MB * NB, tiles128 = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
-    int s256 = 1;
-    if (scratch != nullptr) {   // (as below)
-      s256 = tune_splits > 0 ? tune_splits : (tiles >= 128 ? 1 : (int)((256 + tiles - 1) / tiles));
-      s256 = std::max(1, std::min(s256, std::min(16, KT / 16)));
-      while (s256 > 1 && (size_t)s256 * M * N > scratch_floats) --s256;
-    }
+    const int s256 = splits256(tiles, KT, M, N, scratch, scratch_floats, tune_splits);
     const int s128 = splits128(M, N, K, can_split, scratch_floats);
     mid = pipe_cost(tiles128 * s128, (KT + s128 - 1) / s128, 0.44, s128, M, N) <
           pipe_cost(tiles * s256, (KT + s256 - 1) / s256, 0.71, s256, M, N);
   }
   if (mid) return tp_linear_pipe128(x, w, w_tiled, out, mode, M, N, K, scratch, scratch_floats, rope, defer, splits_out, s);
   // (see tile_of_block) strips of at most eight row blocks, all about as tall; a launch of nb column blocks has
-  // 8 x MB x ceil(nb / 8) blocks
+  // 8 x ceil(MB x nb / 8) blocks
   const int strips = (MB + 7) / 8;
   const int pm = (MB + strips - 1) / strips;
-  auto blocks_for = [&](long nb) { return 8L * MB * ((nb + 7) / 8); };
+  auto blocks_for = [&](long nb) { return 8L * (((long)MB * nb + 7) / 8); };
   const long blocks = blocks_for(NB);
   if (blocks > 0x7fffffffL) return -1;
-  // splits: enough blocks for the 256 CUs, at least sixteen tiles of K each (measured: more splits than
-  // that cost more in partial sums than they gain)
-  int splits = 1;
-  if (scratch != nullptr) {
-    const int tiles = MB * NB, KT = K / BK;
-    splits = tune_splits > 0 ? tune_splits : (tiles >= 128 ? 1 : (256 + tiles - 1) / tiles);
-    splits = std::max(1, std::min(splits, std::min(16, KT / 16)));
-    while (splits > 1 && (size_t)splits * M * N > scratch_floats) --splits;
-    const int per = (KT + splits - 1) / splits;
-    splits = (KT + per - 1) / per;   // no split without a tile
-  }
+  // parts of K: with few tiles, the cheapest number by the cost model, at least sixteen steps of K each
+  const int splits = splits256((long)MB * NB, K / BK, M, N, scratch, scratch_floats, tune_splits);
   const int ldo = mode == OUT_SWIGLU ? N / 2 : N;
   RopeOut rp = {};
   if (rope != nullptr) rp = *rope;

@@ -381,7 +381,7 @@ def _splitk_scratch(x: torch.Tensor, m: int, n: int):
         tiles = -(-m // 256) * -(-n // 128)
         if tiles >= 128:
             return None, 0
-        splits = min(16, -(-256 // tiles))
+        splits = min(16, 2 * -(-256 // tiles))      # (room for the library to choose: it prices the candidates)
     count = splits * m * n
     return torch.empty((count,), dtype=torch.float32, device=x.device), count
 
