@@ -1329,21 +1329,23 @@ int g_pipe_mid = 0;   // tuning: 1 = 128 x 128 blocks for every product of more 
 
 // What a product costs in microseconds, roughly, as `blocks` blocks that take `steps` steps of K each at
 // `step_us` a step, one block on a CU at a time, and a kernel that adds the parts if K is split.  Measured:
-// 0.44 us a step for a block of 128 x 128, 0.71 us for one of 256 x 128; the parts are written and read
-// again at about 3 TB/s.
+// 0.52 us a step for a block of 128 x 128, 0.75 us for one of 256 x 128 (STEP128_US, STEP256_US); the parts are
+// written and read again at about 3 TB/s.
+constexpr double STEP128_US = 0.52, STEP256_US = 0.75;
 static double pipe_cost(long blocks, int steps, double step_us, int splits, int M, int N) {
   const double rounds = (double)((blocks + 255) / 256);
   return rounds * steps * step_us + (splits > 1 ? 3.0 + (splits + 2.0) * M * N * 4.0 / 3e6 : 0.0);
 }
 
 // Into how many parts K (KT steps) is cut for `tiles` result tiles: the cheapest by pipe_cost among whole parts
-// of at least sixteen steps that the scratch memory holds (96 tiles of 256 x 128 and 224 steps: two parts,
-// 192 blocks in one round, not the three that make 288 blocks and a second round).
+// of at least sixteen steps that the scratch memory holds and that make no more blocks than there are CUs (96 tiles
+// of 256 x 128 and 224 steps: two parts, 192 blocks, not the three that make 288 blocks and a second round; parts
+// that fill several rounds measured no better than none).
 static int best_splits(long tiles, int KT, double step_us, int M, int N, size_t scratch_floats) {
   int best = 1;
   double best_cost = pipe_cost(tiles, KT, step_us, 1, M, N);
   const int cap = std::min(16, KT / 16);
-  for (int sp = 2; sp <= cap && (size_t)sp * M * N <= scratch_floats; ++sp) {
+  for (int sp = 2; sp <= cap && sp * tiles <= 256 && (size_t)sp * M * N <= scratch_floats; ++sp) {
     const int per = (KT + sp - 1) / sp;
     if ((KT + per - 1) / per != sp) continue;   // (no part without a step)
     const double c = pipe_cost(tiles * sp, per, step_us, sp, M, N);
@@ -1359,7 +1361,7 @@ static int best_splits(long tiles, int KT, double step_us, int M, int N, size_t 
 static int splits128(int M, int N, int K, bool can_split, size_t scratch_floats) {
   const long tiles = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
   if (!can_split || tiles >= 256) return 1;
-  return best_splits(tiles, K / BK, 0.44, M, N, scratch_floats);
+  return best_splits(tiles, K / BK, STEP128_US, M, N, scratch_floats);
 }
 
 // The parts of K for blocks of 256 x 128: none with 128 tiles or more.
@@ -1372,7 +1374,7 @@ static int splits256(long tiles, int KT, int M, int N, const float* scratch, siz
     return (KT + per - 1) / per;
   }
   if (tiles >= 128) return 1;
-  return best_splits(tiles, KT, 0.71, M, N, scratch_floats);
+  return best_splits(tiles, KT, STEP256_US, M, N, scratch_floats);
 }
 
 // The 128 x 128 blocks.  Returns 0 when launched.
@@ -1419,8 +1421,8 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
     const long tiles = (long)MB * NB, tiles128 = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
     const int s256 = splits256(tiles, KT, M, N, scratch, scratch_floats, tune_splits);
     const int s128 = splits128(M, N, K, can_split, scratch_floats);
-    mid = pipe_cost(tiles128 * s128, (KT + s128 - 1) / s128, 0.44, s128, M, N) <
-          pipe_cost(tiles * s256, (KT + s256 - 1) / s256, 0.71, s256, M, N);
+    mid = pipe_cost(tiles128 * s128, (KT + s128 - 1) / s128, STEP128_US, s128, M, N) <
+          pipe_cost(tiles * s256, (KT + s256 - 1) / s256, STEP256_US, s256, M, N);
   }
   if (mid) return tp_linear_pipe128(x, w, w_tiled, out, mode, M, N, K, scratch, scratch_floats, rope, defer, splits_out, s);
   // (see tile_of_block) strips of at most eight row blocks, all about as tall; a launch of nb column blocks has
