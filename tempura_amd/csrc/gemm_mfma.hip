@@ -832,9 +832,9 @@ int tp_linear_mfma(const void* x, const void* w, void* out, int out_dt, int accu
   } else {
     // large products: 128 x 128 tiles.  Between 17 and 128 rows the weights are still the traffic:
     // 64 x 128 tiles, and K split over blockIdx.z until there are blocks for every CU.
-    // the pipelined kernel: from 129 rows on, and from 65 rows on when there are many column blocks
-    // (measured at 128 rows: N = 28,672 59 us against 77 us, the narrow products a few us slower)
-    const bool pipe = g_tune_order ? g_tune_order == 3 : (M > 128 || (M > 64 && N >= 16384));
+    // the pipelined kernels: from 65 rows on (their 128 x 128 blocks against two 64-row blocks that each fetch
+    // the weights: 72 to 128 rows of the 8B shapes 26 -> 17..21 us, 43 -> 31..34 us, 21 -> 16 us, 52 -> 46 us)
+    const bool pipe = g_tune_order ? g_tune_order == 3 : M > 64;
     const bool pipe64 = !pipe && M <= 128 && scratch != nullptr && g_tune_mid != 2;
     if (pipe && tp_linear_pipe(xb, wb, w_tiled, out, mode, M, N, K, scratch, scratch_floats, g_tune_splits, nullptr, defer_reduce,
                                splits_out, s) == 0) {

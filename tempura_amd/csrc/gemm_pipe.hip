@@ -25,7 +25,7 @@
 // One barrier per 64 of K.  Sizes: K % 64 == 0; any M and N (loads clamp to the last row, stores are
 // masked).  The sum over K runs in ascending order for every output element.
 // Further down: the same pipeline on 256 x 256 block tiles (gemm_pipe_big_kernel; the host mixes both tile
-// sizes so that whole rounds of tiles fill the CUs) and on 64 x 128 tiles for 17..128 rows (gemm_pipe64_kernel).
+// sizes so that whole rounds of tiles fill the CUs) and on 64 x 128 tiles for 17..64 rows (gemm_pipe64_kernel).
 #include <algorithm>
 
 #include "common.h"
@@ -944,7 +944,7 @@ __global__ __launch_bounds__(256) void gemm_pipe_big_kernel(const bf16_t* __rest
   }
 }
 
-// ---- the same pipeline for 17..128 rows -----------------------------------------------------------
+// ---- the same pipeline for 17..64 rows (it takes up to 128) -----------------------------------------------------------
 // Here the weights are the traffic and the matrix core has little to do: a block owns 64 x 128 of the
 // result (a wave 32 x 64), three stages of (64 + 128) rows (72 KB: two blocks per CU), K split over
 // blockIdx.y until there are about two blocks for every CU.  Loads, LDS reads and MFMAs interleave as above.
@@ -1412,10 +1412,10 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   if ((size_t)(BM - 1) * K * 2 + 128 >= ((size_t)1 << 32)) return -1;  // a lane's source offset is 32 bits
   if (mode == OUT_SWIGLU && N % 16 != 0) return -1;
   const int MB = (M + BM - 1) / BM, NB = (N + BN - 1) / BN;
-  // Steps of a few hundred rows, with at most one round of 256 x 128 blocks: blocks of 128 x 128 where they
+  // Steps of 65 to a few hundred rows, with at most one round of 256 x 128 blocks: blocks of 128 x 128 where they
   // are cheaper (more of them, so more CUs at work and K in fewer parts).
   bool mid = g_pipe_mid == 1;
-  if (g_pipe_mid == 0 && M > 128 && (long)MB * NB <= 256) {
+  if (g_pipe_mid == 0 && M > 64 && (long)MB * NB <= 256) {
     const int KT = K / BK;
     const bool can_split = scratch != nullptr && rope == nullptr;
     const long tiles = (long)MB * NB, tiles128 = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
@@ -1502,7 +1502,7 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
 }
 
 int g_pipe64_narrow = 0;   // tuning: 1 = blocks of 64 columns always, 2 = never
-// The 64-row pipeline (17..128 rows).  `defer`: when K is split, leave the partial sums in `scratch` for the
+// The 64-row pipeline (17..64 rows; up to 128 where the other kernels do not take the sizes).  `defer`: when K is split, leave the partial sums in `scratch` for the
 // caller's next kernel and report their number through *splits_out.
 int tp_linear_pipe64(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int mode, int M, int N, int K, float* scratch,
                      size_t scratch_floats, int tune_splits, int defer, int* splits_out, hipStream_t s) {

@@ -372,7 +372,8 @@ def linear_swiglu(x, w: torch.Tensor, blocked_out: bool = False):
 
 def _splitk_scratch(x: torch.Tensor, m: int, n: int):
     """Room for the partial sums of a bfloat16 product whose K is split over blocks: products of 17..128
-    rows, and larger ones with too few result tiles (256 x 128) to give every CU work."""
+    rows (64-row blocks up to 64 rows, 128-row blocks above), and larger ones with too few result tiles (256 x 128)
+    to give every CU work."""
     if x.dtype != torch.bfloat16 or m <= 16:
         return None, 0
     if m <= 128:
