@@ -350,11 +350,19 @@ def main() -> int:
         del eng
         torch.cuda.empty_cache()
         eng3, cfg3, _, wb3 = make_engine(args.mixed_config, None, args.mixed_requests, 2048 + args.mixed_output + 64, args.mixed_chunk)
+        # the named workload: portions of exactly the chunk; then the engine's default, which lengthens portions
+        # with budget that no other request can use
+        eng3.scheduler.config.fill_budget = False
         mixed = mixed_workload(eng3, cfg3, wb3)
         points["mixed_output_tok_s"] = mixed["output_tok_s"]
         points["mixed_ttft_p50_ms"] = mixed["ttft_ms"]["p50"]
         points["mixed_ttft_p95_ms"] = mixed["ttft_ms"]["p95"]
         say(f"mixed {mixed}")
+        eng3.scheduler.config.fill_budget = True
+        filled = mixed_workload(eng3, cfg3, wb3)
+        points["mixed_fill_budget_output_tok_s"] = filled["output_tok_s"]
+        points["mixed_fill_budget_ttft_p50_ms"] = filled["ttft_ms"]["p50"]
+        say(f"mixed, portions lengthened into spare budget {filled}")
 
     out = {
         "metric": f"decode tok/s at batch {args.batch} through the engine, {args.model_config} shape {dshort}, "

@@ -29,7 +29,10 @@ def _add_engine_args(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--kv-blocks", type=int, default=None, help="cache pages (default: from free memory)")
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.9)
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048, help="token budget of one step")
-    ap.add_argument("--prefill-chunk-size", type=int, default=512, help="largest prompt portion in one step")
+    ap.add_argument("--prefill-chunk-size", type=int, default=512,
+                    help="a prompt's portion of one step while other prompts wait for theirs")
+    ap.add_argument("--strict-chunks", action="store_true",
+                    help="never lengthen a prompt portion with budget that nobody else can use")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps as a HIP graph")
     ap.add_argument("--no-chain-steps", action="store_true",
                     help="wait for a step's tokens on the host before queueing the next decode step")
@@ -55,7 +58,7 @@ def _engine_from_args(args):
                   page_size=args.block_size, kv_pages=args.kv_blocks,
                   gpu_memory_utilization=args.gpu_memory_utilization, max_batch_size=args.max_batch_size,
                   max_seq_len=args.max_seq_len, max_num_batched_tokens=args.max_num_batched_tokens,
-                  prefill_chunk_size=args.prefill_chunk_size, use_graph=not args.no_graph,
+                  prefill_chunk_size=args.prefill_chunk_size, fill_budget=not args.strict_chunks, use_graph=not args.no_graph,
                   chain_steps=not args.no_chain_steps)
 
 

@@ -30,11 +30,14 @@ class Engine:
                  gpu_memory_utilization: float = 0.9, max_batch_size: int = 64,
                  max_seq_len: Optional[int] = None, max_num_batched_tokens: int = 2048,
                  prefill_chunk_size: int = 512, device: str = "cuda:0", use_graph: bool = True,
-                 chain_steps: bool = True):
+                 chain_steps: bool = True, fill_budget: bool = True):
         """``model``: a folder with config.json and safetensors, or (with ``random_weights``) a typed
         configuration such as ``LlamaConfig``/``PRESETS[name]``.
         ``kv_pages``: cache pages per group; by default as many as ``gpu_memory_utilization`` of the
         free memory holds, but no more than ``max_batch_size`` requests of ``max_seq_len`` need.
+        ``prefill_chunk_size``: a prompt's share of a step while other prompts wait for theirs; with ``fill_budget``
+        what is left of ``max_num_batched_tokens`` when everybody has had a turn lengthens the portions in the plan
+        (a lone long prompt runs in steps of the whole budget).
         ``chain_steps``: while every running request is decoding and nobody waits, the next step is queued
         behind the sampling kernel (its tokens stay on the device) before the host has read this step's
         tokens, so the GPU does not wait for the host between steps; a request that ends on the token just
@@ -60,7 +63,8 @@ class Engine:
                                   use_graph=use_graph)
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_batch_size, max_num_batched_tokens=max_num_batched_tokens,
-                            prefill_chunk_size=prefill_chunk_size, max_model_len=self.max_seq_len),
+                            prefill_chunk_size=prefill_chunk_size, max_model_len=self.max_seq_len,
+                            fill_budget=fill_budget),
             self.runner.cache)
         self.sampler = Sampler(spec.vocab_size, self.device, default_seed=seed)
         self._ids = itertools.count()

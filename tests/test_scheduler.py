@@ -14,8 +14,9 @@ FULL = CacheSpec("full", 2, 16)
 
 def make(num_pages=64, page_size=8, **cfg):
     cache = CacheManager([FULL], page_size, num_pages, max_requests=cfg.get("max_num_seqs", 8))
+    # (fill_budget off unless a test asks for it: the tests below pin the portions themselves)
     return Scheduler(SchedulerConfig(**{"max_num_seqs": 8, "max_num_batched_tokens": 32, "prefill_chunk_size": 16,
-                                        "max_model_len": 512, **cfg}), cache), cache
+                                        "max_model_len": 512, "fill_budget": False, **cfg}), cache), cache
 
 
 def req(rid, n_prompt, max_new=4, **kw):
@@ -210,3 +211,45 @@ def test_nothing_to_generate_finishes_on_arrival():
     sched.add_request(req("a", 5, max_new=2))
     steps = run(sched, cache)
     assert [s[0][0] for s in steps] == ["a", "a"]
+
+
+def test_budget_nobody_else_can_use_lengthens_the_portions():
+    """With ``fill_budget`` a chunk is a prompt's share while others wait for theirs: what is left of the budget
+    when everybody has had a turn goes to the portions in the plan, in their order, still cut at aligned positions,
+    never beyond the pages that are free; decoding requests keep their single tokens."""
+    sched, cache = make(fill_budget=True)
+    sched.add_request(req("a", 70, max_new=2))
+    steps = run(sched, cache)
+    assert steps[:3] == [[("a", 0, 32, False)], [("a", 32, 32, False)], [("a", 64, 6, True)]]
+    # two prompts: each gets its chunk first, the first of them what is left
+    sched, cache = make(fill_budget=True, max_num_batched_tokens=40)
+    sched.add_request(req("a", 50, max_new=1))
+    sched.add_request(req("b", 20, max_new=1))
+    steps = run(sched, cache)
+    assert steps[0] == [("a", 0, 24, False), ("b", 0, 16, False)]
+    assert steps[1] == [("a", 24, 26, True), ("b", 16, 4, True)]
+    # a decoding request beside a long prompt: one token for it, the rest of the budget for the prompt
+    sched, cache = make(fill_budget=True)
+    sched.add_request(req("d", 3, max_new=30))
+    run_one = sched.schedule()
+    for it in run_one:
+        cache.reserve(it.request.rid, it.count); cache.commit(it.request.rid, it.count); sched.advance(it)
+        sched.append_token(it.request, 7)
+    sched.add_request(req("p", 100, max_new=1))
+    items = sched.schedule()
+    assert [(it.request.rid, it.start, it.count, it.samples) for it in items] == [("d", 3, 1, True), ("p", 0, 24, False)]
+    # few pages: the portion grows only as far as the free pages allow (page size 8, 5 pages)
+    sched, cache = make(num_pages=5, fill_budget=True, max_num_batched_tokens=64, prefill_chunk_size=16)
+    sched.add_request(req("a", 39, max_new=1))
+    sched.add_request(req("b", 30, max_new=1))
+    items = sched.schedule()
+    got = [(it.request.rid, it.start, it.count) for it in items]
+    assert sum(-(-c // 8) for _, _, c in got) <= 5 and got[0][0] == "a" and got[0][2] >= 16
+    # under random traffic nothing is lost and every request still finishes
+    rng = random.Random(5)
+    sched, cache = make(num_pages=24, fill_budget=True, max_num_batched_tokens=48)
+    for i in range(12):
+        sched.add_request(req(f"r{i}", rng.randint(1, 90), max_new=rng.randint(1, 6)))
+    steps = run(sched, cache)
+    assert all(sum(c for _, _, c, _ in st) <= 48 for st in steps)
+    assert cache.free_pages() == [24]
