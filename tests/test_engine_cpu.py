@@ -129,13 +129,16 @@ def test_step_rejects_bad_batches(tiny_dirs):
     runner.cache.check()
 
 
-def test_generate_and_preemption_on_host(tiny_dirs):
+@pytest.mark.parametrize("fill_budget", [True, False])
+def test_generate_and_preemption_on_host(tiny_dirs, fill_budget):
+    """(with and without prompt portions that take up the budget nobody else uses)"""
     from tempura_amd.engine import Engine
     from tempura_amd.sampling import SamplingParams
     cfg, W = tiny_dirs.plain_model("A")
     prompts = [helpers.random_tokens(256, n, seed=700 + n) for n in (5, 17, 33, 26)]
     params = SamplingParams(temperature=0.0, max_new_tokens=12)
-    kw = dict(dtype="float32", device="cpu", page_size=16, max_batch_size=4, max_num_batched_tokens=24, prefill_chunk_size=16)
+    kw = dict(dtype="float32", device="cpu", page_size=16, max_batch_size=4, max_num_batched_tokens=24, prefill_chunk_size=16,
+              fill_budget=fill_budget)
     want = [plain.greedy_generate(cfg, W, p, 12) for p in prompts]
     roomy = Engine(tiny_dirs.path("A"), kv_pages=32, **kw)
     assert roomy.generate(prompts, params) == want
