@@ -1414,8 +1414,8 @@ int tp_linear_pipe(const bf16_t* x, const bf16_t* w, int w_tiled, void* out, int
   const int MB = (M + BM - 1) / BM, NB = (N + BN - 1) / BN;
   // Steps of 65 to a few hundred rows, with at most one round of 256 x 128 blocks: blocks of 128 x 128 where they
   // are cheaper (more of them, so more CUs at work and K in fewer parts).
-  bool mid = g_pipe_mid == 1;
-  if (g_pipe_mid == 0 && M > 64 && (long)MB * NB <= 256) {
+  bool mid = g_pipe_mid == 1 || (g_pipe_mid == 0 && M <= 128);   // (one row block either way, of half the height)
+  if (g_pipe_mid == 0 && M > 128 && (long)MB * NB <= 256) {
     const int KT = K / BK;
     const bool can_split = scratch != nullptr && rope == nullptr;
     const long tiles = (long)MB * NB, tiles128 = (long)((M + BM128 - 1) / BM128) * ((N + BN128 - 1) / BN128);
