@@ -229,6 +229,64 @@ __device__ inline unsigned int select_key(float v, float maxv, float mean_d) {
 // its number, and the copies are summed when the pass is over (8 copies, a row of 128,256 logits, timed from the host: top-k 50
 // 182 -> 143 us, top-p 0.9 256 -> 199 us, typical-p 623 -> 465 us).
 #define SMP_CAND 4096
+// f(value) for every element of x[0, n), the block's threads striding over it.  Sixteen loads of a thread are in
+// flight at a time: one CU walks a row of 128,256 floats, and with four in flight each walk was a chain of 31 trips
+// to memory per thread (about 25 us; a row's top-k sampling has four such walks).  For sums and counts that do not
+// depend on the order.
+template <typename F>
+__device__ inline void walk_row(const float* __restrict__ x, int n, F f) {
+  const int bd = blockDim.x;
+  int j = threadIdx.x;
+  for (; j + 15 * bd < n; j += 16 * bd) {
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = x[j + u * bd];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) f(v[u]);
+  }
+  for (; j + 3 * bd < n; j += 4 * bd) {
+    const float v0 = x[j], v1 = x[j + bd], v2 = x[j + 2 * bd], v3 = x[j + 3 * bd];
+    f(v0);
+    f(v1);
+    f(v2);
+    f(v3);
+  }
+  for (; j < n; j += bd) f(x[j]);
+}
+
+// One wave looks, in index order over x[lo, hi), for the first element of positive mass whose running mass (from c on)
+// exceeds t; every lane returns its index, or -1.  Sixteen groups of 64 elements are loaded before the first is looked
+// at (one group at a time, each load waited for, took 60 us for a wave's 8,016 elements), and a group without mass is
+// passed over without the prefix sum.
+template <typename M>
+__device__ inline int wave_find(const float* __restrict__ x, int lo, int hi, unsigned long long c, unsigned long long t,
+                                M mass_of, int lane) {
+  for (int j0 = lo; j0 < hi; j0 += 16 * TP_WAVE) {
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int j = j0 + u * TP_WAVE + lane;
+      v[u] = j < hi ? x[j] : -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int j = j0 + u * TP_WAVE + lane;
+      const unsigned long long q = j < hi ? mass_of(v[u]) : 0ull;
+      if (__builtin_amdgcn_ballot_w64(q > 0) == 0) continue;
+      unsigned long long inc = q;
+#pragma unroll
+      for (int o = 1; o < TP_WAVE; o <<= 1) {
+        const unsigned long long up = __shfl_up(inc, o, TP_WAVE);
+        if (lane >= o) inc += up;
+      }
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(q > 0 && c + inc > t);
+      if (hit != 0) return j0 + u * TP_WAVE + (int)__builtin_ctzll(hit);   // (the first such lane: index order)
+      c += __shfl(inc, TP_WAVE - 1, TP_WAVE);
+    }
+  }
+  return -1;
+}
+
 #define SMP_REP 8
 template <bool MASS, bool TYP = false>
 __device__ unsigned int radix_select(const float* __restrict__ x, int n, float maxv, unsigned int floor_key,
@@ -257,17 +315,8 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
     };
     if (n_cand >= 0) {
       for (int j = threadIdx.x; j < n_cand; j += blockDim.x) take(cand[j]);
-    } else {   // four loads in flight per thread (counts and fixed-point masses do not depend on the order)
-      const int bd = blockDim.x;
-      int j = threadIdx.x;
-      for (; j + 3 * bd < n; j += 4 * bd) {
-        const float v0 = x[j], v1 = x[j + bd], v2 = x[j + 2 * bd], v3 = x[j + 3 * bd];
-        take(v0);
-        take(v1);
-        take(v2);
-        take(v3);
-      }
-      for (; j < n; j += bd) take(x[j]);
+    } else {   // (counts and fixed-point masses do not depend on the order)
+      walk_row(x, n, take);
     }
     __syncthreads();
     for (int b = threadIdx.x; b < 256; b += blockDim.x) {   // a bin's copies into its first (integers: any order)
@@ -282,18 +331,48 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
       cnt[b * SMP_REP] = cs;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      unsigned long long run = gt;
-      int b = 255;
-      for (; b > 0; --b) {
-        const unsigned long long w = MASS ? hist[b * SMP_REP] : (unsigned long long)cnt[b * SMP_REP];
-        if (run + w >= target) break;
-        run += w;
+    // The bin that holds the target, from the top: the first b in 255 .. 1 with weight(bins above b) + weight(b) >=
+    // target, else bin 0.  One wave, four bins a lane, a prefix sum over the lanes (one thread walking the bins took
+    // 3 to 6 us a pass).
+    if (threadIdx.x < TP_WAVE) {
+      const int lane = threadIdx.x;
+      unsigned long long w[4], local = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int b = 255 - (4 * lane + i);
+        w[i] = MASS ? hist[b * SMP_REP] : (unsigned long long)cnt[b * SMP_REP];
+        local += w[i];
       }
-      sh[0] = run;
-      sh[1] = (unsigned long long)b;
-      sh[2] = (unsigned long long)cnt[b * SMP_REP];
-      sh[3] = 0;            // (the candidates' counter)
+      unsigned long long inc = local;
+#pragma unroll
+      for (int o = 1; o < TP_WAVE; o <<= 1) {
+        const unsigned long long up = __shfl_up(inc, o, TP_WAVE);
+        if (lane >= o) inc += up;
+      }
+      unsigned long long run = gt + inc - local;   // the weight above this lane's first bin
+      int found = -1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int b = 255 - (4 * lane + i);
+        if (found < 0 && b > 0) {
+          if (run + w[i] >= target) found = b;
+          else run += w[i];
+        }
+      }
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(found >= 0);
+      if (hit != 0) {
+        if (lane == (int)__builtin_ctzll(hit)) {
+          sh[0] = run;
+          sh[1] = (unsigned long long)found;
+          sh[2] = (unsigned long long)cnt[found * SMP_REP];
+          sh[3] = 0;            // (the candidates' counter)
+        }
+      } else if (lane == TP_WAVE - 1) {   // bin 0: everything above it is in `run` (the lane's last bin is bin 0)
+        sh[0] = run;
+        sh[1] = 0;
+        sh[2] = (unsigned long long)cnt[0];
+        sh[3] = 0;
+      }
     }
     __syncthreads();
     gt = sh[0];
@@ -307,16 +386,7 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
         const unsigned long long at = atomicAdd(&sh[3], 1ull);
         if (at < (unsigned long long)SMP_CAND) cand[at] = v;
       };
-      const int bd = blockDim.x;
-      int j = threadIdx.x;
-      for (; j + 3 * bd < n; j += 4 * bd) {
-        const float v0 = x[j], v1 = x[j + bd], v2 = x[j + 2 * bd], v3 = x[j + 3 * bd];
-        gather(v0);
-        gather(v1);
-        gather(v2);
-        gather(v3);
-      }
-      for (; j < n; j += bd) gather(x[j]);
+      walk_row(x, n, gather);
       __syncthreads();
       n_cand = (int)sh[3];   // (== sh[2], the bin's count)
     }
@@ -568,26 +638,9 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
       const int lane = threadIdx.x;
       const int per = (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS;
       const int lo = min(vocab, piece * per), hi = min(vocab, lo + per);
-      for (int j0 = lo; j0 < hi; j0 += TP_WAVE) {
-        const int j = j0 + lane;
-        unsigned long long q = 0;
-        if (j < hi) {
-          const float v = x[j];
-          if (float_key(v) >= floor_key) q = fix_mass(v, maxv);
-        }
-        unsigned long long inc = q;
-#pragma unroll
-        for (int o = 1; o < TP_WAVE; o <<= 1) {
-          const unsigned long long up = __shfl_up(inc, o, TP_WAVE);
-          if (lane >= o) inc += up;
-        }
-        const unsigned long long hit = __builtin_amdgcn_ballot_w64(q > 0 && c + inc > t);
-        if (hit != 0) {
-          if (lane == (int)__builtin_ctzll(hit)) out[row] = j;
-          return;
-        }
-        c += __shfl(inc, TP_WAVE - 1, TP_WAVE);
-      }
+      const int at = wave_find(x, lo, hi, c, t,
+                               [&](float v) { return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull; }, lane);
+      if (at >= 0 && lane == 0) out[row] = at;
       return;
     }
   }
@@ -632,14 +685,9 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   const bool need_mass_now = (tp < 1.0f && tp > 0.f) || inf != nullptr || greedy;
   unsigned long long part = 0;
   if (need_mass_now) {
-    auto mass = [&](float v) { return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull; };
-    const int bd = blockDim.x;
-    int j = threadIdx.x;
-    for (; j + 3 * bd < vocab; j += 4 * bd) {   // four loads in flight per thread; integer sums, any order
-      const float v0 = x[j], v1 = x[j + bd], v2 = x[j + 2 * bd], v3 = x[j + 3 * bd];
-      part += mass(v0) + mass(v1) + mass(v2) + mass(v3);
-    }
-    for (; j < vocab; j += bd) part += mass(x[j]);
+    walk_row(x, vocab, [&](float v) {   // (integer sums, any order)
+      if (float_key(v) >= floor_key) part += fix_mass(v, maxv);
+    });
   }
   unsigned long long Z = 0;
   if (need_mass_now) block_excl_scan(part, scan, &Z);
@@ -694,8 +742,18 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull;
   };
   unsigned long long mine = 0;
-  for (int j = wlo + lane; j < whi; j += 4 * TP_WAVE)
-    mine += mass(j) + mass(j + TP_WAVE) + mass(j + 2 * TP_WAVE) + mass(j + 3 * TP_WAVE);
+  {
+    int j = wlo + lane;
+    for (; j + 15 * TP_WAVE < whi; j += 16 * TP_WAVE) {   // sixteen loads in flight (see walk_row)
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = x[j + u * TP_WAVE];
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        if (float_key(v[u]) >= floor_key) mine += fix_mass(v[u], maxv);
+    }
+    for (; j < whi; j += TP_WAVE) mine += mass(j);
+  }
 #pragma unroll
   for (int o = TP_WAVE / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, TP_WAVE);
   __syncthreads();
@@ -722,24 +780,11 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     before += w;
   }
   if (wave == chosen_wave) {
-    unsigned long long c = base;
-    for (int j0 = wlo; j0 < whi; j0 += TP_WAVE) {
-      const unsigned long long q = mass(j0 + lane);
-      unsigned long long inc = q;
-#pragma unroll
-      for (int o = 1; o < TP_WAVE; o <<= 1) {
-        const unsigned long long up = __shfl_up(inc, o, TP_WAVE);
-        if (lane >= o) inc += up;
-      }
-      const unsigned long long hit = __builtin_amdgcn_ballot_w64(q > 0 && c + inc > t);
-      if (hit != 0) {   // (the first lane whose running mass passes the target: index order)
-        if (lane == (int)__builtin_ctzll(hit)) {
-          out[row] = j0 + lane;
-          if (inf != nullptr) inf[3] = (x[j0 + lane] - maxv) - lnZ;
-        }
-        break;
-      }
-      c += __shfl(inc, TP_WAVE - 1, TP_WAVE);
+    const int at = wave_find(x, wlo, whi, base, t,
+                             [&](float v) { return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull; }, lane);
+    if (at >= 0 && lane == 0) {
+      out[row] = at;
+      if (inf != nullptr) inf[3] = (x[at] - maxv) - lnZ;
     }
   }
 }
