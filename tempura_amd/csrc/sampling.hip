@@ -288,11 +288,15 @@ __device__ inline int wave_find(const float* __restrict__ x, int lo, int hi, uns
 }
 
 #define SMP_REP 8
+#define SMP_CHUNKS 32     // pieces of a row that the kernels of many blocks work on
 template <bool MASS, bool TYP = false>
 __device__ unsigned int radix_select(const float* __restrict__ x, int n, float maxv, unsigned int floor_key,
                                      unsigned long long target, unsigned long long* hist /*256 * SMP_REP*/,
                                      unsigned int* cnt /*256 * SMP_REP*/, unsigned long long* sh /*4*/, float* cand /*SMP_CAND*/,
-                                     unsigned long long* gt_out, unsigned int* eq_count, float mean_d = 0.f) {
+                                     unsigned long long* gt_out, unsigned int* eq_count, float mean_d = 0.f,
+                                     const unsigned int* __restrict__ pre_cnt = nullptr) {
+  // pre_cnt (counting only, every finite element takes part): the first pass's counts by bin, SMP_CHUNKS pieces of
+  // the row side by side [SMP_CHUNKS, 256], counted by the kernel of many blocks that scaled the row
   unsigned int prefix = 0;
   unsigned long long gt = 0;
   int n_cand = -1;          // >= 0: the passes run over cand[0 .. n_cand)
@@ -304,6 +308,14 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
       cnt[i] = 0;
     }
     __syncthreads();
+    const bool counted = !MASS && !TYP && pass == 0 && pre_cnt != nullptr;
+    if (counted) {
+      for (int b = threadIdx.x; b < 256; b += blockDim.x) {
+        unsigned int cs = 0;
+        for (int c = 0; c < SMP_CHUNKS; ++c) cs += pre_cnt[c * 256 + b];
+        cnt[b * SMP_REP] = cs;
+      }
+    }
     const unsigned int copy = threadIdx.x % SMP_REP;
     auto take = [&](float v) {
       if (float_key(v) < floor_key) return;
@@ -313,13 +325,15 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
       atomicAdd(&cnt[slot], 1u);
       if (MASS) atomicAdd(&hist[slot], fix_mass(v, maxv));   // (counting: the weight of a bin is its count)
     };
-    if (n_cand >= 0) {
+    if (counted) {
+      // (nothing to walk)
+    } else if (n_cand >= 0) {
       for (int j = threadIdx.x; j < n_cand; j += blockDim.x) take(cand[j]);
     } else {   // (counts and fixed-point masses do not depend on the order)
       walk_row(x, n, take);
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < 256; b += blockDim.x) {   // a bin's copies into its first (integers: any order)
+    for (int b = threadIdx.x; b < 256 && !counted; b += blockDim.x) {   // a bin's copies into its first (integers: any order)
       unsigned long long hs = 0;
       unsigned int cs = 0;
 #pragma unroll
@@ -446,12 +460,22 @@ __device__ void typical_cut(float* __restrict__ x, int n, float maxv, unsigned i
 
 // Step 1 of sample_kernel for a whole row on many CUs: x = logit / temperature (NaN -> -inf), written to `work`,
 // and the maximum of each of SMP_CHUNKS pieces of the row to part_max[row, piece].  grid: (rows, SMP_CHUNKS).
-#define SMP_CHUNKS 32
 __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restrict__ logits, float* __restrict__ work,
                                                            int vocab, const float* __restrict__ temperature,
-                                                           float* __restrict__ part_max) {
+                                                           float* __restrict__ part_max,
+                                                           unsigned int* __restrict__ part_cnt) {
+  // part_cnt (may be null): how many finite elements of the piece fall into each of the 256 bins of radix_select's
+  // first pass, [rows, SMP_CHUNKS, 256]
   __shared__ float fscratch[32];
+  __shared__ unsigned int bins[256 * 4];
   const int row = blockIdx.x, chunk = blockIdx.y;
+  if (part_cnt != nullptr) {
+    for (int i = threadIdx.x; i < 256 * 4; i += blockDim.x) bins[i] = 0;
+    __syncthreads();
+  }
+  auto count = [&](float v) {
+    if (part_cnt != nullptr && v > -INFINITY) atomicAdd(&bins[(float_key(v) >> 24) * 4 + (threadIdx.x & 3)], 1u);
+  };
   const float* lg = logits + (size_t)row * vocab;
   float* x = work + (size_t)row * vocab;
   const float T = temperature[row] > 0.f ? temperature[row] : 1.0f;
@@ -472,14 +496,24 @@ __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restri
     x[j + 2 * bd] = v2;
     x[j + 3 * bd] = v3;
     mx = fmaxf(fmaxf(mx, v0), fmaxf(v1, fmaxf(v2, v3)));
+    count(v0);
+    count(v1);
+    count(v2);
+    count(v3);
   }
   for (; j < hi; j += bd) {
     const float v = scale(lg[j]);
     x[j] = v;
     mx = fmaxf(mx, v);
+    count(v);
   }
   mx = block_max(mx, fscratch);
   if (threadIdx.x == 0) part_max[row * SMP_CHUNKS + chunk] = mx;
+  if (part_cnt != nullptr) {
+    __syncthreads();
+    for (int b = threadIdx.x; b < 256; b += blockDim.x)
+      part_cnt[((size_t)row * SMP_CHUNKS + chunk) * 256 + b] = bins[b * 4] + bins[b * 4 + 1] + bins[b * 4 + 2] + bins[b * 4 + 3];
+  }
 }
 
 // For rows that are only scaled (and perhaps cut by min_p) before the draw: the fixed-point mass of each of the
@@ -521,7 +555,8 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int vocab, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
     const float* __restrict__ typical_p, const float* __restrict__ rnd, int* __restrict__ out,
-    float* __restrict__ info, const float* __restrict__ part_max, const unsigned long long* __restrict__ part_mass) {
+    float* __restrict__ info, const float* __restrict__ part_max, const unsigned long long* __restrict__ part_mass,
+    const unsigned int* __restrict__ part_cnt) {
   __shared__ unsigned long long hist[256 * SMP_REP];
   __shared__ unsigned int cnt[256 * SMP_REP];
   __shared__ unsigned long long sh[4];
@@ -673,7 +708,10 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   if (k > 0 && k < vocab) {
     unsigned long long gt;
     unsigned int eq;
-    const unsigned int K = radix_select<false>(x, vocab, maxv, floor_key, (unsigned long long)k, hist, cnt, sh, cand, &gt, &eq);
+    // (the first pass is counted already when nothing has been cut from the row so far)
+    const bool whole = part_cnt != nullptr && part_max != nullptr && !(mp > 0.f) && !(typ < 1.0f);
+    const unsigned int K = radix_select<false>(x, vocab, maxv, floor_key, (unsigned long long)k, hist, cnt, sh, cand, &gt, &eq,
+                                               0.f, whole ? part_cnt + (size_t)row * SMP_CHUNKS * 256 : nullptr);
     // fewer than k survivors: K lands on the smallest surviving bin and nothing is cut
     if (gt + eq > (unsigned long long)k) drop_surplus_ties(x, vocab, K, (unsigned long long)k - gt, scan);
     if (K > floor_key) floor_key = K;
@@ -855,22 +893,23 @@ __global__ __launch_bounds__(SMP_THREADS) void top_logprobs_kernel(const float* 
 extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p, const float* typical_p,
                          const float* rnd, int* out, float* info, float* part_max, unsigned long long* part_mass,
-                         hipStream_t s) {
+                         unsigned int* part_cnt, hipStream_t s) {
   // part_max: scratch of rows * 32 floats, or null (the row's first step then runs inside the one block per row);
-  // part_mass: scratch of rows * 32 64-bit integers, given when some row is only scaled before the draw
+  // part_mass: scratch of rows * 32 64-bit integers, given when some row is only scaled before the draw;
+  // part_cnt: scratch of rows * 32 * 256 32-bit integers, given when some row is cut by top_k
   TP_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes");
   if (rows == 0) return 0;
   if (part_max != nullptr && vocab >= 4096 && rows <= 65535)
     hipLaunchKernelGGL(sample_scale_kernel, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, logits, work, vocab, temperature,
-                       part_max);
+                       part_max, part_cnt);
   else
-    part_max = nullptr;
+    part_max = nullptr, part_cnt = nullptr;
   if (part_max != nullptr && part_mass != nullptr && info == nullptr)
     hipLaunchKernelGGL(sample_mass_kernel, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, work, vocab, min_p, part_max, part_mass);
   else
     part_mass = nullptr;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, work, vocab, temperature, top_k,
-                     top_p, min_p, typical_p, rnd, out, info, part_max, part_mass);
+                     top_p, min_p, typical_p, rnd, out, info, part_max, part_mass, part_cnt);
   TP_CHECK_LAUNCH("sample");
   return 0;
 }

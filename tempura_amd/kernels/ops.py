@@ -790,11 +790,14 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
     plain_rows = any(t > 0 and not (0 < k < vocab) and not (0.0 < p < 1.0) and not (ty < 1.0)
                      for t, k, p, ty in zip(temperature, top_k, top_p, typical_p))
     part_mass = torch.empty((m * 32,), dtype=torch.int64, device=dev) if plain_rows and info is None else None
+    # rows cut by top_k have the first pass of their selection counted by the kernel of many blocks that scales the row
+    topk_rows = any(t > 0 and 0 < k < vocab for t, k in zip(temperature, top_k))
+    part_cnt = torch.empty((m * 32 * 256,), dtype=torch.int32, device=dev) if topk_rows else None
     if info is not None:
         _dev_ok(info)
         _need(info.dtype == torch.float32 and info.is_contiguous() and tuple(info.shape) == (m, 4), "sample: info must be float32 [m, 4]")
     _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
-          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _ptr(part_max), _ptr(part_mass), _stream())
+          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _ptr(part_max), _ptr(part_mass), _ptr(part_cnt), _stream())
     return out
 
 
