@@ -72,7 +72,7 @@ def _sample(logits, temperature, top_k, top_p, min_p, r, typical_p=1.0):
     return ops.sample(logits.to(DEV), work, full(temperature), full(top_k), full(top_p), full(min_p), full(r), full(typical_p)).tolist()
 
 
-@pytest.mark.parametrize("vocab", [16, 301, 4099])
+@pytest.mark.parametrize("vocab", [16, 301, 4099, 50021])    # (the largest: whole rounds of sixteen loads and their rests)
 @pytest.mark.parametrize("temperature,top_k,top_p,min_p", [(1.0, 0, 1.0, 0.0), (0.8, 0, 1.0, 0.0), (1.0, 5, 1.0, 0.0), (0.7, 50, 0.9, 0.0),
                                                             (1.3, 0, 0.5, 0.0), (1.0, 0, 1.0, 0.1), (0.9, 40, 0.95, 0.05), (0.0, 50, 0.9, 0.0)])
 def test_sample_matches_plain_rules(vocab, temperature, top_k, top_p, min_p):
