@@ -129,6 +129,13 @@ def build(verbose: bool = True) -> str:
                 f.result()
         tmp = os.path.join(out_dir, name + f".{tag}.tmp")
         _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp], "linking")
+        # A kernel whose host stub was not emitted links all the same and fails when the library is loaded: load it
+        # here (in a process of its own; loading needs no GPU), so that a build says so and not the first user.
+        check = subprocess.run([sys.executable, "-c", "import ctypes, sys; ctypes.CDLL(sys.argv[1])", tmp],
+                               capture_output=True, text=True)
+        if check.returncode != 0:
+            os.remove(tmp)
+            raise RuntimeError("the kernel library was linked but does not load:\n" + check.stderr.strip()[-2000:])
         final = os.path.join(out_dir, name)
         os.replace(tmp, final)
     finally:

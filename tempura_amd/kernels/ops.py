@@ -474,7 +474,7 @@ def linear_rope_ok(m: int, n: int, k: int, head_dim: int, rotary_dim: int, page_
     if 0 < m <= 16:
         return k % 32 == 0 and head_dim % 16 == 0
     tiles = -(-m // 128) * -(-n // 128)      # (of 128 x 128, the smallest blocks of the pipelined products)
-    return (rope_in_long_products and m > 128 and tiles >= 128 and k % 64 == 0 and 255 * k * 2 + 128 < 2 ** 32 and head_dim % 64 == 0
+    return (rope_in_long_products and m > 128 and tiles >= 128 and k % 64 == 0 and 255 * k * 2 + 128 < 2 ** 31 and head_dim % 64 == 0
             and rotary_dim % 8 == 0 and page_size % 8 == 0 and not prenormed)
 
 
