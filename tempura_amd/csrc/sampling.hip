@@ -391,12 +391,14 @@ __device__ unsigned int radix_select(const float* __restrict__ x, int n, float m
     __syncthreads();
     gt = sh[0];
     prefix = (prefix << 8) | (unsigned int)sh[1];
-    if (pass == 0 && sh[2] <= (unsigned long long)SMP_CAND) {
-      // gather the chosen bin's elements (their order does not matter: counts and integer masses)
+    if (n_cand < 0 && pass < 3 && sh[2] <= (unsigned long long)SMP_CAND) {
+      // gather the chosen bin's elements (their order does not matter: counts and integer masses): after the first
+      // pass, or after the first one whose bin is small enough (logits that are nearly equal, as a model of random
+      // weights gives them, share their first byte)
       const unsigned int want = prefix;
       auto gather = [&](float v) {
         if (float_key(v) < floor_key) return;
-        if ((select_key<TYP>(v, maxv, mean_d) >> 24) != want) return;
+        if ((select_key<TYP>(v, maxv, mean_d) >> shift) != want) return;
         const unsigned long long at = atomicAdd(&sh[3], 1ull);
         if (at < (unsigned long long)SMP_CAND) cand[at] = v;
       };
