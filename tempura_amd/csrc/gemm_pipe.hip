@@ -1341,7 +1341,10 @@ int g_pipe_mid = 0;   // tuning: 1 = 128 x 128 blocks for every product of more 
 constexpr double STEP128_US = 0.52, STEP256_US = 0.75;
 static double pipe_cost(long blocks, int steps, double step_us, int splits, int M, int N) {
   const double rounds = (double)((blocks + 255) / 256);
-  return rounds * steps * step_us + (splits > 1 ? 3.0 + (splits + 2.0) * M * N * 4.0 / 3e6 : 0.0);
+  // (rows counted in whole blocks of 128: a step of 100 rows and the same step padded to 128 rows for a captured
+  // graph then cut K alike and give the same bits)
+  const double rows = (double)((M + 127) / 128 * 128);
+  return rounds * steps * step_us + (splits > 1 ? 3.0 + (splits + 2.0) * rows * N * 4.0 / 3e6 : 0.0);
 }
 
 // Into how many parts K (KT steps) is cut for `tiles` result tiles: the cheapest by pipe_cost among whole parts

@@ -501,3 +501,30 @@ def test_model_sized_layers_bfloat16_against_float32():
     for r in prompts:
         err = helpers.rel_err(logits["bfloat16"][r], logits["float32"][r].double())
         assert err <= helpers.TOL["bfloat16"], f"request {r}: bfloat16 differs from float32 by {err:.3e}"
+
+
+def test_a_captured_step_padded_to_more_rows_gives_the_bits_of_the_eager_step():
+    """Decode steps replay graphs captured for a power of two of rows; 75 requests run as 128 rows there and as 75
+    rows without graphs.  The products choose their tiles and the parts of K by the rows counted in whole blocks, so
+    that both give the same bits (two layers of the width of Llama-3.2-3B: with random weights the logits lie close
+    together, and a different order of additions moves tokens at once)."""
+    import random
+    from tempura_amd.config import PRESETS, LlamaConfig
+    from tempura_amd.engine import Engine
+    from tempura_amd.kernels import ops
+    from tempura_amd.sampling import SamplingParams
+    ops.set_backend(None)
+    cfg = LlamaConfig.from_dict(PRESETS["llama-3.2-3b"].to_dict())
+    cfg.num_hidden_layers = 2
+    cfg.vocab_size = 8192
+    cfg.validate()
+    g = random.Random(3)
+    prompts = [[g.randrange(cfg.vocab_size) for _ in range(g.choice([40, 64, 90]))] for _ in range(75)]
+    outs = {}
+    for graph in (True, False):
+        eng = Engine(cfg, random_weights=True, seed=11, max_batch_size=128, max_seq_len=256, kv_pages=800, use_graph=graph)
+        outs[graph] = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=8, ignore_eos=True))
+        assert (eng.stats()["graph_steps"] > 0) == graph
+        del eng
+        torch.cuda.empty_cache()
+    assert outs[True] == outs[False]
