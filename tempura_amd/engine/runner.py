@@ -318,9 +318,13 @@ class ModelRunner:
 
     # ---- decode steps as a graph -----------------------------------------
     def _graph_for(self, rows: int, ctx_len: int) -> Optional[_DecodeGraph]:
+        # rows padded to a power of two, beyond 128 to a multiple of 128: the products see as many blocks of rows as
+        # in the unpadded step and so choose the same tiles and parts of K (the same bits as an eager step)
         bucket = 1
-        while bucket < rows:
+        while bucket < min(rows, 128):
             bucket *= 2
+        if rows > 128:
+            bucket = (rows + 127) // 128 * 128
         bound = 256
         while bound < ctx_len:
             bound *= 2
