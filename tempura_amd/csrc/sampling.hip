@@ -460,17 +460,121 @@ __device__ void typical_cut(float* __restrict__ x, int n, float maxv, unsigned i
   __syncthreads();
 }
 
+// ---- rows cut by a small top_k: selection on many CUs -------------------------------------------------------------
+// The k largest of a row all belong to the k largest of their piece of the row.  So each of the SMP_CHUNKS blocks that
+// scale a row also hands over the elements of its piece that are at least as large as the piece's k-th largest (value
+// and index; ties included), and one block per row then works on those few thousand candidates alone: the k-th
+// largest of them, ties at the cut in index order, min_p, top_p and the draw in index order, with the same fixed-point
+// masses as sample_kernel, whose result it reproduces bit for bit.  A row that does not qualify (no or a large
+// top_k, typical_p, a report of probabilities asked for, a piece with more than SMP_CCAP candidates, more than 256 ties
+// at the cut) is left to sample_kernel (`done` 0).
+#define SMP_KMAX 128        // largest top_k of this path
+#define SMP_CCAP 160        // candidates a piece may hand over
+#define SMP_PER_MAX 8192    // elements of a piece (vocabularies up to 262,144)
+
+__device__ inline bool topk_fast_row(float T, int k, int vocab, float typ) {
+  return T > 0.f && k > 0 && k <= SMP_KMAX && k < vocab && !(typ < 1.0f) &&
+         (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS <= SMP_PER_MAX;
+}
+
+__device__ inline float key_float(unsigned int key) {   // float_key's inverse
+  return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+// The target-th largest (counted from 1) of the keys that the threads of the block hold in registers, R each (0: no
+// element there): radix selection from the top with 256 counters, as radix_select does for counts.  *gt: how many keys
+// are larger, *eq: how many are equal.  With fewer than `target` keys the answer is 0 (nothing is cut).  Called by the
+// whole block.
+#define SMP_KBINS 256
+template <int R>
+__device__ inline unsigned int reg_kth_key(const unsigned int (&kreg)[R], unsigned int target, unsigned int* bins /*SMP_KBINS*/,
+                                           unsigned int* sh /*4*/, unsigned int* gt_out, unsigned int* eq_out) {
+  unsigned int prefix = 0, gt = 0;
+  for (int i = threadIdx.x; i < SMP_KBINS; i += blockDim.x) bins[i] = 0;
+  __syncthreads();
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const unsigned int key = kreg[u];
+      if (key != 0 && (pass == 0 || (key >> (shift + 8)) == prefix)) atomicAdd(&bins[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (threadIdx.x < TP_WAVE) {   // the first bin from the top with count(bins above) + count(bin) >= target, else bin 0
+      const int lane = threadIdx.x;
+      unsigned int w[4], local = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        w[i] = bins[255 - (4 * lane + i)];
+        bins[255 - (4 * lane + i)] = 0;   // (clear for the next pass)
+        local += w[i];
+      }
+      unsigned int inc = local;
+#pragma unroll
+      for (int o = 1; o < TP_WAVE; o <<= 1) {
+        const unsigned int up = __shfl_up(inc, o, TP_WAVE);
+        if (lane >= o) inc += up;
+      }
+      unsigned int run = gt + inc - local, wf = 0;
+      int found = -1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int b = 255 - (4 * lane + i);
+        if (found < 0 && b > 0) {
+          if (run + w[i] >= target) {
+            found = b;
+            wf = w[i];
+          } else {
+            run += w[i];
+          }
+        }
+      }
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(found >= 0);
+      if (hit != 0) {
+        if (lane == (int)__builtin_ctzll(hit)) {
+          sh[0] = run;
+          sh[1] = (unsigned int)found;
+          sh[2] = wf;
+        }
+      } else if (lane == TP_WAVE - 1) {
+        sh[0] = run;
+        sh[1] = 0;
+        sh[2] = w[3];   // (bin 0)
+      }
+    }
+    __syncthreads();   // (the next write to sh comes after the next pass's barrier)
+    gt = sh[0];
+    prefix = (prefix << 8) | sh[1];
+  }
+  *gt_out = gt;
+  *eq_out = sh[2];
+  return prefix;
+}
+
 // Step 1 of sample_kernel for a whole row on many CUs: x = logit / temperature (NaN -> -inf), written to `work`,
 // and the maximum of each of SMP_CHUNKS pieces of the row to part_max[row, piece].  grid: (rows, SMP_CHUNKS).
+template <int R>   // R * 256: the most elements of a piece whose row takes the way of a small top_k
 __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restrict__ logits, float* __restrict__ work,
                                                            int vocab, const float* __restrict__ temperature,
                                                            float* __restrict__ part_max,
-                                                           unsigned int* __restrict__ part_cnt) {
+                                                           unsigned int* __restrict__ part_cnt,
+                                                           const int* __restrict__ top_k, const float* __restrict__ typical_p,
+                                                           float* __restrict__ cand_val, int* __restrict__ cand_idx,
+                                                           int* __restrict__ cand_cnt) {
   // part_cnt (may be null): how many finite elements of the piece fall into each of the 256 bins of radix_select's
   // first pass, [rows, SMP_CHUNKS, 256]
+  // cand_* (may be null): the piece's candidates for a row cut by a small top_k (see topk_fast_row),
+  // [rows, SMP_CHUNKS, SMP_CCAP] and their number [rows, SMP_CHUNKS] (more than SMP_CCAP: too many, none usable)
   __shared__ float fscratch[32];
   __shared__ unsigned int bins[256 * 4];
+  __shared__ float xs[R * 256];
+  __shared__ unsigned int kbins[SMP_KBINS];
+  __shared__ unsigned int ksh[4];
+  __shared__ int n_out;
+  static_assert(R * 256 <= SMP_PER_MAX, "sample_topk_kernel takes rows of pieces up to SMP_PER_MAX");
   const int row = blockIdx.x, chunk = blockIdx.y;
+  const bool local_topk = cand_cnt != nullptr && topk_fast_row(temperature[row], top_k[row], vocab, typical_p[row]) &&
+                          (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS <= R * 256;
   if (part_cnt != nullptr) {
     for (int i = threadIdx.x; i < 256 * 4; i += blockDim.x) bins[i] = 0;
     __syncthreads();
@@ -502,15 +606,53 @@ __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restri
     count(v1);
     count(v2);
     count(v3);
+    if (local_topk) {
+      xs[j - lo] = v0;
+      xs[j + bd - lo] = v1;
+      xs[j + 2 * bd - lo] = v2;
+      xs[j + 3 * bd - lo] = v3;
+    }
   }
   for (; j < hi; j += bd) {
     const float v = scale(lg[j]);
     x[j] = v;
     mx = fmaxf(mx, v);
     count(v);
+    if (local_topk) xs[j - lo] = v;
   }
   mx = block_max(mx, fscratch);
   if (threadIdx.x == 0) part_max[row * SMP_CHUNKS + chunk] = mx;
+  if (local_topk) {   // (the same for every thread of the block; xs is whole after block_max's barriers)
+    const int np = hi - lo;
+    const unsigned int finite = float_key(-INFINITY) + 1u;
+    unsigned int kreg[R];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int i = threadIdx.x + u * 256;
+      kreg[u] = 0;
+      if (i < np) {
+        const unsigned int key = float_key(xs[i]);
+        if (key >= finite) kreg[u] = key;
+      }
+    }
+    if (threadIdx.x == 0) n_out = 0;
+    unsigned int gt, eq;
+    unsigned int K = reg_kth_key(kreg, (unsigned int)top_k[row], kbins, ksh, &gt, &eq);   // (barriers: n_out is set)
+    if (K < finite) K = finite;
+    const size_t base = ((size_t)row * SMP_CHUNKS + chunk) * SMP_CCAP;
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      if (kreg[u] >= K) {
+        const int at = atomicAdd(&n_out, 1);
+        if (at < SMP_CCAP) {
+          cand_val[base + at] = key_float(kreg[u]);
+          cand_idx[base + at] = lo + threadIdx.x + u * 256;
+        }
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) cand_cnt[row * SMP_CHUNKS + chunk] = n_out;
+  }
   if (part_cnt != nullptr) {
     __syncthreads();
     for (int b = threadIdx.x; b < 256; b += blockDim.x)
@@ -553,12 +695,165 @@ __global__ __launch_bounds__(256) void sample_mass_kernel(const float* __restric
   if (threadIdx.x == 0) part_mass[row * SMP_CHUNKS + chunk] = wsum[0] + wsum[1] + wsum[2] + wsum[3];
 }
 
+// The candidates of a row cut by a small top_k (see above) -> its token.  grid: rows; done[row] = 1 when the row is
+// settled here, 0 when sample_kernel has to do it.
+#define SMP_TOPK_R (SMP_CHUNKS * SMP_CCAP / 256)
+__global__ __launch_bounds__(256) void sample_topk_kernel(const float* __restrict__ cand_val, const int* __restrict__ cand_idx,
+                                                          const int* __restrict__ cand_cnt, const float* __restrict__ part_max,
+                                                          int vocab, const float* __restrict__ temperature,
+                                                          const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                          const float* __restrict__ min_p, const float* __restrict__ typical_p,
+                                                          const float* __restrict__ rnd, int* __restrict__ out,
+                                                          int* __restrict__ done) {
+  static_assert(SMP_CHUNKS * SMP_CCAP % 256 == 0, "the candidates are spread evenly over the threads");
+  __shared__ int cnts[SMP_CHUNKS];
+  __shared__ unsigned int bins[SMP_KBINS];
+  __shared__ unsigned int sh[4];
+  __shared__ int tl[256];                          // indices of the ties at the cut
+  __shared__ unsigned long long sord[SMP_KMAX];    // survivors: key and index as one number that orders them
+  __shared__ int si[SMP_KMAX];
+  __shared__ unsigned long long sq[SMP_KMAX];      // ... and their masses (0: dropped)
+  __shared__ int s_n, n_tie, s_over;
+  __shared__ float s_max;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  if (tid == 0) done[row] = 0;
+  const int k = top_k[row];
+  if (!topk_fast_row(temperature[row], k, vocab, typical_p[row])) return;
+  if (tid < TP_WAVE) {   // how many candidates each piece brings, and the row's maximum
+    const int c = tid < SMP_CHUNKS ? cand_cnt[row * SMP_CHUNKS + tid] : 0;
+    float mx = tid < SMP_CHUNKS ? part_max[row * SMP_CHUNKS + tid] : -INFINITY;
+    const bool over = __builtin_amdgcn_ballot_w64(c > SMP_CCAP) != 0;
+#pragma unroll
+    for (int o = TP_WAVE / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, TP_WAVE));
+    if (tid < SMP_CHUNKS) cnts[tid] = c;
+    if (tid == 0) {
+      s_n = 0;
+      n_tie = 0;
+      s_over = over;
+      s_max = mx;
+    }
+  }
+  __syncthreads();
+  if (s_over) return;   // some piece had more candidates than it could hand over
+  const float maxv = s_max;
+  if (maxv == -INFINITY) {   // nothing to choose from: the last index, as sample_kernel answers
+    if (tid == 0) {
+      out[row] = vocab - 1;
+      done[row] = 1;
+    }
+    return;
+  }
+  unsigned int floor_key = float_key(-INFINITY) + 1u;
+  const float mp = min_p[row];
+  if (mp > 0.f) {
+    const unsigned int k2 = float_key(maxv + logf(mp));
+    if (k2 > floor_key) floor_key = k2;
+  }
+  // every thread takes its share of the candidates' slots into registers (a slot beyond its piece's count: no element)
+  unsigned int kreg[SMP_TOPK_R];
+  int ireg[SMP_TOPK_R];
+  {
+    const size_t base = (size_t)row * SMP_CHUNKS * SMP_CCAP;
+    float v[SMP_TOPK_R];
+#pragma unroll
+    for (int u = 0; u < SMP_TOPK_R; ++u) {
+      v[u] = cand_val[base + tid + u * 256];
+      ireg[u] = cand_idx[base + tid + u * 256];
+    }
+#pragma unroll
+    for (int u = 0; u < SMP_TOPK_R; ++u) {
+      const int e = tid + u * 256, p = e / SMP_CCAP, i = e - p * SMP_CCAP;
+      const unsigned int key = float_key(v[u]);
+      kreg[u] = (i < cnts[p] && key >= floor_key) ? key : 0u;
+    }
+  }
+  unsigned int gt, eq;
+  const unsigned int K = reg_kth_key(kreg, (unsigned int)k, bins, sh, &gt, &eq);
+  // ties at the cut are admitted in index order, as many as k still allows
+  const bool cut_ties = gt + eq > (unsigned int)k;
+  const unsigned int quota = cut_ties ? (unsigned int)k - gt : eq;
+  if (cut_ties && eq > 256u) return;
+  auto keep = [&](unsigned int key, int idx) {
+    const int at = atomicAdd(&s_n, 1);
+    if (at < SMP_KMAX) {   // (at most k by construction)
+      sord[at] = ((unsigned long long)key << 32) | (unsigned long long)(0xffffffffu - (unsigned int)idx);
+      si[at] = idx;
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < SMP_TOPK_R; ++u) {
+    const unsigned int key = kreg[u];
+    if (key == 0 || key < K) continue;
+    if (key > K || !cut_ties) {
+      keep(key, ireg[u]);
+    } else {
+      const int at = atomicAdd(&n_tie, 1);
+      if (at < 256) tl[at] = ireg[u];
+    }
+  }
+  __syncthreads();
+  if (cut_ties) {
+    if (tid < (int)eq) {
+      const int mine = tl[tid];
+      unsigned int rank = 0;
+      for (int j = 0; j < (int)eq; ++j) rank += tl[j] < mine;
+      if (rank < quota) keep(K, mine);
+    }
+    __syncthreads();
+  }
+  const int S = min(s_n, SMP_KMAX);
+  if (tid < SMP_KMAX) sq[tid] = tid < S ? fix_mass(key_float((unsigned int)(sord[tid] >> 32)), maxv) : 0ull;
+  __syncthreads();
+  // top_p: the survivors in descending order (ties by index) while the mass before one is short of the target
+  const float tp = top_p[row];
+  if (tp < 1.0f && tp > 0.f) {
+    unsigned long long Z = 0;
+#pragma unroll 8
+    for (int j = 0; j < S; ++j) Z += sq[j];
+    unsigned long long target = (unsigned long long)((double)tp * (double)Z);
+    if (target < 1) target = 1;
+    bool drop = false;
+    if (tid < S) {
+      const unsigned long long mine = sord[tid];
+      unsigned long long before = 0;
+#pragma unroll 8
+      for (int j = 0; j < S; ++j) before += sord[j] > mine ? sq[j] : 0ull;
+      drop = before >= target;
+    }
+    __syncthreads();
+    if (drop) sq[tid] = 0;
+    __syncthreads();
+  }
+  // the draw: the first survivor in index order whose cumulative mass exceeds r * Z
+  unsigned long long Z = 0, before = 0;
+  const int mine = tid < S ? si[tid] : 0;
+#pragma unroll 8
+  for (int j = 0; j < S; ++j) {
+    const unsigned long long q = sq[j];
+    Z += q;
+    before += si[j] < mine ? q : 0ull;
+  }
+  if (Z == 0) {   // nothing left to draw from: the last index
+    if (tid == 0) {
+      out[row] = vocab - 1;
+      done[row] = 1;
+    }
+    return;
+  }
+  unsigned long long t = (unsigned long long)((double)rnd[row] * (double)Z);
+  if (t >= Z) t = Z - 1;
+  if (tid < S && before <= t && t < before + sq[tid]) {
+    out[row] = mine;
+    done[row] = 1;
+  }
+}
+
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int vocab, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
     const float* __restrict__ typical_p, const float* __restrict__ rnd, int* __restrict__ out,
     float* __restrict__ info, const float* __restrict__ part_max, const unsigned long long* __restrict__ part_mass,
-    const unsigned int* __restrict__ part_cnt) {
+    const unsigned int* __restrict__ part_cnt, const int* __restrict__ done) {
   __shared__ unsigned long long hist[256 * SMP_REP];
   __shared__ unsigned int cnt[256 * SMP_REP];
   __shared__ unsigned long long sh[4];
@@ -568,6 +863,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   __shared__ int ibest[SMP_WAVES];
   __shared__ float vbest[SMP_WAVES];
   const int row = blockIdx.x;
+  if (done != nullptr && done[row]) return;   // settled by sample_topk_kernel
   const float* lg = logits + (size_t)row * vocab;
   float* x = work + (size_t)row * vocab;
   const bool greedy = !(temperature[row] > 0.f);
@@ -895,23 +1191,35 @@ __global__ __launch_bounds__(SMP_THREADS) void top_logprobs_kernel(const float* 
 extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p, const float* typical_p,
                          const float* rnd, int* out, float* info, float* part_max, unsigned long long* part_mass,
-                         unsigned int* part_cnt, hipStream_t s) {
+                         unsigned int* part_cnt, float* cand_val, int* cand_idx, int* cand_cnt, int* done, hipStream_t s) {
   // part_max: scratch of rows * 32 floats, or null (the row's first step then runs inside the one block per row);
   // part_mass: scratch of rows * 32 64-bit integers, given when some row is only scaled before the draw;
-  // part_cnt: scratch of rows * 32 * 256 32-bit integers, given when some row is cut by top_k
+  // part_cnt: scratch of rows * 32 * 256 32-bit integers, given when some row is cut by top_k;
+  // cand_val, cand_idx (rows * 32 * SMP_CCAP each), cand_cnt (rows * 32), done (rows): scratch for rows cut by a small
+  // top_k (all four or none; not with `info`)
   TP_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes");
   if (rows == 0) return 0;
-  if (part_max != nullptr && vocab >= 4096 && rows <= 65535)
-    hipLaunchKernelGGL(sample_scale_kernel, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, logits, work, vocab, temperature,
-                       part_max, part_cnt);
-  else
+  const bool fast = part_max != nullptr && vocab >= 4096 && rows <= 65535 && info == nullptr && cand_val != nullptr &&
+                    cand_idx != nullptr && cand_cnt != nullptr && done != nullptr;
+  if (!fast) cand_val = nullptr, cand_idx = nullptr, cand_cnt = nullptr, done = nullptr;
+  if (part_max != nullptr && vocab >= 4096 && rows <= 65535) {
+    if (fast && (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS > 16 * 256)
+      hipLaunchKernelGGL(sample_scale_kernel<SMP_PER_MAX / 256>, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, logits, work, vocab,
+                         temperature, part_max, part_cnt, top_k, typical_p, cand_val, cand_idx, cand_cnt);
+    else
+      hipLaunchKernelGGL(sample_scale_kernel<16>, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, logits, work, vocab, temperature,
+                         part_max, part_cnt, top_k, typical_p, cand_val, cand_idx, cand_cnt);
+  } else
     part_max = nullptr, part_cnt = nullptr;
+  if (fast)
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(256), 0, s, cand_val, cand_idx, cand_cnt, part_max, vocab,
+                       temperature, top_k, top_p, min_p, typical_p, rnd, out, done);
   if (part_max != nullptr && part_mass != nullptr && info == nullptr)
     hipLaunchKernelGGL(sample_mass_kernel, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, work, vocab, min_p, part_max, part_mass);
   else
     part_mass = nullptr;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, work, vocab, temperature, top_k,
-                     top_p, min_p, typical_p, rnd, out, info, part_max, part_mass, part_cnt);
+                     top_p, min_p, typical_p, rnd, out, info, part_max, part_mass, part_cnt, done);
   TP_CHECK_LAUNCH("sample");
   return 0;
 }

@@ -791,13 +791,24 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
                      for t, k, p, ty in zip(temperature, top_k, top_p, typical_p))
     part_mass = torch.empty((m * 32,), dtype=torch.int64, device=dev) if plain_rows and info is None else None
     # rows cut by top_k have the first pass of their selection counted by the kernel of many blocks that scales the row
-    topk_rows = any(t > 0 and 0 < k < vocab for t, k in zip(temperature, top_k))
-    part_cnt = torch.empty((m * 32 * 256,), dtype=torch.int32, device=dev) if topk_rows else None
+    # ... unless top_k is small: such a row is settled from the few candidates that each piece of it hands over
+    small = lambda k, ty: 0 < k <= 128 and not (ty < 1.0) and -(-vocab // 32) <= 8192 and info is None
+    topk_rows = [(k, ty) for t, k, ty in zip(temperature, top_k, typical_p) if t > 0 and 0 < k < vocab]
+    part_cnt = None
+    if any(not small(k, ty) for k, ty in topk_rows):
+        part_cnt = torch.empty((m * 32 * 256,), dtype=torch.int32, device=dev)
+    cand_val = cand_idx = cand_cnt = done = None
+    if any(small(k, ty) for k, ty in topk_rows):
+        cand_val = torch.empty((m * 32 * 160,), dtype=torch.float32, device=dev)
+        cand_idx = torch.empty((m * 32 * 160,), dtype=torch.int32, device=dev)
+        cand_cnt = torch.empty((m * 32,), dtype=torch.int32, device=dev)
+        done = torch.empty((m,), dtype=torch.int32, device=dev)
     if info is not None:
         _dev_ok(info)
         _need(info.dtype == torch.float32 and info.is_contiguous() and tuple(info.shape) == (m, 4), "sample: info must be float32 [m, 4]")
     _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
-          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _ptr(part_max), _ptr(part_mass), _ptr(part_cnt), _stream())
+          _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _ptr(part_max), _ptr(part_mass), _ptr(part_cnt),
+          _ptr(cand_val), _ptr(cand_idx), _ptr(cand_cnt), _ptr(done), _stream())
     return out
 
 

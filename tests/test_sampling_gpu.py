@@ -183,6 +183,57 @@ def test_top_k_keeps_at_most_k_even_with_ties():
     assert seen == set(range(40, 64)) | set(range(6))
 
 
+def _sample_one_block(logits, temperature, top_k, top_p, min_p, r):
+    """The same rows through the path of one block per row (a report of probabilities asks for it)."""
+    from tempura_amd.kernels import ops
+    ops.set_backend(None)
+    m, v = logits.shape
+    work = torch.empty(m, v, device=DEV)
+    info = torch.empty(m, 4, device=DEV)
+    full = lambda a: [a] * m if not isinstance(a, (list, tuple)) else list(a)
+    return ops.sample(logits.to(DEV), work, full(temperature), full(top_k), full(top_p), full(min_p), full(r), full(1.0), info).tolist()
+
+
+@pytest.mark.parametrize("vocab", [4099, 50021, 128256])
+def test_small_top_k_from_the_candidates_of_the_pieces(vocab):
+    """A row cut by a small top_k is settled from the candidates that the 32 pieces of the row hand over; the answer
+    is that of the one-block path in every case, and that of the plain rules."""
+    g = torch.Generator().manual_seed(vocab)
+    m = 16
+    rs = [(i + 0.41) / m for i in range(m)]
+    rows = {
+        "random": torch.randn(m, vocab, generator=g) * 3.0,
+        "few levels": (torch.randn(m, vocab, generator=g) * 2.0).round(),          # many ties, also at the cut
+        "flat": torch.zeros(m, vocab),                                             # every piece has too many candidates
+        "one piece holds them all": torch.randn(m, vocab, generator=g) * 0.1,
+        "mostly -inf": torch.full((m, vocab), -math.inf),
+        "nan": torch.randn(m, vocab, generator=g) * 3.0,
+    }
+    per = -(-vocab // 32)
+    rows["one piece holds them all"][:, 3 * per:3 * per + 100] += 10.0            # the k largest lie in one piece
+    rows["one piece holds them all"][:, 3 * per + 7] = rows["one piece holds them all"][:, 3 * per + 9]
+    rows["mostly -inf"][:, [5, vocab // 2, vocab - 1]] = torch.tensor([0.3, 1.0, 0.3])
+    rows["mostly -inf"][m - 1] = -math.inf                                          # nothing at all: the last index
+    rows["nan"][:, ::7] = math.nan
+    for name, lg in rows.items():
+        for t, k, p, mp in [(1.0, 1, 1.0, 0.0), (0.8, 5, 1.0, 0.0), (0.7, 50, 0.9, 0.0), (1.0, 128, 0.95, 0.0), (0.9, 40, 0.95, 0.3),
+                            (1.0, 128, 1.0, 0.0), (1.0, 129, 0.9, 0.0)]:
+            if k >= vocab:
+                continue
+            got = _sample(lg, t, k, p, mp, rs)
+            assert got == _sample_one_block(lg, t, k, p, mp, rs), (name, t, k, p, mp)
+            if name != "nan":
+                want = [plain_sample(lg[i], t, k, p, mp, rs[i]) for i in range(0, m - 1, 5)]
+                assert got[:m - 1:5] == want, (name, t, k, p, mp)
+            if name == "mostly -inf":
+                assert got[m - 1] == vocab - 1
+    # rows of both kinds in one call
+    lg = rows["few levels"]
+    ks = [(3, 200, 0, 64)[i % 4] for i in range(m)]
+    ts = [(1.0, 0.0, 0.9)[i % 3] for i in range(m)]
+    assert _sample(lg, ts, ks, 0.9, 0.0, rs) == _sample_one_block(lg, ts, ks, 0.9, 0.0, rs)
+
+
 def test_frequencies_follow_softmax():
     """Chi-square of 20,000 draws against softmax(logits / T) on a vocabulary of 16."""
     from tempura_amd.sampling import uniform_draw
