@@ -465,12 +465,21 @@ __device__ void typical_cut(float* __restrict__ x, int n, float maxv, unsigned i
 // scale a row also hands over the elements of its piece that are at least as large as the piece's k-th largest (value
 // and index; ties included), and one block per row then works on those few thousand candidates alone: the k-th
 // largest of them, ties at the cut in index order, min_p, top_p and the draw in index order, with the same fixed-point
-// masses as sample_kernel, whose result it reproduces bit for bit.  A row that does not qualify (no or a large
+// masses as sample_kernel, whose result it reproduces bit for bit.  A row that does not qualify (a large
 // top_k, typical_p, a report of probabilities asked for, a piece with more than SMP_CCAP candidates, more than 256 ties
 // at the cut) is left to sample_kernel (`done` 0).
+// A row cut by top_p alone goes the same way with the SMP_KMAX largest of each piece: the candidates hold every element
+// of the row that is at least as large as the largest of the pieces' thresholds, so when the prefix that top_p keeps
+// (against the mass of the whole row, from sample_mass_kernel) ends above that, it is found among them exactly; when
+// it reaches further down, as for a row of nearly equal logits, the row is left to sample_kernel.
 #define SMP_KMAX 128        // largest top_k of this path
 #define SMP_CCAP 160        // candidates a piece may hand over
 #define SMP_PER_MAX 8192    // elements of a piece (vocabularies up to 262,144)
+
+__device__ inline bool topp_fast_row(float T, int k, int vocab, float typ, float tp) {
+  return T > 0.f && !(k > 0 && k < vocab) && !(typ < 1.0f) && tp < 1.0f && tp > 0.f && vocab > SMP_KMAX &&
+         (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS <= SMP_PER_MAX;
+}
 
 __device__ inline bool topk_fast_row(float T, int k, int vocab, float typ) {
   return T > 0.f && k > 0 && k <= SMP_KMAX && k < vocab && !(typ < 1.0f) &&
@@ -551,6 +560,86 @@ __device__ inline unsigned int reg_kth_key(const unsigned int (&kreg)[R], unsign
   return prefix;
 }
 
+// The same with a weight per key (0 where there is no element): the largest key K with weight(keys >= K) >= target,
+// as radix_select<true> finds it.  *gt: the weight of the larger keys, *eq: how many keys are equal to K.
+template <int R>
+__device__ inline unsigned int reg_kth_mass(const unsigned int (&kreg)[R], const unsigned long long (&qreg)[R],
+                                            unsigned long long target, unsigned long long* hist /*256*/,
+                                            unsigned int* cnt /*256*/, unsigned long long* sh /*4*/,
+                                            unsigned long long* gt_out, unsigned int* eq_out) {
+  unsigned int prefix = 0;
+  unsigned long long gt = 0;
+  for (int i = threadIdx.x; i < 256; i += blockDim.x) {
+    hist[i] = 0;
+    cnt[i] = 0;
+  }
+  __syncthreads();
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const unsigned int key = kreg[u];
+      if (key != 0 && (pass == 0 || (key >> (shift + 8)) == prefix)) {
+        atomicAdd(&cnt[(key >> shift) & 255u], 1u);
+        atomicAdd(&hist[(key >> shift) & 255u], qreg[u]);
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < TP_WAVE) {
+      const int lane = threadIdx.x;
+      unsigned long long w[4], local = 0;
+      unsigned int c[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        w[i] = hist[255 - (4 * lane + i)];
+        c[i] = cnt[255 - (4 * lane + i)];
+        hist[255 - (4 * lane + i)] = 0;   // (clear for the next pass)
+        cnt[255 - (4 * lane + i)] = 0;
+        local += w[i];
+      }
+      unsigned long long inc = local;
+#pragma unroll
+      for (int o = 1; o < TP_WAVE; o <<= 1) {
+        const unsigned long long up = __shfl_up(inc, o, TP_WAVE);
+        if (lane >= o) inc += up;
+      }
+      unsigned long long run = gt + inc - local;
+      unsigned int cf = 0;
+      int found = -1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int b = 255 - (4 * lane + i);
+        if (found < 0 && b > 0) {
+          if (run + w[i] >= target) {
+            found = b;
+            cf = c[i];
+          } else {
+            run += w[i];
+          }
+        }
+      }
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(found >= 0);
+      if (hit != 0) {
+        if (lane == (int)__builtin_ctzll(hit)) {
+          sh[0] = run;
+          sh[1] = (unsigned long long)found;
+          sh[2] = cf;
+        }
+      } else if (lane == TP_WAVE - 1) {
+        sh[0] = run;
+        sh[1] = 0;
+        sh[2] = c[3];   // (bin 0)
+      }
+    }
+    __syncthreads();
+    gt = sh[0];
+    prefix = (prefix << 8) | (unsigned int)sh[1];
+  }
+  *gt_out = gt;
+  *eq_out = (unsigned int)sh[2];
+  return prefix;
+}
+
 // Step 1 of sample_kernel for a whole row on many CUs: x = logit / temperature (NaN -> -inf), written to `work`,
 // and the maximum of each of SMP_CHUNKS pieces of the row to part_max[row, piece].  grid: (rows, SMP_CHUNKS).
 template <int R>   // R * 256: the most elements of a piece whose row takes the way of a small top_k
@@ -558,13 +647,15 @@ __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restri
                                                            int vocab, const float* __restrict__ temperature,
                                                            float* __restrict__ part_max,
                                                            unsigned int* __restrict__ part_cnt,
-                                                           const int* __restrict__ top_k, const float* __restrict__ typical_p,
+                                                           const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                           const float* __restrict__ typical_p,
                                                            float* __restrict__ cand_val, int* __restrict__ cand_idx,
-                                                           int* __restrict__ cand_cnt) {
+                                                           int* __restrict__ cand_cnt, unsigned int* __restrict__ cand_thr) {
   // part_cnt (may be null): how many finite elements of the piece fall into each of the 256 bins of radix_select's
   // first pass, [rows, SMP_CHUNKS, 256]
-  // cand_* (may be null): the piece's candidates for a row cut by a small top_k (see topk_fast_row),
-  // [rows, SMP_CHUNKS, SMP_CCAP] and their number [rows, SMP_CHUNKS] (more than SMP_CCAP: too many, none usable)
+  // cand_* (may be null): the piece's candidates for a row cut by a small top_k or by top_p alone (see topk_fast_row,
+  // topp_fast_row), [rows, SMP_CHUNKS, SMP_CCAP], their number [rows, SMP_CHUNKS] (more than SMP_CCAP: too many, none
+  // usable) and the key from which on the piece has handed over everything [rows, SMP_CHUNKS]
   __shared__ float fscratch[32];
   __shared__ unsigned int bins[256 * 4];
   __shared__ float xs[R * 256];
@@ -573,8 +664,10 @@ __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restri
   __shared__ int n_out;
   static_assert(R * 256 <= SMP_PER_MAX, "sample_topk_kernel takes rows of pieces up to SMP_PER_MAX");
   const int row = blockIdx.x, chunk = blockIdx.y;
-  const bool local_topk = cand_cnt != nullptr && topk_fast_row(temperature[row], top_k[row], vocab, typical_p[row]) &&
-                          (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS <= R * 256;
+  const bool by_k = cand_cnt != nullptr && topk_fast_row(temperature[row], top_k[row], vocab, typical_p[row]);
+  const bool by_p = cand_cnt != nullptr && !by_k &&
+                    topp_fast_row(temperature[row], top_k[row], vocab, typical_p[row], top_p[row]);
+  const bool local_topk = (by_k || by_p) && (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS <= R * 256;
   if (part_cnt != nullptr) {
     for (int i = threadIdx.x; i < 256 * 4; i += blockDim.x) bins[i] = 0;
     __syncthreads();
@@ -637,7 +730,8 @@ __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restri
     }
     if (threadIdx.x == 0) n_out = 0;
     unsigned int gt, eq;
-    unsigned int K = reg_kth_key(kreg, (unsigned int)top_k[row], kbins, ksh, &gt, &eq);   // (barriers: n_out is set)
+    unsigned int K = reg_kth_key(kreg, by_k ? (unsigned int)top_k[row] : (unsigned int)SMP_KMAX, kbins, ksh, &gt,
+                                 &eq);   // (barriers: n_out is set)
     if (K < finite) K = finite;
     const size_t base = ((size_t)row * SMP_CHUNKS + chunk) * SMP_CCAP;
 #pragma unroll
@@ -651,7 +745,10 @@ __global__ __launch_bounds__(256) void sample_scale_kernel(const float* __restri
       }
     }
     __syncthreads();
-    if (threadIdx.x == 0) cand_cnt[row * SMP_CHUNKS + chunk] = n_out;
+    if (threadIdx.x == 0) {
+      cand_cnt[row * SMP_CHUNKS + chunk] = n_out;
+      cand_thr[row * SMP_CHUNKS + chunk] = K;
+    }
   }
   if (part_cnt != nullptr) {
     __syncthreads();
@@ -699,7 +796,10 @@ __global__ __launch_bounds__(256) void sample_mass_kernel(const float* __restric
 // settled here, 0 when sample_kernel has to do it.
 #define SMP_TOPK_R (SMP_CHUNKS * SMP_CCAP / 256)
 __global__ __launch_bounds__(256) void sample_topk_kernel(const float* __restrict__ cand_val, const int* __restrict__ cand_idx,
-                                                          const int* __restrict__ cand_cnt, const float* __restrict__ part_max,
+                                                          const int* __restrict__ cand_cnt,
+                                                          const unsigned int* __restrict__ cand_thr,
+                                                          const float* __restrict__ part_max,
+                                                          const unsigned long long* __restrict__ part_mass,
                                                           int vocab, const float* __restrict__ temperature,
                                                           const int* __restrict__ top_k, const float* __restrict__ top_p,
                                                           const float* __restrict__ min_p, const float* __restrict__ typical_p,
@@ -713,24 +813,41 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(const float* __restric
   __shared__ unsigned long long sord[SMP_KMAX];    // survivors: key and index as one number that orders them
   __shared__ int si[SMP_KMAX];
   __shared__ unsigned long long sq[SMP_KMAX];      // ... and their masses (0: dropped)
-  __shared__ int s_n, n_tie, s_over;
+  __shared__ unsigned long long hist[256], sh64[4], pm[SMP_CHUNKS], pl_q[SMP_CCAP], s_Z;   // (rows cut by top_p alone)
+  __shared__ int pl_idx[SMP_CCAP];
+  __shared__ int s_n, n_tie, s_over, n_pl;
+  __shared__ unsigned int s_thr;
   __shared__ float s_max;
   const int row = blockIdx.x, tid = threadIdx.x;
   if (tid == 0) done[row] = 0;
   const int k = top_k[row];
-  if (!topk_fast_row(temperature[row], k, vocab, typical_p[row])) return;
+  const bool by_k = topk_fast_row(temperature[row], k, vocab, typical_p[row]);
+  const bool by_p = !by_k && part_mass != nullptr && topp_fast_row(temperature[row], k, vocab, typical_p[row], top_p[row]);
+  if (!by_k && !by_p) return;
   if (tid < TP_WAVE) {   // how many candidates each piece brings, and the row's maximum
     const int c = tid < SMP_CHUNKS ? cand_cnt[row * SMP_CHUNKS + tid] : 0;
     float mx = tid < SMP_CHUNKS ? part_max[row * SMP_CHUNKS + tid] : -INFINITY;
+    unsigned int thr = tid < SMP_CHUNKS ? cand_thr[row * SMP_CHUNKS + tid] : 0u;
+    unsigned long long z = (by_p && tid < SMP_CHUNKS) ? part_mass[row * SMP_CHUNKS + tid] : 0ull;
     const bool over = __builtin_amdgcn_ballot_w64(c > SMP_CCAP) != 0;
 #pragma unroll
-    for (int o = TP_WAVE / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, TP_WAVE));
-    if (tid < SMP_CHUNKS) cnts[tid] = c;
+    for (int o = TP_WAVE / 2; o > 0; o >>= 1) {
+      mx = fmaxf(mx, __shfl_xor(mx, o, TP_WAVE));
+      thr = max(thr, (unsigned int)__shfl_xor((int)thr, o, TP_WAVE));
+      z += __shfl_xor(z, o, TP_WAVE);
+    }
+    if (tid < SMP_CHUNKS) {
+      cnts[tid] = c;
+      pm[tid] = 0;
+    }
     if (tid == 0) {
       s_n = 0;
       n_tie = 0;
+      n_pl = 0;
       s_over = over;
       s_max = mx;
+      s_thr = thr;
+      s_Z = z;
     }
   }
   __syncthreads();
@@ -766,6 +883,92 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(const float* __restric
       const unsigned int key = float_key(v[u]);
       kreg[u] = (i < cnts[p] && key >= floor_key) ? key : 0u;
     }
+  }
+  if (by_p) {
+    // top_p alone: the prefix by descending value whose mass reaches top_p of the whole row's, then the draw
+    const unsigned long long Zrow = s_Z;
+    if (Zrow == 0) {   // nothing to draw from: the last index
+      if (tid == 0) {
+        out[row] = vocab - 1;
+        done[row] = 1;
+      }
+      return;
+    }
+    unsigned long long qreg[SMP_TOPK_R];
+#pragma unroll
+    for (int u = 0; u < SMP_TOPK_R; ++u) qreg[u] = kreg[u] != 0 ? fix_mass(key_float(kreg[u]), maxv) : 0ull;
+    unsigned long long target = (unsigned long long)((double)top_p[row] * (double)Zrow);
+    if (target < 1) target = 1;
+    unsigned long long gtm;
+    unsigned int eqn;
+    const unsigned int K2 = reg_kth_mass(kreg, qreg, target, hist, bins, sh64, &gtm, &eqn);
+    const unsigned long long q = fix_mass(key_float(K2), maxv);
+    // the candidates are all of the row from s_thr upwards: a prefix that ends there is the row's
+    if (K2 < s_thr || K2 < floor_key || gtm + (unsigned long long)eqn * q < target) return;
+    unsigned long long need = 1;
+    if (q > 0 && target > gtm) need = (target - gtm + q - 1) / q;
+    if (need < 1) need = 1;
+    const bool cut_ties = (unsigned long long)eqn > need;   // each tie has the mass q: as many as the target still needs
+    if (cut_ties && eqn > 256u) return;
+    if (cut_ties) {
+#pragma unroll
+      for (int u = 0; u < SMP_TOPK_R; ++u) {
+        if (kreg[u] == K2) {
+          const int at = atomicAdd(&n_tie, 1);
+          if (at < 256) tl[at] = ireg[u];
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < SMP_TOPK_R; ++u) {
+        if (kreg[u] == K2) {
+          unsigned long long rank = 0;
+          for (int j = 0; j < (int)eqn; ++j) rank += tl[j] < ireg[u];
+          if (rank >= need) kreg[u] = 0;
+        }
+      }
+    }
+    // the survivors' mass piece by piece, the piece that holds the draw, and the survivor there
+#pragma unroll
+    for (int u = 0; u < SMP_TOPK_R; ++u)
+      if (kreg[u] != 0 && kreg[u] >= K2 && qreg[u] != 0) atomicAdd(&pm[(tid + u * 256) / SMP_CCAP], qreg[u]);
+    __syncthreads();
+    unsigned long long Z = 0;
+    for (int i = 0; i < SMP_CHUNKS; ++i) Z += pm[i];
+    if (Z == 0) {
+      if (tid == 0) {
+        out[row] = vocab - 1;
+        done[row] = 1;
+      }
+      return;
+    }
+    unsigned long long t = (unsigned long long)((double)rnd[row] * (double)Z);
+    if (t >= Z) t = Z - 1;
+    unsigned long long c = 0;
+    int piece = 0;
+    for (; piece < SMP_CHUNKS - 1; ++piece) {
+      if (t < c + pm[piece]) break;
+      c += pm[piece];
+    }
+#pragma unroll
+    for (int u = 0; u < SMP_TOPK_R; ++u) {
+      if ((tid + u * 256) / SMP_CCAP == piece && kreg[u] != 0 && kreg[u] >= K2 && qreg[u] != 0) {
+        const int at = atomicAdd(&n_pl, 1);   // (a piece brings at most SMP_CCAP)
+        pl_idx[at] = ireg[u];
+        pl_q[at] = qreg[u];
+      }
+    }
+    __syncthreads();
+    if (tid < n_pl) {
+      const int mine = pl_idx[tid];
+      unsigned long long before = c;
+      for (int j = 0; j < n_pl; ++j) before += pl_idx[j] < mine ? pl_q[j] : 0ull;
+      if (before <= t && t < before + pl_q[tid]) {
+        out[row] = mine;
+        done[row] = 1;
+      }
+    }
+    return;
   }
   unsigned int gt, eq;
   const unsigned int K = reg_kth_key(kreg, (unsigned int)k, bins, sh, &gt, &eq);
@@ -1191,33 +1394,34 @@ __global__ __launch_bounds__(SMP_THREADS) void top_logprobs_kernel(const float* 
 extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p, const float* typical_p,
                          const float* rnd, int* out, float* info, float* part_max, unsigned long long* part_mass,
-                         unsigned int* part_cnt, float* cand_val, int* cand_idx, int* cand_cnt, int* done, hipStream_t s) {
+                         unsigned int* part_cnt, float* cand_val, int* cand_idx, int* cand_cnt, unsigned int* cand_thr,
+                         int* done, hipStream_t s) {
   // part_max: scratch of rows * 32 floats, or null (the row's first step then runs inside the one block per row);
   // part_mass: scratch of rows * 32 64-bit integers, given when some row is only scaled before the draw;
   // part_cnt: scratch of rows * 32 * 256 32-bit integers, given when some row is cut by top_k;
-  // cand_val, cand_idx (rows * 32 * SMP_CCAP each), cand_cnt (rows * 32), done (rows): scratch for rows cut by a small
-  // top_k (all four or none; not with `info`)
+  // cand_val, cand_idx (rows * 32 * SMP_CCAP each), cand_cnt, cand_thr (rows * 32 each), done (rows): scratch for rows
+  // cut by a small top_k or by top_p alone (all five or none; not with `info`; rows cut by top_p alone need part_mass too)
   TP_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes");
   if (rows == 0) return 0;
   const bool fast = part_max != nullptr && vocab >= 4096 && rows <= 65535 && info == nullptr && cand_val != nullptr &&
-                    cand_idx != nullptr && cand_cnt != nullptr && done != nullptr;
-  if (!fast) cand_val = nullptr, cand_idx = nullptr, cand_cnt = nullptr, done = nullptr;
+                    cand_idx != nullptr && cand_cnt != nullptr && cand_thr != nullptr && done != nullptr;
+  if (!fast) cand_val = nullptr, cand_idx = nullptr, cand_cnt = nullptr, cand_thr = nullptr, done = nullptr;
   if (part_max != nullptr && vocab >= 4096 && rows <= 65535) {
     if (fast && (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS > 16 * 256)
       hipLaunchKernelGGL(sample_scale_kernel<SMP_PER_MAX / 256>, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, logits, work, vocab,
-                         temperature, part_max, part_cnt, top_k, typical_p, cand_val, cand_idx, cand_cnt);
+                         temperature, part_max, part_cnt, top_k, top_p, typical_p, cand_val, cand_idx, cand_cnt, cand_thr);
     else
       hipLaunchKernelGGL(sample_scale_kernel<16>, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, logits, work, vocab, temperature,
-                         part_max, part_cnt, top_k, typical_p, cand_val, cand_idx, cand_cnt);
+                         part_max, part_cnt, top_k, top_p, typical_p, cand_val, cand_idx, cand_cnt, cand_thr);
   } else
     part_max = nullptr, part_cnt = nullptr;
-  if (fast)
-    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(256), 0, s, cand_val, cand_idx, cand_cnt, part_max, vocab,
-                       temperature, top_k, top_p, min_p, typical_p, rnd, out, done);
   if (part_max != nullptr && part_mass != nullptr && info == nullptr)
     hipLaunchKernelGGL(sample_mass_kernel, dim3(rows, SMP_CHUNKS), dim3(256), 0, s, work, vocab, min_p, part_max, part_mass);
   else
     part_mass = nullptr;
+  if (fast)
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(256), 0, s, cand_val, cand_idx, cand_cnt, cand_thr, part_max,
+                       part_mass, vocab, temperature, top_k, top_p, min_p, typical_p, rnd, out, done);
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SMP_THREADS), 0, s, logits, work, vocab, temperature, top_k,
                      top_p, min_p, typical_p, rnd, out, info, part_max, part_mass, part_cnt, done);
   TP_CHECK_LAUNCH("sample");

@@ -762,16 +762,20 @@ def apply_penalties(logits: torch.Tensor, rows, tokens, counts, in_window, prese
 
 
 def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, min_p, rnd, typical_p=None,
-           info: Optional[torch.Tensor] = None) -> torch.Tensor:
+           info: Optional[torch.Tensor] = None, settled: Optional[list] = None) -> torch.Tensor:
     """float32 [m, vocab] and per-row options (host arrays) -> int32 [m] chosen tokens.
     ``work`` is float32 scratch of at least [m, vocab].  temperature 0 rows return the argmax.
     ``typical_p`` None leaves that filter off (1.0) in every row.
     ``info``: float32 [m, 4] that receives, per row, what log-probabilities of the filtered distribution need
     (maximum, ln of the normaliser, smallest surviving value) and the chosen token's log-probability in column 3;
-    ``work`` then holds the filtered, scaled logits for ``top_logprobs``."""
+    ``work`` then holds the filtered, scaled logits for ``top_logprobs``.
+    ``settled``: a list that receives, per row, 1 when the row was settled from the candidates of its pieces (a
+    small top_k, or top_p alone on a row whose kept prefix is short) and 0 when the one block per row did it; for tests."""
     if typical_p is None:
         typical_p = [1.0] * len(temperature)
     if _backend is not None:
+        if settled is not None:
+            settled[:] = [0] * len(temperature)
         return _backend.sample(logits, work, temperature, top_k, top_p, min_p, rnd, typical_p, info)
     import numpy as np
     _dev_ok(logits, work)
@@ -789,26 +793,34 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
     # of many blocks; worth it when there is such a row
     plain_rows = any(t > 0 and not (0 < k < vocab) and not (0.0 < p < 1.0) and not (ty < 1.0)
                      for t, k, p, ty in zip(temperature, top_k, top_p, typical_p))
-    part_mass = torch.empty((m * 32,), dtype=torch.int64, device=dev) if plain_rows and info is None else None
+    # rows cut by top_p alone are settled from the candidates of their pieces against the mass of the whole row
+    piece_ok = -(-vocab // 32) <= 8192 and info is None
+    topp_rows = piece_ok and vocab > 128 and any(
+        t > 0 and not (0 < k < vocab) and 0.0 < p < 1.0 and not (ty < 1.0)
+        for t, k, p, ty in zip(temperature, top_k, top_p, typical_p))
+    part_mass = torch.empty((m * 32,), dtype=torch.int64, device=dev) if (plain_rows or topp_rows) and info is None else None
     # rows cut by top_k have the first pass of their selection counted by the kernel of many blocks that scales the row
     # ... unless top_k is small: such a row is settled from the few candidates that each piece of it hands over
-    small = lambda k, ty: 0 < k <= 128 and not (ty < 1.0) and -(-vocab // 32) <= 8192 and info is None
+    small = lambda k, ty: 0 < k <= 128 and not (ty < 1.0) and piece_ok
     topk_rows = [(k, ty) for t, k, ty in zip(temperature, top_k, typical_p) if t > 0 and 0 < k < vocab]
     part_cnt = None
     if any(not small(k, ty) for k, ty in topk_rows):
         part_cnt = torch.empty((m * 32 * 256,), dtype=torch.int32, device=dev)
-    cand_val = cand_idx = cand_cnt = done = None
-    if any(small(k, ty) for k, ty in topk_rows):
+    cand_val = cand_idx = cand_cnt = cand_thr = done = None
+    if topp_rows or any(small(k, ty) for k, ty in topk_rows):
         cand_val = torch.empty((m * 32 * 160,), dtype=torch.float32, device=dev)
         cand_idx = torch.empty((m * 32 * 160,), dtype=torch.int32, device=dev)
         cand_cnt = torch.empty((m * 32,), dtype=torch.int32, device=dev)
+        cand_thr = torch.empty((m * 32,), dtype=torch.int32, device=dev)
         done = torch.empty((m,), dtype=torch.int32, device=dev)
     if info is not None:
         _dev_ok(info)
         _need(info.dtype == torch.float32 and info.is_contiguous() and tuple(info.shape) == (m, 4), "sample: info must be float32 [m, 4]")
     _call("tp_sample", _ptr(logits), _ptr(work), m, vocab, _ptr(fl[0]), _ptr(tk), _ptr(fl[1]), _ptr(fl[2]),
           _ptr(fl[4]), _ptr(fl[3]), _ptr(out), _ptr(info), _ptr(part_max), _ptr(part_mass), _ptr(part_cnt),
-          _ptr(cand_val), _ptr(cand_idx), _ptr(cand_cnt), _ptr(done), _stream())
+          _ptr(cand_val), _ptr(cand_idx), _ptr(cand_cnt), _ptr(cand_thr), _ptr(done), _stream())
+    if settled is not None:
+        settled[:] = [0] * m if done is None else done.tolist()
     return out
 
 

@@ -63,13 +63,14 @@ def plain_sample(logits, temperature, top_k, top_p, min_p, r, typical_p=1.0):
     return int(hit[0]) if hit.numel() else V - 1
 
 
-def _sample(logits, temperature, top_k, top_p, min_p, r, typical_p=1.0):
+def _sample(logits, temperature, top_k, top_p, min_p, r, typical_p=1.0, settled=None):
     from tempura_amd.kernels import ops
     ops.set_backend(None)
     m, v = logits.shape
     work = torch.empty(m, v, device=DEV)
     full = lambda a: [a] * m if not isinstance(a, (list, tuple)) else list(a)
-    return ops.sample(logits.to(DEV), work, full(temperature), full(top_k), full(top_p), full(min_p), full(r), full(typical_p)).tolist()
+    return ops.sample(logits.to(DEV), work, full(temperature), full(top_k), full(top_p), full(min_p), full(r), full(typical_p),
+                      settled=settled).tolist()
 
 
 @pytest.mark.parametrize("vocab", [16, 301, 4099, 50021])    # (the largest: whole rounds of sixteen loads and their rests)
@@ -195,9 +196,10 @@ def _sample_one_block(logits, temperature, top_k, top_p, min_p, r):
 
 
 @pytest.mark.parametrize("vocab", [4099, 50021, 128256])
-def test_small_top_k_from_the_candidates_of_the_pieces(vocab):
-    """A row cut by a small top_k is settled from the candidates that the 32 pieces of the row hand over; the answer
-    is that of the one-block path in every case, and that of the plain rules."""
+def test_small_top_k_and_top_p_from_the_candidates_of_the_pieces(vocab):
+    """A row cut by a small top_k, or by top_p alone when the prefix it keeps is short, is settled from the candidates
+    that the 32 pieces of the row hand over; the answer is that of the one-block path in every case, and that of the
+    plain rules.  Rows that cannot be settled so (nearly equal logits) are left to the one block per row."""
     g = torch.Generator().manual_seed(vocab)
     m = 16
     rs = [(i + 0.41) / m for i in range(m)]
@@ -217,11 +219,17 @@ def test_small_top_k_from_the_candidates_of_the_pieces(vocab):
     rows["nan"][:, ::7] = math.nan
     for name, lg in rows.items():
         for t, k, p, mp in [(1.0, 1, 1.0, 0.0), (0.8, 5, 1.0, 0.0), (0.7, 50, 0.9, 0.0), (1.0, 128, 0.95, 0.0), (0.9, 40, 0.95, 0.3),
-                            (1.0, 128, 1.0, 0.0), (1.0, 129, 0.9, 0.0)]:
+                            (1.0, 128, 1.0, 0.0), (1.0, 129, 0.9, 0.0), (0.8, 0, 0.9, 0.0), (1.0, 0, 0.5, 0.0), (1.0, 0, 0.95, 0.1),
+                            (1.2, 0, 0.999, 0.0), (0.6, 0, 0.01, 0.0)]:
             if k >= vocab:
                 continue
-            got = _sample(lg, t, k, p, mp, rs)
+            settled = []
+            got = _sample(lg, t, k, p, mp, rs, settled=settled)
             assert got == _sample_one_block(lg, t, k, p, mp, rs), (name, t, k, p, mp)
+            if name == "random" and (0 < k <= 128 or (k == 0 and p <= 0.9)):
+                assert settled == [1] * m, (name, t, k, p, mp)
+            if name == "flat" or k > 128:
+                assert settled == [0] * m, (name, t, k, p, mp)
             if name != "nan":
                 want = [plain_sample(lg[i], t, k, p, mp, rs[i]) for i in range(0, m - 1, 5)]
                 assert got[:m - 1:5] == want, (name, t, k, p, mp)
@@ -231,7 +239,8 @@ def test_small_top_k_from_the_candidates_of_the_pieces(vocab):
     lg = rows["few levels"]
     ks = [(3, 200, 0, 64)[i % 4] for i in range(m)]
     ts = [(1.0, 0.0, 0.9)[i % 3] for i in range(m)]
-    assert _sample(lg, ts, ks, 0.9, 0.0, rs) == _sample_one_block(lg, ts, ks, 0.9, 0.0, rs)
+    ps = [(0.9, 1.0, 0.7, 0.9, 0.5)[i % 5] for i in range(m)]
+    assert _sample(lg, ts, ks, ps, 0.0, rs) == _sample_one_block(lg, ts, ks, ps, 0.0, rs)
 
 
 def test_frequencies_follow_softmax():
