@@ -626,10 +626,17 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
         blocks_per_split = num_single * kvh * ((heads // kvh + 15) // 16)
-        # (from 65 blocks per split on, twice the target: two blocks fit a CU, and the blocks of the longest requests,
-        # which set the time when contexts differ, are halved: 16 requests of the 8B shape 4.33 -> 4.25 ms a step,
-        # 32 requests 5.27 -> 5.20, 48 and 64 the same)
-        want = -(-(decode_target_blocks if blocks_per_split <= 64 else 2 * decode_target_blocks) // blocks_per_split)
+        # (two blocks fit a CU, 512 the chip.  From 65 to 256 blocks per split, as many splits as fill it once: measured
+        # alone at 2,100 keys, 16 requests 35.8 -> 33.5 us, 20 requests 47.2 -> 38.5, 32 requests 54.3 -> 52.7, and more
+        # for contexts that differ; through the engine 16 requests of the 8B shape 4.33 -> 4.25 ms a step, 32 requests
+        # 5.27 -> 5.20.  Beyond 256 blocks per split a second split leaves blocks waiting for a place: better for some
+        # batches, worse for others, so none.)
+        if blocks_per_split <= 64:
+            want = -(-decode_target_blocks // blocks_per_split)
+        elif blocks_per_split <= decode_target_blocks:
+            want = max(1, 2 * decode_target_blocks // blocks_per_split)
+        else:
+            want = 1
         if blocks_per_split <= 64:
             want = max(want, decode_min_splits)     # (batch 8 of the 8B shape: eight splits 3.87 ms a step, four 3.94)
         splits = max(1, min(64, want, max(1, max_context_len // 128)))
