@@ -584,6 +584,8 @@ allow_fast_attention = True
 decode_target_blocks = 256
 #: and at least this many splits while a split has at most 64 blocks
 decode_min_splits = 8
+#: measurements: this many splits whatever the batch (0: chosen by the rules below)
+decode_force_splits = 0
 #: portions of prompts with fewer query blocks than this have their keys split over blocks (1: never)
 portion_target_blocks = 1024
 #: in parts of at least this many keys
@@ -629,16 +631,22 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         # (two blocks fit a CU, 512 the chip.  From 65 to 256 blocks per split, as many splits as fill it once: measured
         # alone at 2,100 keys, 16 requests 35.8 -> 33.5 us, 20 requests 47.2 -> 38.5, 32 requests 54.3 -> 52.7, and more
         # for contexts that differ; through the engine 16 requests of the 8B shape 4.33 -> 4.25 ms a step, 32 requests
-        # 5.27 -> 5.20.  Beyond 256 blocks per split a second split leaves blocks waiting for a place: better for some
-        # batches, worse for others, so none.)
+        # 5.27 -> 5.20; 12 requests in five splits against three 4.11 / 4.27, 20 in three against two 4.77 / 4.92, 24 in
+        # two against three 4.97 / 5.21.)
         if blocks_per_split <= 64:
             want = -(-decode_target_blocks // blocks_per_split)
         elif blocks_per_split <= decode_target_blocks:
             want = max(1, 2 * decode_target_blocks // blocks_per_split)
         else:
+            # (more blocks than half the chip's places: no split.  Through the engine, requests of 2,048+ keys of the 8B
+            # shape, one split against two: 36 requests 6.06 / 5.97 ms a step, 40: 6.14 / 6.04, 48: 6.27 / 6.49,
+            # 56: 6.42 / 6.68, 64: 6.62 / 6.89; three splits at 36 and 40 requests, which the kernel timed alone
+            # prefers, 6.07 and 6.13)
             want = 1
         if blocks_per_split <= 64:
             want = max(want, decode_min_splits)     # (batch 8 of the 8B shape: eight splits 3.87 ms a step, four 3.94)
+        if decode_force_splits > 0:
+            want = decode_force_splits
         splits = max(1, min(64, want, max(1, max_context_len // 128)))
         if splits > 1:
             scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
