@@ -1051,6 +1051,64 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(const float* __restric
   }
 }
 
+// The fixed-point mass of the survivors (key >= floor_key) in x[lo, hi), wave by wave: every wave of the block owns
+// a contiguous part of the range (a multiple of 64 elements) and sums it with coalesced loads, sixteen in flight;
+// scan[w] receives wave w's sum.  Returns the range's total; *wlo, *whi: this wave's part.  Called by the whole block.
+__device__ inline unsigned long long range_mass_by_wave(const float* __restrict__ x, int lo, int hi, unsigned int floor_key,
+                                                        float maxv, unsigned long long* scan /*SMP_WAVES*/, int* wlo_out,
+                                                        int* whi_out) {
+  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  const int per_wave = ((hi - lo + SMP_WAVES - 1) / SMP_WAVES + TP_WAVE - 1) / TP_WAVE * TP_WAVE;
+  const int wlo = min(hi, lo + wave * per_wave), whi = min(hi, wlo + per_wave);
+  unsigned long long mine = 0;
+  int j = wlo + lane;
+  for (; j + 15 * TP_WAVE < whi; j += 16 * TP_WAVE) {   // sixteen loads in flight (see walk_row)
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = x[j + u * TP_WAVE];
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      if (float_key(v[u]) >= floor_key) mine += fix_mass(v[u], maxv);
+  }
+  for (; j < whi; j += TP_WAVE) {
+    const float v = x[j];
+    if (float_key(v) >= floor_key) mine += fix_mass(v, maxv);
+  }
+#pragma unroll
+  for (int o = TP_WAVE / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, TP_WAVE);
+  __syncthreads();
+  if (lane == 0) scan[wave] = mine;
+  __syncthreads();
+  unsigned long long total = 0;
+  for (int i = 0; i < SMP_WAVES; ++i) total += scan[i];
+  *wlo_out = wlo;
+  *whi_out = whi;
+  return total;
+}
+
+// After range_mass_by_wave: the first index of the range, in index order, at which the cumulative mass, counted
+// from `base` before the range, exceeds t.  The wave whose part holds it walks that part 64 elements at a time;
+// its lane 0 gets the index, every other thread -1.
+__device__ inline int range_find_by_wave(const float* __restrict__ x, int wlo, int whi, unsigned long long base,
+                                         unsigned long long t, unsigned int floor_key, float maxv,
+                                         const unsigned long long* scan) {
+  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
+  unsigned long long before = base, mine_base = 0;
+  int chosen_wave = -1;
+  for (int i = 0; i < SMP_WAVES; ++i) {
+    const unsigned long long w = scan[i];
+    if (chosen_wave < 0 && t < before + w) {
+      chosen_wave = i;
+      mine_base = before;
+    }
+    before += w;
+  }
+  if (wave != chosen_wave) return -1;
+  const int at = wave_find(x, wlo, whi, mine_base, t,
+                           [&](float v) { return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull; }, lane);
+  return lane == 0 ? at : -1;
+}
+
 __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, float* __restrict__ work, int vocab, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
@@ -1170,13 +1228,13 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
         if (t < c + pm[piece]) break;
         c += pm[piece];
       }
-      if (threadIdx.x >= TP_WAVE) return;      // one wave walks the piece, 64 elements at a time
-      const int lane = threadIdx.x;
+      // the piece's mass wave by wave, then one wave walks its sixteenth of the piece, 64 elements at a time
       const int per = (vocab + SMP_CHUNKS - 1) / SMP_CHUNKS;
       const int lo = min(vocab, piece * per), hi = min(vocab, lo + per);
-      const int at = wave_find(x, lo, hi, c, t,
-                               [&](float v) { return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull; }, lane);
-      if (at >= 0 && lane == 0) out[row] = at;
+      int wlo, whi;
+      range_mass_by_wave(x, lo, hi, floor_key, maxv, scan, &wlo, &whi);
+      const int at = range_find_by_wave(x, wlo, whi, c, t, floor_key, maxv, scan);
+      if (at >= 0) out[row] = at;
       return;
     }
   }
@@ -1272,34 +1330,8 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   // 6. draw: first index (index order) whose cumulative mass exceeds r * Z
   // Every wave owns a contiguous range of the row and sums its mass with coalesced loads; the wave whose range
   // holds the target then walks it 64 elements at a time with a prefix sum over its lanes.
-  const int lane = threadIdx.x % TP_WAVE, wave = threadIdx.x / TP_WAVE;
-  const int per_wave = ((vocab + SMP_WAVES - 1) / SMP_WAVES + TP_WAVE - 1) / TP_WAVE * TP_WAVE;
-  const int wlo = min(vocab, wave * per_wave), whi = min(vocab, wlo + per_wave);
-  auto mass = [&](int j) {
-    if (j >= whi) return 0ull;
-    const float v = x[j];
-    return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull;
-  };
-  unsigned long long mine = 0;
-  {
-    int j = wlo + lane;
-    for (; j + 15 * TP_WAVE < whi; j += 16 * TP_WAVE) {   // sixteen loads in flight (see walk_row)
-      float v[16];
-#pragma unroll
-      for (int u = 0; u < 16; ++u) v[u] = x[j + u * TP_WAVE];
-#pragma unroll
-      for (int u = 0; u < 16; ++u)
-        if (float_key(v[u]) >= floor_key) mine += fix_mass(v[u], maxv);
-    }
-    for (; j < whi; j += TP_WAVE) mine += mass(j);
-  }
-#pragma unroll
-  for (int o = TP_WAVE / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, TP_WAVE);
-  __syncthreads();
-  if (lane == 0) scan[wave] = mine;
-  __syncthreads();
-  unsigned long long total = 0;
-  for (int i = 0; i < SMP_WAVES; ++i) total += scan[i];
+  int wlo, whi;
+  const unsigned long long total = range_mass_by_wave(x, 0, vocab, floor_key, maxv, scan, &wlo, &whi);
   if (!need_mass_now) Z = total;
   if (total == 0 || Z == 0) {       // nothing left to draw from: the last index
     if (threadIdx.x == 0) out[row] = vocab - 1;
@@ -1308,23 +1340,10 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   const float r = rnd[row];
   unsigned long long t = (unsigned long long)((double)r * (double)Z);
   if (t >= Z) t = Z - 1;
-  unsigned long long base = 0, before = 0;
-  int chosen_wave = -1;
-  for (int i = 0; i < SMP_WAVES; ++i) {
-    const unsigned long long w = scan[i];
-    if (chosen_wave < 0 && t < before + w) {
-      chosen_wave = i;
-      base = before;
-    }
-    before += w;
-  }
-  if (wave == chosen_wave) {
-    const int at = wave_find(x, wlo, whi, base, t,
-                             [&](float v) { return float_key(v) >= floor_key ? fix_mass(v, maxv) : 0ull; }, lane);
-    if (at >= 0 && lane == 0) {
-      out[row] = at;
-      if (inf != nullptr) inf[3] = (x[at] - maxv) - lnZ;
-    }
+  const int at = range_find_by_wave(x, wlo, whi, 0ull, t, floor_key, maxv, scan);
+  if (at >= 0) {
+    out[row] = at;
+    if (inf != nullptr) inf[3] = (x[at] - maxv) - lnZ;
   }
 }
 
