@@ -17,6 +17,7 @@ NO_SCRATCH = {
     "gemm_pipe.hip": ["gemm_pipe_kernel", "gemm_pipe_big_kernel", "gemm_pipe64_kernel", "gemm_pipe128_kernel"],
     "gemm_mfma.hip": ["gemm_skinny_mfma_kernel", "gemm_skinny_lds_kernel"],
     "attention_mfma.hip": ["attn_prefill_lds_kernel", "attn_decode_kernel"],
+    "sampling.hip": ["sample_scale_kernel", "sample_topk_kernel"],      # (keys of a piece, or candidates, in registers)
 }
 
 
