@@ -97,6 +97,21 @@ def test_typical_p_matches_plain_rules(vocab, temperature, top_k, top_p, min_p, 
     assert got == want
 
 
+def test_typical_p_and_tie_cuts_on_a_long_row():
+    """The cuts that go through a row in index order (typical_p's last ties, surplus ties of top_k and top_p) on rows
+    long enough for every wave to read several rounds of sixteen groups, with many equal values."""
+    vocab = 50021
+    g = torch.Generator().manual_seed(50021)
+    spread = torch.randn(6, vocab, generator=g) * 2.5
+    levels = (torch.randn(6, vocab, generator=g) * 2.0).round() * 0.5       # ties everywhere
+    rs = [(i + 0.61) / 6 for i in range(6)]
+    for logits in (spread, levels):
+        for t, k, p, ty in [(1.0, 0, 1.0, 0.9), (0.8, 0, 0.9, 0.5), (1.0, 300, 0.9, 1.0), (1.0, 300, 1.0, 1.0), (1.0, 0, 0.7, 1.0)]:
+            got = _sample(logits, t, k, p, 0.0, rs, ty)
+            want = [plain_sample(logits[i], t, k, p, 0.0, rs[i], ty) for i in range(6)]
+            assert got == want, (t, k, p, ty)
+
+
 def test_typical_p_drops_a_likely_but_untypical_token():
     # token 0 holds 30 % of the mass, 700 others share the rest: the entropy is near the information of a tail
     # token, so token 0 is the LEAST typical and leaves first, although every other filter would keep it
