@@ -939,6 +939,18 @@ __global__ __launch_bounds__(256) void sample_topk_kernel(const float* __restric
     for (int u = 0; u < SMP_TOPK_R; ++u) qreg[u] = kreg[u] != 0 ? fix_mass(key_float(kreg[u]), maxv) : 0ull;
     unsigned long long target = (unsigned long long)((double)top_p[row] * (double)Zrow);
     if (target < 1) target = 1;
+    {   // all candidates together short of the target (a row of nearly equal logits): left to sample_kernel at once
+      unsigned long long mine = 0;
+#pragma unroll
+      for (int u = 0; u < SMP_TOPK_R; ++u) mine += qreg[u];
+#pragma unroll
+      for (int o = TP_WAVE / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, TP_WAVE);
+      if (tid % TP_WAVE == 0) sh64[tid / TP_WAVE] = mine;
+      __syncthreads();
+      const unsigned long long all = sh64[0] + sh64[1] + sh64[2] + sh64[3];
+      __syncthreads();   // (sh64 is used again by the selection)
+      if (all < target) return;
+    }
     unsigned long long gtm;
     unsigned int eqn;
     const unsigned int K2 = reg_kth_mass(kreg, qreg, target, hist, bins, sh64, &gtm, &eqn);
@@ -1319,14 +1331,21 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   // needs it earlier: no top_p and no report)
   const float tp = top_p[row];
   const bool need_mass_now = (tp < 1.0f && tp > 0.f) || inf != nullptr || greedy;
+  // (known already when sample_mass_kernel summed the pieces and nothing has been cut since: a row cut by top_p
+  // alone that could not be settled from the candidates of its pieces)
+  const bool mass_known = part_mass != nullptr && !(typ < 1.0f) && !(k > 0 && k < vocab);
   unsigned long long part = 0;
-  if (need_mass_now) {
+  if (need_mass_now && !mass_known) {
     walk_row(x, vocab, [&](float v) {   // (integer sums, any order)
       if (float_key(v) >= floor_key) part += fix_mass(v, maxv);
     });
   }
   unsigned long long Z = 0;
-  if (need_mass_now) block_excl_scan(part, scan, &Z);
+  if (need_mass_now && mass_known) {
+    for (int i = 0; i < SMP_CHUNKS; ++i) Z += part_mass[(size_t)row * SMP_CHUNKS + i];
+  } else if (need_mass_now) {
+    block_excl_scan(part, scan, &Z);
+  }
 
   // 5. top_p: the shortest prefix by descending probability whose mass reaches top_p
   if (tp < 1.0f && tp > 0.f) {
