@@ -30,7 +30,7 @@ class Engine:
                  gpu_memory_utilization: float = 0.9, max_batch_size: int = 64,
                  max_seq_len: Optional[int] = None, max_num_batched_tokens: int = 2048,
                  prefill_chunk_size: int = 512, device: str = "cuda:0", use_graph: bool = True,
-                 chain_steps: bool = True, fill_budget: bool = True):
+                 chain_steps: bool = True, fill_budget: bool = True, admit_headroom: Optional[float] = 0.02):
         """``model``: a folder with config.json and safetensors, or (with ``random_weights``) a typed
         configuration such as ``LlamaConfig``/``PRESETS[name]``.
         ``kv_pages``: cache pages per group; by default as many as ``gpu_memory_utilization`` of the
@@ -41,7 +41,9 @@ class Engine:
         ``chain_steps``: while every running request is decoding and nobody waits, the next step is queued
         behind the sampling kernel (its tokens stay on the device) before the host has read this step's
         tokens, so the GPU does not wait for the host between steps; a request that ends on the token just
-        read has then one row computed for nothing.  What the caller sees does not change."""
+        read has then one row computed for nothing.  What the caller sees does not change.
+        ``admit_headroom``: share of the cache pages that an admission leaves free beside running requests (None:
+        a request comes in as soon as its first portion fits; see ``SchedulerConfig.admit_headroom``)."""
         self.device = torch.device(device)
         if isinstance(model, str):
             if random_weights:
@@ -59,12 +61,14 @@ class Engine:
         self.page_size = int(page_size)
         if kv_pages is None:
             kv_pages = self._pages_from_memory(gpu_memory_utilization, max_batch_size)
-        self.runner = ModelRunner(self.model, self.page_size, int(kv_pages), max_requests=max_batch_size,
+        # (one request slot more than the scheduler hands out: ``forward`` and ``dump`` run their fresh request in it
+        # also while ``max_batch_size`` requests are live)
+        self.runner = ModelRunner(self.model, self.page_size, int(kv_pages), max_requests=max_batch_size + 1,
                                   use_graph=use_graph)
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_batch_size, max_num_batched_tokens=max_num_batched_tokens,
                             prefill_chunk_size=prefill_chunk_size, max_model_len=self.max_seq_len,
-                            fill_budget=fill_budget),
+                            fill_budget=fill_budget, admit_headroom=admit_headroom),
             self.runner.cache)
         self.sampler = Sampler(spec.vocab_size, self.device, default_seed=seed)
         self._ids = itertools.count()
@@ -87,7 +91,7 @@ class Engine:
         free, _total = torch.cuda.mem_get_info(self.device)
         workspace = 2 << 30            # activations of the largest step, logits, sampler scratch
         # the fixed-size state of every request slot comes out of the same memory
-        state_bytes = sum((max_batch_size + 1) * torch.Size(s.shape).numel() * torch.empty((), dtype=s.dtype).element_size()
+        state_bytes = sum((max_batch_size + 2) * torch.Size(s.shape).numel() * torch.empty((), dtype=s.dtype).element_size()
                           for s in m.state_specs.values())
         budget = int(free * utilization) - workspace - state_bytes
         return max(1, min(pages_cap, budget // per_page))
@@ -273,9 +277,13 @@ class Engine:
         if self._ahead is not None:      # a queued step's logits live in a graph's output buffer: keep a copy
             self._ahead = (self._ahead[0], ops.take_rows(self._ahead[1]))
         rid = ("forward", next(self._ids))
-        self.runner.add_request(rid)
+        self.runner.add_request(rid)      # (the slot kept back from the scheduler: free whatever else is live)
         try:
             logits = self.runner.step([StepEntry(rid, list(token_ids), [len(token_ids) - 1])])
+        except PagesExhausted as e:
+            e.args = (f"forward: a prompt of {len(token_ids)} tokens needs {e.need} more cache pages of group {e.group} and "
+                      f"the live requests leave {e.free} free; end some of them or give the engine more pages (kv_pages)",)
+            raise
         finally:
             self.runner.end_request(rid)
         return logits[0].cpu()
@@ -354,6 +362,8 @@ class Engine:
         s["preemptions"] = self.scheduler.num_preemptions
         s["pages_high_water"] = list(self.scheduler.pages_high_water)
         s["pages_total"] = [p.num_pages for p in self.runner.cache.pools]
+        # share of the held token places that hold no token (/root/reference/engine/src/kv_cache.rs:1066-1074)
+        s["waste_ratio"] = self.runner.cache.waste_ratio()
         s["cache_bytes"] = self.runner.pools.bytes()
         s["weight_bytes"] = self.model.weight_bytes()
         s["graph_steps"] = self.runner.graph_steps

@@ -18,6 +18,7 @@ This module is host logic only; it needs a cache manager's bookkeeping, no GPU.
 """
 from __future__ import annotations
 
+import math
 from collections import deque
 from dataclasses import dataclass, field
 from enum import Enum
@@ -85,6 +86,11 @@ class SchedulerConfig:
     max_model_len: int = 4096               # the reference's --max-seq-len
     portion_align: int = 8                  # a prompt portion that is not the last ends at a multiple of this
     fill_budget: bool = True                # budget that no other request can use lengthens the portions in the plan
+    #: share of every page pool that an admission must leave free while other requests run (never less than one page
+    #: for each of them and one for the newcomer): the reference stops admitting below a headroom of free tokens
+    #: "to prevent admit/requeue spinning when the pool is full", with an exception for an idle pool
+    #: (/root/reference/server/src/engine_task.rs:12-16,626-657)
+    admit_headroom: Optional[float] = 0.02  # None: no headroom, a request comes in as soon as its first portion fits
 
 
 @dataclass
@@ -146,27 +152,51 @@ class Scheduler:
         return bool(self.waiting or self.running)
 
     # ---- one step's plan -------------------------------------------------
-    def _portion(self, req: Request, budget: int, alone: bool) -> int:
+    def _portion(self, req: Request, budget: int) -> int:
         """Tokens of the request's prompt for this step: what is left, at most a chunk, at most the budget.  A
-        portion that is cut short of the prompt's end is cut at a multiple of ``portion_align`` positions, so that
-        the next one starts there (cache rows are written in aligned groups of eight where they can be); when
-        not even one such multiple is in reach the request waits for the next step (0), unless the step has no
-        other work (``alone``): then it takes what it can get."""
+        portion that is cut short of the prompt's end is cut at a multiple of ``portion_align`` positions where it
+        reaches one at the price of less than half its tokens, so that the next one starts there (cache rows are
+        written in aligned groups of eight where they can be).  Otherwise (a chunk size or a rest of the budget
+        about as small as the alignment) it takes the tokens all the same: the alignment buys speed, and a request
+        that waited for an aligned cut beside busy decoders would wait for as long as they run."""
         rest = req.num_tokens - req.num_computed
         count = min(rest, self.config.prefill_chunk_size, budget)
         align = self.config.portion_align
         if count < rest and align > 1:
             over = (req.num_computed + count) % align
-            if over < count:
+            if 2 * over <= count:
                 count -= over
-            elif not alone:
-                count = 0
         return count
 
     def _fits(self, req: Request, count: int, planned: List[int]) -> bool:
         need = self.cache.pages_needed(req.rid, count)
         free = self.cache.free_pages()
         return all(n + p <= f for n, p, f in zip(need, planned, free))
+
+    def _admissible(self, req: Request, count: int, planned: List[int]) -> bool:
+        """May a waiting request join the step with a first portion of ``count`` tokens?  Into an idle engine: when
+        that portion fits.  Beside running requests: when every pool can take ALL the tokens it has to compute (the
+        whole prompt, and for a preempted request its output so far), not only the first portion, and still keeps
+        the headroom free: the running requests go on growing by a page each every ``page_size`` steps, and a
+        request admitted into the last free pages would be evicted again a few steps later, its work thrown away
+        (admitted and preempted in turns, such a request cost two tokens computed for every useful one)."""
+        if not self._fits(req, count, planned):
+            return False
+        if not self.running or self.config.admit_headroom is None:
+            return True
+        ps = self.cache.page_size
+        rest = req.num_tokens - req.num_computed
+        step = min(self.config.prefill_chunk_size, self.config.max_num_batched_tokens)
+        free = self.cache.free_pages()
+        for g, pool in enumerate(self.cache.pools):
+            spec = self.cache.groups[g]
+            held = rule_of(spec.kind).held_tokens(spec, rest, step)
+            if held < rest:
+                held = min(rest, held + ps)
+            headroom = max(math.ceil(self.config.admit_headroom * pool.num_pages), len(self.running) + 1) * (1 + req.preemptions)
+            if (held + ps - 1) // ps + headroom + planned[g] > free[g]:
+                return False
+        return True
 
     def _preempt(self, victim: Request) -> None:
         self.cache.release(victim.rid)
@@ -198,7 +228,7 @@ class Scheduler:
                 continue
             if budget <= 0:
                 break
-            count = 1 if req.is_decoding else self._portion(req, budget, not items)
+            count = 1 if req.is_decoding else self._portion(req, budget)
             if count == 0:
                 continue
             while not self._fits(req, count, planned):
@@ -221,8 +251,8 @@ class Scheduler:
                 if len(self.cache.live_requests()) >= self.cache.max_requests:
                     break
                 self.cache.add(req.rid)
-            count = self._portion(req, budget, not items)
-            if count == 0 or not self._fits(req, count, planned):
+            count = self._portion(req, budget)
+            if count == 0 or not self._admissible(req, count, planned):
                 self.cache.release(req.rid)
                 break
             self.waiting.popleft()

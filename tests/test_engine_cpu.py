@@ -142,7 +142,8 @@ def test_generate_and_preemption_on_host(tiny_dirs, fill_budget):
     want = [plain.greedy_generate(cfg, W, p, 12) for p in prompts]
     roomy = Engine(tiny_dirs.path("A"), kv_pages=32, **kw)
     assert roomy.generate(prompts, params) == want
-    tight = Engine(tiny_dirs.path("A"), kv_pages=3, **kw)       # (the longest request alone needs all three pages)
+    # (the longest request alone needs all three pages; without the admission headroom, so that requests are evicted)
+    tight = Engine(tiny_dirs.path("A"), kv_pages=3, admit_headroom=None, **kw)
     assert tight.generate(prompts, params) == want
     assert tight.stats()["preemptions"] > 0 and tight.runner.cache.free_pages() == [3]
 

@@ -80,8 +80,8 @@ def test_mixed_steps_decoding_first_and_budget():
     assert sorted(r.rid for r in sched.finished) == ["a", "b", "c"]
     assert [len(r.output) for r in sorted(sched.finished, key=lambda r: r.rid)] == [30, 2, 2]
     # first step: a's whole prompt (5); b gets what is left of the budget of 20, cut at a multiple of 8 positions;
-    # the 7 that remain reach no multiple of 8 of c's 9 tokens: c waits
-    assert steps[0] == [("a", 0, 5, True), ("b", 0, 8, False)]
+    # the 7 that remain reach no multiple of 8 of c's 9 tokens: c takes them all the same
+    assert steps[0] == [("a", 0, 5, True), ("b", 0, 8, False), ("c", 0, 7, False)]
 
 
 def test_portions_end_at_aligned_positions():
@@ -171,11 +171,83 @@ def test_no_request_lost_under_a_tiny_pool(seed):
             continue
         sched.add_request(req(i, n, max_new=k))
         want[i] = k
-    run(sched, cache)
+    steps = run(sched, cache)
     got = {r.rid: len(r.output) for r in sched.finished}
     assert got == want
     assert cache.free_pages() == [12]
     assert sched.pages_high_water[0] <= 12
+    # and not by computing everything over and over: what preemptions threw away stays below what was kept
+    useful = sum(len(r.prompt) + len(r.output) - 1 for r in sched.finished)
+    assert sum(c for st in steps for _, _, c, _ in st) - useful <= useful // 2
+
+
+def thrash_scenario(**cfg):
+    sched, cache = make(page_size=8, max_num_batched_tokens=256, prefill_chunk_size=128, **cfg)
+    rs = [req(i, 120, max_new=200) for i in range(4)]
+    for r in rs:
+        sched.add_request(r)
+    steps = run(sched, cache, token_of=lambda r: 1000 * r.rid + len(r.output))
+    return sched, rs, sum(c for st in steps for _, _, c, _ in st)
+
+
+def test_admission_keeps_headroom_so_that_a_full_pool_is_not_admit_then_preempt():
+    """Four requests of 120 + 200 tokens in a pool of 512 places: each alone needs 320, so they cannot all run to
+    their ends at once.  Admitted whenever a first portion fits, the later ones were evicted a few steps after every
+    admission (29 preemptions, two tokens recomputed for every useful one).  With the headroom
+    (/root/reference/server/src/engine_task.rs:12-16,626-657) a request comes in only when all it has to compute
+    fits beside a page of growth for everybody: same tokens as with room for all, at most four preemptions, and
+    less thrown away than kept."""
+    sched, rs, ran = thrash_scenario(num_pages=64)
+    roomy, rs_roomy, ran_roomy = thrash_scenario(num_pages=256)
+    assert roomy.num_preemptions == 0 and ran_roomy == 4 * (120 + 199)
+    assert [r.output for r in rs] == [r.output for r in rs_roomy]
+    assert all(len(r.output) == 200 for r in rs)
+    assert sched.num_preemptions <= 4
+    useful = 4 * (120 + 199)
+    assert ran - useful <= useful, f"{ran - useful} tokens recomputed for {useful} useful ones"
+    # the idle-pool exception: a pool that is smaller than prompt + headroom still admits when nothing runs
+    sched, cache = make(num_pages=16, page_size=8, max_num_batched_tokens=256, prefill_chunk_size=128, admit_headroom=0.5)
+    sched.add_request(req("a", 120, max_new=4))
+    sched.add_request(req("b", 120, max_new=4))
+    steps = run(sched, cache)
+    assert sched.num_preemptions == 0 and sorted(r.rid for r in sched.finished) == ["a", "b"]
+    assert all(len({rid for rid, *_ in st}) == 1 for st in steps), "b waits for a: 15 pages + headroom do not fit beside it"
+
+
+def test_a_chunk_or_a_rest_of_the_budget_below_the_alignment_is_still_used():
+    """Alignment buys speed, never a turn: with chunks of 4 tokens (below the alignment of 8) three prompts all
+    advance in every step, and a prompt beside five decoding requests under a budget of 12 takes the 7 tokens left
+    of it step by step instead of waiting until the decoders are done."""
+    sched, cache = make(prefill_chunk_size=4, max_num_batched_tokens=32)
+    for i in range(3):
+        sched.add_request(req(i, 40, max_new=2))
+    steps = run(sched, cache)
+    assert steps[0] == [(0, 0, 4, False), (1, 0, 4, False), (2, 0, 4, False)]
+    firsts = {}
+    for n, st in enumerate(steps):
+        for rid, _, _, samples in st:
+            if samples:
+                firsts.setdefault(rid, n)
+    assert max(firsts.values()) - min(firsts.values()) <= 1, firsts
+    sched, cache = make(max_num_batched_tokens=12, prefill_chunk_size=16)
+    for i in range(5):
+        sched.add_request(req(i, 2, max_new=400))
+    for _ in range(2):                        # the five reach decoding (12 tokens of budget: 2+2+2+2+2)
+        items = sched.schedule()
+        for it in items:
+            cache.reserve(it.request.rid, it.count); cache.commit(it.request.rid, it.count); sched.advance(it)
+            if it.samples:
+                sched.append_token(it.request, 7)
+    sched.add_request(req("late", 30, max_new=1))
+    seen = []
+    for _ in range(6):
+        items = sched.schedule()
+        seen.append([(it.request.rid, it.start, it.count) for it in items if it.request.rid == "late"])
+        for it in items:
+            cache.reserve(it.request.rid, it.count); cache.commit(it.request.rid, it.count); sched.advance(it)
+            if it.samples and sched.append_token(it.request, 7):
+                sched.finish(it.request)
+    assert seen[:5] == [[("late", 0, 7)], [("late", 7, 7)], [("late", 14, 7)], [("late", 21, 7)], [("late", 28, 2)]], seen
 
 
 def test_abort_frees_at_once_wherever_the_request_stands():
