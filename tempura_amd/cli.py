@@ -88,6 +88,14 @@ def cmd_run(args) -> int:
                             presence_penalty=args.presence_penalty, frequency_penalty=args.frequency_penalty,
                             seed=args.sampling_seed, max_new_tokens=args.max_new_tokens,
                             eos_token_id=args.eos_token, ignore_eos=args.ignore_eos)
+    if args.dump_logits:
+        # The logits after each prompt's last token, from a fresh request that runs the whole prompt
+        # (the reference's logits probe: /root/reference/server/src/api.rs:1154-1183; float32 little-endian
+        # rows as /root/reference/tests-ggml/llama_logitprobe.cpp:20-30 writes them), [prompts, vocab].
+        import numpy as np
+        with open(args.dump_logits, "wb") as f:
+            for p in prompts:
+                f.write(np.ascontiguousarray(eng.forward(p).numpy(), dtype="<f4").tobytes())
     t0 = time.time()
     outs = eng.generate(prompts, params)
     dt = time.time() - t0
@@ -182,6 +190,8 @@ def main(argv=None) -> int:
     p.add_argument("--eos-token", type=int, action="append", default=None, help="stop token id (repeatable)")
     p.add_argument("--ignore-eos", action="store_true")
     p.add_argument("--stats", action="store_true", help="print counters to standard error")
+    p.add_argument("--dump-logits", metavar="PATH",
+                   help="write the logits after every prompt's last token to PATH (float32 little-endian, [prompts, vocab])")
     p.set_defaults(fn=cmd_run)
 
     p = sub.add_parser("random-model", help="write a folder with config.json and seeded random weights")

@@ -470,6 +470,12 @@ int cc_fill_step(void* h, int n, const int* reqs, const int* n_new, const int* t
     max_ctx = std::max(max_ctx, (int)end);
     singles += n_new[i] == 1;
     for (int g = 0; g < G; ++g) {
+      // every new position must get a page: a rule whose first visible key lies beyond the query's own position
+      // (a fault of a newly registered rule) would leave the step's first tokens without one; refused here,
+      // before anything is reserved or written
+      if (std::max(c->first_needed(g, r->num_tokens), r->first_live[g]) > r->num_tokens / ps)
+        return fail("entry %d: position %d has no page in group %d (its rule hides the position from its own query)", i,
+                    r->num_tokens, g);
       width[g] = std::max(width[g], std::max((int)r->tables[g].size(), (int)((end + ps - 1) / ps)));
       need[g] += c->pages_needed(*r, g, n_new[i]);
     }

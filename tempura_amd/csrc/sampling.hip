@@ -1468,6 +1468,18 @@ __global__ __launch_bounds__(SMP_THREADS) void top_logprobs_kernel(const float* 
   }
 }
 
+// The sizes that the scratch buffers of tp_sample are laid out by, for the caller that allocates them: pieces of a row,
+// candidates a piece may hand over, largest top_k settled from candidates, most elements of a piece, bins of a counting pass.
+extern "C" int tp_sample_limits(int* out5) {
+  TP_REQUIRE(out5 != nullptr, "sample_limits: no output");
+  out5[0] = SMP_CHUNKS;
+  out5[1] = SMP_CCAP;
+  out5[2] = SMP_KMAX;
+  out5[3] = SMP_PER_MAX;
+  out5[4] = 256;
+  return 0;
+}
+
 extern "C" int tp_sample(const float* logits, float* work, int rows, int vocab, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p, const float* typical_p,
                          const float* rnd, int* out, float* info, float* part_max, unsigned long long* part_mass,

@@ -779,6 +779,22 @@ def apply_penalties(logits: torch.Tensor, rows, tokens, counts, in_window, prese
           _ptr(fl[0]), _ptr(fl[1]), _ptr(fl[2]), n, _stream())
 
 
+_SAMPLE_LIMITS: Optional[tuple] = None
+
+
+def _sample_limits() -> tuple:
+    """(pieces of a row, candidates per piece, largest top_k settled from candidates, most elements of a piece,
+    bins of a counting pass) as the sampling kernels were compiled; ``sample`` sizes their scratch by these."""
+    global _SAMPLE_LIMITS
+    if _SAMPLE_LIMITS is None:
+        buf = (ctypes.c_int * 5)()
+        lib = _Library.get()
+        if lib.tp_sample_limits(buf) != 0:
+            raise KernelError(f"tp_sample_limits: {lib.tp_last_error().decode()}")
+        _SAMPLE_LIMITS = tuple(int(v) for v in buf)
+    return _SAMPLE_LIMITS
+
+
 def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, min_p, rnd, typical_p=None,
            info: Optional[torch.Tensor] = None, settled: Optional[list] = None) -> torch.Tensor:
     """float32 [m, vocab] and per-row options (host arrays) -> int32 [m] chosen tokens.
@@ -806,30 +822,33 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature, top_k, top_p, 
     fl, tk = _Staging.send([np.asarray([temperature, top_p, min_p, rnd, typical_p], dtype=np.float32),
                             np.asarray(top_k, dtype=np.int32)], dev)
     out = torch.empty((m,), dtype=torch.int32, device=dev)
-    part_max = torch.empty((m * 32,), dtype=torch.float32, device=dev)    # (maxima of 32 pieces of each row)
+    # (the scratch buffers are laid out by the library's own sizes, asked of it once: pieces of a row, candidates a
+    # piece may hand over, the largest top_k settled from candidates, the most elements of a piece, bins of a pass)
+    pieces, ccap, kmax, per_max, bins = _sample_limits()
+    part_max = torch.empty((m * pieces,), dtype=torch.float32, device=dev)    # (maxima of the pieces of each row)
     # rows that are only scaled (and cut by min_p) before the draw get the masses of their pieces from a kernel
     # of many blocks; worth it when there is such a row
     plain_rows = any(t > 0 and not (0 < k < vocab) and not (0.0 < p < 1.0) and not (ty < 1.0)
                      for t, k, p, ty in zip(temperature, top_k, top_p, typical_p))
     # rows cut by top_p alone are settled from the candidates of their pieces against the mass of the whole row
-    piece_ok = -(-vocab // 32) <= 8192 and info is None
-    topp_rows = piece_ok and vocab > 128 and any(
+    piece_ok = -(-vocab // pieces) <= per_max and info is None
+    topp_rows = piece_ok and vocab > kmax and any(
         t > 0 and not (0 < k < vocab) and 0.0 < p < 1.0 and not (ty < 1.0)
         for t, k, p, ty in zip(temperature, top_k, top_p, typical_p))
-    part_mass = torch.empty((m * 32,), dtype=torch.int64, device=dev) if (plain_rows or topp_rows) and info is None else None
+    part_mass = torch.empty((m * pieces,), dtype=torch.int64, device=dev) if (plain_rows or topp_rows) and info is None else None
     # rows cut by top_k have the first pass of their selection counted by the kernel of many blocks that scales the row
     # ... unless top_k is small: such a row is settled from the few candidates that each piece of it hands over
-    small = lambda k, ty: 0 < k <= 128 and not (ty < 1.0) and piece_ok
+    small = lambda k, ty: 0 < k <= kmax and not (ty < 1.0) and piece_ok
     topk_rows = [(k, ty) for t, k, ty in zip(temperature, top_k, typical_p) if t > 0 and 0 < k < vocab]
     part_cnt = None
     if any(not small(k, ty) for k, ty in topk_rows):
-        part_cnt = torch.empty((m * 32 * 256,), dtype=torch.int32, device=dev)
+        part_cnt = torch.empty((m * pieces * bins,), dtype=torch.int32, device=dev)
     cand_val = cand_idx = cand_cnt = cand_thr = done = None
     if topp_rows or any(small(k, ty) for k, ty in topk_rows):
-        cand_val = torch.empty((m * 32 * 160,), dtype=torch.float32, device=dev)
-        cand_idx = torch.empty((m * 32 * 160,), dtype=torch.int32, device=dev)
-        cand_cnt = torch.empty((m * 32,), dtype=torch.int32, device=dev)
-        cand_thr = torch.empty((m * 32,), dtype=torch.int32, device=dev)
+        cand_val = torch.empty((m * pieces * ccap,), dtype=torch.float32, device=dev)
+        cand_idx = torch.empty((m * pieces * ccap,), dtype=torch.int32, device=dev)
+        cand_cnt = torch.empty((m * pieces,), dtype=torch.int32, device=dev)
+        cand_thr = torch.empty((m * pieces,), dtype=torch.int32, device=dev)
         done = torch.empty((m,), dtype=torch.int32, device=dev)
     if info is not None:
         _dev_ok(info)

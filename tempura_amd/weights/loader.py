@@ -15,7 +15,10 @@ types) are reported in ONE error; the reference stops at the first
 A folder may hold ``integrity.json``, ``{"tensor_hashes": {name: sha256 of the stored
 bytes}}``; every tensor it names is then verified while it is loaded
 (/root/reference/engine/src/loader.rs:147-182 hashes the widened float32 values; here
-the bytes as stored, so that a bfloat16 checkpoint is never widened just to be hashed).
+the bytes as stored, so that a bfloat16 checkpoint is never widened just to be hashed;
+a digest that fits neither the stored bytes of a BF16 or F16 tensor is tried against the
+widened values before the tensor is refused, so that a manifest made the reference's way
+verifies here too).
 """
 from __future__ import annotations
 
@@ -23,6 +26,7 @@ import glob
 import hashlib
 import json
 import os
+import warnings
 from typing import Callable, Dict, List, Optional
 
 import torch
@@ -88,6 +92,15 @@ class Checkpoint:
     def sha256(self, name: str) -> str:
         """Hex digest of the tensor's bytes as stored."""
         t = self._where[name].tensor(name).contiguous()
+        return hashlib.sha256(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"").hexdigest()
+
+    def sha256_widened(self, name: str) -> Optional[str]:
+        """Hex digest of a BF16 or F16 tensor's values widened (exactly) to little-endian float32, which is what
+        the reference hashes (/root/reference/engine/src/loader.rs:147-182); None for other stored types, whose
+        widened form is the stored one."""
+        if self.dtype_tag(name) not in ("BF16", "F16"):
+            return None
+        t = self._where[name].tensor(name).to(torch.float32).contiguous()
         return hashlib.sha256(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"").hexdigest()
 
     def close(self) -> None:
@@ -175,9 +188,16 @@ def load_into(model, model_dir: str, verify: Optional[bool] = None) -> None:
             raise WeightsError(f"missing tensor {name}", [name])
         if manifest and name in manifest:
             got = ckpt.sha256(name)
-            if got != manifest[name].lower():
+            if got != manifest[name].lower() and ckpt.sha256_widened(name) != manifest[name].lower():
                 raise WeightsError(f"tensor {name} fails its integrity check: expected sha256 {manifest[name]}, got {got}")
         return ckpt.tensor(name)
 
+    # a tied output head reads the embedding matrix; a matrix of its own that the checkpoint still holds is not
+    # an error (/root/reference/engine/src/weights.rs:156-166 falls back to the embedding only when it is absent),
+    # but the user should know that it is not what runs
+    ignored = sorted(n for n, info in expected.items() if info.init == "skip" and n in have)
+    if ignored:
+        warnings.warn(f"checkpoint in {model_dir} holds {', '.join(ignored)}, but the configuration ties that tensor to "
+                      f"another (tie_word_embeddings): the stored tensor is ignored", stacklevel=2)
     model.load_weights(get)
     ckpt.close()

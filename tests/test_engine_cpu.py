@@ -261,3 +261,32 @@ def test_toy_block_arrangements_with_other_parts_register_build_and_step(tmp_pat
     from tempura_amd.parts import part_class
     with pytest.raises(ValueError, match="missing"):
         part_class("block", "prenorm")(LayerSpec("prenorm", {"mixer": spec.layers[1].mixer}), cfg.hidden_size, torch.float32, "cpu")
+
+
+def test_forward_while_every_request_slot_is_live_and_the_waste_ratio(tiny_dirs):
+    """``Engine.forward`` runs a fresh request of its own; the engine keeps one request slot back for it, so it
+    works while ``max_batch_size`` requests are running, and refuses with a message that names the pages when
+    the live requests leave too few.  ``stats()`` reports the share of held cache places that hold no token
+    (/root/reference/engine/src/kv_cache.rs:1066-1074)."""
+    from tempura_amd import Engine, SamplingParams
+    from tempura_amd.cache import PagesExhausted
+    cfg, W = tiny_dirs.plain_model("A")
+    eng = Engine(tiny_dirs.path("A", "float32"), dtype="float32", device="cpu", page_size=16, kv_pages=8, max_batch_size=2)
+    prompts = [helpers.random_tokens(256, n, seed=40 + n) for n in (5, 20)]
+    for p in prompts:
+        eng.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=8))
+    eng.step(); eng.step()
+    assert len(eng.scheduler.running) == 2
+    st = eng.stats()
+    held = 1 * 16 + 2 * 16                       # 5 + 1 cached tokens hold one page, 20 + 1 hold two
+    assert abs(st["waste_ratio"] - (1 - (6 + 21) / held)) < 1e-6
+    probe = helpers.random_tokens(256, 30, seed=99)
+    got = eng.forward(probe)
+    ref = plain.forward(cfg, W, probe)
+    assert float((got.double() - ref[-1]).abs().max() / ref.abs().max()) < 1e-6
+    with pytest.raises(PagesExhausted, match="forward: a prompt of 100 tokens"):
+        eng.forward(helpers.random_tokens(256, 100, seed=98))          # 7 pages, 5 are free
+    while eng.has_unfinished():
+        eng.step()
+    assert [eng.request(i).output for i in range(2)] == [plain.greedy_generate(cfg, W, p, 8) for p in prompts]
+    assert eng.runner.cache.free_pages() == [8] and eng.stats()["waste_ratio"] == 0.0

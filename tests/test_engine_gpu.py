@@ -278,6 +278,20 @@ def test_command_line(tiny_dirs, tmp_path):
     rec = json.loads(p.stdout.strip().splitlines()[-1])
     assert rec["output_ids"] == plain.greedy_generate(cfg, W, prompt, 6) and rec["finish_reason"] == "length"
     assert '"stats"' in p.stderr
+    # --dump-logits: the logits after the last token of every prompt, float32 little-endian, against the plain implementation
+    prompts = [prompt, helpers.random_tokens(256, 21, seed=602)]
+    ids = tmp_path / "ids.txt"
+    ids.write_text("\n".join(" ".join(map(str, q)) for q in prompts) + "\n")
+    out = tmp_path / "logits.f32"
+    p = subprocess.run([sys.executable, tempura, "run", "--model", model, "--dtype", "float32", "--prompt-file", str(ids),
+                        "--max-new-tokens", "2", "--temperature", "0", "--kv-blocks", "16", "--max-batch-size", "2",
+                        "--dump-logits", str(out)], capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    import numpy as np
+    got = torch.from_numpy(np.fromfile(out, dtype="<f4").reshape(2, 256).copy()).double()
+    for row, q in zip(got, prompts):
+        want = plain.forward(cfg, W, q)
+        assert float((row - want[-1]).abs().max() / want.abs().max()) <= helpers.float32_bound(cfg)
     p = subprocess.run([sys.executable, tempura, "profile", "--model", model, "--dtype", "float32", "--prompt-len", "12",
                         "--batch", "2", "--decode-steps", "2", "--kv-blocks", "16", "--max-batch-size", "2", "--json"],
                        capture_output=True, text=True, timeout=600)

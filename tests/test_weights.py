@@ -175,3 +175,43 @@ def test_integrity_manifest(tmp_path):
         json.dump(m, f)
     with pytest.raises(WeightsError, match="ghost"):
         load_into(model, d)
+
+
+def test_a_manifest_of_widened_values_verifies_too(tmp_path):
+    """The reference hashes every tensor as float32 values (/root/reference/engine/src/loader.rs:147-182): a manifest
+    made that way for a bfloat16 checkpoint is accepted, a wrong digest still is not."""
+    import hashlib
+    from tempura_amd.weights.loader import MANIFEST_NAME
+    cfg, model = _model("A")
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=3, dtype="bfloat16")
+    ck = Checkpoint(d)
+    hashes = {n: hashlib.sha256(ck.tensor(n).to(torch.float32).contiguous().numpy().tobytes()).hexdigest() for n in ck.names()}
+    ck.close()
+    with open(os.path.join(d, MANIFEST_NAME), "w") as f:
+        json.dump({"tensor_hashes": hashes}, f)
+    load_into(model, d, verify=True)
+    name = "model.layers.0.self_attn.o_proj.weight"
+    hashes[name] = hashes["model.layers.1.self_attn.o_proj.weight"]
+    with open(os.path.join(d, MANIFEST_NAME), "w") as f:
+        json.dump({"tensor_hashes": hashes}, f)
+    with pytest.raises(WeightsError, match="o_proj.weight fails its integrity check"):
+        load_into(model, d)
+
+
+def test_a_tied_model_warns_about_an_output_matrix_it_ignores(tmp_path):
+    """/root/reference/engine/src/weights.rs:156-166 uses the embedding matrix only when the output matrix is absent;
+    here the configuration's tie decides, and a stored matrix that is not used is said so."""
+    import warnings
+    cfg, model = _model("B")
+    w = dict(random_weights(cfg, 1, dtype="float32"))
+    assert "lm_head.weight" not in w
+    w["lm_head.weight"] = torch.zeros_like(w["model.embed_tokens.weight"])
+    os.makedirs(tmp_path / "m")
+    write_safetensors(str(tmp_path / "m" / "model.safetensors"), w.items())
+    with pytest.warns(UserWarning, match="lm_head.weight.*ignored"):
+        load_into(model, str(tmp_path / "m"))
+    assert model.lm_head.weight.data_ptr() == model.embedding.weight.data_ptr()
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        d = write_random_model(cfg, str(tmp_path / "m2"), seed=1, dtype="float32")
+        load_into(model, d)           # nothing ignored, nothing said
