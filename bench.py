@@ -4,8 +4,11 @@ random weights, synthetic token ids.
 
     python bench.py --gpus 1 --steps K --warmup W
 
-A "step" is one decode step of the whole batch (default 8 requests whose caches hold 2,048 tokens each
-when timing starts).  The headline runs through the engine's own entry point: `Engine.add_request` and
+A "step" is one decode step of the whole batch (default 8 requests).  The timed steps are centred on a cache
+length of 3,072 tokens, the middle of the named sweep from 2,048 to 4,096: the default 2,000 steps cover the
+sweep itself (prompts of 2,048 tokens), a short run (`--steps 20`) starts from prompts of about 3,050 tokens and
+times the steps around 3,072, so that a step reads what a step of the sweep reads on average; `metric` names
+the range that was timed.  The headline runs through the engine's own entry point: `Engine.add_request` and
 `Engine.step`, with its scheduler, step function and sampler (greedy), as `tempura run` does.  Prints ONE
 JSON line: decoded tokens per second (`value`), the step's share of the HBM roofline, the 2,048-token
 prefill, and under `points`: batch 1 and 64 through the engine, the same three batches through the bare
@@ -190,11 +193,13 @@ def main() -> int:
             runner.end_request(rid)
         return batch * n_steps / dt, 1e3 * dt / n_steps
 
-    def prefill_point(eng, cfg, T, runs):
-        """One prompt of T tokens from an empty cache as one step; mean of `runs` after two warm-ups."""
+    def prefill_point(eng, cfg, T, runs, warm=3):
+        """One prompt of T tokens from an empty cache as one step; mean of `runs` after `warm` warm-ups, a fresh
+        request (no cached keys) each time (/root/reference/tools/bench-gpu/src/bench_real_model.rs:160-278: warm-ups,
+        then timed forwards on fresh sessions, tokens a second from the mean time)."""
         runner = eng.runner
         times = []
-        for i in range(2 + runs):
+        for i in range(warm + runs):
             rid = ("p", T, i)
             runner.add_request(rid)
             toks = prompt(cfg.vocab_size, T)
@@ -204,7 +209,7 @@ def main() -> int:
             torch.cuda.synchronize()
             dt = time.perf_counter() - t
             runner.end_request(rid)
-            if i >= 2:
+            if i >= warm:
                 times.append(dt)
         ms = 1e3 * sum(times) / len(times)
         L, H, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
@@ -308,12 +313,18 @@ def main() -> int:
         steps = max(1, args.context - args.prompt_len - warmup - 2)
     points = {}
 
+    def centred(n_warm, n_steps):
+        """The prompt length from which n_warm untimed and n_steps timed steps are centred on the middle of the
+        sweep from --prompt-len to --context (never below --prompt-len)."""
+        mid = (args.prompt_len + args.context) // 2
+        return max(args.prompt_len, mid - n_warm - n_steps // 2)
+
     prefill = None
     if not args.no_prefill:
-        prefill = prefill_point(eng, cfg, args.prompt_len, 5)
+        prefill = prefill_point(eng, cfg, args.prompt_len, 10)
         say(f"prefill {prefill}")
 
-    head = engine_decode(eng, cfg, weight_bytes, args.batch, args.prompt_len, warmup, steps)
+    head = engine_decode(eng, cfg, weight_bytes, args.batch, centred(warmup, steps), warmup, steps)
     say(f"engine decode b{args.batch}: {head['tps']:.1f} tok/s, {head['ms']:.3f} ms/step (p50 {head['p50']:.3f}, p95 {head['p95']:.3f}), KV {head['kv']}")
     achieved = head["bytes"] / (head["ms"] / 1e3) / 1e9
 
@@ -325,18 +336,19 @@ def main() -> int:
     if not args.no_points:
         ps = max(1, min(args.point_steps, steps))
         for b in (1, 64):
-            r = engine_decode(eng, cfg, weight_bytes, b, args.prompt_len, 8, ps)
+            r = engine_decode(eng, cfg, weight_bytes, b, centred(8, ps), 8, ps)
             points[f"decode_b{b}"] = round(r["tps"], 1)
             points[f"decode_b{b}_hbm_frac"] = round(r["bytes"] / (r["ms"] / 1e3) / 1e9 / HBM_PEAK_GBS, 4)
             say(f"engine decode b{b}: {r['tps']:.1f} tok/s, {r['ms']:.3f} ms/step")
         for b in sorted({1, args.batch, 64}):
             # (the same number of steps, so the same range of context lengths, as the engine's figure it stands beside)
-            tps, ms = runner_decode(eng, cfg, b, args.prompt_len, warmup if b == args.batch else 8, steps if b == args.batch else ps)
+            nw, ns = (warmup, steps) if b == args.batch else (8, ps)
+            tps, ms = runner_decode(eng, cfg, b, centred(nw, ns), nw, ns)
             points[f"runner_b{b}"] = round(tps, 1)
             say(f"step function alone b{b}: {tps:.1f} tok/s, {ms:.3f} ms/step")
         if not args.no_long:
             for T in (8192, 32768):
-                p = prefill_point(eng, cfg, T, 2)
+                p = prefill_point(eng, cfg, T, 3 if T <= 8192 else 2, warm=2)
                 points[f"prefill_{T}"] = p["value"]
                 points[f"prefill_{T}_frac"] = p["frac"]
                 say(f"prefill {p}")

@@ -71,7 +71,8 @@ class Engine:
                             fill_budget=fill_budget, admit_headroom=admit_headroom),
             self.runner.cache)
         self.sampler = Sampler(spec.vocab_size, self.device, default_seed=seed)
-        self._ids = itertools.count()
+        self._ids = itertools.count()            # request ids that add_request hands out: 0, 1, 2, ...
+        self._own_ids = itertools.count()        # names of the engine's own short-lived requests (forward, profile)
         self._requests: Dict[Hashable, Request] = {}
         self.counters = {"steps": 0, "prompt_tokens": 0, "generated_tokens": 0, "batched_tokens": 0, "chained_steps": 0}
         self.chain_steps = bool(chain_steps) and self.runner.use_graph     # (a model with parts that cannot be captured runs eagerly)
@@ -276,7 +277,7 @@ class Engine:
         (the reference's ``forward``, /root/reference/engine/src/model.rs:308)."""
         if self._ahead is not None:      # a queued step's logits live in a graph's output buffer: keep a copy
             self._ahead = (self._ahead[0], ops.take_rows(self._ahead[1]))
-        rid = ("forward", next(self._ids))
+        rid = ("forward", next(self._own_ids))
         self.runner.add_request(rid)      # (the slot kept back from the scheduler: free whatever else is live)
         try:
             logits = self.runner.step([StepEntry(rid, list(token_ids), [len(token_ids) - 1])])
@@ -304,7 +305,7 @@ class Engine:
             self._ahead = (self._ahead[0], ops.take_rows(self._ahead[1]))
         g = _random.Random(seed)
         vocab = self.model.spec.vocab_size
-        rids = [("profile", next(self._ids)) for _ in range(batch)]
+        rids = [("profile", next(self._own_ids)) for _ in range(batch)]
         prompts = [[g.randrange(vocab) for _ in range(prompt_len)] for _ in rids]
         runner = self.runner
         keep_graph, runner.use_graph = runner.use_graph, False

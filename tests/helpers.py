@@ -238,3 +238,58 @@ def first_difference(got: torch.Tensor, ref: torch.Tensor, tol: float):
     err = (got.double() - ref.double()).abs().amax(dim=-1) / scale
     bad = torch.nonzero(err > tol)
     return None if bad.numel() == 0 else int(bad[0])
+
+
+# ---- a far key that decides ---------------------------------------------------------------------
+def plant_pointer(cfg: dict, W: Dict[str, torch.Tensor], needles: Sequence[int], probe: int, strength: float = 80.0,
+                  layer: int = 0) -> Dict[str, torch.Tensor]:
+    """Weights (a new dict; float64 values, to be stored in the model's type) in which every head of ``layer``'s
+    attention, at a query that is the token ``probe``, scores about ``strength`` (after the scale) against the key
+    of any token of ``needles``, however far back it lies; every other score stays what the random weights make it
+    (a few units).  The softmax of a probe is then all but one-hot on the needle of its sequence, and a kernel
+    that misses that one key (a page's edge, a split's edge, a page handed to another request) changes the
+    layer's output from the needle's value row to a mixture of the others: the logits move by a large part of
+    their range instead of by rounding.
+
+    How: the rotary pair with the lowest frequency turns by a negligible angle over a few thousand positions
+    (plain.rope_inv_freq), so a product of q and k components in that pair does not depend on the distance.  With
+    x_t the normed embedding of token t (layer 0 sees exactly that), the k rows of that pair's first element get
+    a * g added, g the shortest vector with g . x_n = 1 for every needle n, and the q rows get a * x_p / |x_p|^2,
+    a^2 * scale = strength."""
+    assert layer == 0, "the planted direction is made from normed embeddings, which only layer 0 sees"
+    H = cfg["hidden_size"]
+    nH = cfg["num_attention_heads"]
+    nKV = cfg.get("num_key_value_heads", nH)
+    D = cfg.get("head_dim") or H // nH
+    eps = cfg.get("rms_norm_eps", 1e-5)
+    out = {k: v for k, v in W.items()}
+    emb = W["model.embed_tokens.weight"].double()
+    wn = W["model.layers.0.input_layernorm.weight"].double()
+    xs = plain.rmsnorm(emb[torch.tensor(list(needles) + [probe])], wn, eps)
+    xn, xp = xs[:-1], xs[-1]
+    g = xn.T @ torch.linalg.solve(xn @ xn.T, torch.ones(len(needles), dtype=torch.float64))
+    gp = xp / (xp @ xp)
+    a = (strength * (D ** 0.5)) ** 0.5
+    d = D // 2 - 1                               # the slowest pair's first element, in the checkpoint's split-half order
+    wq = W["model.layers.0.self_attn.q_proj.weight"].double().clone()
+    wk = W["model.layers.0.self_attn.k_proj.weight"].double().clone()
+    for h in range(nH):
+        wq[h * D + d] += a * gp
+    for h in range(nKV):
+        wk[h * D + d] += a * g
+    out["model.layers.0.self_attn.q_proj.weight"] = wq
+    out["model.layers.0.self_attn.k_proj.weight"] = wk
+    return out
+
+
+def pointer_sequence(vocab: int, n: int, needle: int, needle_at: int, probe: int, probes_at: Sequence[int], special: Sequence[int],
+                     seed: int) -> List[int]:
+    """``n`` random tokens that avoid the ``special`` ids, the needle at one place and the probe at others."""
+    g = random.Random(seed)
+    free = [t for t in range(vocab) if t not in set(special)]
+    toks = [g.choice(free) for _ in range(n)]
+    toks[needle_at] = needle
+    for p in probes_at:
+        assert needle_at < p < n
+        toks[p] = probe
+    return toks

@@ -79,8 +79,8 @@ def test_baseline_tiny_workloads(tmp_path):
     and 33 ids, 16 greedy steps, pages of 16) and B with a limit of 256 (prompts of 1, 9, 40, 63 and 120 ids, 24
     steps at temperature 0.8 from seed 2, pages of 8), float32, weights N(0, 0.02) from seeds 0 and 1 with norm
     weights 1.  Greedy tokens equal the plain implementation's; sampled tokens are the same alone and in the
-    batch and every one of them lies in the plain implementation's top 50; and a request that reaches the position
-    limit ends there with the reason max_model_len."""
+    batch and each is the token that the plain sampling rules give on the plain implementation's logits with the
+    same uniform number; and a request that reaches the position limit ends there with the reason max_model_len."""
     from tempura_amd.config import LlamaConfig
     from tempura_amd.engine import Engine
     from tempura_amd.kernels import ops
@@ -110,10 +110,25 @@ def test_baseline_tiny_workloads(tmp_path):
     outs = eng.generate(prompts, params)
     assert all(len(o) == 24 for o in outs)
     assert outs[3] == Engine(db, dtype="float32", page_size=8, kv_pages=32, max_batch_size=1).generate([prompts[3]], params)[0]
-    for p, o in zip(prompts[:3], outs[:3]):
+    # every sampled token is the one that the plain rules give on the plain implementation's logits with the same
+    # uniform number (draw i of the stream with seed 2; /root/reference/kernels/src/sampling.rs:229-333): top-k 50
+    # (the default), temperature 0.8, index-order walk.  The engine's logits are float32, so a draw that lands within
+    # 1e-5 of a step of the cumulative sum may fall on either side; anything else must agree exactly.
+    import numpy as np
+    from tempura_amd.sampling import uniform_draw
+    from test_sampling_gpu import plain_sample
+    checked = 0
+    for p, o in zip(prompts, outs):
         logits = plain.forward(cb, Wb, p + o)
         for i, tok in enumerate(o):
-            assert tok in torch.topk(logits[len(p) + i - 1], 50).indices.tolist(), "a sampled token outside the top 50 (top_k's default)"
+            row = logits[len(p) + i - 1]
+            r = float(np.float32(uniform_draw(2, i)))
+            want = plain_sample(row, 0.8, 50, 1.0, 0.0, r)
+            if tok != want:
+                near = {plain_sample(row, 0.8, 50, 1.0, 0.0, min(max(r + d, 0.0), 1.0 - 1e-9)) for d in (-1e-5, 1e-5)}
+                assert tok in near, f"prompt of {len(p)}: token {i} is {tok}, the plain rules give {want}"
+            checked += 1
+    assert checked == 5 * 24
 
 
 def test_preemption_by_recompute_keeps_tokens(tiny_dirs):
@@ -387,8 +402,11 @@ def test_model_width_mixed_schedule_against_plain(tmp_path):
     some beside single decoded tokens of others, the last 32 tokens of each one by one (decode-only steps replay
     the graph), and so few pages that finished requests' pages are used again; float32 and bfloat16 against the
     plain float64 implementation.  The q and k projections are doubled (scores four times those of N(0, 0.02)
-    weights: a standard deviation of about 6.5 over a few hundred keys), so that attention is sharply peaked and
-    a wrong key or page moves the logits far beyond the bound."""
+    weights: a standard deviation of about 6.5 over a few hundred keys), so that attention is sharply peaked.
+    And every request holds one key that decides (``helpers.plant_pointer``): at its probe positions all of the
+    first layer's attention sits on one far key, at a page's edge, the first key or anywhere, so that a kernel
+    that loses this one key moves those logits by most of their range, far above what bfloat16 explains; the
+    test works out both numbers and compares the probes against the tighter one."""
     from tempura_amd.engine.loading import load_model
     from tempura_amd.engine.runner import ModelRunner
     from tempura_amd.kernels import ops
@@ -399,27 +417,54 @@ def test_model_width_mixed_schedule_against_plain(tmp_path):
     for name in W:
         if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
             W[name] = (W[name].float() * 2.0).to(torch.bfloat16)
+    needles, probe = [8000, 8001, 8002], 8003
+    planted = helpers.plant_pointer(json.loads(cfg.to_json()), W, needles, probe, strength=100.0)
+    for name in ("model.layers.0.self_attn.q_proj.weight", "model.layers.0.self_attn.k_proj.weight"):
+        W[name] = planted[name].to(torch.bfloat16)
+    del planted
     folder = tmp_path / "wide2"
     folder.mkdir()
     (folder / "config.json").write_text(cfg.to_json())
     write_safetensors(str(folder / "model.safetensors"), W.items())
     del W
     pc, PW = plain.read_model_dir(str(folder))
-    lengths = {"w0": 150, "w1": 97, "w2": 210, "w3": 64, "w4": 131, "w5": 40}
-    requests = {rid: helpers.random_tokens(8192, n, seed=300 + i) for i, (rid, n) in enumerate(lengths.items())}
+    # request: (length, needle, its place, probes: in portions and among the last 32 tokens, decoded one by one)
+    layout = {"w0": (150, 8000, 15, [16, 60, 130, 149]), "w1": (97, 8001, 0, [1, 50, 96]), "w2": (210, 8002, 16, [17, 100, 190, 209]),
+              "w3": (64, 8000, 31, [32, 63]), "w4": (131, 8001, 64, [65, 100, 130]), "w5": (40, 8002, 7, [8, 39])}
+    lengths = {rid: n for rid, (n, *_rest) in layout.items()}
+    requests = {rid: helpers.pointer_sequence(8192, n, needle, at, probe, probes, needles + [probe], seed=300 + i)
+                for i, (rid, (n, needle, at, probes)) in enumerate(layout.items())}
     max_tokens = 256 + 192 + 64                 # room for about three requests: pages must come back and be used again
     steps = helpers.schedule_mixed(lengths, max_tokens, seed=9)
     assert max(len(e) for e, _ in steps) >= 3 and any(len(e) > 1 and all(c == 1 for _, _, c in e) for e, _ in steps)
+    missed = {}
+    for rid, (n, needle, at, probes) in layout.items():
+        lost = list(requests[rid])
+        lost[at] = 11
+        missed[rid] = plain.forward(pc, PW, lost)[torch.tensor(probes)]
     for dtype in ("float32", "bfloat16"):
-        refs = {rid: helpers.plain_reference(pc, PW, toks, dtype) for rid, toks in requests.items()}
+        variants = (None,) if dtype == "float32" else (None, plain.as_bfloat16)
+        outs = plain.forward_many(pc, PW, [requests[rid] for rid in layout], variants)
         model = load_model(str(folder), dtype, "cuda:0")
         runner = ModelRunner(model, 16, max_tokens // 16, max_requests=4, use_graph=True)
         got = helpers.run_schedule(runner, requests, steps)
         assert runner.graph_steps > 0 and not runner.cache.live_requests()
-        for rid, (exact, bound) in refs.items():
+        for (rid, (n, needle, at, probes)), res in zip(layout.items(), outs):
+            exact = res[0]
+            scale = float(exact.abs().max())
+            rows = torch.tensor(probes)
+            if dtype == "float32":
+                bound = probe_bound = helpers.float32_bound(pc)
+            else:
+                bound = helpers.BF16_FACTOR * helpers.rel_err(res[1], exact)
+                probe_bound = helpers.BF16_FACTOR * float((res[1][rows] - exact[rows]).abs().max()) / scale
             err = helpers.rel_err(got[rid], exact)
             assert err <= bound, f"{dtype}: request {rid} differs from the plain implementation by {err:.3e} (bound {bound:.3e}), " \
                                  f"first at {helpers.first_difference(got[rid], exact, bound)}"
+            cost = float((missed[rid] - exact[rows]).abs().amax(dim=-1).min()) / scale
+            assert cost >= 10 * probe_bound, f"{rid}: losing the needle moves a probe's logits by {cost:.2e}, the bound is {probe_bound:.2e}"
+            perr = float((got[rid][rows].double() - exact[rows]).abs().max()) / scale
+            assert perr <= probe_bound, f"{dtype}: request {rid}: probes off by {perr:.2e} (bound {probe_bound:.2e}; a lost needle costs {cost:.2e})"
         del model, runner
         torch.cuda.empty_cache()
 

@@ -104,6 +104,62 @@ def test_cutting_modes_against_each_other(tiny_dirs, capsys):
         print("\n  " + "\n  ".join(report))
 
 
+def test_cutting_modes_against_each_other_bfloat16(tiny_dirs, capsys):
+    """The same comparison in bfloat16 on config D, where every fast path runs (products chosen by the step's rows,
+    rotation in the projection's epilogue, matrix-core attention for portions and for single tokens with a split
+    context).  Two things are asked.  (1) Where the tokens lie in the cache is no input at all: the mixed schedule
+    on a pool so small that pages are used again, and on a larger pool whose free list was stirred first and that
+    another live request shares, gives the same BITS at every position, captured steps included.  (2) Between two
+    ways of cutting, the kernels differ (another product for another number of rows; single tokens split their
+    context, portions do not; a probability is rounded to bfloat16 against another running maximum), so the bits
+    differ, and what remains is the noise of the storage type: every mode stays within the request's bound of the
+    whole-prompt run, which is the bound both keep against the plain implementation.  The share of bit-equal
+    positions and the largest difference are printed."""
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner, StepEntry
+    name, dtype = "D", "bfloat16"
+    requests = helpers.requests_for(name)
+    ref = _reference(tiny_dirs, name, dtype)
+    # (1) placement
+    steps, max_tokens = helpers.schedule_for(name, "mixed")
+    tight = _runner(tiny_dirs, name, dtype, max_tokens, helpers.PAGE_SIZE[name], use_graph=True)
+    a = helpers.run_schedule(tight, requests, steps)
+    model = load_model(tiny_dirs.path(name, dtype), dtype, "cuda:0")
+    roomy = ModelRunner(model, helpers.PAGE_SIZE[name], 3 * max_tokens // helpers.PAGE_SIZE[name], max_requests=5, use_graph=True)
+    filler = helpers.random_tokens(helpers.CONFIGS[name].vocab_size, 200, seed=5)
+    for rid, n in (("x", 50), ("y", 90), ("z", 23)):
+        roomy.add_request(rid)
+        roomy.step([StepEntry(rid, filler[:n], [])])
+    roomy.end_request("x")
+    roomy.end_request("z")                       # pages 0..3 and 10, 11 are free again, in that order of return; "y" stays live
+    b = helpers.run_schedule(roomy, requests, steps)
+    assert tight.graph_steps > 0 and roomy.graph_steps == tight.graph_steps
+    for rid in requests:
+        assert torch.equal(a[rid], b[rid]), f"request {rid}: other pages, other bits (first at {helpers.first_difference(a[rid], b[rid], 0.0)})"
+    roomy.end_request("y")
+    # (2) cutting
+    results = {"mixed": a}
+    for mode in ("whole", "bulk_tail", "portions"):
+        steps, max_tokens = helpers.schedule_for(name, mode)
+        results[mode] = helpers.run_schedule(_runner(tiny_dirs, name, dtype, max_tokens, helpers.PAGE_SIZE[name]), requests, steps)
+    report = []
+    for mode in ("bulk_tail", "portions", "mixed"):
+        same = total = 0
+        worst = 0.0
+        for rid in requests:
+            x, y = results["whole"][rid], results[mode][rid]
+            exact, bound = ref[rid]
+            diff = float((x.double() - y.double()).abs().max() / exact.abs().max())
+            worst = max(worst, diff / bound)
+            # (both keep `bound` against the plain implementation; against each other they were measured at a quarter of it)
+            assert diff <= bound / 2, f"{mode} vs whole, request {rid}: {diff:.3e} apart, the storage noise bound is {bound:.3e}"
+            same += int((x == y).all(dim=-1).sum())
+            total += x.shape[0]
+        report.append(f"{mode} vs whole: {same} of {total} positions bit-equal, largest difference {worst:.2f} of the bound")
+    with capsys.disabled():
+        print("\n  " + "\n  ".join(report))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "C", "D"])
 def test_graph_replays_match_eager(tiny_dirs, name, dtype):
