@@ -84,8 +84,8 @@ class Engine:
     def _pages_from_memory(self, utilization: float, max_batch_size: int) -> int:
         m = self.model
         elem = 2 if m.dtype == torch.bfloat16 else 4
-        per_page = sum(n * 2 * g.num_kv_heads * self.page_size * g.head_dim * elem
-                       for g, n in zip(m.cache_groups, m.slots_per_group)) or 1
+        # (what a page costs is the cache spec's to say: every slot of every group holds one page of each plane)
+        per_page = sum(n * g.page_bytes(self.page_size, elem) for g, n in zip(m.cache_groups, m.slots_per_group)) or 1
         pages_cap = max_batch_size * ((self.max_seq_len + self.page_size - 1) // self.page_size)
         if self.device.type != "cuda":
             return pages_cap

@@ -178,12 +178,8 @@ class ModelRunner:
         self.layer_caches: List[LayerCache] = []
         for i, call in enumerate(model.order):
             g, idx = model.slot_group[call.cache]
-            k = v = None
-            if g >= 0:
-                spec = model.cache_groups[g]
-                k = self.pools.kv[g][idx, 0]
-                v = self.pools.kv[g][idx, 1].view(-1, spec.num_kv_heads, spec.head_dim, self.page_size)
-            self.layer_caches.append(LayerCache(g, k, v, model.call_writes[i], self.page_size,
+            planes = self.pools.slot(g, idx) if g >= 0 else {}
+            self.layer_caches.append(LayerCache(g, planes, model.call_writes[i], self.page_size,
                                                 self.pools.state.get(call.cache)))
         self.steps_run = 0
         self.tokens_run = 0

@@ -30,15 +30,37 @@ class WeightInfo:
 class CacheSpec:
     """What a mixer needs of the paged cache.
 
-    ``kind`` is ``"full"`` (every key is kept) or ``"window"`` (only the last
-    ``window`` keys are ever read, so older pages may be given back).
+    ``kind`` names the rule by which pages may be given back: ``"full"`` (every key is kept), ``"window"`` (only
+    the last ``window`` keys are ever read), or any rule registered in cache/rules.py.
     Mixers whose specs are equal share one group of pages.
+
+    The spec also says what a page HOLDS, so that the pools, the runner and the engine's sizing need not know:
+    ``planes(page_size)`` names the tensors a cache slot consists of and the shape of one page of each.  The
+    default is what grouped-query attention keeps: keys ``[kv_heads, page_size, head_dim]`` and values
+    transposed, ``[kv_heads, head_dim, page_size]`` (the attention kernels fetch eight consecutive keys of one
+    value element with one 16-byte load).  A mixer that keeps something else per token (one compressed vector,
+    say) subclasses the spec and overrides ``planes``; its ``forward`` finds the tensors under the same names
+    in ``LayerCache.planes``, each ``[pages + 1, *shape]`` with the page index first.
     """
 
     kind: str
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+
+    def planes(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
+        """name -> shape of one page of that tensor (in elements of the cache dtype)."""
+        return {"k": (self.num_kv_heads, page_size, self.head_dim), "v": (self.num_kv_heads, self.head_dim, page_size)}
+
+    def page_bytes(self, page_size: int, element_size: int) -> int:
+        """Bytes of one page of one cache slot: what a token place costs, times ``page_size``."""
+        total = 0
+        for shape in self.planes(page_size).values():
+            n = 1
+            for d in shape:
+                n *= int(d)
+            total += n
+        return total * element_size
 
 
 @dataclass(frozen=True)

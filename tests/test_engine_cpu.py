@@ -228,6 +228,46 @@ def test_toy_routed_ffn_and_learned_position_register_build_and_step(tmp_path):
     assert runner.cache.free_pages() == [12, 8]
 
 
+def test_toy_mixer_with_pages_of_its_own_layout_registers_builds_and_steps(tmp_path):
+    """A mixer whose pages hold one compressed vector per token instead of keys and values of heads: its cache spec
+    (a subclass defined in the tests) says what a page holds, and pools, runner and engine take it from there.  Its
+    layers form a cache group of their own beside the attention layer's; pages come back and are used again."""
+    import toy_parts
+    from tempura_amd import Engine
+    from tempura_amd.config import load_config
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.weights import write_random_model
+    cfg = toy_parts.ToyLatentConfig()
+    d = write_random_model(cfg, str(tmp_path / "latent"), seed=9, std=0.25, norm_jitter=0.1, dtype="float32")
+    assert type(load_config(d)) is toy_parts.ToyLatentConfig
+    model = load_model(d, "float32", "cpu")
+    assert [type(g).__name__ for g in model.cache_groups] == ["LatentCacheSpec", "CacheSpec"] and model.slots_per_group == [2, 1]
+    assert model.cache_groups[0].page_bytes(8, 4) == 8 * 20 * 4 and model.cache_groups[1].page_bytes(8, 4) == 2 * 2 * 8 * 16 * 4
+    _, W = plain.read_model_dir(d)
+    runner = ModelRunner(model, 8, [9, 9], max_requests=3)
+    assert {n: tuple(t.shape) for n, t in runner.pools.kv[0].items()} == {"c": (2, 10, 8, 20)}
+    assert sorted(runner.layer_caches[0].planes) == ["c"] and runner.layer_caches[0].k is None
+    assert sorted(runner.layer_caches[1].planes) == ["k", "v"]
+    reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=30 + i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30, "s": 12}.items())}
+    ref = {r: toy_parts.plain_latent_forward(cfg, W, t) for r, t in reqs.items()}
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
+             ([("p", 10, 11), ("r", 17, 13)], ["p"]), ([("s", 0, 2)], ["r"]), ([("s", 2, 10)], ["s"])]     # (s takes pages that q and p gave back)
+    got = helpers.run_schedule(runner, reqs, steps)
+    for r in reqs:      # (the toy mixer works in float32: a few 1e-6 of rounding; a vector from a wrong page costs 1e-2 and more)
+        assert helpers.first_difference(got[r], ref[r], helpers.TOL["float32"]) is None, r
+    assert runner.cache.free_pages() == [9, 9]
+    # the engine sizes the pools by what the specs say a page costs, and generates through them
+    eng = Engine(d, dtype="float32", device="cpu", page_size=8, kv_pages=12, max_batch_size=2)
+    assert eng.stats()["cache_bytes"] == 13 * (2 * 8 * 20 + 2 * 2 * 8 * 16) * 4
+    from tempura_amd import SamplingParams
+    out = eng.generate([reqs["q"]], SamplingParams(temperature=0.0, max_new_tokens=3))[0]
+    seq = list(reqs["q"])
+    for tok in out:
+        assert tok == int(torch.argmax(toy_parts.plain_latent_forward(cfg, W, seq)[-1]))
+        seq.append(tok)
+
+
 def test_toy_block_arrangements_with_other_parts_register_build_and_step(tmp_path):
     """Two block arrangements defined in the tests: one with norms before and after the mixer and the feed-forward
     (six named parts), one with a mixer and no feed-forward.  ``LayerSpec`` carries the parts by the names the

@@ -85,7 +85,7 @@ def test_attention_part(dtype, heads, kv, d, hidden, window):
     assert part.cache_spec().kind == ("window" if window else "full")
     kc = torch.zeros(pages + 1, kv, ps, d, dtype=dtype, device=DEV)
     vc = torch.zeros(pages + 1, kv, d, ps, dtype=dtype, device=DEV)
-    cache = LayerCache(0, kc, vc, True, ps, None)
+    cache = LayerCache(0, {"k": kc, "v": vc}, True, ps, None)
     xa = (torch.randn(30, hidden, generator=g)).to(dtype)      # request a: 19 tokens cached first, then 11
     xb = (torch.randn(7, hidden, generator=g)).to(dtype)
     ta, tb = [5, 2, 9, 0], [7, 11]                              # shuffled pages
@@ -157,7 +157,7 @@ def test_block_part(tiny_dirs):
     vc = torch.zeros(5, 3, 48, ps, device=DEV)
     hd = h.clone().to(DEV)
     table = [3, 1, 0]
-    block.forward(hd, _ctx([T], [T], ps, [table], [table[p // ps] * ps + p % ps for p in range(T)]), LayerCache(0, kc, vc, True, ps, None))
+    block.forward(hd, _ctx([T], [T], ps, [table], [table[p // ps] * ps + p % ps for p in range(T)]), LayerCache(0, {"k": kc, "v": vc}, True, ps, None))
     p = "model.layers.1."
     x = plain.rmsnorm(h.double(), W[p + "input_layernorm.weight"], cfg.rms_norm_eps)
     inv = plain.rope_inv_freq(48, cfg.rope_theta, cfg.to_dict()["rope_scaling"])
@@ -227,3 +227,28 @@ def test_toy_routed_ffn_and_learned_position_on_the_gpu(tmp_path):
     for r, t in reqs.items():
         ref = toy_parts.plain_routed_forward(cfg, W, t)
         assert helpers.rel_err(got[r], ref) < helpers.TOL[dtype], r
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_mixer_with_pages_of_its_own_layout_on_the_gpu(tmp_path, dtype):
+    """Registered, built and stepped without a change to the framework: a mixer from the tests whose pages hold one
+    compressed vector per token (its cache spec says so), in a cache group of its own beside an attention layer
+    that uses the HIP kernels; portions and single tokens of four requests, pages given back and used again."""
+    import toy_parts
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.weights import write_random_model
+    cfg = toy_parts.ToyLatentConfig()
+    d = write_random_model(cfg, str(tmp_path / "latent"), seed=9, std=0.25, norm_jitter=0.1, dtype=dtype)
+    model = load_model(d, dtype, "cuda:0")
+    _, W = plain.read_model_dir(d)
+    runner = ModelRunner(model, 8, [9, 9], max_requests=3)
+    assert {n: tuple(t.shape) for n, t in runner.pools.kv[0].items()} == {"c": (2, 10, 8, 20)}
+    reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=30 + i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30, "s": 12}.items())}
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
+             ([("p", 10, 11), ("r", 17, 13)], ["p"]), ([("s", 0, 2)], ["r"]), ([("s", 2, 10)], ["s"])]
+    got = helpers.run_schedule(runner, reqs, steps)
+    for r, t in reqs.items():
+        ref = toy_parts.plain_latent_forward(cfg, W, t)
+        assert helpers.rel_err(got[r], ref) < helpers.TOL[dtype], r
+    assert runner.cache.free_pages() == [9, 9]

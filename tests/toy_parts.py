@@ -6,7 +6,9 @@ nothing under tempura_amd/ knows about them.
   encoding that is not rotary (a learned vector per position, added to queries and keys), in layers beside
   the library's own parts (``ToyRoutedForCausalLM``);
 * a block arrangement with other parts than the library's: norms before AND after the mixer and the feed-forward
-  (six named parts), and a second kind of layer that has a mixer and no feed-forward at all (``ToySandwichForCausalLM``)."""
+  (six named parts), and a second kind of layer that has a mixer and no feed-forward at all (``ToySandwichForCausalLM``);
+* a mixer whose pages hold something else than keys and values of heads: ONE compressed vector per token, declared
+  by a cache spec of its own, in layers beside the library's attention (``ToyLatentForCausalLM``)."""
 from __future__ import annotations
 
 import json
@@ -16,7 +18,7 @@ from typing import Dict, List
 import torch
 
 from tempura_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, register_architecture
-from tempura_amd.parts import ArrangedBlock, FeedForward, Mixer, PositionEncoding, StateSpec, WeightInfo, register_part
+from tempura_amd.parts import ArrangedBlock, CacheSpec, FeedForward, Mixer, PositionEncoding, StateSpec, WeightInfo, register_part
 
 
 class DecaySumMixer(Mixer):
@@ -378,3 +380,131 @@ def plain_sandwich_forward(cfg: ToySandwichConfig, W: Dict[str, torch.Tensor], t
         y = plain.swiglu_ffn(plain.rmsnorm(h, W[f"{p}.n3"], 1e-5), W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
         h = h + plain.rmsnorm(y, W[f"{p}.n4"], 1e-5)
     return plain.rmsnorm(h, W["s.norm"], 1e-5) @ W["s.head"].T
+
+
+# ---- a mixer with another per-token cache layout -------------------------------------------------------------------
+@dataclass(frozen=True)
+class LatentCacheSpec(CacheSpec):
+    """A page holds ``page_size`` compressed vectors of ``latent`` elements and nothing else (no heads, no separate
+    values): one plane, ``c``.  ``num_kv_heads`` and ``head_dim`` are not used."""
+    latent: int = 0
+
+    def planes(self, page_size):
+        return {"c": (page_size, self.latent)}
+
+
+class LatentMixer(Mixer):
+    """c_t = x_t W_c is all a token leaves in the cache; token t's output is softmax_j<=t(q_t . c_j / sqrt(latent))
+    applied to the c_j themselves, times W_out (q_t = x_t W_q)."""
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        self.latent = int(spec.params["latent"])
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        n, w = spec.params["latent"], spec.weights
+        return {w["q"]: WeightInfo((n, hidden_size)), w["c"]: WeightInfo((n, hidden_size)), w["out"]: WeightInfo((hidden_size, n))}
+
+    def load_weights(self, get):
+        w = self.spec.weights
+        self.wq, self.wc, self.wout = (self._to_device(get(w[k]), torch.float32) for k in ("q", "c", "out"))
+
+    def cache_spec(self):
+        return LatentCacheSpec("full", 1, self.latent, None, self.latent)
+
+    def forward(self, x, ctx, cache, residual):
+        xf = x.float()
+        q, c = xf @ self.wq.T, xf @ self.wc.T
+        pool = cache.planes["c"]                                          # [pages + 1, page_size, latent]
+        ps = cache.page_size
+        flat = pool.view(-1, self.latent)
+        flat[ctx.slot_mapping[cache.group].long()] = c.to(pool.dtype)     # this step's vectors into their cache places
+        tables = ctx.block_tables[cache.group].tolist()
+        for r in range(ctx.num_requests):
+            start, n, total = ctx.q_starts[r], ctx.q_lens[r], ctx.ctx_lens[r]
+            rows = torch.tensor([tables[r][j // ps] * ps + j % ps for j in range(total)], device=flat.device)
+            keys = flat[rows].float()                                     # every vector of the request, in order
+            for i in range(n):
+                upto = total - n + i + 1
+                p = torch.softmax(keys[:upto] @ q[start + i] / self.latent ** 0.5, dim=0)
+                residual[start + i] += (p @ keys[:upto]) @ self.wout.T
+
+
+register_part("mixer", "toy_latent", LatentMixer)
+
+
+@dataclass
+class ToyLatentConfig:
+    """Layers 0 and 2: the latent mixer; layer 1: the library's attention.  Two cache groups with different pages."""
+    hidden_size: int = 48
+    vocab_size: int = 110
+    latent: int = 20
+    num_attention_heads: int = 4
+    num_key_value_heads: int = 2
+    head_dim: int = 16
+    intermediate_size: int = 64
+    max_position_embeddings: int = 128
+    architecture: str = "ToyLatentForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        keys = cls.__dataclass_fields__
+        return cls(**{k: v for k, v in d.items() if k in keys})
+
+    def to_json(self):
+        d = {k: getattr(self, k) for k in self.__dataclass_fields__}
+        d["architectures"] = [self.architecture]
+        return json.dumps(d)
+
+    def build_spec(self) -> ModelSpec:
+        norm = lambda n: PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": n})
+        layers = []
+        for l in range(3):
+            p = f"z.{l}"
+            if l == 1:
+                mixer = PartSpec("attention", {"num_heads": self.num_attention_heads, "num_kv_heads": self.num_key_value_heads,
+                                               "head_dim": self.head_dim, "scale": self.head_dim ** -0.5, "window": None,
+                                               "position": PartSpec("rope", {"head_dim": self.head_dim, "theta": 1e4, "scaling": None})},
+                                 {"q": f"{p}.q", "k": f"{p}.k", "v": f"{p}.v", "o": f"{p}.o"})
+            else:
+                mixer = PartSpec("toy_latent", {"latent": self.latent}, {"q": f"{p}.lq", "c": f"{p}.lc", "out": f"{p}.lo"})
+            layers.append(LayerSpec("prenorm", {
+                "mixer": mixer, "mixer_norm": norm(f"{p}.n1"), "ffn_norm": norm(f"{p}.n2"),
+                "ffn": PartSpec("swiglu", {"intermediate_size": self.intermediate_size},
+                                {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"})}))
+        return ModelSpec(self.architecture, self.hidden_size, self.vocab_size, self.max_position_embeddings, layers,
+                         [LayerCall(0), LayerCall(1), LayerCall(2)], norm("z.norm"),
+                         PartSpec("embedding", {}, {"weight": "z.embed"}), PartSpec("lm_head", {"tied": False}, {"weight": "z.head"}))
+
+
+register_architecture("ToyLatentForCausalLM", ToyLatentConfig)
+
+
+def plain_latent_forward(cfg: ToyLatentConfig, W: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
+    """Whole sequence, no cache, float64: the latent toy model written out plainly."""
+    import plain
+    W = {k: v.double() for k, v in W.items()}
+    T = len(tokens)
+    H, KV, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    h = W["z.embed"][torch.tensor(tokens)]
+    inv = plain.rope_inv_freq(D, 1e4, None)
+    pos = torch.arange(T)
+    for l in range(3):
+        p = f"z.{l}"
+        x = plain.rmsnorm(h, W[f"{p}.n1"], 1e-5)
+        if l == 1:
+            q = plain.rope((x @ W[f"{p}.q"].T).reshape(T, H, D), pos, inv)
+            k = plain.rope((x @ W[f"{p}.k"].T).reshape(T, KV, D), pos, inv)
+            v = (x @ W[f"{p}.v"].T).reshape(T, KV, D)
+            h = h + plain.attention(q, k, v, D ** -0.5) @ W[f"{p}.o"].T
+        else:
+            q, c = x @ W[f"{p}.lq"].T, x @ W[f"{p}.lc"].T
+            ys = []
+            for t in range(T):
+                pr = torch.softmax(c[: t + 1] @ q[t] / cfg.latent ** 0.5, dim=0)
+                ys.append((pr @ c[: t + 1]) @ W[f"{p}.lo"].T)
+            h = h + torch.stack(ys)
+        x = plain.rmsnorm(h, W[f"{p}.n2"], 1e-5)
+        h = h + plain.swiglu_ffn(x, W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
+    return plain.rmsnorm(h, W["z.norm"], 1e-5) @ W["z.head"].T
