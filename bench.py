@@ -48,6 +48,7 @@ def parse_args():
     ap.add_argument("--no-points", action="store_true", help="only the headline: no other batches, no bare step function")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-long", action="store_true", help="skip the long prefills and the 32 k decode point")
+    ap.add_argument("--no-large-batches", action="store_true", help="skip decoding at batch 128 and 256")
     ap.add_argument("--no-mixed", action="store_true", help="skip the mixed serving workload")
     ap.add_argument("--no-fingerprint", action="store_true", help="skip the run-to-run determinism check")
     ap.add_argument("--point-steps", type=int, default=500, help="timed steps of the other points")
@@ -304,7 +305,8 @@ def main() -> int:
         }
 
     # =============================================================================================================
-    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    large = [] if (args.no_points or args.no_large_batches) else [128, 256]
+    max_batch = args.batch if args.no_points else max([args.batch, 64] + large)
     long_tokens = 0 if (args.no_long or args.no_points) else 8 * 33536       # eight requests at a 32 k context
     per_request = max(args.context, -(-long_tokens // max_batch))
     eng, cfg, full, weight_bytes = make_engine(args.model_config, args.layers, max_batch, per_request, 2048)
@@ -340,6 +342,12 @@ def main() -> int:
             points[f"decode_b{b}"] = round(r["tps"], 1)
             points[f"decode_b{b}_hbm_frac"] = round(r["bytes"] / (r["ms"] / 1e3) / 1e9 / HBM_PEAK_GBS, 4)
             say(f"engine decode b{b}: {r['tps']:.1f} tok/s, {r['ms']:.3f} ms/step")
+        for b in large:
+            # (their prompts alone are b x 3,000 tokens of prefill: fewer timed steps, around the same cache length)
+            r = engine_decode(eng, cfg, weight_bytes, b, centred(4, 100), 4, 100)
+            points[f"decode_b{b}"] = round(r["tps"], 1)
+            points[f"decode_b{b}_hbm_frac"] = round(r["bytes"] / (r["ms"] / 1e3) / 1e9 / HBM_PEAK_GBS, 4)
+            say(f"engine decode b{b}: {r['tps']:.1f} tok/s, {r['ms']:.3f} ms/step, KV {r['kv']}")
         for b in sorted({1, args.batch, 64}):
             # (the same number of steps, so the same range of context lengths, as the engine's figure it stands beside)
             nw, ns = (warmup, steps) if b == args.batch else (8, ps)
