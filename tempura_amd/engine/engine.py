@@ -68,7 +68,8 @@ class Engine:
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_batch_size, max_num_batched_tokens=max_num_batched_tokens,
                             prefill_chunk_size=prefill_chunk_size, max_model_len=self.max_seq_len,
-                            fill_budget=fill_budget, admit_headroom=admit_headroom),
+                            fill_budget=fill_budget, admit_headroom=admit_headroom,
+                            portion_align=self.model.portion_align()),
             self.runner.cache)
         self.sampler = Sampler(spec.vocab_size, self.device, default_seed=seed)
         self._ids = itertools.count()            # request ids that add_request hands out: 0, 1, 2, ...
@@ -141,15 +142,17 @@ class Engine:
             items = self.scheduler.schedule()
             if not items:
                 return []
-            # Prompt portions go first in the batch, single tokens last: a portion that starts at a multiple of
-            # eight positions then also starts at a multiple of eight rows, which is what lets the projection's
-            # epilogue store eight tokens' values as one piece of the transposed value cache.
+            # Prompt portions go first in the batch, single tokens last: a portion that starts at a multiple of the
+            # alignment the model's parts prefer (attention: eight positions) then also starts at that multiple of
+            # rows, which is what lets the projection's epilogue store eight tokens' values as one piece of the
+            # transposed value cache.
             # Among the single tokens the longest contexts go first: attention hands its blocks out in this order,
             # and a batch of short and long contexts ends sooner when the long ones start first (60 requests of
             # 128 to 2,304 keys: 77 -> 74 us a layer).
-            # (and portions whose length is no multiple of eight, the ends of prompts, go behind the others: every
+            # (and portions whose length is no such multiple, the ends of prompts, go behind the others: every
             # portion behind one of them starts at an odd row)
-            items.sort(key=lambda it: (it.count == 1, it.count % 8 != 0 if it.count > 1 else -it.start))
+            align = self.scheduler.config.portion_align
+            items.sort(key=lambda it: (it.count == 1, it.count % align != 0 if it.count > 1 else -it.start))
             entries = []
             for it in items:
                 toks = it.request.step_tokens(it.start, it.count)

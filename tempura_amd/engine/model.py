@@ -81,6 +81,16 @@ class CausalLM:
                 if mine != theirs:
                     raise ValueError(f"run order entry {i} reads cache slot {call.cache} whose layout differs from its own")
 
+    def portion_align(self) -> int:
+        """The multiple of positions at which the model's parts prefer prompt portions to be cut (the least common
+        multiple of what the mixers say; 1 when none cares)."""
+        import math
+        align = 1
+        for layer in self.layers:
+            for part in layer.parts():
+                align = math.lcm(align, int(getattr(part, "preferred_portion_align", 1)))
+        return align
+
     # ---- weights -------------------------------------------------------
     def expected_weights(self) -> Dict[str, WeightInfo]:
         return expected_weights(self.spec)

@@ -84,7 +84,7 @@ class SchedulerConfig:
     max_num_batched_tokens: int = 2048      # token budget of one step
     prefill_chunk_size: int = 512           # largest prompt portion (engine_task.rs:11)
     max_model_len: int = 4096               # the reference's --max-seq-len
-    portion_align: int = 8                  # a prompt portion that is not the last ends at a multiple of this
+    portion_align: int = 8                  # a prompt portion that is not the last ends at a multiple of this (the engine asks the model's parts)
     fill_budget: bool = True                # budget that no other request can use lengthens the portions in the plan
     #: share of every page pool that an admission must leave free while other requests run (never less than one page
     #: for each of them and one for the newcomer): the reference stops admitting below a headroom of free tokens

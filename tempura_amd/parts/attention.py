@@ -19,6 +19,9 @@ from .base import CacheSpec, Mixer, WeightInfo, build_part, part_class, register
 
 class PagedAttention(Mixer):
     graph_safe = True      # only kernels on device-resident step data: may be captured in a graph
+    #: the value cache is transposed, eight consecutive tokens of one element being one 16-byte piece: a portion that
+    #: starts at a multiple of eight positions (and of eight rows of the batch) has its values stored piece by piece
+    preferred_portion_align = 8
     split_norm = True      # takes rows whose norm its first product finishes; prepares the next norm in its last
 
     def __init__(self, spec, hidden_size, dtype, device):

@@ -108,6 +108,10 @@ class Mixer(Part):
 
     category = "mixer"
 
+    #: a portion of a prompt is best cut at a multiple of this many positions (1: anywhere).  A hint for whoever
+    #: cuts prompts, never a condition: every part takes every cut.
+    preferred_portion_align = 1
+
     def cache_spec(self) -> Optional[CacheSpec]:
         return None
 

@@ -260,6 +260,10 @@ def test_toy_mixer_with_pages_of_its_own_layout_registers_builds_and_steps(tmp_p
     # the engine sizes the pools by what the specs say a page costs, and generates through them
     eng = Engine(d, dtype="float32", device="cpu", page_size=8, kv_pages=12, max_batch_size=2)
     assert eng.stats()["cache_bytes"] == 13 * (2 * 8 * 20 + 2 * 2 * 8 * 16) * 4
+    # where prompts are best cut is the parts' to say: the attention layer prefers multiples of eight, the toy mixer does not care
+    assert eng.scheduler.config.portion_align == 8 == model.portion_align()
+    assert {type(p).__name__: p.preferred_portion_align for l in model.layers for p in l.parts() if p.category == "mixer"} == \
+        {"LatentMixer": 1, "PagedAttention": 8}
     from tempura_amd import SamplingParams
     out = eng.generate([reqs["q"]], SamplingParams(temperature=0.0, max_new_tokens=3))[0]
     seq = list(reqs["q"])
