@@ -405,6 +405,7 @@ def main() -> int:
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "global_batch": args.batch, "seq_len": args.context, "prompt_len": args.prompt_len,
+            "decode_from_kv": head["kv"][0],
             "page_size": args.page_size, "weights": "random N(0,0.02)", "parallelism": "single GPU",
             "graph": not args.no_graph, "steps_queued_ahead": not args.no_chain, "sampling": "greedy",
             "path": "Engine.add_request/step",
