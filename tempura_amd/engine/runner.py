@@ -187,8 +187,9 @@ class ModelRunner:
         #: host time spent packing the inputs of eager steps, and how many such steps there were
         self.host_seconds = {"pack": 0.0}
         self.host_steps = {"pack": 0}
-        # Decode-only steps replay a captured graph when every part of the model allows it.
-        self.use_graph = bool(use_graph) and self.device.type == "cuda" and not model.state_specs and \
+        # Decode-only steps replay a captured graph when every part of the model allows it (a part that keeps
+        # per-request state says so like any other: it then finds its rows through ``ctx.state_slots`` on the device).
+        self.use_graph = bool(use_graph) and self.device.type == "cuda" and \
             all(getattr(p, "graph_safe", False) for layer in model.layers for p in layer.parts())
         self.graph_steps = 0
         self._prepared = None          # (request ids, graph, cache generation) of a decode step staged ahead by prepare_decode
@@ -316,11 +317,7 @@ class ModelRunner:
     def _graph_for(self, rows: int, ctx_len: int) -> Optional[_DecodeGraph]:
         # rows padded to a power of two, beyond 128 to a multiple of 128: the products see as many blocks of rows as
         # in the unpadded step and so choose the same tiles and parts of K (the same bits as an eager step)
-        bucket = 1
-        while bucket < min(rows, 128):
-            bucket *= 2
-        if rows > 128:
-            bucket = (rows + 127) // 128 * 128
+        bucket = ops.decode_rows_padded(rows)
         bound = 256
         while bound < ctx_len:
             bound *= 2
@@ -387,11 +384,17 @@ class ModelRunner:
             self._fill_graph_inputs(g, rids, [0] * n if on_device else tokens)
         if on_device:
             g.packed[:n].copy_(tokens)
+        if self.pools.state:
+            self._clear_state([self.cache.state_slot(r) for r in rids if self.cache.num_tokens(r) == 0])
         if g.graph is None:
             ctx = g.context(self)
             tok = g.view(0)
-            # one eager run first: lazy initialisation must not happen under capture
+            # one eager run first: lazy initialisation must not happen under capture.  (What it writes into the
+            # paged cache the replay writes again; per-request state it would advance twice, so that is put back.)
+            kept = {slot: t.clone() for slot, t in self.pools.state.items()}
             self.model.forward(tok, ctx, self.layer_caches)
+            for slot, t in kept.items():
+                self.pools.state[slot].copy_(t)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):
@@ -404,6 +407,12 @@ class ModelRunner:
         if want_rows is None or len(want_rows) == n:
             return g.logits[:n]
         return ops.take_rows(g.logits, want_rows) if want_rows else g.logits[:0]
+
+    def _clear_state(self, fresh: Sequence[int]) -> None:
+        """A request that starts at position 0 gets a cleared state (also after a recompute)."""
+        if fresh:
+            for t in self.pools.state.values():
+                ops.zero_rows(t, fresh)
 
     def step_chained(self, rids: Sequence, tokens: torch.Tensor) -> torch.Tensor:
         """A step of one token per request whose tokens are still on the device: ``tokens`` int32 [len(rids)],
@@ -449,12 +458,8 @@ class ModelRunner:
             return logits
         self._prepared = None
         tok_dev, ctx = self._pack_step(entries)
-        # A request that starts at position 0 gets a cleared state (also after a recompute).
         if self.pools.state:
-            fresh = [s for s, n, c in zip(ctx.state_slot_list, ctx.q_lens, ctx.ctx_lens) if c == n]
-            if fresh:
-                for t in self.pools.state.values():
-                    ops.zero_rows(t, fresh)
+            self._clear_state([s for s, n, c in zip(ctx.state_slot_list, ctx.q_lens, ctx.ctx_lens) if c == n])
         logits = self.model.forward(tok_dev, ctx, self.layer_caches)
         self.cache.commit_many([e.rid for e in entries], ctx.q_lens)
         self.steps_run += 1

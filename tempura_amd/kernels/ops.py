@@ -582,6 +582,18 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int,
 allow_fast_attention = True
 #: the split decode kernel aims at this many blocks (of four waves) in flight
 decode_target_blocks = 256
+
+
+def decode_rows_padded(rows: int) -> int:
+    """The number of rows a decode step of `rows` requests is sized for: the next power of two up to 128, beyond
+    that the next multiple of 128.  A captured step has that many rows and an eager one chooses its kernels and
+    splits as if it had, so the two give the same bits."""
+    if rows > 128:
+        return (rows + 127) // 128 * 128
+    padded = 1
+    while padded < rows:
+        padded *= 2
+    return padded
 #: and at least this many splits while a split has at most 64 blocks
 decode_min_splits = 8
 #: measurements: this many splits whatever the batch (0: chosen by the rules below)
@@ -627,7 +639,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     splits, scratch = 1, None
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
-        blocks_per_split = num_single * kvh * ((heads // kvh + 15) // 16)
+        blocks_per_split = decode_rows_padded(num_single) * kvh * ((heads // kvh + 15) // 16)
         # (two blocks fit a CU, 512 the chip.  From 65 to 256 blocks per split, as many splits as fill it once: measured
         # alone at 2,100 keys, 16 requests 35.8 -> 33.5 us, 20 requests 47.2 -> 38.5, 32 requests 54.3 -> 52.7, and more
         # for contexts that differ; through the engine 16 requests of the 8B shape 4.33 -> 4.25 ms a step, 32 requests
@@ -647,7 +659,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             want = max(want, decode_min_splits)     # (batch 8 of the 8B shape: eight splits 3.87 ms a step, four 3.94)
         if decode_force_splits > 0:
             want = decode_force_splits
-        splits = max(1, min(64, want, max(1, max_context_len // 128)))
+        # (at least 128 keys a split, by the longest context rounded up to a power of two from 256: a step captured
+        # for a bound on the context and an eager step at the actual length then cut alike and give the same bits)
+        bound = 256
+        while bound < max_context_len:
+            bound *= 2
+        splits = max(1, min(64, want, bound // 128))
         if splits > 1:
             scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
     parts, part_scratch = 1, None

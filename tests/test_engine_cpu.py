@@ -174,24 +174,26 @@ def test_zero_new_tokens_and_a_request_left_out_of_a_step(tiny_dirs):
     assert eng._queue_next(items) is None
 
 
-def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
-    """A mixer defined in the tests, with per-request state and no paged cache, in an architecture of its own."""
+@pytest.mark.parametrize("on_device", [False, True])
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, on_device):
+    """A mixer defined in the tests, with per-request state and no paged cache, in an architecture of its own
+    (``on_device``: the variant that finds its rows of the state through the step's device-side slots)."""
     import toy_parts
     from tempura_amd.config import load_config
     from tempura_amd.engine.loading import load_model
     from tempura_amd.engine.runner import ModelRunner, StepEntry
     from tempura_amd.weights import write_random_model
-    cfg = toy_parts.ToyConfig()
+    cfg = toy_parts.ToyConfig(state_on_device=on_device)
     d = write_random_model(cfg, str(tmp_path / "toy"), seed=4, std=0.2, norm_jitter=0.1, dtype="float32")
-    assert type(load_config(d)) is toy_parts.ToyConfig
+    assert type(load_config(d)) is toy_parts.ToyConfig and load_config(d).state_on_device == on_device
     model = load_model(d, "float32", "cpu")
     assert sorted(model.state_specs) == [0, 2] and model.slots_per_group == [1]     # two state layers, one attention layer
     _, W = plain.read_model_dir(d)
     runner = ModelRunner(model, 8, 12, max_requests=3)
     reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30}.items())}
     ref = {r: toy_parts.plain_toy_forward(cfg, W, t) for r, t in reqs.items()}
-    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
-             ([("p", 10, 11), ("r", 17, 13)], ["p", "r"])]
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1)], ["q"]),
+             ([("p", 10, 1), ("r", 0, 1)], []), ([("p", 11, 1), ("r", 1, 1)], []), ([("p", 12, 9), ("r", 2, 28)], ["p", "r"])]
     got = helpers.run_schedule(runner, reqs, steps)
     for r in reqs:
         assert helpers.first_difference(got[r], ref[r], 1e-6) is None, r

@@ -56,6 +56,26 @@ class DecaySumMixer(Mixer):
 register_part("mixer", "decay_sum", DecaySumMixer)
 
 
+class DecaySumOnDeviceMixer(DecaySumMixer):
+    """The same mixer, declared safe to capture: in a step of one token per request it finds its rows of the state
+    through ``ctx.state_slots`` ON THE DEVICE (rows of a captured step that carry no request point at a spare row)
+    and reads nothing on the host; steps with prompt portions, which are never captured, take the loop above."""
+    graph_safe = True
+
+    def forward(self, x, ctx, cache, residual):
+        if ctx.max_q_len != 1:
+            return super().forward(x, ctx, cache, residual)
+        from tempura_amd.kernels import ops
+        slots = ctx.state_slots.long()
+        u = ops.linear(x.float().contiguous(), self.w_in, torch.float32)
+        s = self.decay * cache.state.index_select(0, slots) + u
+        cache.state.index_copy_(0, slots, s)
+        ops.linear(s, self.w_out, torch.float32, residual=residual)
+
+
+register_part("mixer", "decay_sum_on_device", DecaySumOnDeviceMixer)
+
+
 class TopOneRoutedFFN(FeedForward):
     """Router logits in float32; each token's output is its best expert's two-layer ReLU network times the
     softmax weight of that expert.  Tokens are grouped by expert on the host; a token's result does not
@@ -126,6 +146,7 @@ class ToyConfig:
     head_dim: int = 16
     intermediate_size: int = 64
     max_position_embeddings: int = 256
+    state_on_device: bool = False       # the variant of the stateful mixer that may be captured in a graph
     architecture: str = "ToyForCausalLM"
 
     @classmethod
@@ -143,7 +164,7 @@ class ToyConfig:
         for l in range(self.num_hidden_layers):
             p = f"toy.{l}"
             if l % 2 == 0:      # state layers at even depths, attention at odd ones
-                mixer = PartSpec("decay_sum", {"width": self.width, "decay": self.decay},
+                mixer = PartSpec("decay_sum_on_device" if self.state_on_device else "decay_sum", {"width": self.width, "decay": self.decay},
                                  {"in": f"{p}.mix.in", "out": f"{p}.mix.out"})
             else:
                 mixer = PartSpec("attention", {"num_heads": self.num_attention_heads, "num_kv_heads": 2,
@@ -481,9 +502,13 @@ class ToyLatentConfig:
 register_architecture("ToyLatentForCausalLM", ToyLatentConfig)
 
 
-def plain_latent_forward(cfg: ToyLatentConfig, W: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
-    """Whole sequence, no cache, float64: the latent toy model written out plainly."""
+def plain_latent_forward(cfg: ToyLatentConfig, W: Dict[str, torch.Tensor], tokens: List[int], stored=None) -> torch.Tensor:
+    """Whole sequence, no cache, float64: the latent toy model written out plainly.  ``stored`` (for instance
+    ``plain.as_bfloat16``) is applied to every value that a 16-bit engine keeps in 16 bits (normed rows, rotated
+    queries and keys, values, attention's probabilities and output, the compressed vectors in their pages, gated
+    activations): the distance of that run from the exact one is the noise of the storage type."""
     import plain
+    keep = stored if stored is not None else (lambda t: t)
     W = {k: v.double() for k, v in W.items()}
     T = len(tokens)
     H, KV, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
@@ -492,19 +517,19 @@ def plain_latent_forward(cfg: ToyLatentConfig, W: Dict[str, torch.Tensor], token
     pos = torch.arange(T)
     for l in range(3):
         p = f"z.{l}"
-        x = plain.rmsnorm(h, W[f"{p}.n1"], 1e-5)
+        x = keep(plain.rmsnorm(h, W[f"{p}.n1"], 1e-5))
         if l == 1:
-            q = plain.rope((x @ W[f"{p}.q"].T).reshape(T, H, D), pos, inv)
-            k = plain.rope((x @ W[f"{p}.k"].T).reshape(T, KV, D), pos, inv)
-            v = (x @ W[f"{p}.v"].T).reshape(T, KV, D)
-            h = h + plain.attention(q, k, v, D ** -0.5) @ W[f"{p}.o"].T
+            q = keep(plain.rope((x @ W[f"{p}.q"].T).reshape(T, H, D), pos, inv))
+            k = keep(plain.rope((x @ W[f"{p}.k"].T).reshape(T, KV, D), pos, inv))
+            v = keep((x @ W[f"{p}.v"].T).reshape(T, KV, D))
+            h = h + keep(plain.attention(q, k, v, D ** -0.5, stored=stored)) @ W[f"{p}.o"].T
         else:
-            q, c = x @ W[f"{p}.lq"].T, x @ W[f"{p}.lc"].T
+            q, c = x @ W[f"{p}.lq"].T, keep(x @ W[f"{p}.lc"].T)
             ys = []
             for t in range(T):
                 pr = torch.softmax(c[: t + 1] @ q[t] / cfg.latent ** 0.5, dim=0)
                 ys.append((pr @ c[: t + 1]) @ W[f"{p}.lo"].T)
             h = h + torch.stack(ys)
-        x = plain.rmsnorm(h, W[f"{p}.n2"], 1e-5)
-        h = h + plain.swiglu_ffn(x, W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
-    return plain.rmsnorm(h, W["z.norm"], 1e-5) @ W["z.head"].T
+        x = keep(plain.rmsnorm(h, W[f"{p}.n2"], 1e-5))
+        h = h + plain.swiglu_ffn(x, W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"], stored)
+    return keep(plain.rmsnorm(h, W["z.norm"], 1e-5)) @ W["z.head"].T
