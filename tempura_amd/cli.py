@@ -240,7 +240,12 @@ def main(argv=None) -> int:
             return int(e.code or 0)
         return 0
     args = ap.parse_args(argv)
-    return args.fn(args)
+    from .engine.loading import NoDeviceError
+    try:
+        return args.fn(args)
+    except NoDeviceError as e:
+        print(f"tempura: {e}", file=sys.stderr)
+        return 2
 
 
 if __name__ == "__main__":

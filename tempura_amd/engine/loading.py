@@ -22,8 +22,23 @@ def parse_dtype(dtype) -> torch.dtype:
         raise ValueError(f"dtype must be one of {sorted(_DTYPES)}, got {dtype!r}") from None
 
 
+class NoDeviceError(RuntimeError):
+    """The device that was asked for is not there."""
+
+
+def require_device(device) -> torch.device:
+    """``device`` as a torch.device; one clear error when it names a GPU and none is visible (the engine has no
+    CPU path: on the CPU only the tests' stand-in operations run, with device "cpu")."""
+    device = torch.device(device)
+    if device.type == "cuda" and not torch.cuda.is_available():
+        raise NoDeviceError(f"no GPU is visible to this process (device {str(device)!r} was asked for, "
+                            "torch.cuda.is_available() is False); tempura_amd runs on an AMD MI355X and has no CPU path")
+    return device
+
+
 def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> CausalLM:
     """Read ``config.json``, pick the architecture from the registry, build it, load its weights."""
+    device = require_device(device)
     config = load_config(model_dir)
     model = CausalLM(config.build_spec(), parse_dtype(dtype), torch.device(device))
     model.config = config
@@ -38,6 +53,7 @@ def random_model(config, seed: int = 0, dtype="bfloat16", device="cuda:0", std: 
     GPU) each tensor is filled by a kernel in device memory, with the same values as the host
     generator's that ``write_random_model`` uses.  ``values_as`` (a dtype name) rounds the matrix
     values to that type first, so that a float32 model can hold exactly a bfloat16 model's weights."""
+    device = require_device(device)
     from ..kernels import ops
     from ..weights.random_init import _tensor_seed
     td = parse_dtype(dtype)

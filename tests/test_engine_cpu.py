@@ -336,3 +336,19 @@ def test_forward_while_every_request_slot_is_live_and_the_waste_ratio(tiny_dirs)
         eng.step()
     assert [eng.request(i).output for i in range(2)] == [plain.greedy_generate(cfg, W, p, 8) for p in prompts]
     assert eng.runner.cache.free_pages() == [8] and eng.stats()["waste_ratio"] == 0.0
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="needs a machine without a GPU")
+def test_no_gpu_is_one_clear_error(tiny_dirs, capsys):
+    """Without a GPU the engine says so in one line (it has no CPU path): from the loader, from the entry point
+    and, with exit status 2, from the command line."""
+    from tempura_amd import Engine
+    from tempura_amd.cli import main
+    from tempura_amd.engine.loading import NoDeviceError, load_model
+    d = tiny_dirs.path("A", "float32")
+    with pytest.raises(NoDeviceError, match="no GPU is visible"):
+        load_model(d, "float32", "cuda:0")
+    with pytest.raises(NoDeviceError, match="no CPU path"):
+        Engine(d, dtype="float32")
+    assert main(["run", "--model", d, "--prompt-ids", "1,2,3", "--max-new-tokens", "2"]) == 2
+    assert "no GPU is visible" in capsys.readouterr().err
