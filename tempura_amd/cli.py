@@ -18,8 +18,10 @@ import time
 
 
 def _add_engine_args(ap: argparse.ArgumentParser) -> None:
+    ap.add_argument("model_dir", nargs="?", help="model folder (the same as --model)")
     ap.add_argument("--model", help="model folder (config.json + *.safetensors)")
-    ap.add_argument("--model-config", help="named size for --random-weights (see `tempura random-model --list`)")
+    ap.add_argument("--model-config", "--preset", dest="model_config",
+                    help="named size for --random-weights (see `tempura random-model --list`)")
     ap.add_argument("--random-weights", action="store_true", help="seeded N(0, 0.02) weights instead of a checkpoint")
     ap.add_argument("--seed", type=int, default=0, help="seed of random weights and default sampling seed")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32", "bf16", "fp32"])
@@ -41,6 +43,10 @@ def _add_engine_args(ap: argparse.ArgumentParser) -> None:
 def _engine_from_args(args):
     from .config import PRESETS
     from .engine import Engine
+    if getattr(args, "model_dir", None):
+        if args.model and args.model != args.model_dir:
+            raise SystemExit(f"two model folders given: {args.model_dir!r} and --model {args.model!r}")
+        args.model = args.model_dir
     if args.random_weights:
         if args.model_config:
             if args.model_config not in PRESETS:

@@ -298,7 +298,8 @@ def test_command_line(tiny_dirs, tmp_path):
     ids = tmp_path / "ids.txt"
     ids.write_text("\n".join(" ".join(map(str, q)) for q in prompts) + "\n")
     out = tmp_path / "logits.f32"
-    p = subprocess.run([sys.executable, tempura, "run", "--model", model, "--dtype", "float32", "--prompt-file", str(ids),
+    # (the model folder as the positional argument, as in `tempura inspect`)
+    p = subprocess.run([sys.executable, tempura, "run", model, "--dtype", "float32", "--prompt-file", str(ids),
                         "--max-new-tokens", "2", "--temperature", "0", "--kv-blocks", "16", "--max-batch-size", "2",
                         "--dump-logits", str(out)], capture_output=True, text=True, timeout=600)
     assert p.returncode == 0, p.stderr[-2000:]
