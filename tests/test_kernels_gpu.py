@@ -827,3 +827,71 @@ def test_take_rows_and_zero_rows(dtype, n, width):
     assert torch.equal(d.cpu(), want)
     with pytest.raises(Exception, match="out of range"):
         ops.take_rows(d, [n])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_pages_beyond_two_to_the_31_elements_of_a_pool(dtype):
+    """A layer's key (or value) pool may hold more than 2^31 elements (4 GiB of bfloat16: 2.1 million tokens of 8 kv
+    heads of 128, which a small model's cache reaches on this GPU): every kernel that writes or reads the cache works
+    out its places in 64 bits.  The same step is run twice, on a small pool and on pages that all lie past element
+    2^31 of a large one (a block table with the same pages plus an offset): the rows that the rotation and
+    cache-write kernels store (few rows and a long step, alone and as a projection's epilogue), and what attention
+    then reads for a prompt and for single tokens, must be the same bits."""
+    ops = _ops()
+    from tempura_amd.parts.rope import rotary_inv_freq
+    heads, kv, d, page, hidden = 32, 8, 128, 16, 128
+    small = 150
+    off = 2 ** 31 // (kv * page * d) + 3                   # the first page of the large pool that is used
+    big = off + small
+    g = torch.Generator().manual_seed(11)
+    n = (heads + 2 * kv) * d
+    inv = rotary_inv_freq(d, 500000.0, None, d).to(DEV)
+    w = (torch.randn(n, hidden, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+    m_long, m_few = 2100, 8
+    x_long = torch.randn(m_long, hidden, generator=g).to(torch.bfloat16).to(DEV)
+    x_few = torch.randn(m_few, hidden, generator=g).to(torch.bfloat16).to(DEV)
+    order = torch.randperm(small - 1, generator=g).tolist()            # (the last page stays the tables' filler)
+    sl_long = torch.tensor([order[i // page] * page + i % page for i in range(m_long)], dtype=torch.int32)
+    rest = order[(m_long + page - 1) // page:]
+    sl_few = torch.tensor([rest[i] * page + (5 * i) % page for i in range(m_few)], dtype=torch.int32)
+    pos_long = torch.arange(m_long, dtype=torch.int32).to(DEV)
+    pos_few = torch.randint(0, 100000, (m_few,), generator=g, dtype=torch.int32).to(DEV)
+    # attention afterwards: the prompt as one request, and four requests of one token over parts of its pages
+    width = (m_long + page - 1) // page + 1
+    bt_prompt = torch.full((1, width), small - 1, dtype=torch.int32)
+    bt_prompt[0, : width - 1] = torch.tensor(order[: width - 1], dtype=torch.int32)
+    ctx_single = [m_long, 1500, 333, 17]
+    bt_single = bt_prompt.repeat(4, 1)
+    q_single = (torch.randn(4, heads, d, generator=g) * 1.5).to(dtype).to(DEV)
+    scale = 1.0 / math.sqrt(d)
+
+    def run(pages, shift):
+        kc = torch.empty(pages, kv, page, d, dtype=dtype, device=DEV)
+        vc = torch.empty(pages, kv, d, page, dtype=dtype, device=DEV)
+        kc[shift: shift + small].zero_()
+        vc[shift: shift + small].zero_()
+        a, b = (sl_long + shift * page).to(DEV), (sl_few + shift * page).to(DEV)
+        outs = []
+        if dtype == torch.bfloat16:    # the projections whose epilogue rotates and stores
+            outs.append(ops.linear_rope_kv(x_long, w, pos_long, a, inv, d, 1.0, heads, kv, d, kc, vc, ops.rope_table(pos_long, inv, d, 1.0)))
+            outs.append(ops.linear_rope_kv(x_few, w, pos_few, b, inv, d, 1.0, heads, kv, d, kc, vc))
+        else:                          # the kernels of their own, for a long step and for a few rows
+            outs.append(ops.rope_kv_write(ops.linear(x_long.float(), w.float(), torch.float32), pos_long, a, inv, d, 1.0, heads, kv, d, kc, vc, dtype))
+            outs.append(ops.rope_kv_write(ops.linear(x_few.float(), w.float(), torch.float32), pos_few, b, inv, d, 1.0, heads, kv, d, kc, vc, dtype))
+        q_prompt = outs[0].to(dtype).view(m_long, heads, d)
+        cu = torch.tensor([0, m_long], dtype=torch.int32, device=DEV)
+        outs.append(ops.paged_attention(q_prompt, kc, vc, (bt_prompt + shift).to(DEV), cu, torch.tensor([m_long], dtype=torch.int32, device=DEV),
+                                        torch.zeros(m_long, dtype=torch.int32, device=DEV), scale, 0, m_long, m_long))
+        outs.append(ops.paged_attention(q_single, kc, vc, (bt_single + shift).to(DEV), torch.arange(5, dtype=torch.int32, device=DEV),
+                                        torch.tensor(ctx_single, dtype=torch.int32, device=DEV), torch.arange(4, dtype=torch.int32, device=DEV),
+                                        scale, 0, 1, max(ctx_single)))
+        outs += [kc[shift: shift + small].clone(), vc[shift: shift + small].clone()]
+        return outs
+
+    assert big * kv * page * d > 2 ** 31 and off * kv * page * d >= 2 ** 31
+    low = run(small, 0)
+    high = run(big, off)
+    names = ["q of the long step", "q of the few rows", "attention of the prompt", "attention of single tokens", "key pages", "value pages"]
+    for name, x0, x1 in zip(names, low, high):
+        assert torch.isfinite(x0.float()).all(), name
+        assert torch.equal(x0, x1), f"{name}: other bits on pages past element 2^31"
