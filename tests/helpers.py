@@ -183,6 +183,50 @@ def schedule_mixed(lengths: Dict[str, int], max_tokens: int, seed: int, max_live
     return steps
 
 
+def schedule_random(lengths: Dict[str, int], seed: int):
+    """A schedule drawn from ``seed``: how many requests are live at a time (one to four) and so how small the pool
+    is, in which order the requests come and in which order the entries of a step stand, how long the portions
+    are (1 to 70 tokens, so that they end before, at and behind pages' edges), from where on a request goes token
+    by token, and how often a request sits a step out.  Returns (steps, max_tokens)."""
+    g = random.Random(seed)
+    max_live = g.choice([1, 2, 3, 4, 4])
+    order = list(lengths.items())
+    g.shuffle(order)
+    biggest = sorted(roundup(n, 64) for n in lengths.values())
+    max_tokens = sum(biggest[-max(1, max_live - 1):]) + (64 if max_live > 1 else 0)
+    tail = {rid: g.choice([0, 1, 2, 7, 32, 40]) for rid in lengths}
+    skip = g.choice([0.0, 0.1, 0.3])
+    waiting = list(order)
+    live: Dict[str, int] = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, n = waiting[0]
+            held = sum(roundup(lengths[r], 64) for r in live)
+            if held + roundup(n, 64) > max_tokens:
+                break
+            live[rid] = 0
+            waiting.pop(0)
+        assert live, "max_tokens too small for the next request"
+        entries, end = [], []
+        rids = list(live)
+        g.shuffle(rids)
+        for rid in rids:
+            done, n = live[rid], lengths[rid]
+            if len(live) > 1 and g.random() < skip:
+                continue
+            rest = n - done
+            c = min(g.randint(1, 70), rest - tail[rid]) if rest > tail[rid] else 1
+            entries.append((rid, done, c))
+            live[rid] = done + c
+            if live[rid] == n:
+                end.append(rid)
+                del live[rid]
+        if entries:
+            steps.append((entries, end))
+    return steps, max_tokens
+
+
 # ---- replaying a schedule through a runner -----------------------------------------------------
 LENGTHS = {"A": {"a0": 5, "a1": 17, "a2": 33, "a3": 150, "a4": 97, "a5": 64},
            "B": {"b0": 1, "b1": 9, "b2": 40, "b3": 63, "b4": 120, "b5": 201},

@@ -59,6 +59,23 @@ def test_replay_modes(tiny_dirs, name, dtype, mode):
     _compare(got, _reference(tiny_dirs, name, dtype), dtype, f"{name}/{dtype}/{mode}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+def test_replay_random_schedules(tiny_dirs, name, dtype):
+    """Twelve schedules drawn from seeds (``helpers.schedule_random``: pool size, order of requests and of a step's
+    entries, portion lengths, where single tokens begin, requests sitting out), decode-only steps as replayed
+    graphs: every position of every request against the plain implementation, no page left behind."""
+    requests = helpers.requests_for(name)
+    ref = _reference(tiny_dirs, name, dtype)
+    for seed in range(12):
+        steps, max_tokens = helpers.schedule_random(helpers.LENGTHS[name], seed=100 * seed + ord(name))
+        runner = _runner(tiny_dirs, name, dtype, max_tokens, helpers.PAGE_SIZE[name], use_graph=True)
+        got = helpers.run_schedule(runner, requests, steps)
+        assert not runner.cache.live_requests()
+        assert runner.cache.free_pages() == [p.num_pages for p in runner.cache.pools]
+        _compare(got, ref, dtype, f"{name}/{dtype}/random schedule of seed {seed}")
+
+
 def test_cutting_modes_against_each_other(tiny_dirs, capsys):
     """The four ways of cutting compared with each other, not only with the plain implementation (float32,
     config A).  Every kernel computes a row in an order that does not involve other rows; the one thing that
