@@ -337,3 +337,29 @@ def pointer_sequence(vocab: int, n: int, needle: int, needle_at: int, probe: int
         assert needle_at < p < n
         toks[p] = probe
     return toks
+
+
+def random_arrivals(eng, cfg, W, g, seed: int, n_requests: int = 12) -> None:
+    """Requests of drawn lengths (prompts of 1 to 80 tokens, 1 to 40 new ones) are added to ``eng`` between its
+    steps, none to three at a time, until all are done; asserts that every request got the plain implementation's
+    greedy tokens, that ``finished`` came with the last one, and that no page or request is left in the cache."""
+    from tempura_amd.sampling import SamplingParams
+    todo = [(random_tokens(cfg["vocab_size"], g.randint(1, 80), seed=900 + 20 * seed + i), g.randint(1, 40)) for i in range(n_requests)]
+    got, asked = {}, {}
+    steps = 0
+    while todo or eng.has_unfinished():
+        for _ in range(g.choice([0, 0, 1, 2, 3]) if eng.has_unfinished() else 1):
+            if todo:
+                prompt, n = todo.pop()
+                rid = eng.add_request(prompt, SamplingParams(temperature=0.0, max_new_tokens=n, ignore_eos=True))
+                asked[rid] = (prompt, n)
+                got[rid] = []
+        for rid, tok, finished in eng.step():
+            got[rid].append(tok)
+            assert finished == (len(got[rid]) == asked[rid][1])
+        steps += 1
+        assert steps < 3000, "the engine does not come to an end"
+    cache = eng.runner.cache
+    assert cache.free_pages() == [p.num_pages for p in cache.pools] and not cache.live_requests()
+    for rid, (prompt, n) in asked.items():
+        assert got[rid] == plain.greedy_generate(cfg, W, prompt, n), f"request {rid} (prompt of {len(prompt)}, {n} new tokens)"

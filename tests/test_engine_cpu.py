@@ -148,6 +148,17 @@ def test_generate_and_preemption_on_host(tiny_dirs, fill_budget):
     assert tight.stats()["preemptions"] > 0 and tight.runner.cache.free_pages() == [3]
 
 
+def test_requests_arriving_at_random_times_get_the_plain_tokens(tiny_dirs):
+    """Scheduler, cache manager and step function under requests that arrive while others run, into a pool that holds
+    a third of them (the kernel operations replaced by the stand-ins): the plain implementation's greedy tokens."""
+    import random
+    from tempura_amd.engine import Engine
+    cfg, W = tiny_dirs.plain_model("A")
+    eng = Engine(tiny_dirs.path("A"), dtype="float32", device="cpu", page_size=16, kv_pages=14, max_batch_size=4,
+                 max_num_batched_tokens=24, prefill_chunk_size=8)
+    helpers.random_arrivals(eng, cfg, W, random.Random(3), seed=3, n_requests=8)
+
+
 def test_zero_new_tokens_and_a_request_left_out_of_a_step(tiny_dirs):
     from tempura_amd.engine import Engine
     from tempura_amd.sampling import SamplingParams

@@ -155,29 +155,11 @@ def test_requests_arriving_at_random_times_get_the_plain_tokens(tiny_dirs, seed)
     the host, requests finishing at different times, admission with headroom and, where it comes to that,
     preemption.  Every request gets the plain implementation's greedy tokens, and in the end no page is held."""
     import random
-    from tempura_amd.sampling import SamplingParams
     cfg, W = tiny_dirs.plain_model("A")
     g = random.Random(seed)
     eng = _engine(tiny_dirs, "A", kv_pages=g.choice([14, 20, 28]), max_num_batched_tokens=g.choice([24, 48, 96]),
                   prefill_chunk_size=g.choice([8, 16, 40]))
-    todo = [(helpers.random_tokens(256, g.randint(1, 80), seed=900 + 20 * seed + i), g.randint(1, 40)) for i in range(12)]
-    got, asked = {}, {}
-    steps = 0
-    while todo or eng.has_unfinished():
-        for _ in range(g.choice([0, 0, 1, 2, 3]) if eng.has_unfinished() else 1):
-            if todo:
-                prompt, n = todo.pop()
-                rid = eng.add_request(prompt, SamplingParams(temperature=0.0, max_new_tokens=n, ignore_eos=True))
-                asked[rid] = (prompt, n)
-                got[rid] = []
-        for rid, tok, finished in eng.step():
-            got[rid].append(tok)
-            assert finished == (len(got[rid]) == asked[rid][1])
-        steps += 1
-        assert steps < 3000, "the engine does not come to an end"
-    assert eng.runner.cache.free_pages() == [eng.runner.cache.pools[0].num_pages] and not eng.runner.cache.live_requests()
-    for rid, (prompt, n) in asked.items():
-        assert got[rid] == plain.greedy_generate(cfg, W, prompt, n), f"request {rid} (prompt of {len(prompt)}, {n} new tokens)"
+    helpers.random_arrivals(eng, cfg, W, g, seed)
 
 
 def test_temperature_sampling_seeded(tiny_dirs):
