@@ -303,7 +303,9 @@ def test_toy_block_arrangements_with_other_parts_register_build_and_step(tmp_pat
     d = write_random_model(cfg, str(tmp_path / "sandwich"), seed=8, std=0.2, norm_jitter=0.1, dtype="float32")
     assert type(load_config(d)) is toy_parts.ToySandwichConfig
     model = load_model(d, "float32", "cpu")
-    assert model.slots_per_group == [3] and len(model.expected_weights()) == 3 + 4 * 3 + (4 + 3) * 2 + 1
+    # (embedding, head and the last norm's two tensors; q, k, v, o of three layers; a sandwich layer's two plain and
+    # two centred norms (two tensors each) and its feed-forward; the norm of the layer without a feed-forward)
+    assert model.slots_per_group == [3] and len(model.expected_weights()) == 4 + 4 * 3 + (2 + 2 * 2 + 3) * 2 + 1
     _, W = plain.read_model_dir(d)
     runner = ModelRunner(model, 8, 12, max_requests=3)
     reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=20 + i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30}.items())}

@@ -256,6 +256,38 @@ def test_toy_mixer_with_state_in_captured_steps(tmp_path, dtype):
                 seq.append(tok)
 
 
+def test_toy_block_arrangements_and_norm_on_the_gpu(tmp_path):
+    """Registered, built and stepped without a change to the framework: block arrangements of the tests (norms
+    before and after mixer and feed-forward; a layer without a feed-forward) and a norm of the tests (centred,
+    with a shift; also the model's last norm, which then picks the wanted rows itself), around the library's
+    attention and SwiGLU kernels; and greedy generation through the entry point, decode steps as replayed graphs."""
+    import toy_parts
+    from tempura_amd.engine import Engine
+    from tempura_amd.engine.loading import load_model
+    from tempura_amd.engine.runner import ModelRunner
+    from tempura_amd.sampling import SamplingParams
+    from tempura_amd.weights import write_random_model
+    cfg = toy_parts.ToySandwichConfig()
+    d = write_random_model(cfg, str(tmp_path / "sandwich"), seed=8, std=0.2, norm_jitter=0.1, dtype="float32")
+    model = load_model(d, "float32", "cuda:0")
+    _, W = plain.read_model_dir(d)
+    runner = ModelRunner(model, 8, 12, max_requests=3)
+    reqs = {r: helpers.random_tokens(cfg.vocab_size, n, seed=20 + i) for i, (r, n) in enumerate({"p": 21, "q": 9, "r": 30}.items())}
+    steps = [([("p", 0, 6)], []), ([("p", 6, 3), ("q", 0, 8)], []), ([("p", 9, 1), ("q", 8, 1), ("r", 0, 17)], ["q"]),
+             ([("p", 10, 11), ("r", 17, 13)], ["p", "r"])]
+    got = helpers.run_schedule(runner, reqs, steps)
+    for r, t in reqs.items():
+        assert helpers.rel_err(got[r], toy_parts.plain_sandwich_forward(cfg, W, t)) < helpers.TOL["float32"], r
+    eng = Engine(model, dtype="float32", page_size=8, kv_pages=24, max_batch_size=3)
+    prompts = [reqs["q"], reqs["p"][:5]]
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=6))
+    for prompt, out in zip(prompts, outs):
+        seq = list(prompt)
+        for tok in out:         # greedy by the plain implementation, token by token
+            assert tok == int(torch.argmax(toy_parts.plain_sandwich_forward(cfg, W, seq)[-1]))
+            seq.append(tok)
+
+
 def test_toy_routed_ffn_and_learned_position_on_the_gpu(tmp_path):
     """Registered, built and stepped without a change to the framework: a feed-forward with routing and a
     learned position encoding from the tests, beside the library's kernels (rotary windowed attention, SwiGLU),

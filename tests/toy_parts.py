@@ -6,7 +6,9 @@ nothing under tempura_amd/ knows about them.
   encoding that is not rotary (a learned vector per position, added to queries and keys), in layers beside
   the library's own parts (``ToyRoutedForCausalLM``);
 * a block arrangement with other parts than the library's: norms before AND after the mixer and the feed-forward
-  (six named parts), and a second kind of layer that has a mixer and no feed-forward at all (``ToySandwichForCausalLM``);
+  (six named parts), and a second kind of layer that has a mixer and no feed-forward at all; and a norm that is not
+  the library's (the mean taken out, a scale and a shift), at two of those sites and as the model's last norm
+  (``ToySandwichForCausalLM``);
 * a mixer whose pages hold something else than keys and values of heads: ONE compressed vector per token, declared
   by a cache spec of its own, in layers beside the library's attention (``ToyLatentForCausalLM``)."""
 from __future__ import annotations
@@ -18,7 +20,7 @@ from typing import Dict, List
 import torch
 
 from tempura_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, register_architecture
-from tempura_amd.parts import ArrangedBlock, CacheSpec, FeedForward, Mixer, PositionEncoding, StateSpec, WeightInfo, register_part
+from tempura_amd.parts import ArrangedBlock, CacheSpec, FeedForward, Mixer, Norm, PositionEncoding, StateSpec, WeightInfo, register_part
 
 
 class DecaySumMixer(Mixer):
@@ -307,6 +309,35 @@ def plain_toy_forward(cfg: ToyConfig, W: Dict[str, torch.Tensor], tokens: List[i
     return plain.rmsnorm(h, W["toy.norm"], 1e-5) @ W["toy.embed"].T
 
 
+class CentredNorm(Norm):
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * scale + shift, in float32; two tensors."""
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        self.eps = float(spec.params["eps"])
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        return {spec.weights["scale"]: WeightInfo((hidden_size,), "ones"), spec.weights["shift"]: WeightInfo((hidden_size,))}
+
+    def load_weights(self, get):
+        self.scale = self._to_device(get(self.spec.weights["scale"]), torch.float32)
+        self.shift = self._to_device(get(self.spec.weights["shift"]), torch.float32)
+
+    def forward(self, h, rows=None):
+        x = h if rows is None else h.index_select(0, rows.long())
+        x = x - x.mean(dim=-1, keepdim=True)
+        return (x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + self.eps) * self.scale + self.shift).to(self.dtype)
+
+
+register_part("norm", "toy_centred", CentredNorm)
+
+
+def plain_centred_norm(x, scale, shift, eps):
+    x = x - x.mean(dim=-1, keepdim=True)
+    return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps) * scale + shift
+
+
 class SandwichBlock(ArrangedBlock):
     """h += post_mixer_norm(mixer(pre_mixer_norm(h))); h += post_ffn_norm(ffn(pre_ffn_norm(h))): six parts, two of
     them norms that the library's own arrangement does not have.  A part adds its result into the stream it is
@@ -360,17 +391,19 @@ class ToySandwichConfig:
     def build_spec(self) -> ModelSpec:
         rope = PartSpec("rope", {"head_dim": self.head_dim, "theta": 1e4, "scaling": None})
         norm = lambda n: PartSpec("rmsnorm", {"eps": 1e-5}, {"weight": n})
+        centred = lambda n: PartSpec("toy_centred", {"eps": 1e-4}, {"scale": n + ".scale", "shift": n + ".shift"})
         attn = lambda p: PartSpec("attention", {"num_heads": self.num_attention_heads, "num_kv_heads": self.num_key_value_heads,
                                                 "head_dim": self.head_dim, "scale": self.head_dim ** -0.5, "window": None,
                                                 "position": rope}, {"q": f"{p}.q", "k": f"{p}.k", "v": f"{p}.v", "o": f"{p}.o"})
         swiglu = lambda p: PartSpec("swiglu", {"intermediate_size": self.intermediate_size},
                                     {"gate": f"{p}.gate", "up": f"{p}.up", "down": f"{p}.down"})
+        # (the centred norm after the mixer and before the feed-forward of the sandwich layers, and as the last norm)
         sandwich = lambda p: LayerSpec("toy_sandwich", {
-            "pre_mixer_norm": norm(f"{p}.n1"), "mixer": attn(p), "post_mixer_norm": norm(f"{p}.n2"),
-            "pre_ffn_norm": norm(f"{p}.n3"), "ffn": swiglu(p), "post_ffn_norm": norm(f"{p}.n4")})
+            "pre_mixer_norm": norm(f"{p}.n1"), "mixer": attn(p), "post_mixer_norm": centred(f"{p}.n2"),
+            "pre_ffn_norm": centred(f"{p}.n3"), "ffn": swiglu(p), "post_ffn_norm": norm(f"{p}.n4")})
         layers = [sandwich("s.0"), LayerSpec("toy_mixer_only", {"norm": norm("s.1.n1"), "mixer": attn("s.1")}), sandwich("s.2")]
         return ModelSpec(self.architecture, self.hidden_size, self.vocab_size, self.max_position_embeddings, layers,
-                         [LayerCall(0), LayerCall(1), LayerCall(2)], norm("s.norm"),
+                         [LayerCall(0), LayerCall(1), LayerCall(2)], centred("s.norm"),
                          PartSpec("embedding", {}, {"weight": "s.embed"}), PartSpec("lm_head", {"tied": False}, {"weight": "s.head"}))
 
 
@@ -397,10 +430,11 @@ def plain_sandwich_forward(cfg: ToySandwichConfig, W: Dict[str, torch.Tensor], t
         if l == 1:
             h = h + attend(p, plain.rmsnorm(h, W[f"{p}.n1"], 1e-5))
             continue
-        h = h + plain.rmsnorm(attend(p, plain.rmsnorm(h, W[f"{p}.n1"], 1e-5)), W[f"{p}.n2"], 1e-5)
-        y = plain.swiglu_ffn(plain.rmsnorm(h, W[f"{p}.n3"], 1e-5), W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
+        cn = lambda x, n: plain_centred_norm(x, W[n + ".scale"], W[n + ".shift"], 1e-4)
+        h = h + cn(attend(p, plain.rmsnorm(h, W[f"{p}.n1"], 1e-5)), f"{p}.n2")
+        y = plain.swiglu_ffn(cn(h, f"{p}.n3"), W[f"{p}.gate"], W[f"{p}.up"], W[f"{p}.down"])
         h = h + plain.rmsnorm(y, W[f"{p}.n4"], 1e-5)
-    return plain.rmsnorm(h, W["s.norm"], 1e-5) @ W["s.head"].T
+    return plain_centred_norm(h, W["s.norm.scale"], W["s.norm.shift"], 1e-4) @ W["s.head"].T
 
 
 # ---- a mixer with another per-token cache layout -------------------------------------------------------------------
