@@ -219,6 +219,59 @@ __device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s
   }
 }
 
+// The same arithmetic without a branch (one basic block, so that the scheduler may place another instruction
+// stream's MFMAs between these instructions): alpha is computed always and chosen afterwards; where no maximum
+// moved it is exactly 1 and l * 1 + sum is l + sum.
+template <int NQ, bool MASK>
+__device__ inline void attn_softmax_flat(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const int (&qpos)[NQ],
+                                         float (&m)[NQ], float (&l)[NQ], bf16x8_t (&pf)[NQ], float (&alpha)[NQ], bool (&moved)[NQ]) {
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4;
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    float v[8];
+    float mx = -INFINITY;
+    if (MASK) {
+      const int hi = qpos[nq];
+      const int lo = a.window > 0 ? hi - a.window + 1 : 0;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = j0 + 8 * g + 4 * t + r;
+          v[t * 4 + r] = (key <= hi && key >= lo) ? s[nq][t][r] : -INFINITY;
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[t * 4 + r] = s[nq][t][r];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mx = fmaxf(mx, v[i]);
+    mx = quad_rows_max(mx);
+    const float m_new = fmaxf(m[nq], mx * a.scale_log2);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[i] = __builtin_amdgcn_exp2f(fmaf(v[i], a.scale_log2, -m_use));
+      sum += v[i];
+    }
+    u32x4_t pk;
+    pk[0] = pack_bf16(v[0], v[1]);
+    pk[1] = pack_bf16(v[2], v[3]);
+    pk[2] = pack_bf16(v[4], v[5]);
+    pk[3] = pack_bf16(v[6], v[7]);
+    pf[nq] = frag_of(pk);
+    moved[nq] = __builtin_amdgcn_ballot_w64(m_new != m[nq]) != 0;
+    const float shrink = __builtin_amdgcn_exp2f(m[nq] - m_use);
+    alpha[nq] = moved[nq] ? shrink : 1.0f;
+    l[nq] = fmaf(l[nq], alpha[nq], sum);
+    m[nq] = m_new;     // (where nothing moved, m_new is m)
+  }
+}
+
 template <int D, int NQ>
 __device__ inline void attn_pv(const bf16x8_t (&vf)[D / 16], const bf16x8_t (&pf)[NQ], const float (&alpha)[NQ],
                                const bool (&moved)[NQ], f32x4_t (&o)[NQ][D / 16]) {
@@ -562,26 +615,39 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
       if (s + NS < nsteps) pages_of(s + NS);
     }
     const unsigned base = lds0 + stage * STAGE;
-    // the keys of the following stage are multiplied into the next step's scores before this step's
-    // softmax runs on the vector ALU
-    if (s + 1 < nsteps) {
-      bf16x8_t kf[2][D / 32];
-      read_keys(lds0 + nstage * STAGE, kf);
-      attn_scores<D, NQ>(kf, qf, nxt);
-    }
-    // the value fragments travel while the softmax runs
-    u32x4_t vv[D / 16];
-#define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<(dt >> 1) * 2048 + (dt & 1) * 256>(base + vaddr)
-    ATTN_RV(0); ATTN_RV(1); ATTN_RV(2); ATTN_RV(3); ATTN_RV(4); ATTN_RV(5); ATTN_RV(6); ATTN_RV(7);
-#undef ATTN_RV
+    // The keys of the following stage are multiplied into the next step's scores while this step's softmax runs
+    // on the vector ALU: the two are one block of instructions without a branch, and the scheduler is told to
+    // put a few of the softmax's instructions behind each MFMA (a wave issues in order: sixteen MFMAs in a row
+    // would hold the softmax back for as long as they take).
     bf16x8_t pf[NQ];
     float alpha[NQ];
     bool moved[NQ];
+    u32x4_t vv[D / 16];
     const int j0 = first + s * 32;
-    if (j0 + 31 <= qpos_min && (a.window <= 0 || j0 >= last_pos - a.window + 1))
-      attn_softmax<NQ, false>(a, j0, cur, qpos, m, l, pf, alpha, moved);
-    else
-      attn_softmax<NQ, true>(a, j0, cur, qpos, m, l, pf, alpha, moved);
+    const bool plain_step = j0 + 31 <= qpos_min && (a.window <= 0 || j0 >= last_pos - a.window + 1);
+#define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<(dt >> 1) * 2048 + (dt & 1) * 256>(base + vaddr)
+#define ATTN_BODY(NEXT, MASK)                                                                          \
+  {                                                                                                    \
+    bf16x8_t kf[2][D / 32];                                                                            \
+    if (NEXT) read_keys(lds0 + nstage * STAGE, kf);                                                    \
+    ATTN_RV(0); ATTN_RV(1); ATTN_RV(2); ATTN_RV(3); ATTN_RV(4); ATTN_RV(5); ATTN_RV(6); ATTN_RV(7);    \
+    if (NEXT) attn_scores<D, NQ>(kf, qf, nxt);                                                         \
+    attn_softmax_flat<NQ, MASK>(a, j0, cur, qpos, m, l, pf, alpha, moved);                             \
+    if (NEXT) {                                                                                        \
+      _Pragma("unroll") for (int i = 0; i < 4 * NQ * (D / 32); ++i) {                                  \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                             \
+        __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);                                 \
+      }                                                                                                \
+    }                                                                                                  \
+  }
+    constexpr int VALU_PER_MFMA = 6;
+    if (s + 1 < nsteps) {
+      if (plain_step) ATTN_BODY(true, false) else ATTN_BODY(true, true)
+    } else {
+      if (plain_step) ATTN_BODY(false, false) else ATTN_BODY(false, true)
+    }
+#undef ATTN_BODY
+#undef ATTN_RV
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     bf16x8_t vf[D / 16];
 #pragma unroll
