@@ -148,16 +148,18 @@ def test_preemption_by_recompute_keeps_tokens(tiny_dirs):
         assert tight.runner.cache.free_pages() == [11]
 
 
-@pytest.mark.parametrize("seed", [0, 1, 2])
-def test_requests_arriving_at_random_times_get_the_plain_tokens(tiny_dirs, seed):
-    """Twelve requests of drawn lengths (prompts of 1 to 80 tokens, 1 to 40 new ones: the model has 128 positions) arrive while others run, into an
+@pytest.mark.parametrize("name,seed", [("A", 0), ("A", 1), ("A", 2), ("C", 3), ("D", 4), ("E", 5)])
+def test_requests_arriving_at_random_times_get_the_plain_tokens(tiny_dirs, name, seed):
+    """Twelve requests of drawn lengths (prompts of 1 to 80 tokens, 1 to 40 new ones) arrive while others run, into an
     engine whose pool holds a third of them: prompts in portions beside decoding requests, steps queued ahead of
     the host, requests finishing at different times, admission with headroom and, where it comes to that,
-    preemption.  Every request gets the plain implementation's greedy tokens, and in the end no page is held."""
+    preemption; also with a window whose pages go back while a request runs (C) and with pages of 64 (E).  Every
+    request gets the plain implementation's greedy tokens, and in the end no page is held."""
     import random
-    cfg, W = tiny_dirs.plain_model("A")
+    cfg, W = tiny_dirs.plain_model(name)
     g = random.Random(seed)
-    eng = _engine(tiny_dirs, "A", kv_pages=g.choice([14, 20, 28]), max_num_batched_tokens=g.choice([24, 48, 96]),
+    tokens = g.choice([224, 320, 448])
+    eng = _engine(tiny_dirs, name, kv_pages=tokens // helpers.PAGE_SIZE[name], max_num_batched_tokens=g.choice([24, 48, 96]),
                   prefill_chunk_size=g.choice([8, 16, 40]))
     helpers.random_arrivals(eng, cfg, W, g, seed)
 
