@@ -164,6 +164,48 @@ def test_requests_arriving_at_random_times_get_the_plain_tokens(tiny_dirs, name,
     helpers.random_arrivals(eng, cfg, W, g, seed)
 
 
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("D", "bfloat16"), ("C", "bfloat16")])
+def test_four_hundred_requests_with_aborts_leave_nothing_behind(tiny_dirs, name, dtype):
+    """A long run of the whole engine on a pool that holds a handful of requests: 400 requests of drawn lengths and
+    sampling options (greedy, temperature, top-k, top-p, min-p, repetition penalty) arrive in bursts, one in twenty
+    steps aborts a running or waiting request, requests are preempted and recomputed.  No comparison of tokens here
+    (the other tests have it): every token is a token of the vocabulary, the cache manager's invariants hold
+    throughout, every request ends, and in the end no page and no request slot is held."""
+    import random
+    from tempura_amd.sampling import SamplingParams
+    vocab = helpers.CONFIGS[name].vocab_size
+    g = random.Random(7)
+    ps = helpers.PAGE_SIZE[name]
+    eng = _engine(tiny_dirs, name, dtype=dtype, kv_pages=640 // ps, max_batch_size=6, max_num_batched_tokens=64, prefill_chunk_size=24)
+    live, finished, aborted, added, steps = set(), 0, 0, 0, 0
+    while added < 400 or eng.has_unfinished():
+        for _ in range(g.choice([0, 0, 1, 1, 2, 4])):
+            if added < 400:
+                params = SamplingParams(temperature=g.choice([0.0, 0.7, 1.0]), top_k=g.choice([0, 5, 50]), top_p=g.choice([1.0, 0.9]),
+                                        min_p=g.choice([0.0, 0.05]), repeat_penalty=g.choice([1.0, 1.1]), seed=g.randint(0, 99),
+                                        max_new_tokens=g.randint(1, 60), ignore_eos=True)
+                live.add(eng.add_request(helpers.random_tokens(vocab, g.randint(1, 150), seed=added), params))
+                added += 1
+        if live and g.random() < 0.05:
+            rid = g.choice(sorted(live))
+            eng.abort(rid)
+            live.discard(rid)
+            aborted += 1
+        for rid, tok, fin in eng.step():
+            assert 0 <= tok < vocab and rid in live
+            if fin:
+                live.discard(rid)
+                finished += 1
+        steps += 1
+        if steps % 50 == 0:
+            eng.runner.cache.check()
+        assert steps < 20000, "the engine does not come to an end"
+    cache = eng.runner.cache
+    assert not live and finished + aborted == 400 and aborted > 20
+    assert cache.free_pages() == [p.num_pages for p in cache.pools] and not cache.live_requests()
+    assert eng.stats()["preemptions"] > 0 and eng.runner.graph_steps > 500
+
+
 def test_temperature_sampling_seeded(tiny_dirs):
     from tempura_amd.sampling import SamplingParams
     prompts = [helpers.random_tokens(384, n, seed=500 + n) for n in (1, 9, 40)]
