@@ -641,7 +641,20 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     }                                                                                                  \
   }
     constexpr int VALU_PER_MFMA = 6;
-    if (s + 1 < nsteps) {
+    if constexpr (NQ == 1) {
+      // (one query tile a wave, three blocks a CU: the waves of a SIMD fill one another's gaps, and the interleaved
+      // block would cost registers that this variant does not have: 2,048 tokens 68 us either way)
+      if (s + 1 < nsteps) {
+        bf16x8_t kf[2][D / 32];
+        read_keys(lds0 + nstage * STAGE, kf);
+        attn_scores<D, NQ>(kf, qf, nxt);
+      }
+      ATTN_RV(0); ATTN_RV(1); ATTN_RV(2); ATTN_RV(3); ATTN_RV(4); ATTN_RV(5); ATTN_RV(6); ATTN_RV(7);
+      if (plain_step)
+        attn_softmax<NQ, false>(a, j0, cur, qpos, m, l, pf, alpha, moved);
+      else
+        attn_softmax<NQ, true>(a, j0, cur, qpos, m, l, pf, alpha, moved);
+    } else if (s + 1 < nsteps) {
       if (plain_step) ATTN_BODY(true, false) else ATTN_BODY(true, true)
     } else {
       if (plain_step) ATTN_BODY(false, false) else ATTN_BODY(false, true)
