@@ -219,17 +219,18 @@ __device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s
   }
 }
 
-// The same arithmetic without a branch (one basic block, so that the scheduler may place another instruction
-// stream's MFMAs between these instructions): alpha is computed always and chosen afterwards; where no maximum
-// moved it is exactly 1 and l * 1 + sum is l + sum.
+// The same arithmetic without a branch, in two halves (each one basic block, so that the scheduler may place
+// another instruction stream's MFMAs between these instructions).  The first half needs only the scores: the
+// masked values and the new maximum of every column; it runs while the next step's key fragments travel from LDS.
+// The second half is the exponentials and the sums: alpha is computed always and chosen afterwards; where no
+// maximum moved it is exactly 1 and l * 1 + sum is l + sum.
 template <int NQ, bool MASK>
-__device__ inline void attn_softmax_flat(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const int (&qpos)[NQ],
-                                         float (&m)[NQ], float (&l)[NQ], bf16x8_t (&pf)[NQ], float (&alpha)[NQ], bool (&moved)[NQ]) {
+__device__ inline void attn_softmax_max(const AttnArgs& a, int j0, const f32x4_t (&s)[NQ][2], const int (&qpos)[NQ],
+                                        const float (&m)[NQ], float (&v)[NQ][8], float (&m_new)[NQ]) {
   const int lane = threadIdx.x & 63;
   const int g = lane >> 4;
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
-    float v[8];
     float mx = -INFINITY;
     if (MASK) {
       const int hi = qpos[nq];
@@ -239,36 +240,44 @@ __device__ inline void attn_softmax_flat(const AttnArgs& a, int j0, const f32x4_
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = j0 + 8 * g + 4 * t + r;
-          v[t * 4 + r] = (key <= hi && key >= lo) ? s[nq][t][r] : -INFINITY;
+          v[nq][t * 4 + r] = (key <= hi && key >= lo) ? s[nq][t][r] : -INFINITY;
         }
     } else {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[t * 4 + r] = s[nq][t][r];
+        for (int r = 0; r < 4; ++r) v[nq][t * 4 + r] = s[nq][t][r];
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) mx = fmaxf(mx, v[i]);
+    for (int i = 0; i < 8; ++i) mx = fmaxf(mx, v[nq][i]);
     mx = quad_rows_max(mx);
-    const float m_new = fmaxf(m[nq], mx * a.scale_log2);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    m_new[nq] = fmaxf(m[nq], mx * a.scale_log2);
+  }
+}
+
+template <int NQ>
+__device__ inline void attn_softmax_exp(const AttnArgs& a, float (&v)[NQ][8], const float (&m_new)[NQ], float (&m)[NQ],
+                                        float (&l)[NQ], bf16x8_t (&pf)[NQ], float (&alpha)[NQ], bool (&moved)[NQ]) {
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    const float m_use = (m_new[nq] == -INFINITY) ? 0.f : m_new[nq];
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      v[i] = __builtin_amdgcn_exp2f(fmaf(v[i], a.scale_log2, -m_use));
-      sum += v[i];
+      v[nq][i] = __builtin_amdgcn_exp2f(fmaf(v[nq][i], a.scale_log2, -m_use));
+      sum += v[nq][i];
     }
     u32x4_t pk;
-    pk[0] = pack_bf16(v[0], v[1]);
-    pk[1] = pack_bf16(v[2], v[3]);
-    pk[2] = pack_bf16(v[4], v[5]);
-    pk[3] = pack_bf16(v[6], v[7]);
+    pk[0] = pack_bf16(v[nq][0], v[nq][1]);
+    pk[1] = pack_bf16(v[nq][2], v[nq][3]);
+    pk[2] = pack_bf16(v[nq][4], v[nq][5]);
+    pk[3] = pack_bf16(v[nq][6], v[nq][7]);
     pf[nq] = frag_of(pk);
-    moved[nq] = __builtin_amdgcn_ballot_w64(m_new != m[nq]) != 0;
+    moved[nq] = __builtin_amdgcn_ballot_w64(m_new[nq] != m[nq]) != 0;
     const float shrink = __builtin_amdgcn_exp2f(m[nq] - m_use);
     alpha[nq] = moved[nq] ? shrink : 1.0f;
     l[nq] = fmaf(l[nq], alpha[nq], sum);
-    m[nq] = m_new;     // (where nothing moved, m_new is m)
+    m[nq] = m_new[nq];     // (where nothing moved, m_new is m)
   }
 }
 
@@ -616,8 +625,9 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     }
     const unsigned base = lds0 + stage * STAGE;
     // The keys of the following stage are multiplied into the next step's scores while this step's softmax runs
-    // on the vector ALU: the two are one block of instructions without a branch, and the scheduler is told to
-    // put a few of the softmax's instructions behind each MFMA (a wave issues in order: sixteen MFMAs in a row
+    // on the vector ALU: its first half (the maxima) while the key fragments travel from LDS, its second (the
+    // exponentials) as one block of instructions with the score MFMAs, without a branch, and the scheduler is told
+    // to put a few of the softmax's instructions behind each MFMA (a wave issues in order: sixteen MFMAs in a row
     // would hold the softmax back for as long as they take).
     bf16x8_t pf[NQ];
     float alpha[NQ];
@@ -628,11 +638,31 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
 #define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<(dt >> 1) * 2048 + (dt & 1) * 256>(base + vaddr)
 #define ATTN_BODY(NEXT, MASK)                                                                          \
   {                                                                                                    \
-    bf16x8_t kf[2][D / 32];                                                                            \
-    if (NEXT) read_keys(lds0 + nstage * STAGE, kf);                                                    \
+    u32x4_t kk[2][D / 32];                                                                             \
+    if (NEXT) {                                                                                        \
+      _Pragma("unroll") for (int t2 = 0; t2 < 2; ++t2)                                                 \
+        _Pragma("unroll") for (int dk = 0; dk < D / 32; ++dk)                                          \
+          kk[t2][dk] = attn_lds_read<0>(lds0 + nstage * STAGE + kaddr[t2][dk]);                        \
+    }                                                                                                  \
     ATTN_RV(0); ATTN_RV(1); ATTN_RV(2); ATTN_RV(3); ATTN_RV(4); ATTN_RV(5); ATTN_RV(6); ATTN_RV(7);    \
-    if (NEXT) attn_scores<D, NQ>(kf, qf, nxt);                                                         \
-    attn_softmax_flat<NQ, MASK>(a, j0, cur, qpos, m, l, pf, alpha, moved);                             \
+    float v[NQ][8], m_new[NQ];                                                                         \
+    attn_softmax_max<NQ, MASK>(a, j0, cur, qpos, m, v, m_new);                                         \
+    __builtin_amdgcn_sched_barrier(0);                                                                 \
+    if (NEXT) {                                                                                        \
+      /* the key fragments have arrived (the D / 16 value fragments behind them need not) */           \
+      static_assert(D / 16 <= 8, "value fragments of a step");                                         \
+      if constexpr (D == 128) asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");                       \
+      else if constexpr (D == 64) asm volatile("s_waitcnt lgkmcnt(4)" ::: "memory");                   \
+      else asm volatile("s_waitcnt lgkmcnt(2)" ::: "memory");                                          \
+      bf16x8_t kf[2][D / 32];                                                                          \
+      _Pragma("unroll") for (int t2 = 0; t2 < 2; ++t2)                                                 \
+        _Pragma("unroll") for (int dk = 0; dk < D / 32; ++dk) {                                        \
+          asm volatile("" : "+v"(kk[t2][dk]));                                                         \
+          kf[t2][dk] = frag_of(kk[t2][dk]);                                                            \
+        }                                                                                              \
+      attn_scores<D, NQ>(kf, qf, nxt);                                                                 \
+    }                                                                                                  \
+    attn_softmax_exp<NQ>(a, v, m_new, m, l, pf, alpha, moved);                                         \
     if (NEXT) {                                                                                        \
       _Pragma("unroll") for (int i = 0; i < 4 * NQ * (D / 32); ++i) {                                  \
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                             \
