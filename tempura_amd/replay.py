@@ -40,6 +40,7 @@ def main(argv=None) -> int:
         ap.error("--page-size must divide 64")
 
     import torch
+    from .cache import PagesExhausted
     from .engine.loading import load_model
     from .engine.runner import ModelRunner, StepEntry
     from .kernels import ops
@@ -60,16 +61,24 @@ def main(argv=None) -> int:
         line = line.strip()
         if not line:
             continue
-        rec = json.loads(line)
-        step = rec["step"]
-        entries = []
-        for e in rec.get("entries", []):
-            rid = e["id"]
-            if not runner.has_request(rid):
-                runner.add_request(rid)
-            entries.append(StepEntry(rid, [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+        # (a line that cannot be run ends the replay with one line on standard error and status 2; the steps
+        # before it have been written)
+        rec = None
+        try:
+            rec = json.loads(line)
+            step = rec["step"]
+            entries = []
+            for e in rec.get("entries", []):
+                rid = e["id"]
+                if not runner.has_request(rid):
+                    runner.add_request(rid)
+                entries.append(StepEntry(rid, [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+            logits = runner.step(entries) if entries else None
+        except (ValueError, KeyError, TypeError, PagesExhausted) as err:
+            what = f"step {rec['step']}" if isinstance(rec, dict) and "step" in rec else f"line {line[:60]!r}"
+            print(f"trace_run: {what}: {type(err).__name__}: {err}", file=sys.stderr)
+            return 2
         if entries:
-            logits = runner.step(entries)
             if logits.shape[0] > 0:
                 arr = logits.detach().to("cpu", torch.float32).numpy().astype("<f4", copy=False)
                 tmp = os.path.join(args.out, f".{step}.f32.tmp")

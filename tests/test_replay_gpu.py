@@ -306,6 +306,28 @@ def test_window_layers_give_pages_back(tiny_dirs):
     runner.end_request("x")
 
 
+def test_trace_run_says_what_is_wrong_with_a_step(tiny_dirs, tmp_path):
+    """A step that cannot be run (a token outside the vocabulary, a wanted place outside the entry, more tokens than
+    the pool holds, a line that is no JSON) ends the replay with status 2 and one line that names the step and the
+    fault; the steps before it are done and written."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    good = json.dumps({"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []})
+    bad = {"token id 999": json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [7, 999], "want": [1]}], "end": []}),
+           "wanted place 4": json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [7, 9], "want": [4]}], "end": []}),
+           "PagesExhausted": json.dumps({"step": 1, "entries": [{"id": "b", "tokens": [1] * 100, "want": []}], "end": []}),
+           "JSONDecodeError": "step one"}
+    for marker, line in bad.items():
+        out_dir = tmp_path / marker.replace(" ", "_")
+        p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", tiny_dirs.path("A", "float32"),
+                            "--dtype", "float32", "--out", str(out_dir), "--max-tokens", "64"],
+                           input=good + "\n" + line + "\n", capture_output=True, text=True, timeout=600)
+        assert p.returncode == 2, (marker, p.returncode, p.stderr[-500:])
+        said = [l for l in p.stderr.splitlines() if l.startswith("trace_run:")]
+        assert len(said) == 1 and marker in said[0] and "Traceback" not in p.stderr, (marker, p.stderr[-500:])
+        assert ("step 1" in said[0]) == (marker != "JSONDecodeError")
+        assert p.stdout.splitlines() == ["done 0"] and (out_dir / "0.f32").stat().st_size == 2 * 256 * 4
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(tiny_dirs, tmp_path, dtype):
     """bin/trace_run as a user runs it: JSON steps on standard input, logits files out."""
