@@ -246,11 +246,22 @@ def main(argv=None) -> int:
             return int(e.code or 0)
         return 0
     args = ap.parse_args(argv)
+    # what is wrong with a folder, a configuration, a checkpoint or the machine is one line and status 2
+    # (TEMPURA_TRACEBACK=1 shows where it was raised)
+    import os
+    from .cache import PagesExhausted
+    from .config import ConfigError
     from .engine.loading import NoDeviceError
+    from .weights import SafetensorsError, WeightsError
     try:
         return args.fn(args)
     except NoDeviceError as e:
         print(f"tempura: {e}", file=sys.stderr)
+        return 2
+    except (ConfigError, WeightsError, SafetensorsError, PagesExhausted) as e:
+        if os.environ.get("TEMPURA_TRACEBACK"):
+            raise
+        print(f"tempura: {type(e).__name__}: {e}", file=sys.stderr)
         return 2
 
 

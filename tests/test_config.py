@@ -115,3 +115,20 @@ def test_presets_match_published_sizes():
     assert abs(c.num_parameters() - 8.03e9) < 0.01e9
     assert c.kv_bytes_per_token(2) == 128 * 1024           # 128 KiB per token (/root/reference/AGENTS.md:396-397)
     assert abs(PRESETS["llama-3.1-70b"].num_parameters() - 70.55e9) < 0.05e9
+
+
+def test_the_command_line_says_what_is_wrong_in_one_line(tmp_path, capsys, monkeypatch):
+    """A folder without config.json, an architecture nobody registered: one line on standard error that names
+    the fault, status 2, no traceback (TEMPURA_TRACEBACK=1 raises instead)."""
+    from tempura_amd.cli import main
+    assert main(["inspect", str(tmp_path / "nothing")]) == 2
+    assert capsys.readouterr().err.startswith("tempura: ConfigError: cannot read")
+    odd = tmp_path / "odd"
+    odd.mkdir()
+    (odd / "config.json").write_text('{"architectures": ["NopeForCausalLM"]}')
+    assert main(["inspect", str(odd)]) == 2
+    err = capsys.readouterr().err
+    assert err.startswith("tempura: ConfigError: unknown architecture 'NopeForCausalLM'") and "Traceback" not in err
+    monkeypatch.setenv("TEMPURA_TRACEBACK", "1")
+    with pytest.raises(ConfigError):
+        main(["inspect", str(odd)])
